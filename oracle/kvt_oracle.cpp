@@ -1,0 +1,1296 @@
+// TEST INFRASTRUCTURE -- CPU oracle. NOT part of the product library.
+//
+// A CPU restatement of the reference's KV-transfer hot path: ParseBlock (block
+// table -> byte ranges), merge/validate of the range lists, and the
+// "memcpy per range" pack / unpack that the reference's copy kernels perform.
+// Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py load
+// this file's shared object; the product (llumnix-kv_amd/csrc) never does.
+//
+// Every function cites the reference code it restates (paths relative to the
+// reference checkout, kvtransfer/...). All arithmetic is unsigned 64-bit unless
+// the reference computes a term in 32 bits, in which case the 32-bit product is
+// kept (noted where it happens).
+//
+// Parity status of each part (what pins it):
+//   * every parser:  compared range-for-range against the compiled reference
+//     (oracle/_ref, built from the reference's own sources) on randomized and
+//     config-shaped inputs (tests/test_oracle_vs_ref.py), against the golden
+//     vectors committed under tests/golden/ (written by the compiled reference),
+//     and against the known-answer numbers of the reference's own tests
+//     (tests/test_oracle_known_answers.py).
+//   * valid-rank selection / dispatch: known answers of the reference tests.
+//   * merge: known answers of the reference tests (incl. overlapping prefix).
+//   * pack / unpack: brute-force byte model in numpy + round-trip invariants.
+//   * HND->NHD transposing pack: no reference function exists; pinned by the
+//     textbook permutation in numpy (einsum/transpose) and round trip.
+//   * bf16->fp8: all 65536 bit patterns against torch's float8_e4m3fn cast
+//     (finite values) and the saturating rule of the reference kernel.
+#include <algorithm>
+#include <atomic>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <stdexcept>
+#include <thread>
+#include <vector>
+
+#include "kvt_types.h"
+
+namespace {
+
+typedef uint64_t u64;
+typedef uint32_t u32;
+typedef std::vector<kvt_ipc_block> Runs;
+typedef std::vector<u32> Ids;
+
+struct Bounds {  // parse_block_common.h:19-24
+  u64 src_cap, dst_cap, scale;
+};
+
+// parse_block_common.cpp:9-30 (checked_layer_capacity)
+u64 layer_capacity(const kvt_worker_info& w, u64 idx) {
+  if (idx >= w.n_tensors || w.layer_num_blocks == 0)
+    throw std::out_of_range("capacity metadata mismatch");
+  const u64 b = w.block_sizes[idx];
+  if (b > std::numeric_limits<u64>::max() / w.layer_num_blocks)
+    throw std::overflow_error("capacity overflow");
+  return b * w.layer_num_blocks;
+}
+
+// parse_block_common.cpp:32-41 (make_ipc_block_bounds)
+Bounds make_bounds(const kvt_worker_info& s, const kvt_worker_info& d, u64 idx,
+                   const kvt_parse_opts& o) {
+  Bounds b;
+  b.src_cap = layer_capacity(s, idx);
+  b.dst_cap = layer_capacity(d, idx);
+  b.scale = o.bf16_to_fp8 ? 2 : 1;
+  return b;
+}
+
+// parse_block_common.h:31-68 (append_ipc_block_checked)
+void emit(Runs& out, const Bounds& b, u64 so, u64 dof, u64 len) {
+  const u64 M = std::numeric_limits<u64>::max();
+  const bool ovf = b.scale == 0 || len > M / b.scale;
+  const u64 eff = ovf ? M : len * b.scale;
+  const bool bad_src = len == 0 || ovf || so > b.src_cap || eff > b.src_cap - so;
+  const bool bad_dst = len == 0 || dof > b.dst_cap || len > b.dst_cap - dof;
+  if (bad_src || bad_dst) throw std::out_of_range("range validation failed");
+  out.push_back(kvt_ipc_block{so, dof, len});
+}
+
+u32 at(const Ids& v, u64 i) {  // std::vector::at
+  if (i >= v.size()) throw std::out_of_range("block index");
+  return v[i];
+}
+
+struct Task {
+  u32 seen, fresh;
+  bool last;
+  std::vector<Ids> src, dst;
+};
+
+const Ids& grp(const std::vector<Ids>& g, u64 i) {
+  if (i >= g.size()) throw std::out_of_range("block group");
+  return g[i];
+}
+
+// parse_block_common.cpp:43-79 (do_parse_block_send_p_eq_d). Always group 0.
+void walk_same(u64 B, u64 T, const Task& t, const Bounds& b, Runs& out) {
+  const u32 ntpb = static_cast<u32>(B / T);
+  u32 pos = t.seen, rem = t.fresh;
+  const Ids& sb = grp(t.src, 0);  // the reference indexes [0] unchecked; a task always has >=1 group
+  const Ids& db = grp(t.dst, 0);
+  while (rem > 0) {
+    const u32 bi = pos / ntpb, ti = pos % ntpb;
+    const u64 so = static_cast<u64>(at(sb, bi)) * B + static_cast<u64>(ti) * T;
+    const u32 k = std::min(ntpb - ti, rem);
+    const u64 dof = static_cast<u64>(at(db, bi)) * B + static_cast<u64>(ti) * T;
+    emit(out, b, so, dof, static_cast<u64>(k) * T);
+    pos += k;
+    rem -= k;
+  }
+}
+
+// parse_block_common.cpp:81-129 (parse_block_send_gt)
+void walk_tokens_gt(u64 pT, u64 pK, u64 dT, u32 ntpb, u64 goff, const Ids& pb, const Ids& db,
+                    u32 pos, u32 rem, const Bounds& b, bool swap, bool fp8, Runs& out) {
+  const u64 pB = pT * ntpb, dB = dT * ntpb;
+  if (fp8) pK /= 2;
+  while (rem > 0) {
+    const u32 bi = pos / ntpb, t0 = pos % ntpb;
+    const u64 po = static_cast<u64>(at(pb, bi)) * pB;
+    const u64 dof = static_cast<u64>(at(db, bi)) * dB;
+    const u32 k = std::min(ntpb - t0, rem);
+    for (u32 i = 0; i < k; ++i) {
+      const u32 ti = t0 + i;
+      const u64 pk = po + static_cast<u64>(ti) * pT;
+      const u64 dk = dof + static_cast<u64>(ti) * dT + goff * pK;
+      emit(out, b, swap ? dk : pk, swap ? pk : dk, pK);
+    }
+    pos += k;
+    rem -= k;
+  }
+}
+
+// parse_block_common.cpp:131-147 (emit_zero_fill_segments)
+void zero_fill(u64 zsrc, u64 dof, u64 len, u64 max_seg, const Bounds& b, Runs& out) {
+  u64 done = 0;
+  while (done < len) {
+    const u64 seg = std::min(max_seg, len - done);
+    emit(out, b, zsrc, dof + done, seg);
+    done += seg;
+  }
+}
+
+u32 popcount16(u32 m) { return static_cast<u32>(__builtin_popcount(m & 0xFFFFu)); }
+
+// ---------------------------------------------------------------- RAGGED (shape 1)
+// parse_block_ragged.cpp:29-60
+void ragged_peqd(const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+                 const Task& t, std::vector<Runs>& out) {
+  out.resize(s.n_tensors);
+  const Bounds b = make_bounds(s, d, 0, o);
+  walk_same(s.block_sizes[0], s.token_sizes[0], t, b, out[0]);
+}
+
+// parse_block_ragged.cpp:63-97
+void ragged_pgtd_dpsk(const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+                      const Task& t, std::vector<Runs>& out) {
+  if (s.worker_tp_rank != 0) return;
+  out.resize(s.n_tensors);
+  const Bounds b = make_bounds(s, d, 0, o);
+  walk_same(s.block_sizes[0], s.token_sizes[0], t, b, out[0]);
+}
+
+// parse_block_ragged.cpp:101-175 (do_parse_block_send_internal). `p` is the
+// side with the larger TP (smaller per-rank token row).
+void ragged_split(const kvt_worker_info& p, u32 p_tp, const Ids& pb, const kvt_worker_info& d,
+                  u32 d_tp, const Ids& db, u32 pos, u32 rem, const Bounds& b, bool swap,
+                  const kvt_parse_opts& o, std::vector<Runs>& out) {
+  if (p.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pB = p.block_sizes[0], pT = p.token_sizes[0], dT = d.token_sizes[0];
+  out.resize(p.n_tensors);
+  Runs& r = out[0];
+  const u32 group_n = p_tp / d_tp;
+  const u32 goff = p.worker_tp_rank % group_n;
+  const u64 pK = pT / 2, dK = dT / 2;
+  const u32 ntpb = static_cast<u32>(pB / pT);
+  const size_t n0 = r.size();
+  walk_tokens_gt(pT, pK, dT, ntpb, goff, pb, db, pos, rem, b, swap, o.bf16_to_fp8 != 0, r);
+  const size_t n1 = r.size();
+  for (size_t i = n0; i < n1; ++i) {
+    const kvt_ipc_block k = r[i];
+    emit(r, b, k.src_offset + (swap ? dK : pK), k.dst_offset + (swap ? pK : dK), pK);
+  }
+}
+
+// parse_block_ragged.cpp:178-196
+void ragged_pgtd(const kvt_worker_info& s, const kvt_worker_info& d, u32 kvt_tp_size,
+                 const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  const Bounds b = make_bounds(s, d, 0, o);
+  ragged_split(s, kvt_tp_size, grp(t.src, 0), d, d.engine_tp_size, grp(t.dst, 0), t.seen, t.fresh,
+               b, false, o, out);
+}
+
+// parse_block_ragged.cpp:199-217
+void ragged_pltd(const kvt_worker_info& s, const kvt_worker_info& d, u32 kvt_tp_size,
+                 const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  const Bounds b = make_bounds(s, d, 0, o);
+  ragged_split(d, d.engine_tp_size, grp(t.dst, 0), s, kvt_tp_size, grp(t.src, 0), t.seen, t.fresh,
+               b, true, o, out);
+}
+
+// ---------------------------------------------------------------- FLASH (shape 2)
+// parse_block_flash.cpp:10-62
+void flash_peqd(const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+                const Task& t, std::vector<Runs>& out) {
+  if (s.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 kT = s.token_sizes[0] / 2, kB = s.block_sizes[0] / 2;
+  const u64 s_shift = kB * s.layer_num_blocks, d_shift = kB * d.layer_num_blocks;
+  out.resize(s.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  const size_t n0 = r.size();
+  walk_same(kB, kT, t, b, r);
+  const size_t n1 = r.size();
+  for (size_t i = n0; i < n1; ++i) {
+    const kvt_ipc_block k = r[i];
+    emit(r, b, k.src_offset + s_shift, k.dst_offset + d_shift, k.length);
+  }
+}
+
+// parse_block_flash.cpp:66-130
+void flash_pgtd(const kvt_worker_info& p, const kvt_worker_info& d, u32 valid, u32 kvt_tp_rank,
+                const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  if (!((valid >> p.worker_tp_rank) & 1u)) return;
+  const u32 group_n = popcount16(valid) / d.engine_tp_size;
+  const u32 goff = kvt_tp_rank % group_n;
+  if (p.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pT = p.token_sizes[0], dT = d.token_sizes[0], pB = p.block_sizes[0];
+  const u64 pK = pT / 2, dK = dT / 2;
+  const u32 ntpb = static_cast<u32>(pB / pT);
+  out.resize(p.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(p, d, 0, o);
+  const size_t n0 = r.size();
+  walk_tokens_gt(pK, pK, dK, ntpb, goff, grp(t.src, 0), grp(t.dst, 0), t.seen, t.fresh, b, false,
+                 o.bf16_to_fp8 != 0, r);
+  const size_t n1 = r.size();
+  const u64 ps = static_cast<u64>(ntpb) * pK * p.layer_num_blocks;
+  const u64 ds = static_cast<u64>(ntpb) * dK * d.layer_num_blocks;
+  for (size_t i = n0; i < n1; ++i) {
+    const kvt_ipc_block k = r[i];
+    emit(r, b, k.src_offset + ps, k.dst_offset + ds, k.length);
+  }
+}
+
+// ---------------------------------------------------------------- DPSK V3.2 (shape 4)
+// parse_block_dpsk.cpp:102-143
+void dpsk_peqd(const kvt_worker_info& s, const kvt_worker_info& d, u32 valid,
+               const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  if (!((valid >> s.worker_tp_rank) & 1u)) return;
+  out.resize(s.n_tensors);
+  for (u32 i = 0; i < s.n_tensors; ++i) {
+    const Bounds b = make_bounds(s, d, i, o);
+    walk_same(s.block_sizes[i], s.token_sizes[i], t, b, out[i]);
+  }
+}
+
+// parse_block_dpsk.cpp:16-96 (do_multi_tensor_parse_block_send)
+void dpsk_split(const kvt_worker_info& p, u32 p_tp, const Ids& pb, const kvt_worker_info& d,
+                u32 d_tp, const Ids& db, u32 pos, u32 rem, const kvt_worker_info& real_src,
+                const kvt_worker_info& real_dst, bool swap, const kvt_parse_opts& o,
+                std::vector<Runs>& out) {
+  out.resize(p.n_tensors);
+  for (u32 c = 0; c < p.n_tensors; ++c) {
+    if (c >= d.n_tensors) throw std::out_of_range("tensor index");
+    const u64 pB = p.block_sizes[c], pT = p.token_sizes[c], dT = d.token_sizes[c];
+    Runs& r = out[c];
+    const Bounds b = make_bounds(real_src, real_dst, c, o);
+    const u32 group_n = p_tp / d_tp;
+    const u32 goff = p.worker_tp_rank % group_n;
+    const u64 pK = pT / 2, dK = dT / 2;
+    const u32 ntpb = static_cast<u32>(pB / pT);
+    const size_t n0 = r.size();
+    walk_tokens_gt(pT, pK, dT, ntpb, goff, pb, db, pos, rem, b, swap, o.bf16_to_fp8 != 0, r);
+    const size_t n1 = r.size();
+    for (size_t i = n0; i < n1; ++i) {
+      const kvt_ipc_block k = r[i];
+      emit(r, b, k.src_offset + (swap ? dK : pK), k.dst_offset + (swap ? pK : dK), pK);
+    }
+  }
+}
+
+bool same_token_sizes(const kvt_worker_info& a, const kvt_worker_info& b) {
+  if (a.n_tensors != b.n_tensors) return false;
+  for (u32 i = 0; i < a.n_tensors; ++i)
+    if (a.token_sizes[i] != b.token_sizes[i]) return false;
+  return true;
+}
+
+// parse_block_dpsk.cpp:149-192
+void dpsk_pgtd(const kvt_worker_info& p, const kvt_worker_info& d, u32 kvt_tp_size,
+               const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  if (same_token_sizes(p, d)) {
+    if (p.worker_tp_rank != 0) return;
+    out.resize(p.n_tensors);
+    for (u32 i = 0; i < p.n_tensors; ++i) {
+      const Bounds b = make_bounds(p, d, i, o);
+      walk_same(p.block_sizes[i], p.token_sizes[i], t, b, out[i]);
+    }
+    return;
+  }
+  dpsk_split(p, kvt_tp_size, grp(t.src, 0), d, d.engine_tp_size, grp(t.dst, 0), t.seen, t.fresh,
+             p, d, false, o, out);
+}
+
+// parse_block_dpsk.cpp:198-214
+void dpsk_pltd(const kvt_worker_info& p, const kvt_worker_info& d, u32 kvt_tp_size,
+               const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  dpsk_split(d, d.engine_tp_size, grp(t.dst, 0), p, kvt_tp_size, grp(t.src, 0), t.seen, t.fresh,
+             p, d, true, o, out);
+}
+
+// ---------------------------------------------------------------- FLASHINFER HND (shape 5)
+// parse_block_flashinfer.cpp:15-72 (parse_flashinfer_HND_block)
+void hnd_walk(u64 pT, u64 pB, u64 dB, u32 ntpb, const Ids& sb, const Ids& db, u32 pos, u32 rem,
+              u32 group_off, int heads, const Bounds& b, bool swap, Runs& out) {
+  const u64 hd = pT / 2 / static_cast<u64>(heads);
+  const u64 p_hs = static_cast<u64>(ntpb) * hd, d_hs = p_hs;
+  const u64 p_half = pB / 2, d_half = dB / 2;
+  const u64 per_group = static_cast<u64>(heads) * d_hs;
+  while (rem > 0) {
+    const u32 bi = pos / ntpb, ti = pos % ntpb;
+    const u64 po = static_cast<u64>(at(sb, bi)) * pB;
+    const u64 dof = static_cast<u64>(at(db, bi)) * dB;
+    const u32 k = std::min(ntpb - ti, rem);
+    const u64 len = static_cast<u64>(k) * hd;
+    for (int h = 0; h < heads; ++h) {
+      const u64 pk = po + static_cast<u64>(h) * p_hs + static_cast<u64>(ti) * hd;
+      const u64 pv = pk + p_half;
+      const u64 dk = dof + group_off * per_group + static_cast<u64>(h) * d_hs +
+                     static_cast<u64>(ti) * hd;
+      const u64 dv = dk + d_half;
+      emit(out, b, swap ? dk : pk, swap ? pk : dk, len);
+      emit(out, b, swap ? dv : pv, swap ? pv : dv, len);
+    }
+    pos += k;
+    rem -= k;
+  }
+}
+
+// parse_block_flashinfer.cpp:275-278 / :337-340
+int fi_heads_per_rank(const kvt_worker_info& p) {
+  if (p.num_kv_heads > 0 && static_cast<u32>(p.num_kv_heads) >= p.engine_tp_size)
+    return p.num_kv_heads / static_cast<int>(p.engine_tp_size);
+  return std::max(1, p.num_kv_heads);
+}
+
+// parse_block_flashinfer.cpp:241-298 (P==D) and :304-364 (P>D)
+void flashinfer_any(const kvt_worker_info& p, const kvt_worker_info& d, u32 valid, u32 kvt_tp_rank,
+                    bool gt, const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  u32 group_off = 0;
+  if (gt) {
+    if (!((valid >> p.worker_tp_rank) & 1u)) return;
+    const u32 group_n = popcount16(valid) / d.engine_tp_size;
+    group_off = kvt_tp_rank % group_n;
+  }
+  if (p.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pT = p.token_sizes[0], pB = p.block_sizes[0], dB = d.block_sizes[0];
+  const u32 ntpb = static_cast<u32>(pB / pT);
+  const Ids& sb = grp(t.src, 0);
+  const Ids& db = grp(t.dst, 0);
+  const int heads = fi_heads_per_rank(p);
+  out.resize(1);
+  const Bounds b = make_bounds(p, d, 0, o);
+  hnd_walk(pT, pB, dB, ntpb, sb, db, t.seen, t.fresh, group_off, heads, b, false, out[0]);
+}
+
+// ---------------------------------------------------------------- hybrid pages (shapes 3, 6, 7)
+// parse_block_qwen3_next.cpp:15-84 (do_parse_block_aligned_send)
+void pages_walk(u64 B, const Task& t, const Ids& sb, const Ids& db, u32 ntpb, const Bounds& b,
+                Runs& out) {
+  u32 pos = t.seen, rem = t.fresh;
+  while (rem > 0) {
+    const u32 bi = pos / ntpb, ti = pos % ntpb;
+    const u64 po = static_cast<u64>(at(sb, bi)) * B;
+    const u64 dof = static_cast<u64>(at(db, bi)) * B;
+    const u32 k = std::min(ntpb - ti, rem);
+    u64 len = 0;
+    if (k != ntpb) {
+      if (t.last) len = B;
+      else if (ti == 0) len = 0;
+      else len = (ti + k == ntpb) ? B : 0;
+    } else {
+      len = B;
+    }
+    if (len > 0) emit(out, b, po, dof, len);
+    pos += k;
+    rem -= k;
+  }
+  if (t.last) {
+    const u64 next = (static_cast<u64>(pos) + ntpb - 1) / ntpb;
+    for (u64 i = next; i < sb.size(); ++i)
+      emit(out, b, static_cast<u64>(at(sb, i)) * B, static_cast<u64>(at(db, i)) * B, B);
+  }
+}
+
+// parse_block_qwen3_next.cpp:416-436 and :505-530 (whole state pages, P==D)
+void state_pages_same(u64 B, u64 first_group, u64 n_groups, const Task& t, const Bounds& b,
+                      Runs& out) {
+  for (u64 g = 0; g < n_groups; ++g) {
+    const Ids& sg = grp(t.src, first_group + g);
+    const Ids& dg = grp(t.dst, first_group + g);
+    for (size_t i = 0; i < sg.size(); ++i)
+      emit(out, b, static_cast<u64>(sg[i]) * B, static_cast<u64>(at(dg, i)) * B, B);
+  }
+}
+
+u64 shape_at(const u64* v, u32 n, u32 i) {
+  if (i >= n) throw std::out_of_range("state shape");
+  return v[i];
+}
+
+// parse_block_qwen3_next.cpp:440-502 (parse_hybrid_gdn_block_send_p_gt_d)
+void gdn_pgtd(u64 pB, u64 dB, u64 n_gdn, u32 gn, u32 goff, const kvt_worker_info& s, const Task& t,
+              const Bounds& b, Runs& out) {
+  const u64 e = s.gdn_conv_elem_size;
+  const u64 rows = shape_at(s.conv_state_shape, s.n_conv_state_shape, 1);
+  const u64 p_row = shape_at(s.conv_state_shape, s.n_conv_state_shape, 2) * e;
+  const u64 p_conv = rows * p_row;
+  const u64 p_ssm = shape_at(s.ssm_state_shape, s.n_ssm_state_shape, 1) *
+                    shape_at(s.ssm_state_shape, s.n_ssm_state_shape, 2) *
+                    shape_at(s.ssm_state_shape, s.n_ssm_state_shape, 3) * s.gdn_ssm_elem_size;
+  const u64 d_row = gn * p_row;
+  for (u64 g = 0; g < n_gdn; ++g) {
+    const Ids& sg = grp(t.src, g);
+    const Ids& dg = grp(t.dst, g);
+    for (size_t i = 0; i < sg.size(); ++i) {
+      const u64 po = static_cast<u64>(sg[i]) * pB;
+      const u64 dof = static_cast<u64>(at(dg, i)) * dB;
+      for (u64 r = 0; r < rows; ++r) {
+        u64 inner = 0;
+        for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+          const u64 step = s.gdn_conv_channel_dims[c] * e;
+          emit(out, b, po + r * p_row + inner, dof + r * d_row + gn * inner + goff * step, step);
+          inner += step;
+        }
+      }
+      emit(out, b, po + p_conv, dof + gn * p_conv + goff * p_ssm, p_ssm);
+    }
+  }
+}
+
+// parse_block_qwen3_next.cpp:589-664 (parse_hybrid_gdn_block_send_p_lt_d)
+void gdn_pltd(u64 pB, u64 dB, u64 n_gdn, u32 gn, u32 goff, const kvt_worker_info& s, const Task& t,
+              const Bounds& b, Runs& out) {
+  const u64 e = s.gdn_conv_elem_size;
+  const u64 rows = shape_at(s.conv_state_shape, s.n_conv_state_shape, 1);
+  const u64 p_row = shape_at(s.conv_state_shape, s.n_conv_state_shape, 2) * e;
+  const u64 p_conv = rows * p_row;
+  const u64 p_ssm = shape_at(s.ssm_state_shape, s.n_ssm_state_shape, 1) *
+                    shape_at(s.ssm_state_shape, s.n_ssm_state_shape, 2) *
+                    shape_at(s.ssm_state_shape, s.n_ssm_state_shape, 3) * s.gdn_ssm_elem_size;
+  const u64 d_row = p_row / gn;
+  const u64 d_conv = rows * d_row;
+  const u64 d_ssm = p_ssm / gn;
+  for (u64 g = 0; g < n_gdn; ++g) {
+    const Ids& sg = grp(t.src, g);
+    const Ids& dg = grp(t.dst, g);
+    for (size_t i = 0; i < sg.size(); ++i) {
+      const u64 po = static_cast<u64>(sg[i]) * pB;
+      const u64 dof = static_cast<u64>(at(dg, i)) * dB;
+      for (u64 r = 0; r < rows; ++r) {
+        u64 pin = 0, din = 0;
+        for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+          const u64 ps = s.gdn_conv_channel_dims[c] * e;
+          const u64 ds = ps / gn;
+          emit(out, b, po + r * p_row + pin + goff * ds, dof + r * d_row + din, ds);
+          pin += ps;
+          din += ds;
+        }
+      }
+      emit(out, b, po + p_conv + goff * d_ssm, dof + d_conv, d_ssm);
+    }
+  }
+}
+
+// parse_block_qwen3_next.cpp:532-582 (P>D) and :669-711 (P<D): replicated
+// short-conv (PLE) state; for P>D only the first rank of a subgroup sends.
+void ple_split(u64 pB, u64 dB, bool gt, u32 goff, const kvt_worker_info& s, const Task& t,
+               const Bounds& b, Runs& out) {
+  if (s.num_ple_layers == 0) return;
+  if (gt && goff != 0) return;
+  const u64 sz = shape_at(s.ple_conv_state_shape, s.n_ple_conv_state_shape, 1) *
+                 shape_at(s.ple_conv_state_shape, s.n_ple_conv_state_shape, 2) *
+                 s.ple_conv_elem_size;
+  for (u64 i = 0; i < s.num_ple_layers; ++i) {
+    const Ids& sg = grp(t.src, s.ple_block_group + i);
+    const Ids& dg = grp(t.dst, s.ple_block_group + i);
+    for (size_t j = 0; j < sg.size(); ++j)
+      emit(out, b, static_cast<u64>(sg[j]) * pB, static_cast<u64>(at(dg, j)) * dB, sz);
+  }
+}
+
+// parse_block_qwen3_next.cpp:376-413 (parse_hybrid_indexer_block). The token
+// term and the length are 32-bit products in the reference (uint32 * uint32).
+void indexer_walk(u64 pB, u64 dB, u32 pos, u32 rem, const Ids& sb, const Ids& db, u32 pn, u32 dn,
+                  u32 tok, const Bounds& b, Runs& out) {
+  while (rem > 0) {
+    const u32 sbi = pos / pn, sti = pos % pn, dbi = pos / dn, dti = pos % dn;
+    const u32 k = std::min(std::min(pn - sti, dn - dti), rem);
+    const u64 so = static_cast<u64>(at(sb, sbi)) * pB + static_cast<u32>(sti * tok);
+    const u64 dof = static_cast<u64>(at(db, dbi)) * dB + static_cast<u32>(dti * tok);
+    const u32 len = k * tok;
+    emit(out, b, so, dof, len);
+    pos += k;
+    rem -= k;
+  }
+}
+
+// parse_block_qwen3_next.cpp:108-248 (parse_hybrid_attn_block)
+void hybrid_attn_walk(u32 s_ntpb, u32 d_ntpb, u64 pT, u64 dT, u64 pB, u64 dB, const Ids& sb,
+                      const Ids& db, u32 pos, u32 rem, u32 goff, u32 s_kb, u32 d_kb, u32 pack_in,
+                      const Bounds& b, bool swap, Runs& out) {
+  const u64 p_kbs = static_cast<u64>(s_kb) * pT, d_kbs = static_cast<u64>(d_kb) * dT;
+  const u32 pack = pack_in == 0 ? 1u : pack_in;
+  while (rem > 0) {
+    u32 pbi, dbi, pt0, dt0;
+    u64 p_base, d_base;
+    if (pack == 1) {
+      pbi = pos / s_ntpb;
+      const u32 pki = (pos - pbi * s_ntpb) / s_kb;
+      pt0 = pos % s_kb;
+      dbi = pos / d_ntpb;
+      const u32 dki = (pos - dbi * d_ntpb) / d_kb;
+      dt0 = pos % d_kb;
+      p_base = pki * p_kbs;
+      d_base = dki * d_kbs;
+    } else {
+      const u32 spl = s_ntpb / pack, dpl = d_ntpb / pack;
+      pbi = pos / spl;
+      dbi = pos / dpl;
+      const u32 pki = (pos % spl) / s_kb, dki = (pos % dpl) / d_kb;
+      pt0 = pos % s_kb;
+      dt0 = pos % d_kb;
+      // uint32 * uint32 * size_t in the reference: the first product is 32-bit.
+      p_base = static_cast<u64>(static_cast<u32>(pki * pack)) * p_kbs;
+      d_base = static_cast<u64>(static_cast<u32>(dki * pack)) * d_kbs;
+    }
+    const u32 k = std::min(std::min(s_kb - pt0, d_kb - dt0), rem);
+    const u64 po = static_cast<u64>(at(sb, pbi)) * pB;
+    const u64 dof = static_cast<u64>(at(db, dbi)) * dB;
+    const u64 ps = pT / 2, ds = dT / 2;
+    for (u32 sub = 0; sub < pack; ++sub) {
+      const u64 pk0 = po + p_base + sub * p_kbs;
+      const u64 dk0 = dof + d_base + sub * d_kbs;
+      for (u32 i = 0; i < k; ++i) {
+        const u64 pk = pk0 + static_cast<u64>(pt0 + i) * ps;
+        const u64 pv = pk + p_kbs / 2;
+        const u64 dk = dk0 + static_cast<u64>(dt0 + i) * ds + goff * ps;
+        const u64 dv = dk + d_kbs / 2;
+        emit(out, b, swap ? dk : pk, swap ? pk : dk, ps);
+        emit(out, b, swap ? dv : pv, swap ? pv : dv, ps);
+      }
+    }
+    pos += k;
+    rem -= k;
+  }
+}
+
+// parse_block_qwen3_next.cpp:262-374 (fill_last_hybrid_attn_block)
+void hybrid_attn_fill_last(u32 s_ntpb, u32 d_ntpb, u64 pT, u64 dT, u64 pB, u64 dB, const Ids& sb,
+                           const Ids& db, u32 total, u32 goff, u32 s_kb, u32 d_kb, u32 pack_in,
+                           const Bounds& b, Runs& out) {
+  if (total == 0) return;
+  const u32 pack = pack_in == 0 ? 1u : pack_in;
+  const u32 spl = pack == 1 ? s_ntpb : s_ntpb / pack;
+  const u32 dpl = pack == 1 ? d_ntpb : d_ntpb / pack;
+  (void)spl;
+  const u32 filled = total % dpl;
+  if (filled == 0) return;
+  u32 todo = dpl - filled;
+  const u64 d_kbs = static_cast<u64>(d_kb) * dT;
+  const u64 ps = pT / 2, ds = dT / 2;
+  const u64 zsrc = static_cast<u64>(at(sb, 0)) * pB;
+  u32 dpos = total, spos = 0;
+  while (todo > 0) {
+    u32 dbi, pt0, dt0;
+    u64 d_base;
+    if (pack == 1) {
+      pt0 = spos % s_kb;
+      dbi = dpos / d_ntpb;
+      const u32 dki = (dpos - dbi * d_ntpb) / d_kb;
+      dt0 = dpos % d_kb;
+      d_base = dki * d_kbs;
+    } else {
+      dbi = dpos / dpl;
+      const u32 dki = (dpos % dpl) / d_kb;
+      pt0 = spos % s_kb;
+      dt0 = dpos % d_kb;
+      d_base = static_cast<u64>(static_cast<u32>(dki * pack)) * d_kbs;
+    }
+    const u64 dof = static_cast<u64>(at(db, dbi)) * dB;
+    const u32 k = std::min(std::min(s_kb - pt0, d_kb - dt0), todo);
+    for (u32 sub = 0; sub < pack; ++sub) {
+      const u64 dk0 = dof + d_base + sub * d_kbs;
+      for (u32 i = 0; i < k; ++i) {
+        const u64 dk = dk0 + static_cast<u64>(dt0 + i) * ds + goff * ps;
+        const u64 dv = dk + d_kbs / 2;
+        zero_fill(zsrc, dk, ps, pB, b, out);
+        zero_fill(zsrc, dv, ps, pB, b, out);
+      }
+    }
+    spos += k;
+    dpos += k;
+    todo -= k;
+  }
+}
+
+// parse_block_qwen3_next.cpp:1031-1088 (fill_tail_hybrid_attn_block_p_lt_d)
+void hybrid_attn_fill_tail_pltd(u64 pB, u64 dB, u64 dT, u32 d_ntpb, u32 d_kb, u32 pack_in,
+                                const Ids& sb, const Ids& db, u32 total, const Bounds& b,
+                                Runs& out) {
+  const u32 pack = pack_in == 0 ? 1u : pack_in;
+  const u32 dpl = pack == 1 ? d_ntpb : d_ntpb / pack;
+  const u64 d_kbs = static_cast<u64>(d_kb) * dT;
+  const u64 ds = dT / 2;
+  const u32 end = static_cast<u32>(db.size()) * dpl;
+  if (total >= end) return;
+  const u64 zsrc = static_cast<u64>(at(sb, 0)) * pB;
+  u32 dpos = total;
+  while (dpos < end) {
+    const u32 dbi = dpos / dpl;
+    const u32 dki = (dpos % dpl) / d_kb;
+    const u32 dti = dpos % d_kb;
+    const u32 k = std::min(d_kb - dti, end - dpos);
+    const u64 dof = static_cast<u64>(at(db, dbi)) * dB;
+    const u64 base = static_cast<u64>(dki) * pack * d_kbs;
+    const u64 len = static_cast<u64>(k) * ds;
+    for (u32 sub = 0; sub < pack; ++sub) {
+      const u64 dk = dof + base + sub * d_kbs + static_cast<u64>(dti) * ds;
+      const u64 dv = dk + d_kbs / 2;
+      zero_fill(zsrc, dk, len, pB, b, out);
+      zero_fill(zsrc, dv, len, pB, b, out);
+    }
+    dpos += k;
+  }
+}
+
+// parse_block_qwen3_next.cpp:865-955
+void hybrid_peqd(const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+                 const Task& t, std::vector<Runs>& out) {
+  if (s.n_tensors < 1) throw std::out_of_range("tensor index");
+  out.resize(s.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  const u64 B = s.block_sizes[0], T = s.token_sizes[0];
+  u64 g = s.num_gdn_layers;
+  const u32 pack = s.attn_pack_size == 0 ? 1u : s.attn_pack_size;
+  const u64 attn_ntpb = B / T / pack;
+  const u32 idx_ntpb = s.indexer_blk_ntpb;
+  if (idx_ntpb > 0) {
+    pages_walk(B, t, grp(t.src, g), grp(t.dst, g), idx_ntpb, b, r);
+    g += 1;
+  }
+  pages_walk(B, t, grp(t.src, g), grp(t.dst, g), static_cast<u32>(attn_ntpb), b, r);
+  if (t.last) {
+    state_pages_same(B, 0, s.num_gdn_layers, t, b, r);
+    if (s.num_ple_layers > 0) state_pages_same(B, s.ple_block_group, s.num_ple_layers, t, b, r);
+  }
+}
+
+// parse_block_qwen3_next.cpp:717-859 + :964-1021
+void hybrid_pgtd(const kvt_worker_info& s, const kvt_worker_info& d, u32 valid, u32 kvt_tp_rank,
+                 const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  const u32 gdn_n = s.engine_tp_size / d.engine_tp_size;
+  const u32 gdn_off = s.worker_tp_rank % gdn_n;
+  const u32 attn_n = popcount16(valid) / d.engine_tp_size;
+  const u32 attn_off = kvt_tp_rank % attn_n;
+  if (s.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pT = s.token_sizes[0], dT = d.token_sizes[0];
+  const u32 s_ntpb = static_cast<u32>(s.block_sizes[0] / pT);
+  const u32 d_ntpb = static_cast<u32>(d.block_sizes[0] / dT);
+  out.resize(s.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  const u64 pB = pT * s_ntpb, dB = dT * d_ntpb;
+  const u32 pack = s.attn_pack_size == 0 ? 1u : s.attn_pack_size;
+  const u64 n_gdn = s.num_gdn_layers;
+  if (t.last) {
+    gdn_pgtd(pB, dB, n_gdn, gdn_n, gdn_off, s, t, b, r);
+    ple_split(pB, dB, true, gdn_off, s, t, b, r);
+  }
+  u64 g = n_gdn;
+  if (s.indexer_blk_ntpb > 0 && d.indexer_blk_ntpb > 0) {
+    if (s.worker_tp_rank % gdn_n == 0)
+      indexer_walk(pB, dB, t.seen, t.fresh, grp(t.src, g), grp(t.dst, g), s.indexer_blk_ntpb,
+                   d.indexer_blk_ntpb, s.hybrid_indexer_token_size, b, r);
+    g += 1;
+  }
+  if ((valid >> s.worker_tp_rank) & 1u) {
+    const Ids& sa = grp(t.src, g);
+    const Ids& da = grp(t.dst, g);
+    hybrid_attn_walk(s_ntpb, d_ntpb, pT, dT, pB, dB, sa, da, t.seen, t.fresh, attn_off,
+                     s.attn_kernel_blk_ntpb, d.attn_kernel_blk_ntpb, pack, b, false, r);
+    if (o.pad_last_attn_block && t.last)
+      hybrid_attn_fill_last(s_ntpb, d_ntpb, pT, dT, pB, dB, sa, da, t.seen + t.fresh, attn_off,
+                            s.attn_kernel_blk_ntpb, d.attn_kernel_blk_ntpb, pack, b, r);
+  }
+}
+
+// parse_block_qwen3_next.cpp:1108-1289
+void hybrid_pltd(const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+                 const Task& t, std::vector<Runs>& out) {
+  const u32 p_tp = s.engine_tp_size, d_tp = d.engine_tp_size;
+  const u32 gdn_n = d_tp / p_tp;
+  const u32 gdn_off = d.worker_tp_rank % gdn_n;
+  if (s.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pT = s.token_sizes[0], pB = s.block_sizes[0];
+  const u64 dT = d.token_sizes[0], dB = d.block_sizes[0];
+  out.resize(s.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  u64 g = s.num_gdn_layers;
+  const u32 pack = s.attn_pack_size == 0 ? 1u : s.attn_pack_size;
+  const u32 p_in = s.indexer_blk_ntpb, d_in = d.indexer_blk_ntpb;
+  if (pT == dT) {
+    const u64 attn_ntpb = pB / pT / pack;
+    if (p_in > 0) {
+      pages_walk(pB, t, grp(t.src, g), grp(t.dst, g), p_in, b, r);
+      g += 1;
+    }
+    pages_walk(pB, t, grp(t.src, g), grp(t.dst, g), static_cast<u32>(attn_ntpb), b, r);
+  } else {
+    const u32 attn_n = static_cast<u32>(pT / dT);
+    const u32 replicas = d_tp / (p_tp * attn_n);
+    const u32 attn_off = (d.worker_tp_rank / replicas) % attn_n;
+    const u32 s_ntpb = static_cast<u32>(pB / pT), d_ntpb = static_cast<u32>(dB / dT);
+    if (p_in > 0) {
+      indexer_walk(pB, dB, t.seen, t.fresh, grp(t.src, g), grp(t.dst, g), p_in, d_in,
+                   s.hybrid_indexer_token_size, b, r);
+      g += 1;
+    }
+    const Ids& sa = grp(t.src, g);
+    const Ids& da = grp(t.dst, g);
+    hybrid_attn_walk(d_ntpb, s_ntpb, dT, pT, dB, pB, da, sa, t.seen, t.fresh, attn_off,
+                     d.attn_kernel_blk_ntpb, s.attn_kernel_blk_ntpb, pack, b, true, r);
+    if (o.pad_last_attn_block && t.last)
+      hybrid_attn_fill_tail_pltd(pB, dB, dT, d_ntpb, d.attn_kernel_blk_ntpb, pack, sa, da,
+                                 t.seen + t.fresh, b, r);
+  }
+  if (t.last) {
+    gdn_pltd(pB, dB, s.num_gdn_layers, gdn_n, gdn_off, s, t, b, r);
+    ple_split(pB, dB, false, gdn_off, s, t, b, r);
+  }
+}
+
+// parse_block_flashinfer.cpp:82-161 (parse_hybrid_flashinfer_HND_block)
+void hybrid_hnd_walk(u64 pT, u64 dT, u64 pB, u64 dB, u32 p_ntpb, u32 d_ntpb, const Ids& sb,
+                     const Ids& db, u32 pos, u32 rem, u32 goff, u32 s_kb, u32 d_kb, int heads,
+                     const Bounds& b, bool swap, Runs& out) {
+  const u64 p_kbs = static_cast<u64>(s_kb) * pT, d_kbs = static_cast<u64>(d_kb) * dT;
+  const u64 p_half = p_kbs / 2, d_half = d_kbs / 2;
+  const u64 hd = pT / 2 / static_cast<u64>(heads);
+  const u64 p_hs = static_cast<u64>(s_kb) * hd, d_hs = static_cast<u64>(d_kb) * hd;
+  const u64 per_group = static_cast<u64>(heads) * d_hs;
+  while (rem > 0) {
+    const u32 pbi = pos / p_ntpb;
+    const u32 pki = (pos - pbi * p_ntpb) / s_kb;
+    const u32 pt0 = pos % s_kb;
+    const u32 dbi = pos / d_ntpb;
+    const u32 dki = (pos - dbi * d_ntpb) / d_kb;
+    const u32 dt0 = pos % d_kb;
+    const u64 pk0 = static_cast<u64>(at(sb, pbi)) * pB + pki * p_kbs;
+    const u64 dk0 = static_cast<u64>(at(db, dbi)) * dB + dki * d_kbs;
+    const u32 k = std::min(std::min(s_kb - pt0, d_kb - dt0), rem);
+    const u64 len = static_cast<u64>(k) * hd;
+    for (int h = 0; h < heads; ++h) {
+      const u64 pk = pk0 + static_cast<u64>(h) * p_hs + pt0 * hd;
+      const u64 pv = pk + p_half;
+      const u64 dk = dk0 + goff * per_group + static_cast<u64>(h) * d_hs + dt0 * hd;
+      const u64 dv = dk + d_half;
+      emit(out, b, swap ? dk : pk, swap ? pk : dk, len);
+      emit(out, b, swap ? dv : pv, swap ? pv : dv, len);
+    }
+    pos += k;
+    rem -= k;
+  }
+}
+
+// parse_block_flashinfer.cpp:175-235 (fill_last_hybrid_flashinfer_HND_block)
+void hybrid_hnd_fill_last(u64 pT, u64 dT, u64 pB, u64 dB, u32 d_ntpb, const Ids& sb, const Ids& db,
+                          u32 total, u32 goff, int heads, const Bounds& b, Runs& out) {
+  if (total == 0) return;
+  const u32 filled = total % d_ntpb;
+  if (filled == 0) return;
+  const u32 remaining = d_ntpb - filled;
+  const u32 dbi = total / d_ntpb;
+  const u64 hd = pT / 2 / static_cast<u64>(heads);
+  const u64 d_hs = static_cast<u64>(d_ntpb) * hd;
+  const u64 d_half = static_cast<u64>(d_ntpb) * dT / 2;
+  const u64 per_group = static_cast<u64>(heads) * d_hs;
+  const u64 len = static_cast<u64>(remaining) * hd;
+  const u64 zsrc = static_cast<u64>(at(sb, 0)) * pB;
+  const u64 dof = static_cast<u64>(at(db, dbi)) * dB;
+  for (int h = 0; h < heads; ++h) {
+    const u64 dk = dof + goff * per_group + static_cast<u64>(h) * d_hs + filled * hd;
+    const u64 dv = dk + d_half;
+    zero_fill(zsrc, dk, len, pB, b, out);
+    zero_fill(zsrc, dv, len, pB, b, out);
+  }
+}
+
+// parse_block_qwen3_next_flashinfer.cpp:12-16
+int hybrid_fi_heads(const kvt_worker_info& w) {
+  return std::max(1, w.num_kv_heads / static_cast<int>(w.engine_tp_size));
+}
+
+// parse_block_qwen3_next_flashinfer.cpp:35-122
+void hybrid_fi_peqd(const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+                    const Task& t, std::vector<Runs>& out) {
+  if (s.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pT = s.token_sizes[0], pB = s.block_sizes[0];
+  const u32 ntpb = static_cast<u32>(pB / pT);
+  out.resize(s.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  u64 g = s.num_gdn_layers;
+  if (s.indexer_blk_ntpb > 0) {
+    pages_walk(pB, t, grp(t.src, g), grp(t.dst, g), s.indexer_blk_ntpb, b, r);
+    g += 1;
+  }
+  pages_walk(pB, t, grp(t.src, g), grp(t.dst, g), ntpb, b, r);
+  if (t.last) {
+    state_pages_same(pB, 0, s.num_gdn_layers, t, b, r);
+    if (s.num_ple_layers > 0) state_pages_same(pB, s.ple_block_group, s.num_ple_layers, t, b, r);
+  }
+}
+
+// parse_block_qwen3_next_flashinfer.cpp:128-271
+void hybrid_fi_pgtd(const kvt_worker_info& s, const kvt_worker_info& d, u32 valid, u32 kvt_tp_rank,
+                    const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  const u32 gdn_n = s.engine_tp_size / d.engine_tp_size;
+  const u32 gdn_off = s.worker_tp_rank % gdn_n;
+  const u32 attn_n = popcount16(valid) / d.engine_tp_size;
+  const u32 attn_off = attn_n > 0 ? kvt_tp_rank % attn_n : 0;
+  if (s.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pT = s.token_sizes[0], dT = d.token_sizes[0];
+  const u64 pB = s.block_sizes[0], dB = d.block_sizes[0];
+  const int heads = hybrid_fi_heads(s);
+  const u32 s_ntpb = static_cast<u32>(pB / pT), d_ntpb = static_cast<u32>(dB / dT);
+  out.resize(s.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  const u64 n_gdn = s.num_gdn_layers;
+  if (t.last) {
+    gdn_pgtd(pB, dB, n_gdn, gdn_n, gdn_off, s, t, b, r);
+    ple_split(pB, dB, true, gdn_off, s, t, b, r);
+  }
+  u64 g = n_gdn;
+  if (s.indexer_blk_ntpb > 0 && d.indexer_blk_ntpb > 0) {
+    if (s.worker_tp_rank % gdn_n == 0)
+      indexer_walk(pB, dB, t.seen, t.fresh, grp(t.src, g), grp(t.dst, g), s.indexer_blk_ntpb,
+                   d.indexer_blk_ntpb, s.hybrid_indexer_token_size, b, r);
+    g += 1;
+  }
+  if ((valid >> s.worker_tp_rank) & 1u) {
+    const Ids& sa = grp(t.src, g);
+    const Ids& da = grp(t.dst, g);
+    hybrid_hnd_walk(pT, dT, pB, dB, s_ntpb, d_ntpb, sa, da, t.seen, t.fresh, attn_off,
+                    s.attn_kernel_blk_ntpb, d.attn_kernel_blk_ntpb, heads, b, false, r);
+    if (o.pad_last_attn_block && t.last)
+      hybrid_hnd_fill_last(pT, dT, pB, dB, d_ntpb, sa, da, t.seen + t.fresh, attn_off, heads, b, r);
+  }
+}
+
+// parse_block_qwen3_next_flashinfer.cpp:278-322 (fill_tail_..._p_lt_d)
+void hybrid_hnd_fill_tail_pltd(u64 pB, u64 dB, u32 d_ntpb, u64 hd, int d_heads, const Ids& sb,
+                               const Ids& db, u32 total, const Bounds& b, Runs& out) {
+  const u32 end = static_cast<u32>(db.size()) * d_ntpb;
+  if (total >= end) return;
+  const u64 d_hs = static_cast<u64>(d_ntpb) * hd;
+  const u64 d_half = dB / 2;
+  const u64 zsrc = static_cast<u64>(at(sb, 0)) * pB;
+  u32 dpos = total;
+  while (dpos < end) {
+    const u32 dbi = dpos / d_ntpb, dti = dpos % d_ntpb;
+    const u32 k = std::min(d_ntpb - dti, end - dpos);
+    const u64 dof = static_cast<u64>(at(db, dbi)) * dB;
+    const u64 len = static_cast<u64>(k) * hd;
+    for (int h = 0; h < d_heads; ++h) {
+      const u64 dk = dof + static_cast<u64>(h) * d_hs + dti * hd;
+      const u64 dv = dk + d_half;
+      zero_fill(zsrc, dk, len, pB, b, out);
+      zero_fill(zsrc, dv, len, pB, b, out);
+    }
+    dpos += k;
+  }
+}
+
+// parse_block_qwen3_next_flashinfer.cpp:342-533
+void hybrid_fi_pltd(const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+                    const Task& t, std::vector<Runs>& out) {
+  const u32 p_tp = s.engine_tp_size, d_tp = d.engine_tp_size;
+  const u32 gdn_n = d_tp / p_tp;
+  const u32 gdn_off = d.worker_tp_rank % gdn_n;
+  if (s.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 pT = s.token_sizes[0], pB = s.block_sizes[0];
+  const u64 dT = d.token_sizes[0], dB = d.block_sizes[0];
+  const u32 s_ntpb = static_cast<u32>(pB / pT), d_ntpb = static_cast<u32>(dB / dT);
+  out.resize(s.n_tensors);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  u64 g = s.num_gdn_layers;
+  const u32 p_in = s.indexer_blk_ntpb, d_in = d.indexer_blk_ntpb;
+  if (pT == dT) {
+    if (p_in > 0) {
+      pages_walk(pB, t, grp(t.src, g), grp(t.dst, g), p_in, b, r);
+      g += 1;
+    }
+    pages_walk(pB, t, grp(t.src, g), grp(t.dst, g), s_ntpb, b, r);
+  } else {
+    const u32 attn_n = static_cast<u32>(pT / dT);
+    const u32 replicas = d_tp / (p_tp * attn_n);
+    const u32 attn_off = (d.worker_tp_rank / replicas) % attn_n;
+    const int heads = s.num_kv_heads;
+    const int d_heads = static_cast<u32>(heads) >= d_tp ? heads / static_cast<int>(d_tp) : 1;
+    const u64 hd = dT / 2 / static_cast<u64>(d_heads);
+    if (p_in > 0) {
+      indexer_walk(pB, dB, t.seen, t.fresh, grp(t.src, g), grp(t.dst, g), p_in, d_in,
+                   s.hybrid_indexer_token_size, b, r);
+      g += 1;
+    }
+    const Ids& sa = grp(t.src, g);
+    const Ids& da = grp(t.dst, g);
+    hybrid_hnd_walk(dT, pT, dB, pB, d_ntpb, s_ntpb, da, sa, t.seen, t.fresh, attn_off,
+                    d.attn_kernel_blk_ntpb, s.attn_kernel_blk_ntpb, d_heads, b, true, r);
+    if (o.pad_last_attn_block && t.last)
+      hybrid_hnd_fill_tail_pltd(pB, dB, d_ntpb, hd, d_heads, sa, da, t.seen + t.fresh, b, r);
+  }
+  if (t.last) {
+    gdn_pltd(pB, dB, s.num_gdn_layers, gdn_n, gdn_off, s, t, b, r);
+    ple_split(pB, dB, false, gdn_off, s, t, b, r);
+  }
+}
+
+std::vector<Ids> split_groups(const u32* ids, const u32* lens, u32 n) {
+  std::vector<Ids> g(n);
+  size_t p = 0;
+  for (u32 i = 0; i < n; ++i) {
+    g[i].assign(ids + p, ids + p + lens[i]);
+    p += lens[i];
+  }
+  return g;
+}
+
+int run_parser(int id, const kvt_worker_info& s, const kvt_worker_info& d, u32 valid,
+               u32 kvt_tp_size, u32 kvt_tp_rank, const kvt_parse_opts& o, const Task& t,
+               std::vector<Runs>& out) {
+  switch (id) {
+    case KVT_PARSER_RAGGED_PEQD: ragged_peqd(s, d, o, t, out); break;
+    case KVT_PARSER_RAGGED_PGTD: ragged_pgtd(s, d, kvt_tp_size, o, t, out); break;
+    case KVT_PARSER_RAGGED_PGTD_DPSK: ragged_pgtd_dpsk(s, d, o, t, out); break;
+    case KVT_PARSER_RAGGED_PLTD: ragged_pltd(s, d, kvt_tp_size, o, t, out); break;
+    case KVT_PARSER_FLASH_PEQD: flash_peqd(s, d, o, t, out); break;
+    case KVT_PARSER_FLASH_PGTD: flash_pgtd(s, d, valid, kvt_tp_rank, o, t, out); break;
+    case KVT_PARSER_TURBOQUANT_PEQD:  // parse_block_turboquant.cpp:9-22
+    case KVT_PARSER_HYBRID_PEQD: hybrid_peqd(s, d, o, t, out); break;
+    case KVT_PARSER_TURBOQUANT_PGTD:  // parse_block_turboquant.cpp:25-39
+    case KVT_PARSER_HYBRID_PGTD: hybrid_pgtd(s, d, valid, kvt_tp_rank, o, t, out); break;
+    case KVT_PARSER_HYBRID_PLTD: hybrid_pltd(s, d, o, t, out); break;
+    case KVT_PARSER_DPSK_PEQD: dpsk_peqd(s, d, valid, o, t, out); break;
+    case KVT_PARSER_DPSK_PGTD: dpsk_pgtd(s, d, kvt_tp_size, o, t, out); break;
+    case KVT_PARSER_DPSK_PLTD: dpsk_pltd(s, d, kvt_tp_size, o, t, out); break;
+    case KVT_PARSER_FLASHINFER_PEQD: flashinfer_any(s, d, valid, kvt_tp_rank, false, o, t, out); break;
+    case KVT_PARSER_FLASHINFER_PGTD: flashinfer_any(s, d, valid, kvt_tp_rank, true, o, t, out); break;
+    case KVT_PARSER_HYBRID_FI_PEQD: hybrid_fi_peqd(s, d, o, t, out); break;
+    case KVT_PARSER_HYBRID_FI_PGTD: hybrid_fi_pgtd(s, d, valid, kvt_tp_rank, o, t, out); break;
+    case KVT_PARSER_HYBRID_FI_PLTD: hybrid_fi_pltd(s, d, o, t, out); break;
+    default: return KVT_ERR_UNSUPPORTED;  // KDA / Kimi-K3 parsers are not restated here
+  }
+  return KVT_OK;
+}
+
+// kvtransfer/src/copy_kernels.cu:287-334, the path taken when <cuda_fp8.h> is
+// present: round-to-nearest-even to E4M3 with saturation to +-448
+// (__NV_SATFINITE); NaN -> 0x7F | sign.
+uint8_t bf16_to_e4m3_satfinite(uint16_t bits) {
+  const uint8_t sign = static_cast<uint8_t>((bits >> 15) << 7);
+  const int e = (bits >> 7) & 0xFF;
+  const u32 m = bits & 0x7F;
+  if (e == 0xFF) return m ? static_cast<uint8_t>(sign | 0x7F) : static_cast<uint8_t>(sign | 0x7E);
+  if (e == 0) return sign;  // zero and bf16 subnormals (< 2^-126) underflow to zero
+  const int ue = e - 127;   // value = 1.m * 2^ue
+  // work with a 8-bit significand S = 1mmmmmmm (value = S * 2^(ue-7))
+  const u32 S = 0x80 | m;
+  int shift;  // number of low bits of S dropped
+  int out_e;  // biased e4m3 exponent before rounding
+  if (ue >= -6) {
+    shift = 4;  // keep 1 + 3 bits
+    out_e = ue + 7;
+  } else {
+    shift = 4 + (-6 - ue);  // subnormal: value = M * 2^-9, M in [0,8)
+    out_e = 0;
+  }
+  if (shift > 12) return sign;
+  u32 q = S >> shift;
+  const u32 rem = S & ((1u << shift) - 1);
+  const u32 half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (q & 1))) q += 1;
+  u32 code;
+  if (out_e == 0) {
+    code = q;  // q in [0,8]; 8 == smallest normal (exp 1, mant 0)
+  } else {
+    code = (static_cast<u32>(out_e) << 3) + (q - 8);  // q in [8,16]; 16 carries into the exponent
+  }
+  if (code > 0x7E) code = 0x7E;  // saturate (0x7F is NaN)
+  return static_cast<uint8_t>(sign | code);
+}
+
+}  // namespace
+
+extern "C" {
+
+// tx_stub.cpp:201-205 (loop over the batch's tasks appending into one list).
+int kvto_parse(int parser_id, const kvt_worker_info* src, const kvt_worker_info* dst,
+               uint32_t valid_mask, uint32_t kvt_tp_size, uint32_t kvt_tp_rank,
+               const kvt_parse_opts* opts, const kvt_task* tasks, uint32_t n_tasks, uint32_t cap,
+               kvt_ipc_block** out, uint64_t* n_out, uint32_t* n_tensors) {
+  std::vector<Runs> lists;
+  try {
+    for (u32 i = 0; i < n_tasks; ++i) {
+      Task t;
+      t.seen = tasks[i].seen_tokens;
+      t.fresh = tasks[i].new_tokens;
+      t.last = tasks[i].reach_last_token != 0;
+      t.src = split_groups(tasks[i].src_blocks, tasks[i].src_group_len, tasks[i].n_src_groups);
+      t.dst = split_groups(tasks[i].dst_blocks, tasks[i].dst_group_len, tasks[i].n_dst_groups);
+      const int rc = run_parser(parser_id, *src, *dst, valid_mask, kvt_tp_size, kvt_tp_rank, *opts,
+                                t, lists);
+      if (rc != KVT_OK) return rc;
+    }
+  } catch (const std::out_of_range&) {
+    return KVT_ERR_OUT_OF_RANGE;
+  } catch (const std::overflow_error&) {
+    return KVT_ERR_OVERFLOW;
+  } catch (const std::exception&) {
+    return KVT_ERR_INVALID;
+  }
+  *n_tensors = static_cast<u32>(lists.size());
+  for (u32 t = 0; t < lists.size() && t < cap; ++t) {
+    n_out[t] = lists[t].size();
+    out[t] = static_cast<kvt_ipc_block*>(std::malloc(sizeof(kvt_ipc_block) * (lists[t].size() + 1)));
+    if (!lists[t].empty())
+      std::memcpy(out[t], lists[t].data(), sizeof(kvt_ipc_block) * lists[t].size());
+  }
+  return KVT_OK;
+}
+
+void kvto_free(void* p) { std::free(p); }
+
+// tx_stub.cpp:18-81 (compute_valid_ranks_pd)
+uint32_t kvto_valid_ranks(uint32_t p_tp, uint32_t d_tp, int num_kv_heads) {
+  u32 m = 0;
+  if (p_tp < d_tp || num_kv_heads <= 0 || static_cast<u32>(num_kv_heads) >= p_tp) {
+    for (u32 i = 0; i < p_tp; ++i) m |= 1u << i;
+    return m;
+  }
+  if (d_tp <= static_cast<u32>(num_kv_heads)) {
+    const u32 stride = p_tp / static_cast<u32>(num_kv_heads);
+    for (int i = 0; i < num_kv_heads; ++i) m |= 1u << (static_cast<u32>(i) * stride);
+    return m;
+  }
+  const u32 per_d = p_tp / d_tp;
+  for (u32 r = 0; r < d_tp; ++r) m |= 1u << (r * per_d);
+  return m;
+}
+
+// tx_stub.cpp:105-114 (selection_p_tp) and :451-590 (dispatch in refresh_dst_info)
+int kvto_select(int cache_shape, const kvt_worker_info* src, const kvt_worker_info* dst,
+                uint32_t* valid_mask, uint32_t* kvt_tp_size, uint32_t* kvt_tp_rank,
+                int* parser_id, int* tp_kind) {
+  const u32 valid = kvto_valid_ranks(src->engine_tp_size, dst->engine_tp_size, src->num_kv_heads);
+  const u32 eff = popcount16(valid);
+  const u32 below = popcount16(valid & ((1u << src->worker_tp_rank) - 1u));
+  *valid_mask = valid;
+  *kvt_tp_size = eff;
+  *kvt_tp_rank = below;
+  const bool engine_based = cache_shape == KVT_SHAPE_QWEN3_NEXT_FLASH ||
+                            cache_shape == KVT_SHAPE_QWEN3_NEXT_FLASHINFER ||
+                            cache_shape == KVT_SHAPE_KIMI_K3_MLA;
+  const u32 p = engine_based ? src->engine_tp_size : eff;
+  const u32 d = dst->engine_tp_size;
+  const int rel = p == d ? 0 : (p > d ? 1 : -1);
+  int id = -1, kind = KVT_TP_UNKNOWN;
+  switch (cache_shape) {
+    case KVT_SHAPE_RAGGED_FLASH:
+      if (rel == 0) { id = KVT_PARSER_RAGGED_PEQD; kind = KVT_TP_PEQD; }
+      else if (rel > 0) {
+        if (same_token_sizes(*src, *dst)) { id = KVT_PARSER_RAGGED_PGTD_DPSK; kind = KVT_TP_PEQD; }
+        else { id = KVT_PARSER_RAGGED_PGTD; kind = KVT_TP_PGTD; }
+      } else { id = KVT_PARSER_RAGGED_PLTD; kind = KVT_TP_PLTD; }
+      break;
+    case KVT_SHAPE_FLASH:
+      if (rel == 0) { id = KVT_PARSER_FLASH_PEQD; kind = KVT_TP_PEQD; }
+      else if (rel > 0) { id = KVT_PARSER_FLASH_PGTD; kind = KVT_TP_PGTD; }
+      break;
+    case KVT_SHAPE_QWEN3_NEXT_FLASH:
+      if (rel == 0) { id = KVT_PARSER_HYBRID_PEQD; kind = KVT_TP_PEQD; }
+      else if (rel > 0) { id = KVT_PARSER_HYBRID_PGTD; kind = KVT_TP_PGTD; }
+      else { id = KVT_PARSER_HYBRID_PLTD; kind = KVT_TP_PLTD; }
+      break;
+    case KVT_SHAPE_DPSK_V32_SPARSE_MLA:  // TPKind is PEQD for all three (tx_stub.cpp:521-535)
+      kind = KVT_TP_PEQD;
+      id = rel == 0 ? KVT_PARSER_DPSK_PEQD : (rel > 0 ? KVT_PARSER_DPSK_PGTD : KVT_PARSER_DPSK_PLTD);
+      break;
+    case KVT_SHAPE_FLASHINFER:
+      if (rel == 0) { id = KVT_PARSER_FLASHINFER_PEQD; kind = KVT_TP_PEQD; }
+      else if (rel > 0) { id = KVT_PARSER_FLASHINFER_PGTD; kind = KVT_TP_PGTD; }
+      break;
+    case KVT_SHAPE_QWEN3_NEXT_FLASHINFER:
+      if (rel == 0) { id = KVT_PARSER_HYBRID_FI_PEQD; kind = KVT_TP_PEQD; }
+      else if (rel > 0) { id = KVT_PARSER_HYBRID_FI_PGTD; kind = KVT_TP_PGTD; }
+      else { id = KVT_PARSER_HYBRID_FI_PLTD; kind = KVT_TP_PLTD; }
+      break;
+    case KVT_SHAPE_KIMI_K3_MLA:
+      if (rel == 0) { id = KVT_PARSER_KIMI_K3_PEQD; kind = KVT_TP_PEQD; }
+      else if (rel > 0) { id = KVT_PARSER_KIMI_K3_PGTD; kind = KVT_TP_PGTD; }
+      else { id = KVT_PARSER_KIMI_K3_PLTD; kind = KVT_TP_PLTD; }
+      break;
+    case KVT_SHAPE_TURBOQUANT:
+      if (rel == 0) { id = KVT_PARSER_TURBOQUANT_PEQD; kind = KVT_TP_PEQD; }
+      else if (rel > 0) { id = KVT_PARSER_TURBOQUANT_PGTD; kind = KVT_TP_PGTD; }
+      break;
+    default: break;
+  }
+  if (id < 0) return KVT_ERR_UNSUPPORTED;  // tx_stub.cpp:590
+  *parser_id = id;
+  *tp_kind = kind;
+  return KVT_OK;
+}
+
+// channel.cpp:53-98 (merge_interval) followed by the erase of zero-length
+// entries its callers do (tcp_channel.cpp:388-391). The reference sorts with an
+// unstable std::sort keyed on src_offset only; this restatement sorts stably,
+// which is the same order whenever source offsets are distinct. stats =
+// {min, max, total, count}. Returns the compacted length.
+uint64_t kvto_merge(kvt_ipc_block* v, uint64_t n, uint64_t stats[4]) {
+  std::stable_sort(v, v + n, [](const kvt_ipc_block& a, const kvt_ipc_block& b) {
+    return a.src_offset < b.src_offset;
+  });
+  u64 mn = std::numeric_limits<u64>::max(), mx = 0, tot = 0, cnt = 0, prev = 0;
+  for (u64 i = 1; i < n; ++i) {
+    kvt_ipc_block& p = v[prev];
+    kvt_ipc_block& c = v[i];
+    if (c.src_offset == p.src_offset + p.length && c.dst_offset == p.dst_offset + p.length) {
+      p.length += c.length;
+      c.length = 0;
+    } else {
+      mn = std::min(mn, p.length);
+      mx = std::max(mx, p.length);
+      tot += p.length;
+      cnt += 1;
+      prev = i;
+    }
+  }
+  if (prev < n) {
+    mn = std::min(mn, v[prev].length);
+    mx = std::max(mx, v[prev].length);
+    tot += v[prev].length;
+    cnt += 1;
+  }
+  if (stats) { stats[0] = mn; stats[1] = mx; stats[2] = tot; stats[3] = cnt; }
+  u64 w = 0;
+  for (u64 i = 0; i < n; ++i)
+    if (v[i].length != 0) v[w++] = v[i];
+  return w;
+}
+
+// channel.cpp:11-50 (validate_ipc_block_bounds). which: 0 = source, 1 = destination.
+// Returns KVT_OK or KVT_ERR_OUT_OF_RANGE with *bad_idx set.
+int kvto_validate(const kvt_ipc_block* v, uint64_t n, uint64_t capacity, int which,
+                  uint64_t length_scale, uint64_t* bad_idx) {
+  const u64 M = std::numeric_limits<u64>::max();
+  for (u64 i = 0; i < n; ++i) {
+    const u64 off = which == 0 ? v[i].src_offset : v[i].dst_offset;
+    const bool ovf = length_scale == 0 || v[i].length > M / length_scale;
+    const u64 eff = ovf ? M : v[i].length * length_scale;
+    if (v[i].length == 0 || ovf || off > capacity || eff > capacity - off) {
+      if (bad_idx) *bad_idx = i;
+      return KVT_ERR_OUT_OF_RANGE;
+    }
+  }
+  return KVT_OK;
+}
+
+// Pack = tcp_channel.cpp:517-555 + copy_kernels.cpp:384-397: the blob is the
+// ranges' source bytes concatenated in list order (host offset = running sum).
+void kvto_pack(const uint8_t* layer, const kvt_ipc_block* v, uint64_t n, uint8_t* blob) {
+  u64 cur = 0;
+  for (u64 i = 0; i < n; ++i) {
+    std::memcpy(blob + cur, layer + v[i].src_offset, v[i].length);
+    cur += v[i].length;
+  }
+}
+
+// Unpack = tcp_channel.cpp:190-256: range i of the blob goes to dst_offset.
+void kvto_unpack(uint8_t* layer, const kvt_ipc_block* v, uint64_t n, const uint8_t* blob) {
+  u64 cur = 0;
+  for (u64 i = 0; i < n; ++i) {
+    std::memcpy(layer + v[i].dst_offset, blob + cur, v[i].length);
+    cur += v[i].length;
+  }
+}
+
+// The same pack over `n_layers` layers (layer l at layers[l], blob l at
+// blob + l * blob_stride) with `threads` host threads striding over layers.
+// threads == 1 is the reference's situation: one "clisend" thread per
+// destination walks the layers (tx_stub.cpp:395-415, client.cpp:94-104).
+void kvto_pack_layers(const uint8_t* const* layers, uint32_t n_layers, const kvt_ipc_block* v,
+                      uint64_t n, uint8_t* blob, uint64_t blob_stride, uint32_t threads) {
+  if (threads <= 1) {
+    for (u32 l = 0; l < n_layers; ++l) kvto_pack(layers[l], v, n, blob + l * blob_stride);
+    return;
+  }
+  std::atomic<u32> next(0);
+  std::vector<std::thread> pool;
+  for (u32 t = 0; t < threads; ++t)
+    pool.emplace_back([&]() {
+      for (;;) {
+        const u32 l = next.fetch_add(1);
+        if (l >= n_layers) break;
+        kvto_pack(layers[l], v, n, blob + l * blob_stride);
+      }
+    });
+  for (auto& th : pool) th.join();
+}
+
+void kvto_unpack_layers(uint8_t* const* layers, uint32_t n_layers, const kvt_ipc_block* v,
+                        uint64_t n, const uint8_t* blob, uint64_t blob_stride, uint32_t threads) {
+  if (threads <= 1) {
+    for (u32 l = 0; l < n_layers; ++l) kvto_unpack(layers[l], v, n, blob + l * blob_stride);
+    return;
+  }
+  std::atomic<u32> next(0);
+  std::vector<std::thread> pool;
+  for (u32 t = 0; t < threads; ++t)
+    pool.emplace_back([&]() {
+      for (;;) {
+        const u32 l = next.fetch_add(1);
+        if (l >= n_layers) break;
+        kvto_unpack(layers[l], v, n, blob + l * blob_stride);
+      }
+    });
+  for (auto& th : pool) th.join();
+}
+
+// Transposing pack HND -> NHD (no reference function; the reference never
+// changes layout). For each block id in list order, the block's K half then V
+// half, each stored [heads][ntpb][row] in the cache, is written [ntpb][heads][row]
+// into the blob. block_bytes = 2 * heads * ntpb * row_bytes.
+void kvto_pack_hnd_to_nhd(const uint8_t* layer, const uint32_t* block_ids, uint64_t n_blocks,
+                          uint32_t heads, uint32_t ntpb, uint32_t row_bytes, uint8_t* blob) {
+  const u64 half = static_cast<u64>(heads) * ntpb * row_bytes;
+  for (u64 i = 0; i < n_blocks; ++i)
+    for (u32 kv = 0; kv < 2; ++kv)
+      for (u32 h = 0; h < heads; ++h)
+        for (u32 t = 0; t < ntpb; ++t)
+          std::memcpy(blob + (2 * i + kv) * half + (static_cast<u64>(t) * heads + h) * row_bytes,
+                      layer + (2 * static_cast<u64>(block_ids[i]) + kv) * half +
+                          (static_cast<u64>(h) * ntpb + t) * row_bytes,
+                      row_bytes);
+}
+
+// Inverse: NHD blob -> HND cache blocks.
+void kvto_unpack_nhd_to_hnd(uint8_t* layer, const uint32_t* block_ids, uint64_t n_blocks,
+                            uint32_t heads, uint32_t ntpb, uint32_t row_bytes,
+                            const uint8_t* blob) {
+  const u64 half = static_cast<u64>(heads) * ntpb * row_bytes;
+  for (u64 i = 0; i < n_blocks; ++i)
+    for (u32 kv = 0; kv < 2; ++kv)
+      for (u32 h = 0; h < heads; ++h)
+        for (u32 t = 0; t < ntpb; ++t)
+          std::memcpy(layer + (2 * static_cast<u64>(block_ids[i]) + kv) * half +
+                          (static_cast<u64>(h) * ntpb + t) * row_bytes,
+                      blob + (2 * i + kv) * half + (static_cast<u64>(t) * heads + h) * row_bytes,
+                      row_bytes);
+}
+
+uint8_t kvto_bf16_to_fp8(uint16_t bits) { return bf16_to_e4m3_satfinite(bits); }
+
+// Converting pack = copy_kernels.cu:369-481 as driven by tcp_channel.cpp:536-547:
+// each range's bf16 source (2 * length bytes at src_offset) becomes `length`
+// fp8 bytes, concatenated in list order.
+void kvto_pack_bf16_to_fp8(const uint8_t* layer, const kvt_ipc_block* v, uint64_t n,
+                           uint8_t* blob) {
+  u64 cur = 0;
+  for (u64 i = 0; i < n; ++i) {
+    const uint16_t* s = reinterpret_cast<const uint16_t*>(layer + v[i].src_offset);
+    for (u64 j = 0; j < v[i].length; ++j) blob[cur + j] = bf16_to_e4m3_satfinite(s[j]);
+    cur += v[i].length;
+  }
+}
+
+}  // extern "C"

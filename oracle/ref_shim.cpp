@@ -1,0 +1,164 @@
+// TEST INFRASTRUCTURE -- not part of the product.
+//
+// C-ABI shim around the *reference's own* ParseBlock implementation. It is
+// compiled (by oracle/Makefile, target `ref`) together with the reference
+// sources where they lie under /root/reference/kvtransfer -- nothing of the
+// reference is copied into this repository -- and the result goes to
+// oracle/_ref/libkvt_ref.so. The shim only converts the plain-C structs of
+// include/kvt_types.h into the reference's C++ types and calls the reference
+// function selected by `parser_id`
+// (declarations: kvtransfer/include/parse_block_common.h:143-388,
+//  kvtransfer/include/parse_block_turboquant.h).
+//
+// Used by tests/ to validate the CPU restatement in oracle/kvt_oracle.cpp and
+// by tests/golden/make_golden.py to write golden vectors.
+#include <bitset>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "parse_block_common.h"
+#include "parse_block_turboquant.h"
+
+#include "kvt_types.h"
+
+using namespace blade_llm;
+
+namespace {
+
+WorkerInfo to_ref(const kvt_worker_info& w) {
+  WorkerInfo r;
+  r.inst_id = "inst";
+  r.worker_id = 0;
+  r.engine_tp_size = w.engine_tp_size;
+  r.worker_tp_rank = w.worker_tp_rank;
+  r.block_sizes.assign(w.block_sizes, w.block_sizes + w.n_tensors);
+  r.token_sizes.assign(w.token_sizes, w.token_sizes + w.n_tensors);
+  r.layer_num_blocks = w.layer_num_blocks;
+  r.num_layers = w.num_layers;
+  r.attn_kernel_blk_ntpb = w.attn_kernel_blk_ntpb;
+  r.indexer_blk_ntpb = w.indexer_blk_ntpb;
+  r.attn_pack_size = w.attn_pack_size;
+  r.num_kv_heads = w.num_kv_heads;
+  r.num_gdn_layers = w.num_gdn_layers;
+  r.hybrid_indexer_token_size = w.hybrid_indexer_token_size;
+  r.gdn_conv_elem_size = w.gdn_conv_elem_size;
+  r.gdn_ssm_elem_size = w.gdn_ssm_elem_size;
+  r.conv_state_shape.assign(w.conv_state_shape, w.conv_state_shape + w.n_conv_state_shape);
+  r.ssm_state_shape.assign(w.ssm_state_shape, w.ssm_state_shape + w.n_ssm_state_shape);
+  r.gdn_conv_channel_dims.assign(w.gdn_conv_channel_dims,
+                                 w.gdn_conv_channel_dims + w.n_gdn_conv_channel_dims);
+  r.num_ple_layers = w.num_ple_layers;
+  r.ple_block_group = w.ple_block_group;
+  r.ple_conv_elem_size = w.ple_conv_elem_size;
+  r.ple_conv_state_shape.assign(w.ple_conv_state_shape,
+                                w.ple_conv_state_shape + w.n_ple_conv_state_shape);
+  r.ple_conv_channel_dims.assign(w.ple_conv_channel_dims,
+                                 w.ple_conv_channel_dims + w.n_ple_conv_channel_dims);
+  r.kda_conv_dim_first = w.kda_conv_dim_first != 0;
+  r.hybrid_attn_token_size = w.hybrid_attn_token_size;
+  r.kda_page_stride = w.kda_page_stride;
+  return r;
+}
+
+BlockIds to_groups(const uint32_t* ids, const uint32_t* lens, uint32_t n) {
+  BlockIds out(n);
+  size_t pos = 0;
+  for (uint32_t g = 0; g < n; ++g) {
+    out[g].assign(ids + pos, ids + pos + lens[g]);
+    pos += lens[g];
+  }
+  return out;
+}
+
+ParseBlockFunc pick(int id) {
+  switch (id) {
+    case KVT_PARSER_RAGGED_PEQD: return parse_block_send_p_eq_d;
+    case KVT_PARSER_RAGGED_PGTD: return parse_block_send_p_gt_d;
+    case KVT_PARSER_RAGGED_PGTD_DPSK: return parse_block_send_p_gt_d_dpsk;
+    case KVT_PARSER_RAGGED_PLTD: return parse_block_send_p_lt_d;
+    case KVT_PARSER_FLASH_PEQD: return vllm_parse_block_send_p_eq_d;
+    case KVT_PARSER_FLASH_PGTD: return vllm_parse_block_send_p_gt_d;
+    case KVT_PARSER_HYBRID_PEQD: return vllm_parse_hybrid_block_send_p_eq_d_block_aligned;
+    case KVT_PARSER_HYBRID_PGTD: return vllm_parse_hybrid_block_send_p_gt_d;
+    case KVT_PARSER_HYBRID_PLTD: return vllm_parse_hybrid_block_send_p_lt_d;
+    case KVT_PARSER_DPSK_PEQD: return vllm_parse_block_send_multi_tensor_p_eq_d;
+    case KVT_PARSER_DPSK_PGTD: return vllm_parse_block_send_multi_tensor_p_gt_d;
+    case KVT_PARSER_DPSK_PLTD: return vllm_parse_block_send_multi_tensor_p_lt_d;
+    case KVT_PARSER_FLASHINFER_PEQD: return vllm_parse_flashinfer_block_send_p_eq_d;
+    case KVT_PARSER_FLASHINFER_PGTD: return vllm_parse_flashinfer_block_send_p_gt_d;
+    case KVT_PARSER_HYBRID_FI_PEQD: return vllm_parse_qwen3_next_flashinfer_block_send_p_eq_d;
+    case KVT_PARSER_HYBRID_FI_PGTD: return vllm_parse_qwen3_next_flashinfer_block_send_p_gt_d;
+    case KVT_PARSER_HYBRID_FI_PLTD: return vllm_parse_qwen3_next_flashinfer_block_send_p_lt_d;
+    case KVT_PARSER_KDA_PEQD: return parse_kda_block_send_p_eq_d;
+    case KVT_PARSER_KDA_PGTD: return parse_kda_block_send_p_gt_d;
+    case KVT_PARSER_KDA_PLTD: return parse_kda_block_send_p_lt_d;
+    case KVT_PARSER_KIMI_K3_PEQD: return parse_kimi_k3_mla_block_send_p_eq_d;
+    case KVT_PARSER_KIMI_K3_PGTD: return parse_kimi_k3_mla_block_send_p_gt_d;
+    case KVT_PARSER_KIMI_K3_PLTD: return parse_kimi_k3_mla_block_send_p_lt_d;
+    case KVT_PARSER_TURBOQUANT_PEQD: return turboquant_parse_block_send_p_eq_d;
+    case KVT_PARSER_TURBOQUANT_PGTD: return turboquant_parse_block_send_p_gt_d;
+    default: return nullptr;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+// Runs the reference parser over `n_tasks` tasks, appending into one
+// send_blocks vector exactly as KvSendStub::TaskContext::do_task does
+// (kvtransfer/src/tx_stub.cpp:201-205). On success *n_tensors is the outer
+// size and out[t] / n_out[t] (t < min(*n_tensors, cap)) is a malloc'd array the
+// caller releases with kvtref_free. Returns a KVT_* code.
+int kvtref_parse(int parser_id, const kvt_worker_info* src, const kvt_worker_info* dst,
+                 uint32_t valid_mask, uint32_t kvt_tp_size, uint32_t kvt_tp_rank,
+                 const kvt_task* tasks, uint32_t n_tasks, uint32_t cap,
+                 kvt_ipc_block** out, uint64_t* n_out, uint32_t* n_tensors) {
+  ParseBlockFunc fn = pick(parser_id);
+  if (fn == nullptr) return KVT_ERR_UNSUPPORTED;
+  const WorkerInfo s = to_ref(*src);
+  const WorkerInfo d = to_ref(*dst);
+  const std::bitset<MAX_TP_SIZE> valid(valid_mask);
+  std::vector<std::vector<IpcBlock>> send_blocks;
+  try {
+    for (uint32_t i = 0; i < n_tasks; ++i) {
+      const kvt_task& t = tasks[i];
+      auto req = std::make_shared<RequestInfo>(
+          "dst", 0u, "req" + std::to_string(i),
+          to_groups(t.src_blocks, t.src_group_len, t.n_src_groups),
+          to_groups(t.dst_blocks, t.dst_group_len, t.n_dst_groups));
+      ReqSendTask task(req, t.seen_tokens, t.new_tokens, t.reach_last_token != 0);
+      fn(&s, &d, valid, kvt_tp_size, kvt_tp_rank, &task, send_blocks);
+    }
+  } catch (const std::out_of_range&) {
+    return KVT_ERR_OUT_OF_RANGE;
+  } catch (const std::overflow_error&) {
+    return KVT_ERR_OVERFLOW;
+  } catch (const std::exception&) {
+    return KVT_ERR_INVALID;
+  }
+  *n_tensors = static_cast<uint32_t>(send_blocks.size());
+  for (uint32_t t = 0; t < send_blocks.size() && t < cap; ++t) {
+    const auto& v = send_blocks[t];
+    n_out[t] = v.size();
+    out[t] = static_cast<kvt_ipc_block*>(std::malloc(sizeof(kvt_ipc_block) * (v.size() + 1)));
+    for (size_t i = 0; i < v.size(); ++i) {
+      out[t][i].src_offset = v[i].src_offset;
+      out[t][i].dst_offset = v[i].dst_offset;
+      out[t][i].length = v[i].length;
+    }
+  }
+  return KVT_OK;
+}
+
+void kvtref_free(void* p) { std::free(p); }
+
+// The two environment switches the reference latches on first use.
+int kvtref_env_bf16_to_fp8(void) { return env_bf162fp8_conversion() ? 1 : 0; }
+int kvtref_env_pad_last_attn_block(void) { return env_pad_last_attn_block() ? 1 : 0; }
+
+}  // extern "C"
