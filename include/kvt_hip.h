@@ -1,0 +1,288 @@
+/*
+ * kvt_hip.h -- C ABI of libkvt_hip.so: the MI355X (gfx950) implementation of
+ * Blade-KVT's ParseBlock + block-copy (pack / unpack) path.
+ *
+ * Conventions
+ *   - every function returns a KVT_* code (kvt_types.h); kvt_last_error() gives
+ *     the message of the calling thread's most recent failure. No exception
+ *     crosses this boundary.
+ *   - hipStream_t / hipEvent_t travel as void* so that the header needs no HIP
+ *     include; NULL stream = the device's default stream.
+ *   - "cache offset" always means a byte offset relative to one layer tensor's
+ *     base address, exactly like IpcBlock offsets in the reference.
+ *   - every GPU entry point fails with KVT_ERR_NO_DEVICE when no gfx950 device
+ *     is usable; there is no CPU fallback inside this library.
+ *
+ * Each declaration cites the reference interface it replaces (paths relative
+ * to the reference checkout).
+ */
+#ifndef KVT_HIP_H_
+#define KVT_HIP_H_
+
+#include "kvt_types.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ misc */
+
+const char* kvt_last_error(void);
+/* sizeof() of the ABI structs as compiled, for binding self-checks:
+ * which = 0 kvt_ipc_block, 1 kvt_worker_info, 2 kvt_task, 3 kvt_parse_opts,
+ * 4 kvt_xform. */
+uint64_t kvt_abi_sizeof(int which);
+/* Number of usable gfx950 devices (0 when none / no driver). */
+int kvt_device_count(void);
+
+/* ---------------------------------------------------- ParseBlock (host) */
+
+/* replaces compute_valid_ranks_pd()            kvtransfer/src/tx_stub.cpp:18-81 */
+uint32_t kvt_compute_valid_ranks_pd(uint32_t p_tp, uint32_t d_tp, int32_t num_kv_heads);
+
+/* replaces the per-destination dispatch of KvSendStub::TaskContext::
+ * refresh_dst_info()                            kvtransfer/src/tx_stub.cpp:451-590
+ * (valid ranks, effective kvt_tp_size / kvt_tp_rank, parser and TPKind).
+ * KVT_ERR_UNSUPPORTED where the reference throws "unsupported cache_shape". */
+int kvt_select_parser(int cache_shape, const kvt_worker_info* src, const kvt_worker_info* dst,
+                      uint32_t* valid_mask, uint32_t* kvt_tp_size, uint32_t* kvt_tp_rank,
+                      int* parser_id, int* tp_kind);
+
+/* A compiled parser: the per-destination part of ParseBlock (all divisions,
+ * strides and rank gating) resolved once, the way refresh_dst_info() picks a
+ * ParseBlockFunc once per destination. */
+typedef struct kvt_parser kvt_parser;
+int kvt_parser_create(int parser_id, const kvt_worker_info* src, const kvt_worker_info* dst,
+                      uint32_t valid_mask, uint32_t kvt_tp_size, uint32_t kvt_tp_rank,
+                      const kvt_parse_opts* opts, kvt_parser** out);
+void kvt_parser_destroy(kvt_parser* p);
+
+/* Growable per-tensor range lists: the C stand-in for the caller-owned
+ * std::vector<std::vector<IpcBlock>>& send_blocks of ParseBlockFunc. */
+typedef struct kvt_block_lists kvt_block_lists;
+int kvt_block_lists_create(kvt_block_lists** out);
+void kvt_block_lists_destroy(kvt_block_lists* l);
+void kvt_block_lists_clear(kvt_block_lists* l);
+uint32_t kvt_block_lists_num_tensors(const kvt_block_lists* l);
+/* Borrowed view of tensor t's list; valid until the next mutation. */
+int kvt_block_lists_view(const kvt_block_lists* l, uint32_t tensor, const kvt_ipc_block** data,
+                         uint64_t* n);
+
+/* Appends n caller-supplied ranges to tensor `tensor`'s list (growing the outer
+ * size as needed). The receiving side uses it for the IpcBlock arrays that
+ * arrive in a layer message                      kvtransfer/src/tcp_channel.cpp:190-221. */
+int kvt_block_lists_append(kvt_block_lists* l, uint32_t tensor, const kvt_ipc_block* blocks,
+                           uint64_t n);
+
+/* replaces one ParseBlockFunc call              kvtransfer/include/parse_block_common.h:86-94
+ * as issued per request by do_task()            kvtransfer/src/tx_stub.cpp:201-205.
+ * APPENDS the task's ranges to `lists` (outer size grows to the parser's
+ * tensor count). Errors: KVT_ERR_OUT_OF_RANGE where the reference throws
+ * std::out_of_range (range validation of append_ipc_block_checked,
+ * parse_block_common.h:31-68; bad block index), KVT_ERR_OVERFLOW for the
+ * capacity overflow (parse_block_common.cpp:20-29). On error the lists keep
+ * whatever was appended before the failing range, like the reference. */
+int kvt_parse_block(const kvt_parser* p, const kvt_task* task, kvt_block_lists* lists);
+
+/* replaces merge_interval() + the erase of zero-length entries its callers do
+ *                                               kvtransfer/src/channel.cpp:53-98,
+ *                                               kvtransfer/src/tcp_channel.cpp:376-392
+ * In place; returns the compacted count in *n_out and {min,max,total,count}
+ * in stats (may be NULL). Sorting is stable on src_offset. */
+int kvt_merge_interval(kvt_ipc_block* blocks, uint64_t n, uint64_t* n_out, uint64_t stats[4]);
+/* Same, applied to every tensor of `lists` (what register_data does for PEQD). */
+int kvt_block_lists_merge(kvt_block_lists* l);
+
+/* replaces validate_ipc_block_bounds()          kvtransfer/src/channel.cpp:11-50
+ * which: 0 = check src_offset, 1 = check dst_offset. *bad_idx (may be NULL)
+ * receives the first offending index. */
+int kvt_validate_ipc_block_bounds(const kvt_ipc_block* blocks, uint64_t n, uint64_t capacity,
+                                  int which, uint64_t length_scale, uint64_t* bad_idx);
+
+/* ------------------------------------------- registered cache (device) */
+
+/* The `layers[layer][tensor]` base pointers Python hands to
+ * init_kv_transfer_client                       kvtransfer/kvtransfer_pybind.cpp:131-199
+ * (flattened by _flatten_cache,                 blade_kvt/hybrid_connector/kvtbackend.py:594-629).
+ * ptrs is a host array of n_layers * n_tensors device pointers
+ * (ptrs[layer * n_tensors + tensor]); capacity[t] is tensor t's size in bytes
+ * (block_sizes[t] * layer_num_blocks). The table is copied to the device once. */
+typedef struct kvt_cache kvt_cache;
+int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, uint32_t n_tensors,
+                       const uint64_t* capacity, kvt_cache** out);
+void kvt_cache_destroy(kvt_cache* c);
+
+/* --------------------------------------------------- copy plan (device) */
+
+/* Optional intra-page layout transform applied while packing / unpacking.
+ * KVT_XFORM_HND_NHD: the cache holds pages [2][heads][ntpb][row_bytes] (FlashInfer
+ * HND) while the packed buffer holds them [2][ntpb][heads][row_bytes] (NHD).
+ * Only valid for plans whose ranges are whole pages (page_bytes = 2 * heads *
+ * ntpb * row_bytes, offsets and lengths multiples of it). The reference has no
+ * layout-changing copy; this is an addition of this library. */
+enum { KVT_XFORM_NONE = 0, KVT_XFORM_HND_NHD = 1 };
+typedef struct kvt_xform {
+  uint32_t kind;
+  uint32_t heads;
+  uint32_t ntpb;
+  uint32_t row_bytes;
+} kvt_xform;
+
+/* A plan = the batch's merged range lists, split into bounded chunks and made
+ * resident on the device once; every layer of the step replays it. Replaces
+ * what IChannel::register_data() prepares      kvtransfer/src/tcp_channel.cpp:348-475
+ * and the per-launch metadata upload of copy_handle_data_kernel_direct()
+ *                                               kvtransfer/src/copy_kernels.cpp:363-439.
+ *
+ * `lists` is consumed as-is (call kvt_block_lists_merge first for PEQD).
+ * src_capacity / dst_capacity: per-tensor byte sizes the ranges were validated
+ * against; pack refuses a cache smaller than src_capacity, unpack one smaller
+ * than dst_capacity. chunk_bytes = 0 selects the default. */
+typedef struct kvt_plan kvt_plan;
+int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
+                    const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
+                    kvt_plan** out);
+void kvt_plan_destroy(kvt_plan* p);
+uint32_t kvt_plan_num_tensors(const kvt_plan* p);
+uint64_t kvt_plan_num_chunks(const kvt_plan* p);
+/* Packed bytes of tensor t in one layer (sum of its range lengths), and the
+ * byte offset of its blob inside a layer's packed area (blobs are laid out
+ * back to back, each start rounded up to 256 bytes). */
+uint64_t kvt_plan_tensor_bytes(const kvt_plan* p, uint32_t tensor);
+uint64_t kvt_plan_tensor_offset(const kvt_plan* p, uint32_t tensor);
+/* Bytes one layer occupies in the packed buffer (incl. the rounding above). */
+uint64_t kvt_plan_layer_bytes(const kvt_plan* p);
+
+/* Pack = TCPChannel::send_data body             kvtransfer/src/tcp_channel.cpp:517-560
+ * (+ RDMAStagedChannel::send_data               kvtransfer/src/rdma_staged_channel.cpp:246-265):
+ * for layers [first_layer, first_layer + n_layers): tensor t's blob =
+ * concatenation of cache[src_offset : +length] in list order, written to
+ * packed + (layer - first_layer) * layer_stride + kvt_plan_tensor_offset(t).
+ * One kernel launch for all requested layers; asynchronous on `stream`.
+ * `packed` may be device memory or device-visible pinned host memory. */
+int kvt_pack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, uint32_t n_layers,
+             void* packed, uint64_t layer_stride, void* stream);
+
+/* Unpack = TCPServer handle_kv_cache_data       kvtransfer/src/tcp_channel.cpp:190-261
+ * (+ RDMAStagedServer                           kvtransfer/src/rdma_staged_server.cpp:441-463):
+ * cache[dst_offset : +length] = next `length` bytes of the blob. */
+int kvt_unpack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, uint32_t n_layers,
+               const void* packed, uint64_t layer_stride, void* stream);
+
+/* --------------------------- drop-ins for the reference copy entry points */
+
+/* replaces launch_copy_d2h_direct_kernel()      kvtransfer/src/copy_kernels.cu:268-281
+ * gather: dst[dst_offsets[i] : +lengths[i]] = gpu_src_base[src_offsets[i] : ...].
+ * The three arrays live in device memory. num_wg / threads_per_wg <= 0 pick
+ * this library's launch shape. */
+int kvt_launch_copy_d2h_direct(const void* gpu_src_base, void* dst, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream);
+/* replaces launch_copy_h2d_direct_kernel()      kvtransfer/src/copy_kernels.cu:179-192 */
+int kvt_launch_copy_h2d_direct(const void* src, void* gpu_dst_base, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream);
+/* replaces launch_copy_d2h_bf16_to_fp8_kernel() kvtransfer/src/copy_kernels.cu:467-481
+ * lengths are ELEMENT counts, src offsets in bf16 bytes, dst offsets in fp8 bytes. */
+int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
+                                    const int64_t* src_offsets, const int64_t* dst_offsets,
+                                    const int64_t* lengths, int64_t n, int num_wg,
+                                    int threads_per_wg, void* stream);
+
+enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
+/* replaces copy_handle_data_with_kernel()       kvtransfer/include/copy_kernels.h:87-97,
+ *                                               kvtransfer/src/copy_kernels.cpp:733-827
+ * Same calling convention: blocks[i].dst_offset is the GPU-side offset for BOTH
+ * directions, the contiguous side advances by blocks[i].length (running sum),
+ * tensor_data_size must equal the sum of lengths. dev_meta / host_meta are the
+ * caller's metadata buffers (>= 3 * 8 * max_block_num bytes each, host_meta
+ * pinned); more than max_block_num ranges are processed in batches with a
+ * stream synchronisation after each, like the reference. max_block_num <= 0
+ * means 8192 (BLLM_KVTRANS_KERNEL_COPY_MAX_BLOCK_NUM's default). */
+int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
+                                     const kvt_ipc_block* blocks, uint64_t n,
+                                     uint64_t tensor_data_size, int direction, int device,
+                                     void* stream, int64_t* dev_meta, int64_t* host_meta,
+                                     int64_t max_block_num);
+/* replaces copy_d2h_bf16_to_fp8()               kvtransfer/include/copy_kernels.h:112-121,
+ *                                               kvtransfer/src/copy_kernels.cpp:833-959
+ * blocks[i].length = bf16 bytes at the source; the contiguous side receives
+ * length / 2 fp8 (E4M3, round-to-nearest-even, saturating) bytes per range. */
+int kvt_copy_d2h_bf16_to_fp8(void* tensor_buf, const void* layer_gpu_ptr,
+                             const kvt_ipc_block* blocks, uint64_t n, uint64_t tensor_data_size,
+                             int device, void* stream, int64_t* dev_meta, int64_t* host_meta,
+                             int64_t max_block_num);
+
+/* ------------------------------------- per-layer gating on a side stream */
+
+/* Replaces Step / StepGuard / CudaEventBarrier  kvtransfer/include/step.h, src/step.cpp:49-69,
+ *                                               kvtransfer/src/context.cpp:18-20
+ * and the host-side wait in do_send()           kvtransfer/src/tx_stub.cpp:395-415:
+ * the reference parks a host thread in cudaEventSynchronize per layer; here the
+ * dependency stays on the device (event record on the compute stream, stream
+ * wait on a side stream, pack launch, done event), so the sequence can be
+ * captured into a hipGraph together with the forward pass. */
+typedef struct kvt_session kvt_session;
+int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packed,
+                       uint64_t layer_stride, kvt_session** out);
+void kvt_session_destroy(kvt_session* s);
+/* save_kv_layer hook: layer `layer` of the cache is complete once the work
+ * already queued on compute_stream has run. Never blocks the host. */
+int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream);
+/* Host-blocking wait until layer's packed bytes are complete (what the
+ * transport thread calls before send_data(layer)); not capturable. */
+int kvt_session_wait_layer(kvt_session* s, uint32_t layer);
+/* Makes `stream` wait for every pack issued so far (joins the side stream
+ * back; required before ending a capture that included save_layer calls). */
+int kvt_session_join(kvt_session* s, void* stream);
+/* hipStream_t of the side stream (for tests / profiling). */
+void* kvt_session_side_stream(kvt_session* s);
+
+/* ------------------------------------ pinned-host staging (KVStore path) */
+
+/* A ring of pinned host slots fed by hipMemcpyAsync on its own copy stream, so
+ * that D2H of layer L overlaps the pack of layer L+1 (and H2D of L+1 overlaps
+ * the unpack of L). Stands where the reference's KVStore backends hand packed
+ * layers to a host-side store                   blade_kvt/hybrid_connector/kvsbackend.py:268-357,
+ *                                               blade_kvt/hybrid_connector/file_backend.py:222-283.
+ * slot_bytes bounds one transfer; n_slots >= 2. */
+typedef struct kvt_stager kvt_stager;
+int kvt_stager_create(int device, uint64_t slot_bytes, uint32_t n_slots, kvt_stager** out);
+void kvt_stager_destroy(kvt_stager* s);
+void* kvt_stager_slot(kvt_stager* s, uint32_t slot);
+void* kvt_stager_copy_stream(kvt_stager* s);
+/* Device -> slot: waits (on the copy stream) for everything queued on
+ * `producer_stream`, then copies `bytes` from dev into the slot. */
+int kvt_stager_save(kvt_stager* s, uint32_t slot, const void* dev, uint64_t bytes,
+                    void* producer_stream);
+/* Slot -> device on the copy stream, then makes consumer_stream wait for it. */
+int kvt_stager_load(kvt_stager* s, uint32_t slot, void* dev, uint64_t bytes,
+                    void* consumer_stream);
+/* Host-blocking: the slot's last save/load has completed. */
+int kvt_stager_wait(kvt_stager* s, uint32_t slot);
+/* Measured plain pinned<->device copy rate in bytes/s (direction: KVT_COPY_*),
+ * the ceiling the staging path is reported against. */
+int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats,
+                     double* bytes_per_s);
+
+/* ------------------------------------------------------------- utilities */
+
+/* Plain device-to-device copy kernel with the same vector width and launch
+ * shape as the gather kernel; used to calibrate profiler counters and as the
+ * "no scatter" bandwidth reference. */
+int kvt_copy_linear(void* dst, const void* src, uint64_t bytes, void* stream);
+/* Average duration in milliseconds of the GPU work queued on `stream` between
+ * two internally created events around `fn`-less region helpers: */
+int kvt_event_create(void** ev);
+int kvt_event_destroy(void* ev);
+int kvt_event_record(void* ev, void* stream);
+int kvt_event_synchronize(void* ev);
+int kvt_event_elapsed_ms(void* start, void* stop, float* ms);
+int kvt_stream_create(void** stream);
+int kvt_stream_destroy(void* stream);
+int kvt_stream_synchronize(void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* KVT_HIP_H_ */

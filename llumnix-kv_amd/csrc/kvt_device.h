@@ -1,0 +1,46 @@
+// Types and launcher declarations shared between the HIP translation units.
+#ifndef KVT_DEVICE_H_
+#define KVT_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace kvt {
+
+// One bounded piece of a range, resident in device memory. 32 bytes.
+struct __attribute__((aligned(16))) Chunk {
+  uint64_t cache_src;  // byte offset in the sender-side layer tensor (pack reads here)
+  uint64_t cache_dst;  // byte offset in the receiver-side layer tensor (unpack writes here)
+  uint64_t packed;     // byte offset inside one layer's packed area
+  uint32_t len;        // bytes
+  uint16_t tensor;     // cache tensor index within the layer
+  uint16_t t0;         // layout transform only: first token of the half page covered
+};
+static_assert(sizeof(Chunk) == 32, "Chunk must stay 32 bytes");
+
+// Device-side constants of the HND <-> NHD page transform.
+struct XformDev {
+  uint32_t heads, ntpb, vrow;     // vrow = 16-byte vectors per (token, head) row
+  uint32_t inv_vrow, inv_heads;   // floor(2^32 / d) + 1: exact quotients for operands < 2^16
+};
+
+hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
+                              uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                              uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                              hipStream_t stream);
+hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
+                               uint8_t* const* layer_ptrs, uint32_t n_tensors,
+                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
+                               uint64_t layer_stride, const XformDev& x, hipStream_t stream);
+hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
+                              const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,
+                              int parts, bool wave_per_range, hipStream_t stream);
+hipError_t launch_convert_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
+                                 const int64_t* dst_off, const int64_t* lens, int64_t n,
+                                 int num_wg, int parts, hipStream_t stream);
+hipError_t launch_copy_linear(void* dst, const void* src, uint64_t bytes, hipStream_t stream);
+
+}  // namespace kvt
+
+#endif  // KVT_DEVICE_H_

@@ -1,0 +1,750 @@
+// Host side of the device path: registered caches, copy plans, pack / unpack
+// launches, the reference-shaped copy entry points, per-layer gating sessions
+// and pinned-host staging.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "kvt_device.h"
+#include "kvt_internal.h"
+
+namespace kvt {
+namespace {
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(KVT_ERR_HIP, std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define KVT_HIP(call)                                  \
+  do {                                                 \
+    const hipError_t _e = (call);                      \
+    if (_e != hipSuccess) return hip_fail(_e, #call);  \
+  } while (0)
+
+// Number of devices, or a negative KVT error. Only gfx950 parts are accepted:
+// the code objects in this library are built for that target alone.
+int usable_devices() {
+  static int cached = -2;
+  static std::once_flag once;
+  std::call_once(once, []() {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      cached = 0;
+      return;
+    }
+    int ok = 0;
+    for (int i = 0; i < n; ++i) {
+      hipDeviceProp_t p;
+      if (hipGetDeviceProperties(&p, i) != hipSuccess) break;
+      if (std::strncmp(p.gcnArchName, "gfx950", 6) != 0) break;
+      ++ok;
+    }
+    cached = ok;
+  });
+  return cached;
+}
+
+int check_device(int device) {
+  const int n = usable_devices();
+  if (n <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+  if (device < 0 || device >= n) return fail(KVT_ERR_INVALID, "device index out of range");
+  return KVT_OK;
+}
+
+struct DeviceGuard {
+  int prev = -1;
+  bool switched = false;
+  int enter(int device) {
+    if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+    if (prev != device) {
+      const hipError_t e = hipSetDevice(device);
+      if (e != hipSuccess) return hip_fail(e, "hipSetDevice");
+      switched = true;
+    }
+    return KVT_OK;
+  }
+  ~DeviceGuard() {
+    if (switched && prev >= 0) (void)hipSetDevice(prev);
+  }
+};
+
+uint64_t round_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+constexpr uint32_t kDefaultChunk = 32768;
+constexpr uint64_t kBlobAlign = 256;
+
+}  // namespace
+}  // namespace kvt
+
+using namespace kvt;
+
+struct kvt_cache {
+  int device = 0;
+  uint32_t n_layers = 0, n_tensors = 0;
+  std::vector<uint64_t> capacity;
+  std::vector<void*> host_ptrs;
+  uint8_t** dev_ptrs = nullptr;
+};
+
+struct kvt_plan {
+  int device = 0;
+  uint32_t n_tensors = 0;
+  uint64_t n_chunks = 0;
+  std::vector<uint64_t> tensor_bytes, tensor_offset, src_cap, dst_cap;
+  uint64_t layer_bytes = 0;
+  bool xform = false;
+  XformDev xdev{};
+  Chunk* dev_chunks = nullptr;
+};
+
+struct kvt_session {
+  const kvt_plan* plan = nullptr;
+  const kvt_cache* cache = nullptr;
+  void* packed = nullptr;
+  uint64_t layer_stride = 0;
+  hipStream_t side = nullptr;
+  std::vector<hipEvent_t> ready, done;
+  hipEvent_t last_done = nullptr;
+};
+
+struct kvt_stager {
+  int device = 0;
+  uint64_t slot_bytes = 0;
+  uint32_t n_slots = 0;
+  uint8_t* pinned = nullptr;
+  hipStream_t copy = nullptr;
+  std::vector<hipEvent_t> slot_done;
+  hipEvent_t fence = nullptr;
+};
+
+extern "C" {
+
+int kvt_device_count(void) { return std::max(0, usable_devices()); }
+
+// ------------------------------------------------------------------- cache
+
+int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, uint32_t n_tensors,
+                       const uint64_t* capacity, kvt_cache** out) {
+  return guarded([&]() -> int {
+    if (!ptrs || !capacity || !out || n_layers == 0 || n_tensors == 0)
+      return fail(KVT_ERR_INVALID, "kvt_cache_register: bad argument");
+    if (n_tensors > KVT_MAX_TENSORS)
+      return fail(KVT_ERR_INVALID, "kvt_cache_register: too many tensors per layer");
+    if (int rc = check_device(device)) return rc;
+    const uint64_t n = static_cast<uint64_t>(n_layers) * n_tensors;
+    for (uint64_t i = 0; i < n; ++i)
+      if (!ptrs[i]) return fail(KVT_ERR_INVALID, "kvt_cache_register: null layer pointer");
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    std::unique_ptr<kvt_cache> c(new kvt_cache());
+    c->device = device;
+    c->n_layers = n_layers;
+    c->n_tensors = n_tensors;
+    c->capacity.assign(capacity, capacity + n_tensors);
+    c->host_ptrs.resize(n);
+    for (uint64_t i = 0; i < n; ++i) c->host_ptrs[i] = const_cast<void*>(ptrs[i]);
+    KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c->dev_ptrs), n * sizeof(void*)));
+    const hipError_t e =
+        hipMemcpy(c->dev_ptrs, c->host_ptrs.data(), n * sizeof(void*), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      (void)hipFree(c->dev_ptrs);
+      return hip_fail(e, "hipMemcpy(layer pointer table)");
+    }
+    *out = c.release();
+    return KVT_OK;
+  });
+}
+
+void kvt_cache_destroy(kvt_cache* c) {
+  if (!c) return;
+  if (c->dev_ptrs) (void)hipFree(c->dev_ptrs);
+  delete c;
+}
+
+// -------------------------------------------------------------------- plan
+
+int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
+                    const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
+                    kvt_plan** out) {
+  return guarded([&]() -> int {
+    if (!lists || !src_capacity || !dst_capacity || !out)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create: null argument");
+    if (lists->tensors.empty() || lists->tensors.size() > KVT_MAX_TENSORS)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create: tensor count out of range");
+    if (int rc = check_device(device)) return rc;
+    if (chunk_bytes == 0) chunk_bytes = kDefaultChunk;
+    if (chunk_bytes % 256 != 0 || chunk_bytes > (1u << 20))
+      return fail(KVT_ERR_INVALID, "kvt_plan_create: chunk_bytes must be a multiple of 256, <= 1 MiB");
+
+    std::unique_ptr<kvt_plan> p(new kvt_plan());
+    p->device = device;
+    p->n_tensors = static_cast<uint32_t>(lists->tensors.size());
+    p->src_cap.assign(src_capacity, src_capacity + p->n_tensors);
+    p->dst_cap.assign(dst_capacity, dst_capacity + p->n_tensors);
+
+    uint64_t half = 0, tok_bytes = 0;
+    if (xform && xform->kind != KVT_XFORM_NONE) {
+      if (xform->kind != KVT_XFORM_HND_NHD) return fail(KVT_ERR_INVALID, "unknown layout transform");
+      if (p->n_tensors != 1) return fail(KVT_ERR_INVALID, "layout transform needs a single tensor");
+      if (xform->heads == 0 || xform->ntpb == 0 || xform->row_bytes == 0 ||
+          xform->row_bytes % 16 != 0 || xform->ntpb > 65535 || xform->heads > 65535)
+        return fail(KVT_ERR_INVALID, "layout transform: rows must be multiples of 16 bytes");
+      tok_bytes = static_cast<uint64_t>(xform->heads) * xform->row_bytes;
+      half = tok_bytes * xform->ntpb;
+      if (tok_bytes > (1u << 19)) return fail(KVT_ERR_INVALID, "layout transform: token row too large");
+      p->xform = true;
+      p->xdev.heads = xform->heads;
+      p->xdev.ntpb = xform->ntpb;
+      p->xdev.vrow = xform->row_bytes / 16;
+      p->xdev.inv_vrow = static_cast<uint32_t>((1ull << 32) / p->xdev.vrow) + 1u;
+      p->xdev.inv_heads = static_cast<uint32_t>((1ull << 32) / p->xdev.heads) + 1u;
+    }
+
+    std::vector<Chunk> chunks;
+    uint64_t cursor = 0;
+    for (uint32_t t = 0; t < p->n_tensors; ++t) {
+      cursor = round_up(cursor, kBlobAlign);
+      p->tensor_offset.push_back(cursor);
+      uint64_t bad = 0;
+      const RunList& runs = lists->tensors[t];
+      if (kvt_validate_ipc_block_bounds(runs.data(), runs.size(), p->src_cap[t], 0, 1, &bad) ||
+          kvt_validate_ipc_block_bounds(runs.data(), runs.size(), p->dst_cap[t], 1, 1, &bad))
+        return fail(KVT_ERR_OUT_OF_RANGE, "kvt_plan_create: range " + std::to_string(bad) +
+                                              " of tensor " + std::to_string(t) +
+                                              " exceeds the stated capacity");
+      uint64_t blob = 0;
+      for (const kvt_ipc_block& r : runs) {
+        if (!p->xform) {
+          for (uint64_t o = 0; o < r.length; o += chunk_bytes) {
+            Chunk c{};
+            c.cache_src = r.src_offset + o;
+            c.cache_dst = r.dst_offset + o;
+            c.packed = cursor + blob + o;
+            c.len = static_cast<uint32_t>(std::min<uint64_t>(chunk_bytes, r.length - o));
+            c.tensor = static_cast<uint16_t>(t);
+            chunks.push_back(c);
+          }
+        } else {
+          const uint64_t page = 2 * half;
+          if (r.src_offset % page || r.dst_offset % page || r.length % page)
+            return fail(KVT_ERR_INVALID, "layout transform: ranges must be whole pages");
+          const uint32_t tok_per_chunk =
+              static_cast<uint32_t>(std::max<uint64_t>(1, std::min<uint64_t>(chunk_bytes, 1u << 19) / tok_bytes));
+          for (uint64_t o = 0; o < r.length; o += half) {  // one K or V half page at a time
+            for (uint32_t t0 = 0; t0 < xform->ntpb; t0 += tok_per_chunk) {
+              const uint32_t nt = std::min(tok_per_chunk, xform->ntpb - t0);
+              Chunk c{};
+              c.cache_src = r.src_offset + o;
+              c.cache_dst = r.dst_offset + o;
+              c.packed = cursor + blob + o + static_cast<uint64_t>(t0) * tok_bytes;
+              c.len = static_cast<uint32_t>(nt * tok_bytes);
+              c.tensor = 0;
+              c.t0 = static_cast<uint16_t>(t0);
+              chunks.push_back(c);
+            }
+          }
+        }
+        blob += r.length;
+      }
+      p->tensor_bytes.push_back(blob);
+      cursor += blob;
+    }
+    p->layer_bytes = round_up(cursor, kBlobAlign);
+    p->n_chunks = chunks.size();
+    if (p->n_chunks > 0x7FFFFFFFull) return fail(KVT_ERR_INVALID, "kvt_plan_create: too many chunks");
+
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    if (!chunks.empty()) {
+      KVT_HIP(hipMalloc(reinterpret_cast<void**>(&p->dev_chunks), chunks.size() * sizeof(Chunk)));
+      const hipError_t e = hipMemcpy(p->dev_chunks, chunks.data(), chunks.size() * sizeof(Chunk),
+                                     hipMemcpyHostToDevice);
+      if (e != hipSuccess) {
+        (void)hipFree(p->dev_chunks);
+        return hip_fail(e, "hipMemcpy(chunk table)");
+      }
+    }
+    *out = p.release();
+    return KVT_OK;
+  });
+}
+
+void kvt_plan_destroy(kvt_plan* p) {
+  if (!p) return;
+  if (p->dev_chunks) (void)hipFree(p->dev_chunks);
+  delete p;
+}
+
+uint32_t kvt_plan_num_tensors(const kvt_plan* p) { return p ? p->n_tensors : 0; }
+uint64_t kvt_plan_num_chunks(const kvt_plan* p) { return p ? p->n_chunks : 0; }
+uint64_t kvt_plan_tensor_bytes(const kvt_plan* p, uint32_t t) {
+  return (p && t < p->n_tensors) ? p->tensor_bytes[t] : 0;
+}
+uint64_t kvt_plan_tensor_offset(const kvt_plan* p, uint32_t t) {
+  return (p && t < p->n_tensors) ? p->tensor_offset[t] : 0;
+}
+uint64_t kvt_plan_layer_bytes(const kvt_plan* p) { return p ? p->layer_bytes : 0; }
+
+static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer,
+                    uint32_t n_layers, void* packed, uint64_t layer_stride, void* stream) {
+  if (!p || !cache || (!packed && p->n_chunks))
+    return fail(KVT_ERR_INVALID, "kvt_pack/unpack: null argument");
+  if (p->device != cache->device) return fail(KVT_ERR_INVALID, "plan and cache are on different devices");
+  if (p->n_tensors != cache->n_tensors)
+    return fail(KVT_ERR_INVALID, "plan and cache disagree on tensors per layer");
+  if (static_cast<uint64_t>(first_layer) + n_layers > cache->n_layers)
+    return fail(KVT_ERR_OUT_OF_RANGE, "layer range exceeds the registered cache");
+  if (n_layers > 65535) return fail(KVT_ERR_INVALID, "at most 65535 layers per launch");
+  if (n_layers > 1 && layer_stride < p->layer_bytes)
+    return fail(KVT_ERR_INVALID, "layer_stride smaller than one packed layer");
+  const std::vector<uint64_t>& need = pack ? p->src_cap : p->dst_cap;
+  for (uint32_t t = 0; t < p->n_tensors; ++t)
+    if (cache->capacity[t] < need[t])
+      return fail(KVT_ERR_OUT_OF_RANGE, "registered cache is smaller than the plan's capacity");
+  DeviceGuard g;
+  if (int rc = g.enter(p->device)) return rc;
+  const hipStream_t s = static_cast<hipStream_t>(stream);
+  const hipError_t e =
+      p->xform ? launch_xform_chunks(pack, p->dev_chunks, static_cast<uint32_t>(p->n_chunks),
+                                     cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
+                                     static_cast<uint8_t*>(packed), layer_stride, p->xdev, s)
+               : launch_copy_chunks(pack, p->dev_chunks, static_cast<uint32_t>(p->n_chunks),
+                                    cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
+                                    static_cast<uint8_t*>(packed), layer_stride, s);
+  if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
+  return KVT_OK;
+}
+
+int kvt_pack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, uint32_t n_layers,
+             void* packed, uint64_t layer_stride, void* stream) {
+  return guarded([&]() { return run_plan(true, p, cache, first_layer, n_layers, packed, layer_stride, stream); });
+}
+
+int kvt_unpack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, uint32_t n_layers,
+               const void* packed, uint64_t layer_stride, void* stream) {
+  return guarded([&]() {
+    return run_plan(false, p, cache, first_layer, n_layers, const_cast<void*>(packed), layer_stride, stream);
+  });
+}
+
+// ------------------------------------------- reference-shaped entry points
+
+static int range_launch_shape(int64_t n, int num_wg, int* wgs) {
+  if (n > 0x7FFFFFFFll) return fail(KVT_ERR_INVALID, "too many ranges");
+  int w = num_wg > 0 ? num_wg : static_cast<int>(std::min<int64_t>(n, 16384));
+  *wgs = std::max(1, w);
+  return KVT_OK;
+}
+
+static int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so,
+                         const int64_t* dof, const int64_t* len, int64_t n, int num_wg,
+                         int threads_per_wg, void* stream) {
+  (void)threads_per_wg;  // workgroups are always 256 lanes (4 wavefronts)
+  if (n == 0) return KVT_OK;
+  if (n < 0 || !src || !dst || !so || !dof || !len)
+    return fail(KVT_ERR_INVALID, "launch_copy: bad argument");
+  if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+  int wgs = 0;
+  if (int rc = range_launch_shape(n, num_wg, &wgs)) return rc;
+  // With fewer ranges than a wave of workgroups fills the chip, cut each range
+  // into parts so that about 2048 workgroups exist.
+  int parts = 1;
+  if (n < 2048) parts = static_cast<int>(std::min<int64_t>(64, (2048 + n - 1) / n));
+  const hipStream_t s = static_cast<hipStream_t>(stream);
+  const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, parts, s)
+                               : launch_copy_ranges(src, dst, so, dof, len, n, wgs, parts, false, s);
+  if (e != hipSuccess) return hip_fail(e, "range copy launch");
+  return KVT_OK;
+}
+
+int kvt_launch_copy_d2h_direct(const void* gpu_src_base, void* dst, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(false, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+int kvt_launch_copy_h2d_direct(const void* src, void* gpu_dst_base, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(false, src, gpu_dst_base, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
+                                    const int64_t* src_offsets, const int64_t* dst_offsets,
+                                    const int64_t* lengths, int64_t n, int num_wg,
+                                    int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(true, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+// Shared body of the two "handle data" entry points. `halve`: converting
+// gather (contiguous side advances by length / 2, lengths passed to the kernel
+// are element counts).
+static int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks,
+                       uint64_t n, uint64_t tensor_data_size, int direction, bool halve,
+                       int device, void* stream, int64_t* dev_meta, int64_t* host_meta,
+                       int64_t max_block_num) {
+  if (n == 0) return KVT_OK;
+  if (!tensor_buf || !layer_gpu_ptr || !blocks || !dev_meta || !host_meta)
+    return fail(KVT_ERR_INVALID, "copy_handle_data: null argument");
+  if (direction != KVT_COPY_H2D && direction != KVT_COPY_D2H)
+    return fail(KVT_ERR_INVALID, "copy_handle_data: bad direction");
+  if (int rc = check_device(device)) return rc;
+  if (max_block_num <= 0) max_block_num = 8192;
+  uint64_t total = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    if (blocks[i].length == 0) return fail(KVT_ERR_INVALID, "copy_handle_data: zero-length range");
+    if (halve && (blocks[i].length & 1)) return fail(KVT_ERR_INVALID, "odd bf16 byte length");
+    total += blocks[i].length;
+  }
+  if (total != tensor_data_size)
+    return fail(KVT_ERR_INVALID, "copy_handle_data: tensor_data_size != sum of range lengths");
+  DeviceGuard g;
+  if (int rc = g.enter(device)) return rc;
+  const hipStream_t s = static_cast<hipStream_t>(stream);
+  uint64_t host_cursor = 0;
+  for (uint64_t first = 0; first < n; first += static_cast<uint64_t>(max_block_num)) {
+    const uint64_t m = std::min<uint64_t>(static_cast<uint64_t>(max_block_num), n - first);
+    int64_t* contig = host_meta;
+    int64_t* gpu = host_meta + m;
+    int64_t* lens = host_meta + 2 * m;
+    uint64_t longest = 0;
+    for (uint64_t i = 0; i < m; ++i) {
+      const kvt_ipc_block& b = blocks[first + i];
+      contig[i] = static_cast<int64_t>(host_cursor);
+      gpu[i] = static_cast<int64_t>(b.dst_offset);
+      lens[i] = static_cast<int64_t>(halve ? b.length / 2 : b.length);
+      host_cursor += halve ? b.length / 2 : b.length;
+      longest = std::max<uint64_t>(longest, b.length);
+    }
+    KVT_HIP(hipMemcpyAsync(dev_meta, host_meta, 3 * m * sizeof(int64_t), hipMemcpyHostToDevice, s));
+    const int64_t* d_contig = dev_meta;
+    const int64_t* d_gpu = dev_meta + m;
+    const int64_t* d_lens = dev_meta + 2 * m;
+    const int wgs = static_cast<int>(std::min<uint64_t>(m, 16384));
+    // about 32 KiB per workgroup, but enough workgroups to cover the chip
+    uint64_t parts = std::max<uint64_t>(1, (longest + 32767) / 32768);
+    if (m * parts < 2048) parts = std::min<uint64_t>(64, (2048 + m - 1) / m);
+    parts = std::min<uint64_t>(parts, 1024);
+    hipError_t e;
+    if (halve)
+      e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
+                                static_cast<int64_t>(m), wgs, static_cast<int>(parts), s);
+    else if (direction == KVT_COPY_D2H)
+      e = launch_copy_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
+                             static_cast<int64_t>(m), wgs, static_cast<int>(parts), false, s);
+    else
+      e = launch_copy_ranges(tensor_buf, layer_gpu_ptr, d_contig, d_gpu, d_lens,
+                             static_cast<int64_t>(m), wgs, static_cast<int>(parts), false, s);
+    if (e != hipSuccess) return hip_fail(e, "copy_handle_data launch");
+    // the metadata buffers are reused by the next batch
+    if (first + m < n) KVT_HIP(hipStreamSynchronize(s));
+  }
+  return KVT_OK;
+}
+
+int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
+                                     const kvt_ipc_block* blocks, uint64_t n,
+                                     uint64_t tensor_data_size, int direction, int device,
+                                     void* stream, int64_t* dev_meta, int64_t* host_meta,
+                                     int64_t max_block_num) {
+  return guarded([&]() {
+    return handle_data(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction, false,
+                       device, stream, dev_meta, host_meta, max_block_num);
+  });
+}
+
+int kvt_copy_d2h_bf16_to_fp8(void* tensor_buf, const void* layer_gpu_ptr,
+                             const kvt_ipc_block* blocks, uint64_t n, uint64_t tensor_data_size,
+                             int device, void* stream, int64_t* dev_meta, int64_t* host_meta,
+                             int64_t max_block_num) {
+  return guarded([&]() {
+    return handle_data(tensor_buf, const_cast<void*>(layer_gpu_ptr), blocks, n, tensor_data_size,
+                       KVT_COPY_D2H, true, device, stream, dev_meta, host_meta, max_block_num);
+  });
+}
+
+// ----------------------------------------------------------------- session
+
+int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packed,
+                       uint64_t layer_stride, kvt_session** out) {
+  return guarded([&]() -> int {
+    if (!plan || !cache || !packed || !out)
+      return fail(KVT_ERR_INVALID, "kvt_session_create: null argument");
+    if (layer_stride < plan->layer_bytes)
+      return fail(KVT_ERR_INVALID, "kvt_session_create: layer_stride smaller than one packed layer");
+    if (int rc = check_device(plan->device)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(plan->device)) return rc;
+    std::unique_ptr<kvt_session> s(new kvt_session());
+    s->plan = plan;
+    s->cache = cache;
+    s->packed = packed;
+    s->layer_stride = layer_stride;
+    KVT_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));
+    s->ready.resize(cache->n_layers);
+    s->done.resize(cache->n_layers);
+    for (uint32_t l = 0; l < cache->n_layers; ++l) {
+      KVT_HIP(hipEventCreateWithFlags(&s->ready[l], hipEventDisableTiming));
+      KVT_HIP(hipEventCreateWithFlags(&s->done[l], hipEventDisableTiming));
+    }
+    *out = s.release();
+    return KVT_OK;
+  });
+}
+
+void kvt_session_destroy(kvt_session* s) {
+  if (!s) return;
+  if (s->side) {
+    (void)hipStreamSynchronize(s->side);
+    (void)hipStreamDestroy(s->side);
+  }
+  for (hipEvent_t e : s->ready)
+    if (e) (void)hipEventDestroy(e);
+  for (hipEvent_t e : s->done)
+    if (e) (void)hipEventDestroy(e);
+  delete s;
+}
+
+int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_save_layer: null session");
+    if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    DeviceGuard g;
+    if (int rc = g.enter(s->plan->device)) return rc;
+    KVT_HIP(hipEventRecord(s->ready[layer], static_cast<hipStream_t>(compute_stream)));
+    KVT_HIP(hipStreamWaitEvent(s->side, s->ready[layer], 0));
+    uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
+    if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
+    KVT_HIP(hipEventRecord(s->done[layer], s->side));
+    s->last_done = s->done[layer];
+    return KVT_OK;
+  });
+}
+
+int kvt_session_wait_layer(kvt_session* s, uint32_t layer) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_wait_layer: null session");
+    if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    KVT_HIP(hipEventSynchronize(s->done[layer]));
+    return KVT_OK;
+  });
+}
+
+int kvt_session_join(kvt_session* s, void* stream) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_join: null session");
+    if (s->last_done) KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), s->last_done, 0));
+    return KVT_OK;
+  });
+}
+
+void* kvt_session_side_stream(kvt_session* s) { return s ? s->side : nullptr; }
+
+// ------------------------------------------------------------------ stager
+
+int kvt_stager_create(int device, uint64_t slot_bytes, uint32_t n_slots, kvt_stager** out) {
+  return guarded([&]() -> int {
+    if (!out || slot_bytes == 0 || n_slots < 2)
+      return fail(KVT_ERR_INVALID, "kvt_stager_create: need >= 2 slots of > 0 bytes");
+    if (int rc = check_device(device)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    std::unique_ptr<kvt_stager> s(new kvt_stager());
+    s->device = device;
+    s->slot_bytes = round_up(slot_bytes, 4096);
+    s->n_slots = n_slots;
+    KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&s->pinned), s->slot_bytes * n_slots,
+                          hipHostMallocDefault));
+    KVT_HIP(hipStreamCreateWithFlags(&s->copy, hipStreamNonBlocking));
+    s->slot_done.resize(n_slots);
+    for (uint32_t i = 0; i < n_slots; ++i)
+      KVT_HIP(hipEventCreateWithFlags(&s->slot_done[i], hipEventDisableTiming));
+    KVT_HIP(hipEventCreateWithFlags(&s->fence, hipEventDisableTiming));
+    *out = s.release();
+    return KVT_OK;
+  });
+}
+
+void kvt_stager_destroy(kvt_stager* s) {
+  if (!s) return;
+  if (s->copy) {
+    (void)hipStreamSynchronize(s->copy);
+    (void)hipStreamDestroy(s->copy);
+  }
+  for (hipEvent_t e : s->slot_done)
+    if (e) (void)hipEventDestroy(e);
+  if (s->fence) (void)hipEventDestroy(s->fence);
+  if (s->pinned) (void)hipHostFree(s->pinned);
+  delete s;
+}
+
+void* kvt_stager_slot(kvt_stager* s, uint32_t slot) {
+  return (s && slot < s->n_slots) ? s->pinned + static_cast<uint64_t>(slot) * s->slot_bytes : nullptr;
+}
+void* kvt_stager_copy_stream(kvt_stager* s) { return s ? s->copy : nullptr; }
+
+int kvt_stager_save(kvt_stager* s, uint32_t slot, const void* dev, uint64_t bytes,
+                    void* producer_stream) {
+  return guarded([&]() -> int {
+    if (!s || !dev) return fail(KVT_ERR_INVALID, "kvt_stager_save: null argument");
+    if (slot >= s->n_slots || bytes > s->slot_bytes)
+      return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_save: slot index or size out of range");
+    DeviceGuard g;
+    if (int rc = g.enter(s->device)) return rc;
+    KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(producer_stream)));
+    KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));
+    KVT_HIP(hipMemcpyAsync(kvt_stager_slot(s, slot), dev, bytes, hipMemcpyDeviceToHost, s->copy));
+    KVT_HIP(hipEventRecord(s->slot_done[slot], s->copy));
+    return KVT_OK;
+  });
+}
+
+int kvt_stager_load(kvt_stager* s, uint32_t slot, void* dev, uint64_t bytes,
+                    void* consumer_stream) {
+  return guarded([&]() -> int {
+    if (!s || !dev) return fail(KVT_ERR_INVALID, "kvt_stager_load: null argument");
+    if (slot >= s->n_slots || bytes > s->slot_bytes)
+      return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_load: slot index or size out of range");
+    DeviceGuard g;
+    if (int rc = g.enter(s->device)) return rc;
+    // the device buffer may still be read by earlier work of the consumer
+    KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(consumer_stream)));
+    KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));
+    KVT_HIP(hipMemcpyAsync(dev, kvt_stager_slot(s, slot), bytes, hipMemcpyHostToDevice, s->copy));
+    KVT_HIP(hipEventRecord(s->slot_done[slot], s->copy));
+    KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream), s->slot_done[slot], 0));
+    return KVT_OK;
+  });
+}
+
+int kvt_stager_wait(kvt_stager* s, uint32_t slot) {
+  return guarded([&]() -> int {
+    if (!s || slot >= s->n_slots) return fail(KVT_ERR_INVALID, "kvt_stager_wait: bad argument");
+    KVT_HIP(hipEventSynchronize(s->slot_done[slot]));
+    return KVT_OK;
+  });
+}
+
+int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats,
+                     double* bytes_per_s) {
+  return guarded([&]() -> int {
+    if (!bytes_per_s || bytes == 0 || repeats == 0)
+      return fail(KVT_ERR_INVALID, "kvt_measure_pcie: bad argument");
+    if (int rc = check_device(device)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    void *host = nullptr, *dev = nullptr;
+    hipStream_t st = nullptr;
+    hipEvent_t a = nullptr, b = nullptr;
+    int rc = KVT_OK;
+    auto cleanup = [&]() {
+      if (a) (void)hipEventDestroy(a);
+      if (b) (void)hipEventDestroy(b);
+      if (st) (void)hipStreamDestroy(st);
+      if (dev) (void)hipFree(dev);
+      if (host) (void)hipHostFree(host);
+    };
+#define KVT_TRY(call)                         \
+  do {                                        \
+    const hipError_t _e = (call);             \
+    if (_e != hipSuccess) {                   \
+      rc = hip_fail(_e, #call);               \
+      cleanup();                              \
+      return rc;                              \
+    }                                         \
+  } while (0)
+    KVT_TRY(hipHostMalloc(&host, bytes, hipHostMallocDefault));
+    KVT_TRY(hipMalloc(&dev, bytes));
+    std::memset(host, 0x5a, bytes);
+    KVT_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    KVT_TRY(hipEventCreate(&a));
+    KVT_TRY(hipEventCreate(&b));
+    const bool d2h = direction == KVT_COPY_D2H;
+    KVT_TRY(hipMemcpyAsync(d2h ? host : dev, d2h ? dev : host, bytes,
+                           d2h ? hipMemcpyDeviceToHost : hipMemcpyHostToDevice, st));
+    KVT_TRY(hipEventRecord(a, st));
+    for (uint32_t i = 0; i < repeats; ++i)
+      KVT_TRY(hipMemcpyAsync(d2h ? host : dev, d2h ? dev : host, bytes,
+                             d2h ? hipMemcpyDeviceToHost : hipMemcpyHostToDevice, st));
+    KVT_TRY(hipEventRecord(b, st));
+    KVT_TRY(hipEventSynchronize(b));
+    float ms = 0;
+    KVT_TRY(hipEventElapsedTime(&ms, a, b));
+#undef KVT_TRY
+    *bytes_per_s = static_cast<double>(bytes) * repeats / (ms * 1e-3);
+    cleanup();
+    return KVT_OK;
+  });
+}
+
+// --------------------------------------------------------------- utilities
+
+int kvt_copy_linear(void* dst, const void* src, uint64_t bytes, void* stream) {
+  return guarded([&]() -> int {
+    if ((!dst || !src) && bytes) return fail(KVT_ERR_INVALID, "kvt_copy_linear: null argument");
+    if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+    if (bytes > (0x7FFFFFFFull * 32768ull)) return fail(KVT_ERR_INVALID, "kvt_copy_linear: too large");
+    const hipError_t e = launch_copy_linear(dst, src, bytes, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "linear copy launch");
+    return KVT_OK;
+  });
+}
+
+int kvt_event_create(void** ev) {
+  if (!ev) return fail(KVT_ERR_INVALID, "kvt_event_create: null argument");
+  if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+  hipEvent_t e;
+  KVT_HIP(hipEventCreate(&e));
+  *ev = e;
+  return KVT_OK;
+}
+int kvt_event_destroy(void* ev) {
+  if (ev) KVT_HIP(hipEventDestroy(static_cast<hipEvent_t>(ev)));
+  return KVT_OK;
+}
+int kvt_event_record(void* ev, void* stream) {
+  KVT_HIP(hipEventRecord(static_cast<hipEvent_t>(ev), static_cast<hipStream_t>(stream)));
+  return KVT_OK;
+}
+int kvt_event_synchronize(void* ev) {
+  KVT_HIP(hipEventSynchronize(static_cast<hipEvent_t>(ev)));
+  return KVT_OK;
+}
+int kvt_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!ms) return fail(KVT_ERR_INVALID, "kvt_event_elapsed_ms: null argument");
+  KVT_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return KVT_OK;
+}
+int kvt_stream_create(void** stream) {
+  if (!stream) return fail(KVT_ERR_INVALID, "kvt_stream_create: null argument");
+  if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+  hipStream_t s;
+  KVT_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = s;
+  return KVT_OK;
+}
+int kvt_stream_destroy(void* stream) {
+  if (stream) KVT_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return KVT_OK;
+}
+int kvt_stream_synchronize(void* stream) {
+  KVT_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return KVT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,338 @@
+"""ctypes declarations for every symbol of include/kvt_hip.h plus small RAII wrappers."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from .ctypes_defs import IpcBlock, ParseOpts, Task, WorkerInfo
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "libkvt_hip.so")
+
+_vp = C.c_void_p
+_u32, _u64, _i64, _int = C.c_uint32, C.c_uint64, C.c_int64, C.c_int
+_P = C.POINTER
+
+
+class Xform(C.Structure):
+    _fields_ = [("kind", _u32), ("heads", _u32), ("ntpb", _u32), ("row_bytes", _u32)]
+
+
+# name -> (restype, argtypes); this table is also what tests/test_abi.py checks
+# against the declarations in include/kvt_hip.h.
+SIGNATURES = {
+    "kvt_last_error": (C.c_char_p, []),
+    "kvt_abi_sizeof": (_u64, [_int]),
+    "kvt_device_count": (_int, []),
+    "kvt_compute_valid_ranks_pd": (_u32, [_u32, _u32, C.c_int32]),
+    "kvt_select_parser": (_int, [_int, _P(WorkerInfo), _P(WorkerInfo), _P(_u32), _P(_u32),
+                                 _P(_u32), _P(_int), _P(_int)]),
+    "kvt_parser_create": (_int, [_int, _P(WorkerInfo), _P(WorkerInfo), _u32, _u32, _u32,
+                                 _P(ParseOpts), _P(_vp)]),
+    "kvt_parser_destroy": (None, [_vp]),
+    "kvt_block_lists_create": (_int, [_P(_vp)]),
+    "kvt_block_lists_destroy": (None, [_vp]),
+    "kvt_block_lists_clear": (None, [_vp]),
+    "kvt_block_lists_num_tensors": (_u32, [_vp]),
+    "kvt_block_lists_view": (_int, [_vp, _u32, _P(_P(IpcBlock)), _P(_u64)]),
+    "kvt_block_lists_append": (_int, [_vp, _u32, _vp, _u64]),
+    "kvt_parse_block": (_int, [_vp, _P(Task), _vp]),
+    "kvt_merge_interval": (_int, [_vp, _u64, _P(_u64), _P(_u64)]),
+    "kvt_block_lists_merge": (_int, [_vp]),
+    "kvt_validate_ipc_block_bounds": (_int, [_vp, _u64, _u64, _int, _u64, _P(_u64)]),
+    "kvt_cache_register": (_int, [_int, _P(_vp), _u32, _u32, _P(_u64), _P(_vp)]),
+    "kvt_cache_destroy": (None, [_vp]),
+    "kvt_plan_create": (_int, [_int, _vp, _P(_u64), _P(_u64), _P(Xform), _u32, _P(_vp)]),
+    "kvt_plan_destroy": (None, [_vp]),
+    "kvt_plan_num_tensors": (_u32, [_vp]),
+    "kvt_plan_num_chunks": (_u64, [_vp]),
+    "kvt_plan_tensor_bytes": (_u64, [_vp, _u32]),
+    "kvt_plan_tensor_offset": (_u64, [_vp, _u32]),
+    "kvt_plan_layer_bytes": (_u64, [_vp]),
+    "kvt_pack": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _vp]),
+    "kvt_unpack": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _vp]),
+    "kvt_launch_copy_d2h_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
+    "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
+    "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
+    "kvt_copy_handle_data_with_kernel": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp, _vp,
+                                               _vp, _i64]),
+    "kvt_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _vp, _vp, _vp, _i64]),
+    "kvt_session_create": (_int, [_vp, _vp, _vp, _u64, _P(_vp)]),
+    "kvt_session_destroy": (None, [_vp]),
+    "kvt_session_save_layer": (_int, [_vp, _u32, _vp]),
+    "kvt_session_wait_layer": (_int, [_vp, _u32]),
+    "kvt_session_join": (_int, [_vp, _vp]),
+    "kvt_session_side_stream": (_vp, [_vp]),
+    "kvt_stager_create": (_int, [_int, _u64, _u32, _P(_vp)]),
+    "kvt_stager_destroy": (None, [_vp]),
+    "kvt_stager_slot": (_vp, [_vp, _u32]),
+    "kvt_stager_copy_stream": (_vp, [_vp]),
+    "kvt_stager_save": (_int, [_vp, _u32, _vp, _u64, _vp]),
+    "kvt_stager_load": (_int, [_vp, _u32, _vp, _u64, _vp]),
+    "kvt_stager_wait": (_int, [_vp, _u32]),
+    "kvt_measure_pcie": (_int, [_int, _int, _u64, _u32, _P(C.c_double)]),
+    "kvt_copy_linear": (_int, [_vp, _vp, _u64, _vp]),
+    "kvt_event_create": (_int, [_P(_vp)]),
+    "kvt_event_destroy": (_int, [_vp]),
+    "kvt_event_record": (_int, [_vp, _vp]),
+    "kvt_event_synchronize": (_int, [_vp]),
+    "kvt_event_elapsed_ms": (_int, [_vp, _vp, _P(C.c_float)]),
+    "kvt_stream_create": (_int, [_P(_vp)]),
+    "kvt_stream_destroy": (_int, [_vp]),
+    "kvt_stream_synchronize": (_int, [_vp]),
+}
+
+
+class KvtError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("kvt error %d: %s" % (code, message))
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """Loads libkvt_hip.so (built in-tree by ``make -C llumnix-kv_amd``)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise KvtError(-1, "libkvt_hip.so is not built: run `make -C llumnix-kv_amd` "
+                               "(or __graft_entry__.build())")
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise KvtError(rc, (lib().kvt_last_error() or b"").decode())
+
+
+def device_count():
+    return lib().kvt_device_count()
+
+
+def compute_valid_ranks_pd(p_tp, d_tp, heads):
+    return lib().kvt_compute_valid_ranks_pd(p_tp, d_tp, heads)
+
+
+def select_parser(cache_shape, src, dst):
+    """-> (valid_mask, kvt_tp_size, kvt_tp_rank, parser_id, tp_kind)"""
+    v, s, r, pid, kind = _u32(), _u32(), _u32(), _int(), _int()
+    check(lib().kvt_select_parser(cache_shape, C.byref(src), C.byref(dst), C.byref(v), C.byref(s),
+                                  C.byref(r), C.byref(pid), C.byref(kind)))
+    return v.value, s.value, r.value, pid.value, kind.value
+
+
+def merge_interval(runs):
+    """runs: (n,3) uint64 -> (merged (m,3) array, (min,max,total,count))"""
+    a = np.ascontiguousarray(runs, dtype=np.uint64).reshape(-1, 3).copy()
+    n_out = _u64()
+    stats = (_u64 * 4)()
+    check(lib().kvt_merge_interval(a.ctypes.data, len(a), C.byref(n_out), stats))
+    return a[:n_out.value].copy(), tuple(stats)
+
+
+def validate_bounds(runs, capacity, which, scale=1):
+    """-> (rc, bad_index)"""
+    a = np.ascontiguousarray(runs, dtype=np.uint64).reshape(-1, 3)
+    bad = _u64(0)
+    rc = lib().kvt_validate_ipc_block_bounds(a.ctypes.data, len(a), capacity, which, scale,
+                                             C.byref(bad))
+    return rc, bad.value
+
+
+class BlockLists:
+    def __init__(self):
+        self.h = _vp()
+        check(lib().kvt_block_lists_create(C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().kvt_block_lists_destroy(self.h)
+            self.h = _vp()
+
+    __del__ = close
+
+    def clear(self):
+        lib().kvt_block_lists_clear(self.h)
+
+    def merge(self):
+        check(lib().kvt_block_lists_merge(self.h))
+
+    def num_tensors(self):
+        return lib().kvt_block_lists_num_tensors(self.h)
+
+    def append(self, t, runs):
+        a = np.ascontiguousarray(runs, dtype=np.uint64).reshape(-1, 3)
+        check(lib().kvt_block_lists_append(self.h, t, a.ctypes.data, len(a)))
+
+    def tensor(self, t):
+        """-> (n,3) uint64 copy of tensor t's ranges"""
+        data = _P(IpcBlock)()
+        n = _u64()
+        check(lib().kvt_block_lists_view(self.h, t, C.byref(data), C.byref(n)))
+        if n.value == 0:
+            return np.zeros((0, 3), dtype=np.uint64)
+        arr = np.ctypeslib.as_array(C.cast(data, _P(_u64)), shape=(n.value, 3))
+        return arr.copy()
+
+    def all(self):
+        return [self.tensor(t) for t in range(self.num_tensors())]
+
+
+class Parser:
+    def __init__(self, parser_id, src, dst, valid, tp_size, tp_rank, fp8=False, pad=True):
+        self.h = _vp()
+        opts = ParseOpts(1 if fp8 else 0, 1 if pad else 0)
+        check(lib().kvt_parser_create(parser_id, C.byref(src), C.byref(dst), valid, tp_size,
+                                      tp_rank, C.byref(opts), C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().kvt_parser_destroy(self.h)
+            self.h = _vp()
+
+    __del__ = close
+
+    def parse(self, task_struct, lists):
+        """Appends one task's ranges; returns the KVT_* code (0 = ok)."""
+        return lib().kvt_parse_block(self.h, C.byref(task_struct), lists.h)
+
+
+def _ptr(x):
+    """device / host pointer of a torch tensor, numpy array, int or None"""
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    if hasattr(x, "ctypes"):
+        return x.ctypes.data
+    raise TypeError(type(x))
+
+
+class Cache:
+    """Registered layer-tensor base pointers (layers[layer][tensor])."""
+
+    def __init__(self, device, layers, capacity):
+        n_layers, n_tensors = len(layers), len(layers[0])
+        flat = (_vp * (n_layers * n_tensors))(*[_ptr(t) for l in layers for t in l])
+        cap = (_u64 * n_tensors)(*capacity)
+        self.h = _vp()
+        self._keep = layers
+        check(lib().kvt_cache_register(device, flat, n_layers, n_tensors, cap, C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().kvt_cache_destroy(self.h)
+            self.h = _vp()
+
+    __del__ = close
+
+
+class Plan:
+    def __init__(self, device, lists, src_capacity, dst_capacity, xform=None, chunk_bytes=0):
+        n = lists.num_tensors()
+        sc = (_u64 * max(1, n))(*src_capacity)
+        dc = (_u64 * max(1, n))(*dst_capacity)
+        xf = None
+        if xform is not None:
+            xf = C.byref(Xform(1, *xform))
+        self.h = _vp()
+        check(lib().kvt_plan_create(device, lists.h, sc, dc, xf, chunk_bytes, C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().kvt_plan_destroy(self.h)
+            self.h = _vp()
+
+    __del__ = close
+
+    @property
+    def layer_bytes(self):
+        return lib().kvt_plan_layer_bytes(self.h)
+
+    @property
+    def num_chunks(self):
+        return lib().kvt_plan_num_chunks(self.h)
+
+    def tensor_bytes(self, t):
+        return lib().kvt_plan_tensor_bytes(self.h, t)
+
+    def tensor_offset(self, t):
+        return lib().kvt_plan_tensor_offset(self.h, t)
+
+    def pack(self, cache, first_layer, n_layers, packed, layer_stride, stream=None):
+        check(lib().kvt_pack(self.h, cache.h, first_layer, n_layers, _ptr(packed), layer_stride,
+                             _ptr(stream)))
+
+    def unpack(self, cache, first_layer, n_layers, packed, layer_stride, stream=None):
+        check(lib().kvt_unpack(self.h, cache.h, first_layer, n_layers, _ptr(packed), layer_stride,
+                               _ptr(stream)))
+
+
+class Session:
+    def __init__(self, plan, cache, packed, layer_stride):
+        self.h = _vp()
+        self._keep = (plan, cache, packed)
+        check(lib().kvt_session_create(plan.h, cache.h, _ptr(packed), layer_stride,
+                                       C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().kvt_session_destroy(self.h)
+            self.h = _vp()
+
+    __del__ = close
+
+    def save_layer(self, layer, compute_stream=None):
+        check(lib().kvt_session_save_layer(self.h, layer, _ptr(compute_stream)))
+
+    def wait_layer(self, layer):
+        check(lib().kvt_session_wait_layer(self.h, layer))
+
+    def join(self, stream=None):
+        check(lib().kvt_session_join(self.h, _ptr(stream)))
+
+    @property
+    def side_stream(self):
+        return lib().kvt_session_side_stream(self.h)
+
+
+class Stager:
+    def __init__(self, device, slot_bytes, n_slots):
+        self.h = _vp()
+        self.slot_bytes, self.n_slots = slot_bytes, n_slots
+        check(lib().kvt_stager_create(device, slot_bytes, n_slots, C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().kvt_stager_destroy(self.h)
+            self.h = _vp()
+
+    __del__ = close
+
+    def slot_ptr(self, slot):
+        return lib().kvt_stager_slot(self.h, slot)
+
+    def slot_array(self, slot, nbytes):
+        buf = (C.c_uint8 * nbytes).from_address(self.slot_ptr(slot))
+        return np.frombuffer(buf, dtype=np.uint8)
+
+    @property
+    def copy_stream(self):
+        return lib().kvt_stager_copy_stream(self.h)
+
+    def save(self, slot, dev, nbytes, producer_stream=None):
+        check(lib().kvt_stager_save(self.h, slot, _ptr(dev), nbytes, _ptr(producer_stream)))
+
+    def load(self, slot, dev, nbytes, consumer_stream=None):
+        check(lib().kvt_stager_load(self.h, slot, _ptr(dev), nbytes, _ptr(consumer_stream)))
+
+    def wait(self, slot):
+        check(lib().kvt_stager_wait(self.h, slot))

@@ -1,0 +1,30 @@
+"""Host-side flow of one send step, mirroring KvSendStub::TaskContext::do_task
+(reference: kvtransfer/src/tx_stub.cpp:158-263): pick the parser for the
+destination, run ParseBlock for every request of the batch into one range list
+per cache tensor, merge when the TP relation is P==D (what register_data does,
+kvtransfer/src/tcp_channel.cpp:376-392) and make the result resident on the GPU
+as a copy plan."""
+from . import binding
+from .ctypes_defs import TP_PEQD
+
+
+def parse_batch(cache_shape, src, dst, task_bufs, fp8=False, pad=True):
+    """-> (BlockLists, tp_kind). Raises KvtError on the first failing request."""
+    valid, tp_size, tp_rank, parser_id, tp_kind = binding.select_parser(cache_shape, src, dst)
+    parser = binding.Parser(parser_id, src, dst, valid, tp_size, tp_rank, fp8=fp8, pad=pad)
+    lists = binding.BlockLists()
+    for t in task_bufs:
+        binding.check(parser.parse(t.struct, lists))
+    parser.close()
+    if tp_kind == TP_PEQD:
+        lists.merge()
+    return lists, tp_kind
+
+
+def build_plan(workload, device=0, chunk_bytes=0):
+    """Workload -> (Plan, BlockLists). The lists stay valid for wire metadata."""
+    src, dst = workload.worker_infos()
+    lists, _ = parse_batch(workload.cache_shape, src, dst, workload.task_bufs())
+    plan = binding.Plan(device, lists, workload.capacities("src"), workload.capacities("dst"),
+                        xform=workload.xform, chunk_bytes=chunk_bytes)
+    return plan, lists

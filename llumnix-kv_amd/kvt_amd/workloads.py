@@ -1,0 +1,158 @@
+"""Seeded synthetic workloads shaped like the five benchmark configurations.
+
+A workload is plain host data (numpy / python): cache geometry, per-request
+block tables and the ParseBlock inputs. Device memory is the caller's business.
+Every builder takes scale parameters so that tests can run the same code on
+small pools while bench.py uses the full sizes.
+"""
+from dataclasses import dataclass, field
+
+import numpy as np
+
+from .ctypes_defs import (PARSER, SHAPE_DPSK_V32_SPARSE_MLA, SHAPE_FLASH, SHAPE_FLASHINFER,
+                          SHAPE_QWEN3_NEXT_FLASH, TaskBuf, make_worker_info)
+
+
+@dataclass
+class Workload:
+    name: str
+    cache_shape: int
+    parser: str
+    n_layers: int
+    src_info: dict                 # make_worker_info kwargs (sender)
+    dst_info: dict                 # make_worker_info kwargs (receiver)
+    tasks: list                    # [seen, new, last, src_groups, dst_groups] per request
+    elem_dtype: str = "bf16"       # "bf16" | "fp8" | "f32"
+    xform: tuple = None            # (heads, ntpb, row_bytes) for the HND<->NHD transposing pack
+    seed: int = 0
+    notes: dict = field(default_factory=dict)
+
+    def worker_infos(self):
+        return make_worker_info(**self.src_info), make_worker_info(**self.dst_info)
+
+    def task_bufs(self):
+        return [TaskBuf(*t) for t in self.tasks]
+
+    @property
+    def n_tensors(self):
+        return len(self.src_info["block_sizes"])
+
+    def capacities(self, side="src"):
+        info = self.src_info if side == "src" else self.dst_info
+        return [b * info["layer_num_blocks"] for b in info["block_sizes"]]
+
+
+def _tables(rng, n_req, lens_tokens, ntpb, src_pool, dst_pool, disjoint_dst=True):
+    """Per request: src ids sampled without replacement inside the request (requests
+    may share source blocks, reads only); dst ids disjoint across the whole batch."""
+    n_blocks = [(int(t) + ntpb - 1) // ntpb for t in lens_tokens]
+    total = sum(n_blocks)
+    if disjoint_dst:
+        if total > dst_pool:
+            raise ValueError("destination pool too small for disjoint tables: %d > %d"
+                             % (total, dst_pool))
+        perm = rng.permutation(dst_pool)[:total]
+    src, dst, pos = [], [], 0
+    for nb in n_blocks:
+        src.append([int(x) for x in rng.choice(src_pool, size=nb, replace=False)])
+        if disjoint_dst:
+            dst.append([int(x) for x in perm[pos:pos + nb]])
+        else:
+            dst.append([int(x) for x in rng.choice(dst_pool, size=nb, replace=False)])
+        pos += nb
+    return src, dst
+
+
+def llama8b_single(n_layers=32, pool=1024, tokens=512, seed=20251):
+    """Config 1: FlashAttention layout [2, pool, 16, 8, 128] bf16, one request."""
+    rng = np.random.default_rng(seed)
+    T, ntpb = 2 * 8 * 128 * 2, 16
+    src, dst = _tables(rng, 1, [tokens], ntpb, pool, pool)
+    info = dict(block_sizes=[T * ntpb], token_sizes=[T], layer_num_blocks=pool, num_kv_heads=8,
+                num_layers=n_layers)
+    return Workload("llama3-8b FA 1x%d tok" % tokens, SHAPE_FLASH, "FLASH_PEQD", n_layers, info,
+                    dict(info), [[0, tokens, True, [src[0]], [dst[0]]]], seed=seed)
+
+
+def llama8b_batch(n_layers=32, src_pool=16384, dst_pool=24576, n_req=64, min_tok=1024,
+                  max_tok=8192, seed=20252):
+    """Config 2: same geometry, 64 requests with lengths uniform in [1k, 8k]."""
+    rng = np.random.default_rng(seed)
+    T, ntpb = 4096, 16
+    lens = rng.integers(min_tok, max_tok + 1, size=n_req)
+    src, dst = _tables(rng, n_req, lens, ntpb, src_pool, dst_pool)
+    s_info = dict(block_sizes=[T * ntpb], token_sizes=[T], layer_num_blocks=src_pool,
+                  num_kv_heads=8, num_layers=n_layers)
+    d_info = dict(s_info, layer_num_blocks=dst_pool)
+    tasks = [[0, int(n), True, [s], [d]] for n, s, d in zip(lens, src, dst)]
+    return Workload("llama3-8b FA %dreq x %d-%d tok" % (n_req, min_tok, max_tok), SHAPE_FLASH,
+                    "FLASH_PEQD", n_layers, s_info, d_info, tasks, seed=seed,
+                    notes=dict(tokens=int(lens.sum())))
+
+
+def llama70b_flashinfer(n_layers=80, pool=8192, n_req=32, tokens=4096, transpose=True,
+                        seed=20253):
+    """Config 3: FlashInfer pages, HND in the cache ([pool, 2, 8, 16, 128] bf16).
+
+    transpose=True: whole-page plan (the page parse of the NHD page layout) with
+    the HND->NHD transform applied while packing. transpose=False: the plain
+    FlashInfer HND parse (per-head ranges, merged)."""
+    rng = np.random.default_rng(seed)
+    T, ntpb, heads, row = 4096, 16, 8, 256
+    src, dst = _tables(rng, n_req, [tokens] * n_req, ntpb, pool, pool)
+    info = dict(block_sizes=[T * ntpb], token_sizes=[T], layer_num_blocks=pool, num_kv_heads=heads,
+                num_layers=n_layers, num_gdn_layers=0)
+    tasks = [[0, tokens, True, [s], [d]] for s, d in zip(src, dst)]
+    if transpose:
+        return Workload("llama3-70b FlashInfer HND->NHD %dreq x %d tok" % (n_req, tokens),
+                        SHAPE_QWEN3_NEXT_FLASH, "HYBRID_PEQD", n_layers, info, dict(info), tasks,
+                        xform=(heads, ntpb, row), seed=seed)
+    return Workload("llama3-70b FlashInfer HND %dreq x %d tok" % (n_req, tokens), SHAPE_FLASHINFER,
+                    "FLASHINFER_PEQD", n_layers, info, dict(info), tasks, seed=seed)
+
+
+def deepseek_mla(n_layers=61, pool=4608, n_req=16, tokens=16384, seed=20254):
+    """Config 4: MLA latent (576 B/token) + DSA indexer keys (128 B/token), fp8, 64 tokens/block."""
+    rng = np.random.default_rng(seed)
+    ntpb = 64
+    src, dst = _tables(rng, n_req, [tokens] * n_req, ntpb, pool, pool)
+    info = dict(block_sizes=[576 * ntpb, 128 * ntpb], token_sizes=[576, 128],
+                layer_num_blocks=pool, num_kv_heads=1, num_layers=n_layers)
+    tasks = [[0, tokens, True, [s], [d]] for s, d in zip(src, dst)]
+    return Workload("deepseek-v3 MLA+indexer fp8 %dreq x %d tok" % (n_req, tokens),
+                    SHAPE_DPSK_V32_SPARSE_MLA, "DPSK_PEQD", n_layers, info, dict(info), tasks,
+                    elem_dtype="fp8", seed=seed)
+
+
+def qwen3next_attn(n_layers=12, pool=36864, n_req=128, tokens=4096, seed=20255):
+    """Config 5, full-attention part: NHD pages of 2 KV heads x 256 bf16, 16 tokens (32 KiB)."""
+    rng = np.random.default_rng(seed)
+    T, ntpb = 2 * 2 * 256 * 2, 16
+    src, dst = _tables(rng, n_req, [tokens] * n_req, ntpb, pool, pool)
+    info = dict(block_sizes=[T * ntpb], token_sizes=[T], layer_num_blocks=pool, num_kv_heads=2,
+                num_layers=n_layers, num_gdn_layers=0)
+    tasks = [[0, tokens, True, [s], [d]] for s, d in zip(src, dst)]
+    return Workload("qwen3-next full-attn pages %dreq x %d tok" % (n_req, tokens),
+                    SHAPE_QWEN3_NEXT_FLASH, "HYBRID_PEQD", n_layers, info, dict(info), tasks,
+                    seed=seed)
+
+
+def qwen3next_gdn(n_layers=36, slots=256, n_req=128, seed=20256):
+    """Config 5, linear-attention part: one 2 MiB fp32 state (32 x 128 x 128) per request and
+    layer, kept in its own pool of state slots. A state is one whole page of that pool and is
+    sent when the request completes (the whole-page rule of the hybrid P==D parser, with the
+    page size set to the slot stride)."""
+    rng = np.random.default_rng(seed)
+    state = 32 * 128 * 128 * 4
+    perm_s = rng.permutation(slots)[:n_req]
+    perm_d = rng.permutation(slots)[:n_req]
+    info = dict(block_sizes=[state], token_sizes=[state], layer_num_blocks=slots, num_kv_heads=2,
+                num_layers=n_layers, num_gdn_layers=0)
+    # one "token" per request in a pool whose page holds one token: exactly one whole page
+    tasks = [[0, 1, True, [[int(s)]], [[int(d)]]] for s, d in zip(perm_s, perm_d)]
+    return Workload("qwen3-next GDN state %dreq" % n_req, SHAPE_QWEN3_NEXT_FLASH, "HYBRID_PEQD",
+                    n_layers, info, dict(info), tasks, elem_dtype="f32", seed=seed)
+
+
+def parser_id(w):
+    return PARSER[w.parser]

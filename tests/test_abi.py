@@ -1,0 +1,73 @@
+"""CPU-side checks of the C ABI: the library loads without a GPU, exports every
+symbol include/kvt_hip.h declares, struct sizes agree with the ctypes mirrors,
+and device entry points fail loudly (never fall back) when no gfx950 is present."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+import kvt_amd
+from kvt_amd import binding
+from kvt_amd.ctypes_defs import IpcBlock, ParseOpts, Task, WorkerInfo, make_worker_info
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "kvt_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(kvt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_what_the_binding_binds():
+    assert _declared_symbols() == sorted(binding.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = kvt_amd.lib()
+    for name in _declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_struct_sizes_match():
+    lib = kvt_amd.lib()
+    assert lib.kvt_abi_sizeof(0) == C.sizeof(IpcBlock) == 24
+    assert lib.kvt_abi_sizeof(1) == C.sizeof(WorkerInfo)
+    assert lib.kvt_abi_sizeof(2) == C.sizeof(Task)
+    assert lib.kvt_abi_sizeof(3) == C.sizeof(ParseOpts)
+    assert lib.kvt_abi_sizeof(4) == C.sizeof(binding.Xform)
+
+
+def test_null_arguments_are_errors_not_crashes():
+    lib = kvt_amd.lib()
+    assert lib.kvt_parse_block(None, None, None) == 3
+    assert lib.kvt_block_lists_view(None, 0, None, None) == 3
+    assert b"null" in lib.kvt_last_error()
+    lists = kvt_amd.BlockLists()
+    data, n = C.POINTER(IpcBlock)(), C.c_uint64()
+    assert lib.kvt_block_lists_view(lists.h, 0, C.byref(data), C.byref(n)) == 1
+
+
+def test_unbuilt_parsers_are_refused():
+    w = make_worker_info([16384], [1024], 8)
+    for pid in range(17, 23):  # KDA / Kimi-K3
+        with pytest.raises(kvt_amd.KvtError) as e:
+            kvt_amd.Parser(pid, w, w, 1, 1, 0)
+        assert e.value.code == 4
+
+
+@pytest.mark.skipif(kvt_amd.device_count() > 0, reason="this check is for machines without a GPU")
+def test_gpu_entry_points_fail_loudly_without_a_device():
+    w = make_worker_info([65536], [4096], 8)
+    lists = kvt_amd.BlockLists()
+    p = kvt_amd.Parser(4, w, w, 1, 1, 0)
+    from kvt_amd.ctypes_defs import TaskBuf
+    assert p.parse(TaskBuf(0, 16, True, [[1]], [[2]]).struct, lists) == 0
+    with pytest.raises(kvt_amd.KvtError) as e:
+        kvt_amd.Plan(0, lists, [65536 * 8], [65536 * 8])
+    assert e.value.code == 6
+    with pytest.raises(kvt_amd.KvtError) as e:
+        kvt_amd.Stager(0, 4096, 2)
+    assert e.value.code == 6
+    assert kvt_amd.lib().kvt_copy_linear(1, 1, 16, None) == 6

@@ -1,0 +1,499 @@
+"""GPU parity tests: the HIP pack / unpack path, called through the C ABI of
+libkvt_hip.so, against the CPU oracle on identical seeded caches and block
+tables. Bit-exact (byte work). Needs a real MI355X: run with `-m gpu`."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import checkers
+import kvt_amd
+from kvt_amd import pipeline, workloads
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _dev_bytes(n, seed=None, dtype="bf16"):
+    """n bytes of seeded cache content on the GPU (as a uint8 tensor)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0 if seed is None else seed)
+    if dtype == "bf16":
+        t = (torch.rand(n // 2, generator=g, device="cuda") * 2 - 1).to(torch.bfloat16)
+        return t.view(torch.uint8)
+    if dtype == "fp8":
+        t = torch.randn(n, generator=g, device="cuda").clamp_(-448, 448).to(torch.float8_e4m3fn)
+        return t.view(torch.uint8)
+    if dtype == "f32":
+        return torch.randn(n // 4, generator=g, device="cuda").view(torch.uint8)
+    return torch.randint(0, 256, (n,), generator=g, device="cuda", dtype=torch.uint8)
+
+
+def _host(t):
+    return t.cpu().numpy()
+
+
+def _make_caches(w, side, seed, dtype=None, fill=True):
+    caps = w.capacities(side)
+    layers = []
+    for l in range(w.n_layers):
+        row = []
+        for t, cap in enumerate(caps):
+            if fill:
+                row.append(_dev_bytes(cap, seed * 1000 + l * 8 + t, dtype or w.elem_dtype))
+            else:
+                row.append(torch.full((cap,), 0xA5, dtype=torch.uint8, device="cuda"))
+        layers.append(row)
+    return layers
+
+
+def _oracle_lists(w):
+    """merged per-tensor range lists from the oracle (independent of the product parser)"""
+    src, dst = w.worker_infos()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, src, dst)
+    assert rc == 0
+    rc, outs = checkers.oracle_parse(pid, src, dst, valid, tps, tpr, w.task_bufs())
+    assert rc == 0
+    if kind == 0:
+        outs = [checkers.oracle_merge(o)[0] for o in outs]
+    return outs
+
+
+def _check_pack_unpack(w, seed=1, chunk_bytes=0, layers_per_launch=None):
+    plan, lists = pipeline.build_plan(w, 0, chunk_bytes)
+    o_lists = _oracle_lists(w)
+    for t in range(w.n_tensors):
+        assert np.array_equal(lists.tensor(t), o_lists[t])
+    src_layers = _make_caches(w, "src", seed)
+    dst_layers = _make_caches(w, "dst", seed + 1, fill=False)
+    src_cache = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dst_cache = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    step = layers_per_launch or w.n_layers
+    for first in range(0, w.n_layers, step):
+        n = min(step, w.n_layers - first)
+        plan.pack(src_cache, first, n, packed.data_ptr() + first * stride, stride)
+    torch.cuda.synchronize()
+    packed_h = _host(packed)
+    for l in range(w.n_layers):
+        for t in range(w.n_tensors):
+            blob = checkers.oracle_pack(_host(src_layers[l][t]), o_lists[t])
+            off = l * stride + plan.tensor_offset(t)
+            assert plan.tensor_bytes(t) == len(blob)
+            assert np.array_equal(packed_h[off:off + len(blob)], blob), (l, t)
+    for first in range(0, w.n_layers, step):
+        n = min(step, w.n_layers - first)
+        plan.unpack(dst_cache, first, n, packed.data_ptr() + first * stride, stride)
+    torch.cuda.synchronize()
+    for l in range(w.n_layers):
+        for t in range(w.n_tensors):
+            exp = np.full(w.capacities("dst")[t], 0xA5, dtype=np.uint8)
+            off = l * stride + plan.tensor_offset(t)
+            checkers.oracle_unpack(exp, o_lists[t], packed_h[off:off + plan.tensor_bytes(t)])
+            assert np.array_equal(_host(dst_layers[l][t]), exp), (l, t)
+    return plan
+
+
+def test_config1_llama8b_single_request_full_size():
+    w = workloads.llama8b_single()  # 32 layers x 64 MiB, 1 request x 512 tokens
+    plan = _check_pack_unpack(w)
+    assert plan.layer_bytes == 2 * 1024 * 1024
+    assert plan.num_chunks == 64
+
+
+@pytest.mark.parametrize("chunk", [0, 4096, 65536])
+def test_config2_shape_reduced_pool(chunk):
+    w = workloads.llama8b_batch(n_layers=3, src_pool=512, dst_pool=768, n_req=6, min_tok=100,
+                                max_tok=1500)
+    _check_pack_unpack(w, chunk_bytes=chunk, layers_per_launch=2)
+
+
+def test_config3_plain_hnd_ranges():
+    w = workloads.llama70b_flashinfer(n_layers=2, pool=256, n_req=3, tokens=600, transpose=False)
+    _check_pack_unpack(w)
+
+
+def test_config4_mla_and_indexer_two_tensors():
+    w = workloads.deepseek_mla(n_layers=3, pool=64, n_req=3, tokens=1000)
+    plan = _check_pack_unpack(w)
+    assert plan.tensor_offset(1) % 256 == 0 and plan.tensor_offset(1) >= plan.tensor_bytes(0)
+
+
+def test_config5_attention_pages_and_gdn_states():
+    _check_pack_unpack(workloads.qwen3next_attn(n_layers=2, pool=512, n_req=5, tokens=700))
+    _check_pack_unpack(workloads.qwen3next_gdn(n_layers=2, slots=12, n_req=5), chunk_bytes=65536)
+
+
+def test_chunked_prefill_steps_and_ragged_tail():
+    # two chunked-prefill steps of one request + a second request, ragged last block
+    w = workloads.llama8b_single(n_layers=2, pool=64, tokens=100)
+    src, dst = w.tasks[0][3], w.tasks[0][4]
+    w.tasks = [[0, 37, False, src, dst], [37, 63, True, src, dst]]
+    _check_pack_unpack(w)
+
+
+def _transposing(w_t, seed=3):
+    heads, ntpb, row = w_t.xform
+    plan, lists = pipeline.build_plan(w_t, 0)
+    runs = lists.tensor(0)
+    B = 2 * heads * ntpb * row
+    ids = np.concatenate([np.arange(r[0] // B, (r[0] + r[2]) // B) for r in runs]).astype(np.uint32)
+    dst_ids = np.concatenate([np.arange(r[1] // B, (r[1] + r[2]) // B) for r in runs]).astype(np.uint32)
+    src_layers = _make_caches(w_t, "src", seed)
+    dst_layers = _make_caches(w_t, "dst", seed + 1, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w_t.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w_t.capacities("dst"))
+    stride = plan.layer_bytes
+    packed = torch.zeros(w_t.n_layers * stride, dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, w_t.n_layers, packed, stride)
+    plan.unpack(dc, 0, w_t.n_layers, packed, stride)
+    torch.cuda.synchronize()
+    lib = checkers.oracle()
+    ph = _host(packed)
+    for l in range(w_t.n_layers):
+        hnd = _host(src_layers[l][0])
+        blob = np.zeros(len(ids) * B, dtype=np.uint8)
+        lib.kvto_pack_hnd_to_nhd(hnd.ctypes.data, ids.ctypes.data, len(ids), heads, ntpb, row,
+                                 blob.ctypes.data)
+        assert np.array_equal(ph[l * stride:l * stride + len(blob)], blob), l
+        # same bytes as a plain pack of an NHD cache holding the same logical values
+        nhd = np.ascontiguousarray(
+            hnd.reshape(-1, 2, heads, ntpb, row).transpose(0, 1, 3, 2, 4)).reshape(-1)
+        assert np.array_equal(blob, checkers.oracle_pack(nhd, runs))
+        exp = np.full(w_t.capacities("dst")[0], 0xA5, dtype=np.uint8)
+        lib.kvto_unpack_nhd_to_hnd(exp.ctypes.data, dst_ids.ctypes.data, len(ids), heads, ntpb,
+                                   row, blob.ctypes.data)
+        assert np.array_equal(_host(dst_layers[l][0]), exp), l
+        # round trip: destination pages hold the source pages' bytes, still HND
+        got = _host(dst_layers[l][0]).reshape(-1, B)
+        assert np.array_equal(got[dst_ids], hnd.reshape(-1, B)[ids])
+
+
+def test_config3_transposing_pack_hnd_to_nhd():
+    _transposing(workloads.llama70b_flashinfer(n_layers=2, pool=128, n_req=3, tokens=500))
+
+
+@pytest.mark.parametrize("heads,ntpb,row", [(1, 16, 256), (3, 5, 48), (8, 16, 16), (2, 64, 128)])
+def test_transposing_pack_other_geometries(heads, ntpb, row):
+    w = workloads.llama70b_flashinfer(n_layers=1, pool=40, n_req=2, tokens=3 * ntpb)
+    T = 2 * heads * row
+    for info in (w.src_info, w.dst_info):
+        info["block_sizes"], info["token_sizes"], info["num_kv_heads"] = [T * ntpb], [T], heads
+    rng = np.random.default_rng(5)
+    w.tasks = [[0, 3 * ntpb, True, [[int(x) for x in rng.choice(40, 3, replace=False)]],
+                [[int(x) for x in 3 * i + np.arange(3)]]] for i in range(2)]
+    w.xform = (heads, ntpb, row)
+    _transposing(w)
+
+
+def test_arbitrary_ranges_including_misaligned():
+    rng = np.random.default_rng(42)
+    cap = 1 << 20
+    runs, used, pos = [], np.zeros(cap, dtype=bool), 0
+    for ln in list(rng.integers(1, 5000, size=200)) + [1, 2, 3, 15, 16, 17, 255, 257, 70001]:
+        ln = int(ln)
+        for _ in range(100):
+            d = int(rng.integers(0, cap - ln))
+            if not used[d:d + ln].any():
+                break
+        used[d:d + ln] = True
+        s = int(rng.integers(0, cap - ln))
+        if rng.random() < 0.5:
+            s, d2 = s & ~15, d
+        runs.append((s, d, ln))
+    runs = np.array(runs, dtype=np.uint64)
+    lists = kvt_amd.BlockLists()
+    lists.append(0, runs)
+    plan = kvt_amd.Plan(0, lists, [cap], [cap], chunk_bytes=8192)
+    src = _dev_bytes(cap, 9, "raw")
+    dst = torch.full((cap,), 0x11, dtype=torch.uint8, device="cuda")
+    sc, dc = kvt_amd.Cache(0, [[src]], [cap]), kvt_amd.Cache(0, [[dst]], [cap])
+    packed = torch.zeros(plan.layer_bytes, dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, 1, packed, plan.layer_bytes)
+    plan.unpack(dc, 0, 1, packed, plan.layer_bytes)
+    torch.cuda.synchronize()
+    blob = checkers.oracle_pack(_host(src), runs)
+    assert np.array_equal(_host(packed)[:len(blob)], blob)
+    exp = np.full(cap, 0x11, dtype=np.uint8)
+    checkers.oracle_unpack(exp, runs, blob)
+    assert np.array_equal(_host(dst), exp)
+
+
+def test_plan_refuses_ranges_beyond_capacity_and_small_caches():
+    lists = kvt_amd.BlockLists()
+    lists.append(0, [(0, 0, 4096), (8192, 61440, 8192)])
+    with pytest.raises(kvt_amd.KvtError) as e:
+        kvt_amd.Plan(0, lists, [65536], [65536])
+    assert e.value.code == 1
+    plan = kvt_amd.Plan(0, lists, [65536], [131072])
+    buf = torch.zeros(65536, dtype=torch.uint8, device="cuda")
+    small = kvt_amd.Cache(0, [[buf]], [65536])
+    packed = torch.zeros(plan.layer_bytes, dtype=torch.uint8, device="cuda")
+    plan.pack(small, 0, 1, packed, plan.layer_bytes)          # source side fits
+    with pytest.raises(kvt_amd.KvtError) as e:
+        plan.unpack(small, 0, 1, packed, plan.layer_bytes)    # destination side does not
+    assert e.value.code == 1
+    with pytest.raises(kvt_amd.KvtError):
+        plan.pack(small, 1, 1, packed, plan.layer_bytes)      # layer out of range
+    torch.cuda.synchronize()
+
+
+def test_empty_plan_is_a_no_op():
+    lists = kvt_amd.BlockLists()
+    lists.append(0, np.zeros((0, 3), dtype=np.uint64))
+    plan = kvt_amd.Plan(0, lists, [4096], [4096])
+    assert plan.num_chunks == 0 and plan.layer_bytes == 0
+    buf = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    plan.pack(kvt_amd.Cache(0, [[buf]], [4096]), 0, 1, buf, 0)
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------ reference-shaped entry points
+
+def _soa(runs_contig_gpu_len):
+    a = np.ascontiguousarray(runs_contig_gpu_len, dtype=np.int64)
+    return [torch.from_numpy(np.ascontiguousarray(a[:, i])).cuda() for i in range(3)]
+
+
+@pytest.mark.parametrize("n,maxlen", [(5, 200000), (300, 5000), (5000, 700)])
+def test_launch_copy_direct_gather_and_scatter(n, maxlen):
+    rng = np.random.default_rng(n)
+    cap = 8 << 20
+    lens = rng.integers(1, maxlen, size=n) // 16 * 16 + rng.choice([0, 16, 7], size=n)
+    lens = np.maximum(lens, 1)
+    gpu_off = np.sort(rng.choice(cap // 1024 - maxlen // 1024 - 2, size=n, replace=False)) * 1024
+    lens = np.minimum(lens, np.diff(np.append(gpu_off, cap)))
+    contig = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    total = int(lens.sum())
+    src = _dev_bytes(cap, 77, "raw")
+    out = torch.zeros(total, dtype=torch.uint8, device="cuda")
+    so, do, ln = _soa(np.stack([gpu_off, contig, lens], axis=1))
+    lib = kvt_amd.lib()
+    rc = lib.kvt_launch_copy_d2h_direct(src.data_ptr(), out.data_ptr(), so.data_ptr(),
+                                        do.data_ptr(), ln.data_ptr(), n, 0, 0, None)
+    assert rc == 0, lib.kvt_last_error()
+    torch.cuda.synchronize()
+    runs = np.stack([gpu_off, gpu_off, lens], axis=1).astype(np.uint64)
+    blob = checkers.oracle_pack(_host(src), runs)
+    assert np.array_equal(_host(out), blob)
+    dst = torch.full((cap,), 0x3C, dtype=torch.uint8, device="cuda")
+    rc = lib.kvt_launch_copy_h2d_direct(out.data_ptr(), dst.data_ptr(), do.data_ptr(),
+                                        so.data_ptr(), ln.data_ptr(), n, 64, 256, None)
+    assert rc == 0, lib.kvt_last_error()
+    torch.cuda.synchronize()
+    exp = np.full(cap, 0x3C, dtype=np.uint8)
+    checkers.oracle_unpack(exp, runs, blob)
+    assert np.array_equal(_host(dst), exp)
+
+
+@pytest.mark.parametrize("max_block_num", [0, 7])
+def test_copy_handle_data_with_kernel_pinned_host_buffer(max_block_num):
+    w = workloads.llama8b_single(n_layers=1, pool=64, tokens=300)
+    runs = _oracle_lists(w)[0]
+    cap = w.capacities("src")[0]
+    layer = _dev_bytes(cap, 5)
+    total = int(runs[:, 2].sum())
+    pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
+    n = len(runs)
+    meta_n = 3 * max(n, 8192)
+    dev_meta = torch.zeros(meta_n, dtype=torch.int64, device="cuda")
+    host_meta = torch.zeros(meta_n, dtype=torch.int64).pin_memory()
+    # sender convention: kernel blocks carry the GPU offset in dst_offset (tcp_channel.cpp:538-542)
+    kb = np.stack([np.zeros(n, dtype=np.uint64), runs[:, 0], runs[:, 2]], axis=1).copy()
+    lib = kvt_amd.lib()
+    st = torch.cuda.Stream()
+    rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(), kb.ctypes.data,
+                                              n, total, 1, 0, st.cuda_stream, dev_meta.data_ptr(),
+                                              host_meta.data_ptr(), max_block_num)
+    assert rc == 0, lib.kvt_last_error()
+    st.synchronize()
+    blob = checkers.oracle_pack(_host(layer), runs)
+    assert np.array_equal(pinned.numpy(), blob)
+    # receiver: scatter from the pinned buffer by dst_offset
+    dst = torch.full((cap,), 0x77, dtype=torch.uint8, device="cuda")
+    rb = np.ascontiguousarray(runs)
+    rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), dst.data_ptr(), rb.ctypes.data, n,
+                                              total, 0, 0, st.cuda_stream, dev_meta.data_ptr(),
+                                              host_meta.data_ptr(), max_block_num)
+    assert rc == 0, lib.kvt_last_error()
+    st.synchronize()
+    exp = np.full(cap, 0x77, dtype=np.uint8)
+    checkers.oracle_unpack(exp, runs, blob)
+    assert np.array_equal(_host(dst), exp)
+    # wrong total is refused before anything is launched
+    assert lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), dst.data_ptr(), rb.ctypes.data,
+                                                n, total + 1, 0, 0, None, dev_meta.data_ptr(),
+                                                host_meta.data_ptr(), 0) == 3
+
+
+def test_bf16_to_fp8_all_bit_patterns_and_converting_gather():
+    lib = kvt_amd.lib()
+    o = checkers.oracle()
+    bits = np.arange(65536, dtype=np.uint16)
+    src = torch.from_numpy(bits.view(np.int16).copy()).cuda()
+    out = torch.zeros(65536, dtype=torch.uint8, device="cuda")
+    so = torch.tensor([0, 2 * 40000], dtype=torch.int64, device="cuda")
+    do = torch.tensor([0, 40000], dtype=torch.int64, device="cuda")
+    ln = torch.tensor([40000, 25536], dtype=torch.int64, device="cuda")
+    assert lib.kvt_launch_copy_d2h_bf16_to_fp8(src.data_ptr(), out.data_ptr(), so.data_ptr(),
+                                               do.data_ptr(), ln.data_ptr(), 2, 0, 0, None) == 0
+    torch.cuda.synchronize()
+    exp = np.array([o.kvto_bf16_to_fp8(int(b)) for b in bits], dtype=np.uint8)
+    assert np.array_equal(_host(out), exp)
+    # unaligned element offsets take the scalar path
+    so2 = torch.tensor([2 * 3], dtype=torch.int64, device="cuda")
+    do2 = torch.tensor([5], dtype=torch.int64, device="cuda")
+    ln2 = torch.tensor([1001], dtype=torch.int64, device="cuda")
+    out2 = torch.zeros(2000, dtype=torch.uint8, device="cuda")
+    assert lib.kvt_launch_copy_d2h_bf16_to_fp8(src.data_ptr(), out2.data_ptr(), so2.data_ptr(),
+                                               do2.data_ptr(), ln2.data_ptr(), 1, 0, 0, None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(_host(out2)[5:1006], exp[3:1004])
+    # the "handle data" form: lengths are bf16 bytes, the pinned side gets half
+    w = workloads.llama8b_single(n_layers=1, pool=32, tokens=200)
+    runs = _oracle_lists(w)[0]
+    layer = _dev_bytes(w.capacities("src")[0], 8)
+    total = int(runs[:, 2].sum())
+    pinned = torch.zeros(total // 2, dtype=torch.uint8).pin_memory()
+    n = len(runs)
+    dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
+    host_meta = torch.zeros(3 * 8192, dtype=torch.int64).pin_memory()
+    kb = np.stack([np.zeros(n, dtype=np.uint64), runs[:, 0], runs[:, 2]], axis=1).copy()
+    assert lib.kvt_copy_d2h_bf16_to_fp8(pinned.data_ptr(), layer.data_ptr(), kb.ctypes.data, n,
+                                        total, 0, None, dev_meta.data_ptr(), host_meta.data_ptr(),
+                                        0) == 0
+    torch.cuda.synchronize()
+    fp8_runs = np.stack([runs[:, 0], runs[:, 1], runs[:, 2] // 2], axis=1).astype(np.uint64).copy()
+    exp = np.zeros(total // 2, dtype=np.uint8)
+    o.kvto_pack_bf16_to_fp8(_host(layer).ctypes.data, fp8_runs.ctypes.data, n, exp.ctypes.data)
+    assert np.array_equal(pinned.numpy(), exp)
+
+
+# ------------------------------------------------------- gating and staging
+
+def test_per_layer_session_on_side_stream():
+    w = workloads.llama8b_batch(n_layers=6, src_pool=256, dst_pool=256, n_req=3, min_tok=200,
+                                max_tok=900)
+    plan, lists = pipeline.build_plan(w, 0)
+    layers = [[torch.zeros(w.capacities("src")[0], dtype=torch.uint8, device="cuda")]
+              for _ in range(w.n_layers)]
+    cache = kvt_amd.Cache(0, layers, w.capacities("src"))
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    sess = kvt_amd.Session(plan, cache, packed, stride)
+    compute = torch.cuda.Stream()
+    fresh = [_dev_bytes(w.capacities("src")[0], 50 + l) for l in range(w.n_layers)]
+    with torch.cuda.stream(compute):
+        for l in range(w.n_layers):
+            layers[l][0].copy_(fresh[l])           # the "forward pass" writes layer l
+            sess.save_layer(l, compute.cuda_stream)
+    for l in range(w.n_layers):
+        sess.wait_layer(l)                         # what the transport thread does per layer
+        blob = checkers.oracle_pack(_host(fresh[l]), lists.tensor(0))
+        got = packed[l * stride:l * stride + len(blob)].cpu().numpy()
+        assert np.array_equal(got, blob), l
+    sess.join(compute.cuda_stream)
+    compute.synchronize()
+    sess.close()
+
+
+def test_session_inside_hip_graph_replays():
+    w = workloads.llama8b_single(n_layers=4, pool=64, tokens=200)
+    plan, lists = pipeline.build_plan(w, 0)
+    cap = w.capacities("src")[0]
+    layers = [[torch.zeros(cap, dtype=torch.uint8, device="cuda")] for _ in range(w.n_layers)]
+    staging = [torch.zeros(cap, dtype=torch.uint8, device="cuda") for _ in range(w.n_layers)]
+    cache = kvt_amd.Cache(0, layers, [cap])
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    sess = kvt_amd.Session(plan, cache, packed, stride)
+    graph = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        with torch.cuda.graph(graph, stream=s):
+            for l in range(w.n_layers):
+                layers[l][0].copy_(staging[l])
+                sess.save_layer(l, s.cuda_stream)
+            sess.join(s.cuda_stream)
+    for rep in range(3):
+        contents = [_dev_bytes(cap, 900 + 10 * rep + l) for l in range(w.n_layers)]
+        for l in range(w.n_layers):
+            staging[l].copy_(contents[l])
+        packed.fill_(0)                                # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for l in range(w.n_layers):
+            blob = checkers.oracle_pack(_host(contents[l]), lists.tensor(0))
+            got = packed[l * stride:l * stride + len(blob)].cpu().numpy()
+            assert np.array_equal(got, blob), (rep, l)
+    sess.close()
+
+
+def test_stager_save_load_round_trip_overlapped_with_packing():
+    w = workloads.llama70b_flashinfer(n_layers=4, pool=64, n_req=2, tokens=300)
+    plan, lists = pipeline.build_plan(w, 0)
+    src_layers = _make_caches(w, "src", 21)
+    dst_layers = _make_caches(w, "dst", 22, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    nbytes = plan.layer_bytes
+    stager = kvt_amd.Stager(0, nbytes, 2)
+    dev_buf = [torch.zeros(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    pack_stream = torch.cuda.Stream()
+    store = []                                    # the "KV store": host copies per layer
+    for l in range(w.n_layers):
+        slot = l % 2
+        if l >= 2:
+            stager.wait(slot)                     # slot's previous D2H done -> consume it
+            store.append(stager.slot_array(slot, nbytes).copy())
+        plan.pack(sc, l, 1, dev_buf[slot], nbytes, pack_stream.cuda_stream)
+        stager.save(slot, dev_buf[slot], nbytes, pack_stream.cuda_stream)
+    for l in range(w.n_layers - 2, w.n_layers):
+        stager.wait(l % 2)
+        store.append(stager.slot_array(l % 2, nbytes).copy())
+    o_runs = _oracle_lists(w)[0]
+    assert np.array_equal(o_runs, lists.tensor(0))
+    # what was stored is the NHD-ordered packed layer
+    heads, ntpb, row = w.xform
+    B = 2 * heads * ntpb * row
+    ids = np.concatenate([np.arange(r[0] // B, (r[0] + r[2]) // B) for r in o_runs]).astype(np.uint32)
+    lib = checkers.oracle()
+    for l in range(w.n_layers):
+        blob = np.zeros(len(ids) * B, dtype=np.uint8)
+        lib.kvto_pack_hnd_to_nhd(_host(src_layers[l][0]).ctypes.data, ids.ctypes.data, len(ids),
+                                 heads, ntpb, row, blob.ctypes.data)
+        assert np.array_equal(store[l][:len(blob)], blob), l
+    # load path: host -> slot -> device -> unpack
+    un_stream = torch.cuda.Stream()
+    for l in range(w.n_layers):
+        slot = l % 2
+        stager.wait(slot)
+        un_stream.synchronize()                   # device buffer of this slot is free again
+        stager.slot_array(slot, nbytes)[:] = store[l]
+        stager.load(slot, dev_buf[slot], nbytes, un_stream.cuda_stream)
+        plan.unpack(dc, l, 1, dev_buf[slot], nbytes, un_stream.cuda_stream)
+    un_stream.synchronize()
+    dst_ids = np.concatenate([np.arange(r[1] // B, (r[1] + r[2]) // B) for r in o_runs])
+    for l in range(w.n_layers):
+        got = _host(dst_layers[l][0]).reshape(-1, B)
+        assert np.array_equal(got[dst_ids], _host(src_layers[l][0]).reshape(-1, B)[ids])
+    stager.close()
+
+
+def test_measure_pcie_reports_a_plausible_rate():
+    lib = kvt_amd.lib()
+    for direction in (0, 1):
+        r = C.c_double()
+        assert lib.kvt_measure_pcie(0, direction, 64 << 20, 3, C.byref(r)) == 0
+        assert 1e9 < r.value < 2e11
+
+
+def test_copy_linear():
+    a = _dev_bytes((1 << 20) + 48, 1, "raw")
+    b = torch.zeros_like(a)
+    assert kvt_amd.lib().kvt_copy_linear(b.data_ptr(), a.data_ptr(), a.numel(), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
