@@ -1,6 +1,8 @@
 """ctypes declarations for every symbol of include/kvt_hip.h plus small RAII wrappers."""
 import ctypes as C
+import importlib.util
 import os
+import sys
 
 import numpy as np
 
@@ -91,6 +93,26 @@ class KvtError(RuntimeError):
 _lib = None
 
 
+def _preload_hip_runtime():
+    """A process must hold ONE HIP runtime. PyTorch wheels bundle their own
+    libamdhip64 (same SONAME as the system one); if this library were loaded
+    first it would bind the system runtime and a later ``import torch`` would
+    bring in a second one that then finds no device. So when PyTorch is
+    installed but not imported yet, its runtime is mapped first and the
+    dynamic loader resolves this library's dependency to it by SONAME."""
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.origin:
+        return
+    cand = os.path.join(os.path.dirname(spec.origin), "lib", "libamdhip64.so")
+    if os.path.exists(cand):
+        C.CDLL(cand, mode=C.RTLD_GLOBAL)
+
+
 def lib():
     """Loads libkvt_hip.so (built in-tree by ``make -C llumnix-kv_amd``)."""
     global _lib
@@ -98,6 +120,7 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise KvtError(-1, "libkvt_hip.so is not built: run `make -C llumnix-kv_amd` "
                                "(or __graft_entry__.build())")
+        _preload_hip_runtime()
         handle = C.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)

@@ -191,17 +191,20 @@ def test_transposing_pack_other_geometries(heads, ntpb, row):
 def test_arbitrary_ranges_including_misaligned():
     rng = np.random.default_rng(42)
     cap = 1 << 20
-    runs, used, pos = [], np.zeros(cap, dtype=bool), 0
-    for ln in list(rng.integers(1, 5000, size=200)) + [1, 2, 3, 15, 16, 17, 255, 257, 70001]:
+    runs, used = [], np.zeros(cap, dtype=bool)
+    # destination ranges must not overlap (overlapping scatters race); largest first
+    for ln in [70001, 257, 255, 17, 16, 15, 3, 2, 1] + list(rng.integers(1, 5000, size=200)):
         ln = int(ln)
-        for _ in range(100):
+        while True:
             d = int(rng.integers(0, cap - ln))
             if not used[d:d + ln].any():
                 break
         used[d:d + ln] = True
         s = int(rng.integers(0, cap - ln))
         if rng.random() < 0.5:
-            s, d2 = s & ~15, d
+            s &= ~15
+        if rng.random() < 0.3:
+            s = (s & ~15) | (d & 15)          # same misalignment on both sides
         runs.append((s, d, ln))
     runs = np.array(runs, dtype=np.uint64)
     lists = kvt_amd.BlockLists()
@@ -367,7 +370,8 @@ def test_bf16_to_fp8_all_bit_patterns_and_converting_gather():
     torch.cuda.synchronize()
     fp8_runs = np.stack([runs[:, 0], runs[:, 1], runs[:, 2] // 2], axis=1).astype(np.uint64).copy()
     exp = np.zeros(total // 2, dtype=np.uint8)
-    o.kvto_pack_bf16_to_fp8(_host(layer).ctypes.data, fp8_runs.ctypes.data, n, exp.ctypes.data)
+    layer_h = _host(layer)
+    o.kvto_pack_bf16_to_fp8(layer_h.ctypes.data, fp8_runs.ctypes.data, n, exp.ctypes.data)
     assert np.array_equal(pinned.numpy(), exp)
 
 
@@ -463,8 +467,9 @@ def test_stager_save_load_round_trip_overlapped_with_packing():
     lib = checkers.oracle()
     for l in range(w.n_layers):
         blob = np.zeros(len(ids) * B, dtype=np.uint8)
-        lib.kvto_pack_hnd_to_nhd(_host(src_layers[l][0]).ctypes.data, ids.ctypes.data, len(ids),
-                                 heads, ntpb, row, blob.ctypes.data)
+        src_h = _host(src_layers[l][0])
+        lib.kvto_pack_hnd_to_nhd(src_h.ctypes.data, ids.ctypes.data, len(ids), heads, ntpb, row,
+                                 blob.ctypes.data)
         assert np.array_equal(store[l][:len(blob)], blob), l
     # load path: host -> slot -> device -> unpack
     un_stream = torch.cuda.Stream()
@@ -476,7 +481,8 @@ def test_stager_save_load_round_trip_overlapped_with_packing():
         stager.load(slot, dev_buf[slot], nbytes, un_stream.cuda_stream)
         plan.unpack(dc, l, 1, dev_buf[slot], nbytes, un_stream.cuda_stream)
     un_stream.synchronize()
-    dst_ids = np.concatenate([np.arange(r[1] // B, (r[1] + r[2]) // B) for r in o_runs])
+    dst_ids = np.concatenate([np.arange(r[1] // B, (r[1] + r[2]) // B) for r in o_runs]).astype(np.int64)
+    ids = ids.astype(np.int64)
     for l in range(w.n_layers):
         got = _host(dst_layers[l][0]).reshape(-1, B)
         assert np.array_equal(got[dst_ids], _host(src_layers[l][0]).reshape(-1, B)[ids])
