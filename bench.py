@@ -1,0 +1,371 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV-cache pack/unpack hot path on one MI355X.
+
+One *step* = one pass of the hot path over one batch: ParseBlock for every
+request of the batch, merge, plan upload, then ONE pack launch (all layers) and
+ONE unpack launch (all layers). Inputs (caches, block tables) are resident
+before the timed region. Steps are issued the way a serving loop issues them:
+the host prepares step k+1 while the GPU still runs step k.
+
+Prints one JSON line; see DESIGN.md for the meaning of every field.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path[:0] = [os.path.join(ROOT, "llumnix-kv_amd"), os.path.join(ROOT, "tests")]
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_workload(cfg, scale):
+    from kvt_amd import workloads as W
+    if cfg == 1:
+        return [W.llama8b_single()]
+    if cfg == 2:
+        if scale < 1.0:
+            return [W.llama8b_batch(n_layers=max(2, int(32 * scale)),
+                                    src_pool=max(1024, int(16384 * scale)),
+                                    dst_pool=max(1536, int(24576 * scale)),
+                                    n_req=max(2, int(64 * scale)),
+                                    min_tok=max(64, int(1024 * scale)),
+                                    max_tok=max(128, int(8192 * scale)))]
+        return [W.llama8b_batch()]
+    if cfg == 3:
+        return [W.llama70b_flashinfer(n_layers=max(2, int(80 * scale)),
+                                      pool=max(512, int(8192 * scale)),
+                                      n_req=max(2, int(32 * scale)))]
+    if cfg == 4:
+        return [W.deepseek_mla(n_layers=max(2, int(61 * scale)), pool=max(512, int(4608 * scale)),
+                               n_req=max(2, int(16 * scale)))]
+    if cfg == 5:
+        return [W.qwen3next_attn(n_layers=max(2, int(12 * scale)),
+                                 pool=max(512, int(36864 * scale)), n_req=max(2, int(128 * scale))),
+                W.qwen3next_gdn(n_layers=max(2, int(36 * scale)), slots=max(4, int(256 * scale)),
+                                n_req=max(2, int(128 * scale)))]
+    raise SystemExit("unknown --config %r" % cfg)
+
+
+class DeviceSide:
+    """Caches and packed buffer of one workload, resident in HBM."""
+
+    def __init__(self, torch, kvt, w, seed):
+        self.w = w
+        g = torch.Generator(device="cuda")
+        self.src, self.dst = [], []
+        for l in range(w.n_layers):
+            row_s, row_d = [], []
+            for t, (cs, cd) in enumerate(zip(w.capacities("src"), w.capacities("dst"))):
+                g.manual_seed(seed * 100003 + l * 16 + t)
+                if w.elem_dtype == "bf16":
+                    x = torch.empty(cs // 2, dtype=torch.bfloat16, device="cuda")
+                    step = 1 << 28
+                    for o in range(0, x.numel(), step):  # bounded fp32 temporaries
+                        n = min(step, x.numel() - o)
+                        x[o:o + n] = torch.rand(n, generator=g, device="cuda") * 2 - 1
+                    row_s.append(x.view(torch.uint8))
+                elif w.elem_dtype == "fp8":
+                    x = torch.randn(cs, generator=g, device="cuda").clamp_(-448, 448)
+                    row_s.append(x.to(torch.float8_e4m3fn).view(torch.uint8))
+                else:
+                    row_s.append(torch.randn(cs // 4, generator=g, device="cuda").view(torch.uint8))
+                row_d.append(torch.zeros(cd, dtype=torch.uint8, device="cuda"))
+            self.src.append(row_s)
+            self.dst.append(row_d)
+        self.src_cache = kvt.Cache(0, self.src, w.capacities("src"))
+        self.dst_cache = kvt.Cache(0, self.dst, w.capacities("dst"))
+
+
+def ev_ms(lib, a, b):
+    ms = C.c_float()
+    rc = lib.kvt_event_elapsed_ms(a, b, C.byref(ms))
+    assert rc == 0, lib.kvt_last_error()
+    return ms.value
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=2, help="BASELINE.json configs[] index + 1")
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")
+    ap.add_argument("--chunk-bytes", type=int, default=0)
+    ap.add_argument("--cpu-layers", type=int, default=4, help="layers in the CPU baseline sample")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py: this build measures ONE MI355X; the path has no inter-GPU "
+                         "part, so --gpus N with N > 1 is not supported (see DESIGN.md, sharding).")
+
+    import numpy as np
+    import torch
+
+    import kvt_amd as kvt
+    from kvt_amd import pipeline
+
+    lib = kvt.lib()
+    if kvt.device_count() < 1:
+        raise SystemExit("bench.py: no usable MI355X (gfx950) device; there is no CPU fallback")
+
+    wls = build_workload(args.config, args.scale)
+    t_init = time.time()
+    sides = [DeviceSide(torch, kvt, w, 7 + i) for i, w in enumerate(wls)]
+    torch.cuda.synchronize()
+    log("caches resident in %.1fs" % (time.time() - t_init))
+
+    infos = [w.worker_infos() for w in wls]
+    tasks = [w.task_bufs() for w in wls]
+
+    def prepare(i):
+        """host part of a step for workload i: ParseBlock + merge + plan upload"""
+        w = wls[i]
+        lists, _ = pipeline.parse_batch(w.cache_shape, infos[i][0], infos[i][1], tasks[i])
+        plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
+                        chunk_bytes=args.chunk_bytes)
+        return plan, lists
+
+    first = [prepare(i) for i in range(len(wls))]
+    strides = [p.layer_bytes for p, _ in first]
+    payload = [sum(p.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
+               for (p, _), w in zip(first, wls)]
+    P = sum(payload)
+    packed = [torch.empty(max(1, s * w.n_layers), dtype=torch.uint8, device="cuda")
+              for s, w in zip(strides, wls)]
+    log("payload per step: %.3f GiB, chunks per layer: %s" %
+        (P / 2**30, [p.num_chunks for p, _ in first]))
+
+    stream = torch.cuda.Stream()
+    sh = stream.cuda_stream
+
+    def new_event():
+        e = C.c_void_p()
+        assert lib.kvt_event_create(C.byref(e)) == 0, lib.kvt_last_error()
+        return e
+
+    def launch(plans, evs):
+        lib.kvt_event_record(evs[0], sh)
+        for i, (plan, _) in enumerate(plans):
+            plan.pack(sides[i].src_cache, 0, wls[i].n_layers, packed[i], strides[i], sh)
+        lib.kvt_event_record(evs[1], sh)
+        for i, (plan, _) in enumerate(plans):
+            plan.unpack(sides[i].dst_cache, 0, wls[i].n_layers, packed[i], strides[i], sh)
+        lib.kvt_event_record(evs[2], sh)
+
+    keep = [first]
+    plans = first
+    for _ in range(args.warmup):
+        launch(plans, [new_event() for _ in range(3)])
+        plans = [prepare(i) for i in range(len(wls))]
+        keep.append(plans)
+    torch.cuda.synchronize()
+
+    events, host_ms = [], []
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        evs = [new_event() for _ in range(3)]
+        events.append(evs)
+        launch(plans, evs)
+        # host side of the following step (ParseBlock + merge + plan upload) overlaps this
+        # step's GPU work; every timed step pays for one such preparation
+        h0 = time.perf_counter()
+        plans = [prepare(i) for i in range(len(wls))]
+        keep.append(plans)
+        host_ms.append((time.perf_counter() - h0) * 1e3)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+    pack_ms = [ev_ms(lib, e[0], e[1]) for e in events]
+    unpack_ms = [ev_ms(lib, e[1], e[2]) for e in events]
+    pack_avg, unpack_avg = statistics.mean(pack_ms), statistics.mean(unpack_ms)
+    value = 4.0 * P / (ms_per_step * 1e-3) / 1e9
+    achieved = 2.0 * P / (pack_avg * 1e-3) / 1e9
+    log("pack %.3f ms  unpack %.3f ms  host %.3f ms/step  wall %.3f ms/step" %
+        (pack_avg, unpack_avg, statistics.mean(host_ms), ms_per_step))
+
+    out = {
+        "metric": "pack+unpack GB/s (bytes read + bytes written per second, whole job)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": "; ".join(w.name for w in wls), "baseline_config": args.config,
+                   "scale": args.scale, "layers": [w.n_layers for w in wls],
+                   "requests": [len(w.tasks) for w in wls], "payload_bytes_per_step": P,
+                   "chunk_bytes": args.chunk_bytes or 32768},
+        "frac_hbm_peak": round(value * 1e9 / HBM_PEAK, 4),
+        "pack_ms": round(pack_avg, 4),
+        "unpack_ms": round(unpack_avg, 4),
+        "pack_gbps": round(achieved, 1),
+        "unpack_gbps": round(2.0 * P / (unpack_avg * 1e-3) / 1e9, 1),
+        "host_parse_plan_ms": round(statistics.mean(host_ms), 4),
+        "roofline": {"bound": "hbm", "kernel": "copy_chunks_kernel<pack>" if not wls[0].xform
+                     else "xform_chunks_kernel<pack>",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None},
+    }
+
+    # ---------------------------------------------------------------- parity spot check + CPU leg
+    if not args.skip_cpu:
+        import checkers
+        w, side = wls[0], sides[0]
+        L = max(1, min(args.cpu_layers, w.n_layers))
+        s_info, d_info = infos[0]
+        rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, s_info, d_info)
+        assert rc == 0
+        olib = checkers.oracle()
+        host_src = [[t.cpu().numpy() for t in side.src[l]] for l in range(L)]
+        host_dst = [[np.zeros(c, dtype=np.uint8) for c in w.capacities("dst")] for _ in range(L)]
+        stride = strides[0]
+        gpu_packed = packed[0][:L * stride].cpu().numpy()
+        plan0 = first[0][0]
+
+        def cpu_pass():
+            t_a = time.perf_counter()
+            rc, outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, tasks[0])
+            assert rc == 0
+            if kind == 0:
+                outs = [checkers.oracle_merge(o)[0] for o in outs]
+            t_b = time.perf_counter()
+            blobs = []
+            for l in range(L):
+                blobs.append([checkers.oracle_pack(host_src[l][t], outs[t])
+                              for t in range(w.n_tensors)])
+            t_c = time.perf_counter()
+            if w.xform is None:
+                for l in range(L):
+                    for t in range(w.n_tensors):
+                        checkers.oracle_unpack(host_dst[l][t], outs[t], blobs[l][t])
+            t_d = time.perf_counter()
+            return (t_b - t_a, t_c - t_b, t_d - t_c), outs, blobs
+
+        reps = [cpu_pass() for _ in range(3)]
+        times = sorted(r[0] for r in reps)
+        parse_s, pack_s, unpack_s = times[1]
+        outs, blobs = reps[-1][1], reps[-1][2]
+        parity = True
+        if w.xform is None:
+            for l in range(L):
+                for t in range(w.n_tensors):
+                    off = l * stride + plan0.tensor_offset(t)
+                    parity &= bool(np.array_equal(gpu_packed[off:off + len(blobs[l][t])],
+                                                  blobs[l][t]))
+            gpu_dst = [[x.cpu().numpy() for x in side.dst[l]] for l in range(L)]
+            for l in range(L):
+                for t in range(w.n_tensors):
+                    parity &= bool(np.array_equal(gpu_dst[l][t], host_dst[l][t]))
+        P_s = sum(int(o[:, 2].sum()) for o in outs) * L
+        total_s = parse_s + pack_s + unpack_s
+        out["parity_vs_oracle"] = parity if w.xform is None else "n/a (transposing pack is checked in tests/)"
+        out["cpu_baseline"] = {
+            "value": round(4.0 * P_s / total_s / 1e9, 2), "unit": "GB/s", "cores": 1,
+            "kind": "port",
+            "sample": "%d of %d layers of the same batch (%d requests): ParseBlock+merge %.1f ms, "
+                      "pack %.1f ms, unpack %.1f ms; median of 3" %
+                      (L, w.n_layers, len(w.tasks), parse_s * 1e3, pack_s * 1e3, unpack_s * 1e3),
+            "host_cores_available": os.cpu_count(),
+        }
+        # all host cores, threads striding over layers (not the reference's threading model)
+        nthr = min(16, os.cpu_count() or 1, L)
+        if nthr > 1 and w.xform is None and w.n_tensors == 1:
+            ptrs = (C.c_void_p * L)(*[host_src[l][0].ctypes.data for l in range(L)])
+            runs0 = np.ascontiguousarray(outs[0])
+            tb = int(runs0[:, 2].sum())
+            blob = np.empty(L * tb, dtype=np.uint8)
+            tt = []
+            for _ in range(3):
+                a = time.perf_counter()
+                olib.kvto_pack_layers(ptrs, L, runs0.ctypes.data, len(runs0), blob.ctypes.data, tb,
+                                      nthr)
+                tt.append(time.perf_counter() - a)
+            out["cpu_baseline_threads"] = {"pack_gbps": round(2.0 * tb * L / sorted(tt)[1] / 1e9, 2),
+                                           "cores": nthr}
+        log("cpu baseline done, parity:", out.get("parity_vs_oracle"))
+        del host_src, host_dst, gpu_packed
+
+    # ---------------------------------------------------------------- per-request latency, staging
+    if not args.skip_extras:
+        w, side = wls[0], sides[0]
+        lat = []
+        reqs = list(range(len(w.tasks)))
+        for r in reqs:
+            lists, _ = pipeline.parse_batch(w.cache_shape, infos[0][0], infos[0][1], [tasks[0][r]])
+            plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
+                            chunk_bytes=args.chunk_bytes)
+            keep.append(plan)
+            a, b = new_event(), new_event()
+            for rep in range(2):   # second run is the measurement
+                lib.kvt_event_record(a, sh)
+                plan.pack(side.src_cache, 0, w.n_layers, packed[0], plan.layer_bytes, sh)
+                lib.kvt_event_record(b, sh)
+            lib.kvt_event_synchronize(b)
+            lat.append(ev_ms(lib, a, b) * 1e3)
+        out["latency_p50_us"] = round(statistics.median(lat), 2)
+        out["latency_note"] = "per request: one pack launch covering all %d layers, GPU time" % w.n_layers
+
+        # pinned-host staging of packed layers, double buffered against the pack kernel
+        plan = first[0][0]
+        nbytes = plan.layer_bytes
+        Ls = min(w.n_layers, 8)
+        if nbytes > 0 and nbytes < (3 << 30):
+            ceil = {}
+            for name, d in (("d2h", 1), ("h2d", 0)):
+                r = C.c_double()
+                assert lib.kvt_measure_pcie(0, d, min(nbytes, 1 << 30), 5, C.byref(r)) == 0
+                ceil[name] = r.value
+            stg = kvt.Stager(0, nbytes, 2)
+            bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
+            ps = torch.cuda.Stream()
+            for phase in ("warm", "timed"):
+                torch.cuda.synchronize()
+                a = time.perf_counter()
+                for l in range(Ls):
+                    slot = l % 2
+                    if l >= 2:
+                        stg.wait(slot)
+                    plan.pack(side.src_cache, l, 1, bufs[slot], nbytes, ps.cuda_stream)
+                    stg.save(slot, bufs[slot], nbytes, ps.cuda_stream)
+                stg.wait(0)
+                stg.wait(1)
+                d2h_s = time.perf_counter() - a
+            for phase in ("warm", "timed"):
+                torch.cuda.synchronize()
+                a = time.perf_counter()
+                for l in range(Ls):
+                    slot = l % 2
+                    stg.load(slot, bufs[slot], nbytes, ps.cuda_stream)
+                    plan.unpack(side.dst_cache, l, 1, bufs[slot], nbytes, ps.cuda_stream)
+                ps.synchronize()
+                h2d_s = time.perf_counter() - a
+            pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * Ls
+            out["staging"] = {
+                "save_gbps": round(pay / d2h_s / 1e9, 2), "load_gbps": round(pay / h2d_s / 1e9, 2),
+                "pcie_d2h_gbps": round(ceil["d2h"] / 1e9, 2), "pcie_h2d_gbps": round(ceil["h2d"] / 1e9, 2),
+                "save_frac_of_pcie": round(pay / d2h_s / ceil["d2h"], 4),
+                "load_frac_of_pcie": round(pay / h2d_s / ceil["h2d"], 4),
+                "sample": "%d layers x %.1f MiB through 2 pinned slots" % (Ls, nbytes / 2**20),
+            }
+            stg.close()
+
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
