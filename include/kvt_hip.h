@@ -137,7 +137,9 @@ typedef struct kvt_xform {
  * `lists` is consumed as-is (call kvt_block_lists_merge first for PEQD).
  * src_capacity / dst_capacity: per-tensor byte sizes the ranges were validated
  * against; pack refuses a cache smaller than src_capacity, unpack one smaller
- * than dst_capacity. chunk_bytes = 0 selects the default. */
+ * than dst_capacity. chunk_bytes bounds one table entry: a power of two in
+ * [4096, 524288], or 0 to derive it from the median range length (at most
+ * 32 KiB). Every entry is moved by ceil(len / 4096) workgroups. */
 typedef struct kvt_plan kvt_plan;
 int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
                     const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,

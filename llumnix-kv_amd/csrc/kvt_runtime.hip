@@ -76,7 +76,7 @@ struct DeviceGuard {
 
 uint64_t round_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
-constexpr uint32_t kDefaultChunk = 32768;
+constexpr uint32_t kMinChunk = 4096, kMaxAutoChunk = 32768, kMaxChunk = 1u << 19;
 constexpr uint64_t kBlobAlign = 256;
 
 }  // namespace
@@ -100,7 +100,8 @@ struct kvt_plan {
   uint64_t layer_bytes = 0;
   bool xform = false;
   XformDev xdev{};
-  Chunk* dev_chunks = nullptr;
+  uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
+  Chunk* dev_chunks = nullptr;     // [0, n_chunks): pack order; [n_chunks, 2 n_chunks): unpack order
 };
 
 struct kvt_session {
@@ -178,9 +179,10 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
     if (lists->tensors.empty() || lists->tensors.size() > KVT_MAX_TENSORS)
       return fail(KVT_ERR_INVALID, "kvt_plan_create: tensor count out of range");
     if (int rc = check_device(device)) return rc;
-    if (chunk_bytes == 0) chunk_bytes = kDefaultChunk;
-    if (chunk_bytes % 256 != 0 || chunk_bytes > (1u << 20))
-      return fail(KVT_ERR_INVALID, "kvt_plan_create: chunk_bytes must be a multiple of 256, <= 1 MiB");
+    if (chunk_bytes != 0 && (chunk_bytes < kMinChunk || chunk_bytes > kMaxChunk ||
+                             (chunk_bytes & (chunk_bytes - 1)) != 0))
+      return fail(KVT_ERR_INVALID,
+                  "kvt_plan_create: chunk_bytes must be a power of two in [4096, 524288]");
 
     std::unique_ptr<kvt_plan> p(new kvt_plan());
     p->device = device;
@@ -197,7 +199,7 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
         return fail(KVT_ERR_INVALID, "layout transform: rows must be multiples of 16 bytes");
       tok_bytes = static_cast<uint64_t>(xform->heads) * xform->row_bytes;
       half = tok_bytes * xform->ntpb;
-      if (tok_bytes > (1u << 19)) return fail(KVT_ERR_INVALID, "layout transform: token row too large");
+      if (tok_bytes > kMaxChunk) return fail(KVT_ERR_INVALID, "layout transform: token row too large");
       p->xform = true;
       p->xdev.heads = xform->heads;
       p->xdev.ntpb = xform->ntpb;
@@ -206,7 +208,30 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       p->xdev.inv_heads = static_cast<uint32_t>((1ull << 32) / p->xdev.heads) + 1u;
     }
 
-    std::vector<Chunk> chunks;
+    if (chunk_bytes == 0) {
+      // Largest power of two not above the median range length, within [4 KiB, 32 KiB]: ranges
+      // shorter than a chunk leave workgroups idle, longer chunks only save table entries.
+      std::vector<uint64_t> lens;
+      for (const RunList& runs : lists->tensors)
+        for (const kvt_ipc_block& r : runs) lens.push_back(p->xform ? half : r.length);
+      uint64_t median = kMaxAutoChunk;
+      if (!lens.empty()) {
+        std::nth_element(lens.begin(), lens.begin() + lens.size() / 2, lens.end());
+        median = lens[lens.size() / 2];
+      }
+      chunk_bytes = kMinChunk;
+      while (chunk_bytes * 2 <= median && chunk_bytes * 2 <= kMaxAutoChunk) chunk_bytes *= 2;
+    }
+    if (p->xform)  // a chunk holds whole tokens
+      while (chunk_bytes < tok_bytes) chunk_bytes *= 2;
+    while ((kMinChunk << p->sub_shift) < chunk_bytes) ++p->sub_shift;
+
+    struct Piece {
+      uint64_t src, dst, packed;
+      uint32_t len;
+      uint16_t tensor, t0;
+    };
+    std::vector<Piece> pieces;
     uint64_t cursor = 0;
     for (uint32_t t = 0; t < p->n_tensors; ++t) {
       cursor = round_up(cursor, kBlobAlign);
@@ -221,34 +246,23 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       uint64_t blob = 0;
       for (const kvt_ipc_block& r : runs) {
         if (!p->xform) {
-          for (uint64_t o = 0; o < r.length; o += chunk_bytes) {
-            Chunk c{};
-            c.cache_src = r.src_offset + o;
-            c.cache_dst = r.dst_offset + o;
-            c.packed = cursor + blob + o;
-            c.len = static_cast<uint32_t>(std::min<uint64_t>(chunk_bytes, r.length - o));
-            c.tensor = static_cast<uint16_t>(t);
-            chunks.push_back(c);
-          }
+          for (uint64_t o = 0; o < r.length; o += chunk_bytes)
+            pieces.push_back(Piece{r.src_offset + o, r.dst_offset + o, cursor + blob + o,
+                                   static_cast<uint32_t>(std::min<uint64_t>(chunk_bytes, r.length - o)),
+                                   static_cast<uint16_t>(t), 0});
         } else {
           const uint64_t page = 2 * half;
           if (r.src_offset % page || r.dst_offset % page || r.length % page)
             return fail(KVT_ERR_INVALID, "layout transform: ranges must be whole pages");
-          const uint32_t tok_per_chunk =
-              static_cast<uint32_t>(std::max<uint64_t>(1, std::min<uint64_t>(chunk_bytes, 1u << 19) / tok_bytes));
-          for (uint64_t o = 0; o < r.length; o += half) {  // one K or V half page at a time
+          const uint32_t tok_per_chunk = static_cast<uint32_t>(chunk_bytes / tok_bytes);
+          for (uint64_t o = 0; o < r.length; o += half)  // one K or V half page at a time
             for (uint32_t t0 = 0; t0 < xform->ntpb; t0 += tok_per_chunk) {
               const uint32_t nt = std::min(tok_per_chunk, xform->ntpb - t0);
-              Chunk c{};
-              c.cache_src = r.src_offset + o;
-              c.cache_dst = r.dst_offset + o;
-              c.packed = cursor + blob + o + static_cast<uint64_t>(t0) * tok_bytes;
-              c.len = static_cast<uint32_t>(nt * tok_bytes);
-              c.tensor = 0;
-              c.t0 = static_cast<uint16_t>(t0);
-              chunks.push_back(c);
+              pieces.push_back(Piece{r.src_offset + o, r.dst_offset + o,
+                                     cursor + blob + o + static_cast<uint64_t>(t0) * tok_bytes,
+                                     static_cast<uint32_t>(nt * tok_bytes), 0,
+                                     static_cast<uint16_t>(t0)});
             }
-          }
         }
         blob += r.length;
       }
@@ -256,14 +270,37 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       cursor += blob;
     }
     p->layer_bytes = round_up(cursor, kBlobAlign);
-    p->n_chunks = chunks.size();
-    if (p->n_chunks > 0x7FFFFFFFull) return fail(KVT_ERR_INVALID, "kvt_plan_create: too many chunks");
+    p->n_chunks = pieces.size();
+    if ((p->n_chunks << p->sub_shift) > 0x7FFFFFF0ull)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create: too many chunks for one launch");
+
+    // Two tables, each walked in ascending cache address of its own direction.
+    std::vector<Chunk> table(2 * pieces.size());
+    std::vector<uint32_t> order(pieces.size());
+    for (int dir = 0; dir < 2; ++dir) {
+      for (uint32_t i = 0; i < order.size(); ++i) order[i] = i;
+      std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
+        const Piece &x = pieces[a], &y = pieces[b];
+        if (x.tensor != y.tensor) return x.tensor < y.tensor;
+        return dir == 0 ? x.src < y.src : x.dst < y.dst;
+      });
+      for (size_t i = 0; i < order.size(); ++i) {
+        const Piece& q = pieces[order[i]];
+        Chunk& c = table[dir * pieces.size() + i];
+        c.cache = dir == 0 ? q.src : q.dst;
+        c.packed = q.packed;
+        c.len = q.len;
+        c.tensor = q.tensor;
+        c.t0 = q.t0;
+        c.reserved = 0;
+      }
+    }
 
     DeviceGuard g;
     if (int rc = g.enter(device)) return rc;
-    if (!chunks.empty()) {
-      KVT_HIP(hipMalloc(reinterpret_cast<void**>(&p->dev_chunks), chunks.size() * sizeof(Chunk)));
-      const hipError_t e = hipMemcpy(p->dev_chunks, chunks.data(), chunks.size() * sizeof(Chunk),
+    if (!table.empty()) {
+      KVT_HIP(hipMalloc(reinterpret_cast<void**>(&p->dev_chunks), table.size() * sizeof(Chunk)));
+      const hipError_t e = hipMemcpy(p->dev_chunks, table.data(), table.size() * sizeof(Chunk),
                                      hipMemcpyHostToDevice);
       if (e != hipSuccess) {
         (void)hipFree(p->dev_chunks);
@@ -310,13 +347,15 @@ static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
   DeviceGuard g;
   if (int rc = g.enter(p->device)) return rc;
   const hipStream_t s = static_cast<hipStream_t>(stream);
+  const Chunk* table = p->dev_chunks + (pack ? 0 : p->n_chunks);
+  const uint32_t n = static_cast<uint32_t>(p->n_chunks);
   const hipError_t e =
-      p->xform ? launch_xform_chunks(pack, p->dev_chunks, static_cast<uint32_t>(p->n_chunks),
-                                     cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
-                                     static_cast<uint8_t*>(packed), layer_stride, p->xdev, s)
-               : launch_copy_chunks(pack, p->dev_chunks, static_cast<uint32_t>(p->n_chunks),
-                                    cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
-                                    static_cast<uint8_t*>(packed), layer_stride, s);
+      p->xform ? launch_xform_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
+                                     first_layer, n_layers, static_cast<uint8_t*>(packed),
+                                     layer_stride, p->xdev, s)
+               : launch_copy_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
+                                    first_layer, n_layers, static_cast<uint8_t*>(packed),
+                                    layer_stride, s);
   if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
   return KVT_OK;
 }
@@ -337,7 +376,7 @@ int kvt_unpack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, 
 
 static int range_launch_shape(int64_t n, int num_wg, int* wgs) {
   if (n > 0x7FFFFFFFll) return fail(KVT_ERR_INVALID, "too many ranges");
-  int w = num_wg > 0 ? num_wg : static_cast<int>(std::min<int64_t>(n, 16384));
+  int w = num_wg > 0 ? num_wg : static_cast<int>(std::min<int64_t>(n, 1 << 20));
   *wgs = std::max(1, w);
   return KVT_OK;
 }
@@ -352,13 +391,11 @@ static int launch_ranges(bool convert, const void* src, void* dst, const int64_t
   if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
   int wgs = 0;
   if (int rc = range_launch_shape(n, num_wg, &wgs)) return rc;
-  // With fewer ranges than a wave of workgroups fills the chip, cut each range
-  // into parts so that about 2048 workgroups exist.
-  int parts = 1;
-  if (n < 2048) parts = static_cast<int>(std::min<int64_t>(64, (2048 + n - 1) / n));
+  // The range lengths live on the device; eight workgroups stride over each range's slices.
+  const int rows = 8;
   const hipStream_t s = static_cast<hipStream_t>(stream);
-  const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, parts, s)
-                               : launch_copy_ranges(src, dst, so, dof, len, n, wgs, parts, false, s);
+  const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, s)
+                               : launch_copy_ranges(src, dst, so, dof, len, n, wgs, rows, s);
   if (e != hipSuccess) return hip_fail(e, "range copy launch");
   return KVT_OK;
 }
@@ -435,21 +472,20 @@ static int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
     const int64_t* d_contig = dev_meta;
     const int64_t* d_gpu = dev_meta + m;
     const int64_t* d_lens = dev_meta + 2 * m;
-    const int wgs = static_cast<int>(std::min<uint64_t>(m, 16384));
-    // about 32 KiB per workgroup, but enough workgroups to cover the chip
-    uint64_t parts = std::max<uint64_t>(1, (longest + 32767) / 32768);
-    if (m * parts < 2048) parts = std::min<uint64_t>(64, (2048 + m - 1) / m);
-    parts = std::min<uint64_t>(parts, 1024);
+    const int wgs = static_cast<int>(m);
+    // one workgroup per 4 KiB slice of the longest range (bounded; longer ranges are strided)
+    const uint64_t unit = halve ? 8192 : 4096;
+    const int rows = static_cast<int>(std::min<uint64_t>(std::max<uint64_t>(1, (longest + unit - 1) / unit), 512));
     hipError_t e;
     if (halve)
       e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
-                                static_cast<int64_t>(m), wgs, static_cast<int>(parts), s);
+                                static_cast<int64_t>(m), wgs, rows, s);
     else if (direction == KVT_COPY_D2H)
       e = launch_copy_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
-                             static_cast<int64_t>(m), wgs, static_cast<int>(parts), false, s);
+                             static_cast<int64_t>(m), wgs, rows, s);
     else
       e = launch_copy_ranges(tensor_buf, layer_gpu_ptr, d_contig, d_gpu, d_lens,
-                             static_cast<int64_t>(m), wgs, static_cast<int>(parts), false, s);
+                             static_cast<int64_t>(m), wgs, rows, s);
     if (e != hipSuccess) return hip_fail(e, "copy_handle_data launch");
     // the metadata buffers are reused by the next batch
     if (first + m < n) KVT_HIP(hipStreamSynchronize(s));
@@ -698,7 +734,7 @@ int kvt_copy_linear(void* dst, const void* src, uint64_t bytes, void* stream) {
   return guarded([&]() -> int {
     if ((!dst || !src) && bytes) return fail(KVT_ERR_INVALID, "kvt_copy_linear: null argument");
     if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
-    if (bytes > (0x7FFFFFFFull * 32768ull)) return fail(KVT_ERR_INVALID, "kvt_copy_linear: too large");
+    if (bytes > (0x7FFFFFF0ull << 12)) return fail(KVT_ERR_INVALID, "kvt_copy_linear: too large");
     const hipError_t e = launch_copy_linear(dst, src, bytes, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "linear copy launch");
     return KVT_OK;

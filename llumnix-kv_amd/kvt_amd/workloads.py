@@ -42,23 +42,25 @@ class Workload:
         return [b * info["layer_num_blocks"] for b in info["block_sizes"]]
 
 
-def _tables(rng, n_req, lens_tokens, ntpb, src_pool, dst_pool, disjoint_dst=True):
-    """Per request: src ids sampled without replacement inside the request (requests
-    may share source blocks, reads only); dst ids disjoint across the whole batch."""
+def _tables(rng, n_req, lens_tokens, ntpb, src_pool, dst_pool):
+    """Block tables the way a paged allocator hands them out: every request gets blocks
+    nobody else holds, drawn from one seeded permutation of the pool. Destination tables
+    are always disjoint (a scatter into shared blocks would race). When the batch needs
+    more source blocks than the source pool has, the permutation wraps around, i.e. the
+    last requests share blocks with the first ones (reads only, as with a shared prefix)."""
     n_blocks = [(int(t) + ntpb - 1) // ntpb for t in lens_tokens]
     total = sum(n_blocks)
-    if disjoint_dst:
-        if total > dst_pool:
-            raise ValueError("destination pool too small for disjoint tables: %d > %d"
-                             % (total, dst_pool))
-        perm = rng.permutation(dst_pool)[:total]
+    if total > dst_pool:
+        raise ValueError("destination pool too small for disjoint tables: %d > %d"
+                         % (total, dst_pool))
+    dperm = rng.permutation(dst_pool)[:total]
+    sperm = rng.permutation(src_pool)
     src, dst, pos = [], [], 0
     for nb in n_blocks:
-        src.append([int(x) for x in rng.choice(src_pool, size=nb, replace=False)])
-        if disjoint_dst:
-            dst.append([int(x) for x in perm[pos:pos + nb]])
-        else:
-            dst.append([int(x) for x in rng.choice(dst_pool, size=nb, replace=False)])
+        if nb > src_pool:
+            raise ValueError("request larger than the source pool")
+        src.append([int(sperm[(pos + i) % src_pool]) for i in range(nb)])
+        dst.append([int(x) for x in dperm[pos:pos + nb]])
         pos += nb
     return src, dst
 
