@@ -22,6 +22,11 @@ sys.path[:0] = [os.path.join(ROOT, "llumnix-kv_amd"), os.path.join(ROOT, "tests"
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 
+# HBM bytes moved by ONE pack launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# file (each counter scaled by what it reads for the plain copy kernel of known size); see
+# profiles/copy_chunks_kernel_config2_hbm_traffic.md. Keyed by (config, scale, chunk_bytes).
+MEASURED_PACK_TRAFFIC = {(2, 1.0, 0): 70.966e9}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -103,6 +108,9 @@ def main():
     ap.add_argument("--cpu-layers", type=int, default=4, help="layers in the CPU baseline sample")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
+    ap.add_argument("--calibrate-copy-gib", type=float, default=0.0,
+                    help="only run the plain linear copy kernel on this many GiB (profiler "
+                         "counter calibration: its HBM traffic is known, 1 read + 1 write)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py: this build measures ONE MI355X; the path has no inter-GPU "
@@ -117,6 +125,21 @@ def main():
     lib = kvt.lib()
     if kvt.device_count() < 1:
         raise SystemExit("bench.py: no usable MI355X (gfx950) device; there is no CPU fallback")
+
+    if args.calibrate_copy_gib > 0:
+        n = int(args.calibrate_copy_gib * 2**30)
+        a = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
+        b = torch.empty(n, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            assert lib.kvt_copy_linear(b.data_ptr(), a.data_ptr(), n, None) == 0
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        assert torch.equal(a, b)
+        print(json.dumps({"calibration": "kvt_copy_linear", "bytes": n, "launches": args.steps,
+                          "gbps_read_plus_write": round(2 * n / dt / 1e9, 1)}))
+        return
 
     wls = build_workload(args.config, args.scale)
     t_init = time.time()
@@ -219,7 +242,9 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "copy_chunks_kernel<pack>" if not wls[0].xform
                      else "xform_chunks_kernel<pack>",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "traffic": None},
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4),
+                     "traffic": MEASURED_PACK_TRAFFIC.get((args.config, args.scale,
+                                                           args.chunk_bytes))},
     }
 
     # ---------------------------------------------------------------- parity spot check + CPU leg
