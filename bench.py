@@ -191,6 +191,10 @@ def main():
         launch(plans, [new_event() for _ in range(3)])
         plans = [prepare(i) for i in range(len(wls))]
         keep.append(plans)
+        if len(keep) > 3:
+            for pl, ls in keep.pop(1):
+                pl.close()
+                ls.close()
     torch.cuda.synchronize()
 
     events, host_ms = [], []
@@ -204,6 +208,10 @@ def main():
         h0 = time.perf_counter()
         plans = [prepare(i) for i in range(len(wls))]
         keep.append(plans)
+        if len(keep) > 3:               # plans of finished steps go back to the library's pool
+            for pl, ls in keep.pop(1):
+                pl.close()
+                ls.close()
         host_ms.append((time.perf_counter() - h0) * 1e3)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0

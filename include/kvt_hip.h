@@ -145,6 +145,10 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
                     const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
                     kvt_plan** out);
 void kvt_plan_destroy(kvt_plan* p);
+/* The table upload is asynchronous; launches order themselves after it on
+ * their stream. Host-blocking wait for it -- needed only before the plan is
+ * used inside a stream capture (kvt_session_create does it itself). */
+int kvt_plan_ready(const kvt_plan* p);
 uint32_t kvt_plan_num_tensors(const kvt_plan* p);
 uint64_t kvt_plan_num_chunks(const kvt_plan* p);
 /* Packed bytes of tensor t in one layer (sum of its range lengths), and the

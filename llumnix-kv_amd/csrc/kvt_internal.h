@@ -45,6 +45,13 @@ int guarded(F&& body) {
 
 typedef std::vector<kvt_ipc_block> RunList;
 
+// Stable permutation that orders `keys` ascending: LSD radix sort on 11-bit
+// digits, skipping digits that are constant over the input. Returns early with
+// the identity when the keys are already ascending (the common case for a
+// sender's list that was merged before). O(n) instead of O(n log n): the lists
+// of a large batch hold tens of thousands of ranges.
+void stable_order_by_key(const std::vector<uint64_t>& keys, std::vector<uint32_t>& order);
+
 }  // namespace kvt
 
 struct kvt_block_lists {

@@ -17,12 +17,55 @@ int fail(int code, const std::string& msg) {
 }
 void clear_error() { g_last_error.clear(); }
 
+void stable_order_by_key(const std::vector<uint64_t>& keys, std::vector<uint32_t>& order) {
+  const size_t n = keys.size();
+  order.resize(n);
+  for (size_t i = 0; i < n; ++i) order[i] = static_cast<uint32_t>(i);
+  uint64_t all_or = 0, all_and = ~0ull;
+  bool sorted = true;
+  for (size_t i = 0; i < n; ++i) {
+    all_or |= keys[i];
+    all_and &= keys[i];
+    if (i && keys[i] < keys[i - 1]) sorted = false;
+  }
+  if (sorted || n < 2) return;
+  const uint64_t varying = all_or ^ all_and;  // bits that differ somewhere
+  constexpr int kBits = 11;
+  constexpr size_t kBuckets = size_t(1) << kBits;
+  std::vector<uint32_t> tmp(n);
+  std::vector<uint32_t> count(kBuckets);
+  for (int shift = 0; shift < 64; shift += kBits) {
+    if (((varying >> shift) & (kBuckets - 1)) == 0) continue;
+    std::fill(count.begin(), count.end(), 0u);
+    for (size_t i = 0; i < n; ++i) ++count[(keys[order[i]] >> shift) & (kBuckets - 1)];
+    uint32_t run = 0;
+    for (size_t b = 0; b < kBuckets; ++b) {
+      const uint32_t c = count[b];
+      count[b] = run;
+      run += c;
+    }
+    for (size_t i = 0; i < n; ++i) tmp[count[(keys[order[i]] >> shift) & (kBuckets - 1)]++] = order[i];
+    order.swap(tmp);
+  }
+}
+
 // Sort by source offset (stable) and fold a range into its predecessor when it
 // continues it on both sides. Returns {min, max, total, count} of the result.
 static void merge_runs(RunList& v, uint64_t stats[4]) {
-  std::stable_sort(v.begin(), v.end(), [](const kvt_ipc_block& a, const kvt_ipc_block& b) {
-    return a.src_offset < b.src_offset;
-  });
+  if (v.size() > 0xFFFFFFF0ull) throw InvalidError("range list too long");
+  {
+    std::vector<uint64_t> keys(v.size());
+    for (size_t i = 0; i < v.size(); ++i) keys[i] = v[i].src_offset;
+    std::vector<uint32_t> order;
+    stable_order_by_key(keys, order);
+    bool identity = true;
+    for (size_t i = 0; i < order.size() && identity; ++i) identity = order[i] == i;
+    if (!identity) {
+      RunList sorted(v.size());
+      for (size_t i = 0; i < v.size(); ++i) sorted[i] = v[order[i]];
+      v.swap(sorted);
+    }
+  }
   size_t w = 0;  // index of the run being grown
   for (size_t i = 1; i < v.size(); ++i) {
     kvt_ipc_block& head = v[w];

@@ -76,6 +76,103 @@ struct DeviceGuard {
 
 uint64_t round_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
+// Chunk tables are uploaded once per batch and die with the batch. hipMalloc /
+// hipFree per batch would stall (hipFree waits for the whole device), so table
+// storage is recycled: a buffer = device memory + a pinned host twin of the same
+// size + an event that marks its last use on the GPU. A released buffer is handed
+// out again only once that event has completed.
+struct TableBuf {
+  int device = -1;
+  size_t cap = 0;
+  void* dev = nullptr;
+  void* host = nullptr;          // pinned staging for the asynchronous upload
+  hipEvent_t last_use = nullptr; // recorded after every launch that reads `dev`
+  bool used = false;             // last_use has been recorded at least once
+  bool captured = false;         // read by a kernel recorded into a hipGraph
+};
+
+class TablePool {
+ public:
+  int acquire(int device, size_t bytes, TableBuf** out) {
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      size_t best = idle_.size();
+      for (size_t i = 0; i < idle_.size(); ++i) {
+        TableBuf* b = idle_[i];
+        if (b->device != device || b->cap < bytes) continue;
+        if (b->used && hipEventQuery(b->last_use) != hipSuccess) {
+          (void)hipGetLastError();
+          continue;  // still being read by a queued kernel
+        }
+        if (best == idle_.size() || b->cap < idle_[best]->cap) best = i;
+      }
+      if (best != idle_.size()) {
+        *out = idle_[best];
+        idle_.erase(idle_.begin() + best);
+        (*out)->used = false;
+        return KVT_OK;
+      }
+    }
+    std::unique_ptr<TableBuf> b(new TableBuf());
+    b->device = device;
+    b->cap = 65536;
+    while (b->cap < bytes) b->cap *= 2;
+    KVT_HIP(hipMalloc(&b->dev, b->cap));
+    hipError_t e = hipHostMalloc(&b->host, b->cap, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&b->last_use, hipEventDisableTiming);
+    if (e != hipSuccess) {
+      destroy(b.get());
+      return hip_fail(e, "table buffer allocation");
+    }
+    *out = b.release();
+    return KVT_OK;
+  }
+
+  void release(TableBuf* b) {
+    if (!b) return;
+    if (b->captured) {  // a graph may replay the kernel later: never recycle, free for good
+      destroy(b);
+      delete b;
+      return;
+    }
+    std::lock_guard<std::mutex> lock(mu_);
+    if (idle_.size() >= 64) {
+      TableBuf* victim = idle_.front();
+      idle_.erase(idle_.begin());
+      if (victim->used) (void)hipEventSynchronize(victim->last_use);
+      destroy(victim);
+      delete victim;
+    }
+    idle_.push_back(b);
+  }
+
+  // One upload stream per device, created on first use.
+  int upload_stream(int device, hipStream_t* out) {
+    std::lock_guard<std::mutex> lock(mu_);
+    if (device >= static_cast<int>(streams_.size())) streams_.resize(device + 1, nullptr);
+    if (!streams_[device]) KVT_HIP(hipStreamCreateWithFlags(&streams_[device], hipStreamNonBlocking));
+    *out = streams_[device];
+    return KVT_OK;
+  }
+
+ private:
+  static void destroy(TableBuf* b) {
+    if (b->dev) (void)hipFree(b->dev);
+    if (b->host) (void)hipHostFree(b->host);
+    if (b->last_use) (void)hipEventDestroy(b->last_use);
+    b->dev = b->host = nullptr;
+    b->last_use = nullptr;
+  }
+  std::mutex mu_;
+  std::vector<TableBuf*> idle_;
+  std::vector<hipStream_t> streams_;
+};
+
+TablePool& table_pool() {
+  static TablePool* pool = new TablePool();  // intentionally leaked: outlives static destruction
+  return *pool;
+}
+
 constexpr uint32_t kMinChunk = 4096, kMaxAutoChunk = 32768, kMaxChunk = 1u << 19;
 constexpr uint64_t kBlobAlign = 256;
 
@@ -102,6 +199,9 @@ struct kvt_plan {
   XformDev xdev{};
   uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
   Chunk* dev_chunks = nullptr;     // [0, n_chunks): pack order; [n_chunks, 2 n_chunks): unpack order
+  TableBuf* buf = nullptr;         // storage of dev_chunks (recycled through the table pool)
+  hipEvent_t uploaded = nullptr;   // completes when the table has reached the device
+  mutable bool upload_seen = false;  // a launch has already observed `uploaded` as complete
 };
 
 struct kvt_session {
@@ -209,18 +309,24 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
     }
 
     if (chunk_bytes == 0) {
-      // Largest power of two not above the median range length, within [4 KiB, 32 KiB]: ranges
-      // shorter than a chunk leave workgroups idle, longer chunks only save table entries.
-      std::vector<uint64_t> lens;
-      for (const RunList& runs : lists->tensors)
-        for (const kvt_ipc_block& r : runs) lens.push_back(p->xform ? half : r.length);
-      uint64_t median = kMaxAutoChunk;
-      if (!lens.empty()) {
-        std::nth_element(lens.begin(), lens.begin() + lens.size() / 2, lens.end());
-        median = lens[lens.size() / 2];
-      }
+      // Every table entry is served by chunk_bytes / 4096 workgroups, of which only
+      // ceil(len / 4096) have bytes to move. Take the largest entry size (fewest table
+      // entries) that leaves at most 2 % of the launched workgroups idle.
       chunk_bytes = kMinChunk;
-      while (chunk_bytes * 2 <= median && chunk_bytes * 2 <= kMaxAutoChunk) chunk_bytes *= 2;
+      for (uint32_t cand = kMaxAutoChunk; cand > kMinChunk; cand /= 2) {
+        uint64_t launched = 0, useful = 0;
+        for (const RunList& runs : lists->tensors)
+          for (const kvt_ipc_block& r : runs) {
+            const uint64_t len = p->xform ? half : r.length;
+            const uint64_t reps = p->xform ? r.length / std::max<uint64_t>(half, 1) : 1;
+            launched += reps * ((len + cand - 1) / cand) * (cand / kMinChunk);
+            useful += reps * ((len + kMinChunk - 1) / kMinChunk);
+          }
+        if (launched * 100 <= useful * 102) {
+          chunk_bytes = cand;
+          break;
+        }
+      }
     }
     if (p->xform)  // a chunk holds whole tokens
       while (chunk_bytes < tok_bytes) chunk_bytes *= 2;
@@ -274,16 +380,18 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
     if ((p->n_chunks << p->sub_shift) > 0x7FFFFFF0ull)
       return fail(KVT_ERR_INVALID, "kvt_plan_create: too many chunks for one launch");
 
-    // Two tables, each walked in ascending cache address of its own direction.
+    // Two tables, each walked in ascending cache address of its own direction
+    // (tensor-major: different tensors are different allocations).
     std::vector<Chunk> table(2 * pieces.size());
-    std::vector<uint32_t> order(pieces.size());
+    std::vector<uint32_t> order;
+    std::vector<uint64_t> keys(pieces.size());
     for (int dir = 0; dir < 2; ++dir) {
-      for (uint32_t i = 0; i < order.size(); ++i) order[i] = i;
-      std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
-        const Piece &x = pieces[a], &y = pieces[b];
-        if (x.tensor != y.tensor) return x.tensor < y.tensor;
-        return dir == 0 ? x.src < y.src : x.dst < y.dst;
-      });
+      for (size_t i = 0; i < pieces.size(); ++i) {
+        const uint64_t off = dir == 0 ? pieces[i].src : pieces[i].dst;
+        if (off >> 56) return fail(KVT_ERR_INVALID, "kvt_plan_create: offset beyond 2^56");
+        keys[i] = (static_cast<uint64_t>(pieces[i].tensor) << 56) | off;
+      }
+      stable_order_by_key(keys, order);
       for (size_t i = 0; i < order.size(); ++i) {
         const Piece& q = pieces[order[i]];
         Chunk& c = table[dir * pieces.size() + i];
@@ -299,12 +407,25 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
     DeviceGuard g;
     if (int rc = g.enter(device)) return rc;
     if (!table.empty()) {
-      KVT_HIP(hipMalloc(reinterpret_cast<void**>(&p->dev_chunks), table.size() * sizeof(Chunk)));
-      const hipError_t e = hipMemcpy(p->dev_chunks, table.data(), table.size() * sizeof(Chunk),
-                                     hipMemcpyHostToDevice);
+      // Asynchronous upload: fill the pinned twin, copy on the library's upload stream; the
+      // first launch that uses the plan waits for `uploaded` on its own stream.
+      const size_t bytes = table.size() * sizeof(Chunk);
+      if (int rc = table_pool().acquire(device, bytes, &p->buf)) return rc;
+      std::memcpy(p->buf->host, table.data(), bytes);
+      p->dev_chunks = static_cast<Chunk*>(p->buf->dev);
+      hipStream_t up = nullptr;
+      if (int rc = table_pool().upload_stream(device, &up)) {
+        table_pool().release(p->buf);
+        return rc;
+      }
+      hipError_t e = hipEventCreateWithFlags(&p->uploaded, hipEventDisableTiming);
+      if (e == hipSuccess) e = hipMemcpyAsync(p->buf->dev, p->buf->host, bytes, hipMemcpyHostToDevice, up);
+      if (e == hipSuccess) e = hipEventRecord(p->uploaded, up);
       if (e != hipSuccess) {
-        (void)hipFree(p->dev_chunks);
-        return hip_fail(e, "hipMemcpy(chunk table)");
+        (void)hipStreamSynchronize(up);
+        if (p->uploaded) (void)hipEventDestroy(p->uploaded);
+        table_pool().release(p->buf);
+        return hip_fail(e, "chunk table upload");
       }
     }
     *out = p.release();
@@ -314,8 +435,23 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
 
 void kvt_plan_destroy(kvt_plan* p) {
   if (!p) return;
-  if (p->dev_chunks) (void)hipFree(p->dev_chunks);
+  if (p->uploaded) {
+    (void)hipEventSynchronize(p->uploaded);  // the upload reads the pinned twin
+    (void)hipEventDestroy(p->uploaded);
+  }
+  table_pool().release(p->buf);
   delete p;
+}
+
+int kvt_plan_ready(const kvt_plan* p) {
+  return guarded([&]() -> int {
+    if (!p) return fail(KVT_ERR_INVALID, "kvt_plan_ready: null plan");
+    if (p->uploaded && !p->upload_seen) {
+      KVT_HIP(hipEventSynchronize(p->uploaded));
+      p->upload_seen = true;
+    }
+    return KVT_OK;
+  });
 }
 
 uint32_t kvt_plan_num_tensors(const kvt_plan* p) { return p ? p->n_tensors : 0; }
@@ -347,6 +483,21 @@ static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
   DeviceGuard g;
   if (int rc = g.enter(p->device)) return rc;
   const hipStream_t s = static_cast<hipStream_t>(stream);
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &cap) != hipSuccess) (void)hipGetLastError();
+  const bool capturing = cap != hipStreamCaptureStatusNone;
+  if (p->uploaded && !p->upload_seen) {
+    if (capturing)  // event queries and waits on outside events are not allowed inside a capture
+      return fail(KVT_ERR_INVALID,
+                  "the plan's table upload has not been observed yet: call kvt_plan_ready() "
+                  "before using the plan inside a stream capture");
+    if (hipEventQuery(p->uploaded) == hipSuccess) {
+      p->upload_seen = true;
+    } else {
+      (void)hipGetLastError();
+      KVT_HIP(hipStreamWaitEvent(s, p->uploaded, 0));
+    }
+  }
   const Chunk* table = p->dev_chunks + (pack ? 0 : p->n_chunks);
   const uint32_t n = static_cast<uint32_t>(p->n_chunks);
   const hipError_t e =
@@ -357,6 +508,15 @@ static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
                                     first_layer, n_layers, static_cast<uint8_t*>(packed),
                                     layer_stride, s);
   if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
+  if (p->buf) {
+    // remember when the table is last read, so that its storage is not recycled too early
+    if (capturing) {
+      p->buf->captured = true;
+    } else {
+      KVT_HIP(hipEventRecord(p->buf->last_use, s));
+      p->buf->used = true;
+    }
+  }
   return KVT_OK;
 }
 
@@ -526,6 +686,7 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
     if (int rc = check_device(plan->device)) return rc;
     DeviceGuard g;
     if (int rc = g.enter(plan->device)) return rc;
+    if (int rc = kvt_plan_ready(plan)) return rc;  // save_layer may run inside a stream capture
     std::unique_ptr<kvt_session> s(new kvt_session());
     s->plan = plan;
     s->cache = cache;

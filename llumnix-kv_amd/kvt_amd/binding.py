@@ -45,6 +45,7 @@ SIGNATURES = {
     "kvt_cache_destroy": (None, [_vp]),
     "kvt_plan_create": (_int, [_int, _vp, _P(_u64), _P(_u64), _P(Xform), _u32, _P(_vp)]),
     "kvt_plan_destroy": (None, [_vp]),
+    "kvt_plan_ready": (_int, [_vp]),
     "kvt_plan_num_tensors": (_u32, [_vp]),
     "kvt_plan_num_chunks": (_u64, [_vp]),
     "kvt_plan_tensor_bytes": (_u64, [_vp, _u32]),
@@ -275,6 +276,9 @@ class Plan:
             self.h = _vp()
 
     __del__ = close
+
+    def ready(self):
+        check(lib().kvt_plan_ready(self.h))
 
     @property
     def layer_bytes(self):
