@@ -108,7 +108,16 @@ struct FillOp {
   u64 d_head_stride = 0;
 };
 
-enum OpKind { OP_WALK, OP_PAGES, OP_STATE, OP_GDN, OP_FILL };
+// Real MLA prefix of KDA-sized physical pages (Kimi-K3): whole manager blocks
+// when both sides use the same TP, kernel pages plus a zero-filled tail otherwise.
+struct MlaOp {
+  u32 group = 0;
+  bool equal_tp = true, pad = true;
+  u32 s_mgr_tok = 1, d_mgr_tok = 1, kernel_tok = 1;
+  u64 s_page = 0, d_page = 0, kernel_bytes = 0, tok_bytes = 0;
+};
+
+enum OpKind { OP_WALK, OP_PAGES, OP_STATE, OP_GDN, OP_FILL, OP_MLA };
 
 struct Op {
   OpKind kind;
@@ -119,6 +128,7 @@ struct Op {
   StateOp state;
   GdnOp gdn;
   FillOp fill;
+  MlaOp mla;
 };
 
 }  // namespace
@@ -630,6 +640,97 @@ struct Builder {
     ple_split(h.pB, h.dB, false, gdn_off);
   }
 
+  // ---- KDA state pages ([conv][recurrent][padding], SD or DS conv layout)
+  u64 kda_stride(const kvt_worker_info& w) const {
+    if (w.kda_page_stride != 0) return w.kda_page_stride;
+    if (w.n_tensors < 1) throw RangeError("no cache tensor registered");
+    return w.block_sizes[0];
+  }
+
+  // rel: 0 P==D, +1 P>D, -1 P<D. The page stride is looked up before the
+  // "last chunk only" gate for P==D and after it otherwise (a missing tensor is
+  // then reported on the last chunk only), as the reference orders it.
+  void kda_state(int rel) {
+    set_lists(1);
+    if (rel == 0) {
+      const u64 sp = kda_stride(s), dp = kda_stride(d);
+      cap(0);
+      state(0, s.num_gdn_layers, sp, dp, sp);
+      return;
+    }
+    need(s.engine_tp_size > 0 && d.engine_tp_size > 0, "bad TP relation");
+    const u32 gn = rel > 0 ? s.engine_tp_size / d.engine_tp_size : d.engine_tp_size / s.engine_tp_size;
+    need(gn > 0, "bad TP relation");
+    const u32 goff = (rel > 0 ? s.worker_tp_rank : d.worker_tp_rank) % gn;
+    const size_t at = out->ops.size();
+    push(OP_GDN, true);
+    try {
+      GdnOp& g = out->ops[at].gdn;
+      g.n_groups = s.num_gdn_layers;
+      g.s_page = kda_stride(s);
+      g.d_page = kda_stride(d);
+      const u64 e = s.gdn_conv_elem_size;
+      const bool ds = s.kda_conv_dim_first != 0;
+      const u64 state_len = dim(s.conv_state_shape, s.n_conv_state_shape, ds ? 2 : 1);
+      const u64 qkv = dim(s.conv_state_shape, s.n_conv_state_shape, ds ? 1 : 2);
+      const u64 conv = state_len * qkv * e;
+      const u64 rec = dim(s.ssm_state_shape, s.n_ssm_state_shape, 1) *
+                      dim(s.ssm_state_shape, s.n_ssm_state_shape, 2) *
+                      dim(s.ssm_state_shape, s.n_ssm_state_shape, 3) * s.gdn_ssm_elem_size;
+      // DS keeps each channel's history contiguous: one "row" whose pieces are whole
+      // components; SD repeats the q/k/v placement for every history row.
+      g.rows = ds ? 1 : state_len;
+      const u64 per_piece = ds ? state_len * e : e;
+      g.s_row = qkv * e;
+      u64 s_in = 0, d_in = 0;
+      if (rel > 0) {
+        g.d_row = gn * g.s_row;
+        for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+          const u64 comp = s.gdn_conv_channel_dims[c] * per_piece;
+          g.row_pieces.push_back(Piece{s_in, gn * s_in + goff * comp, comp});
+          s_in += comp;
+        }
+        g.ssm = Piece{conv, gn * conv + goff * rec, rec};
+      } else {
+        g.d_row = g.s_row / gn;
+        for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+          const u64 comp = (s.gdn_conv_channel_dims[c] / gn) * per_piece;
+          g.row_pieces.push_back(Piece{s_in + goff * comp, d_in, comp});
+          s_in += gn * comp;
+          d_in += comp;
+        }
+        g.ssm = Piece{conv + goff * (rec / gn), ds ? d_in : conv / gn, rec / gn};
+      }
+    } catch (const RangeError&) {
+      out->ops[at].bad_shape = true;
+    }
+    cap(0);
+  }
+
+  void kimi_mla() {
+    if (!src_rank_valid()) return;
+    const size_t at = out->ops.size();
+    MlaOp& m = push(OP_MLA).mla;
+    m.group = s.num_gdn_layers;
+    if (s.n_tensors < 1 || d.n_tensors < 1) {
+      out->ops[at].bad_shape = true;
+      return;
+    }
+    need(s.token_sizes[0] > 0 && d.token_sizes[0] > 0, "token size must be positive");
+    m.s_mgr_tok = static_cast<u32>(s.block_sizes[0] / s.token_sizes[0]);
+    m.d_mgr_tok = static_cast<u32>(d.block_sizes[0] / d.token_sizes[0]);
+    m.kernel_tok = s.attn_kernel_blk_ntpb;
+    need(m.s_mgr_tok > 0 && m.d_mgr_tok > 0 && m.kernel_tok > 0, "tokens per block must be positive");
+    m.tok_bytes = s.hybrid_attn_token_size;
+    m.kernel_bytes = static_cast<u64>(m.kernel_tok) * m.tok_bytes;
+    m.s_page = s.kda_page_stride != 0 ? s.kda_page_stride : s.block_sizes[0];
+    m.d_page = d.kda_page_stride != 0 ? d.kda_page_stride : d.block_sizes[0];
+    m.equal_tp = s.engine_tp_size == d.engine_tp_size;
+    m.pad = opts.pad_last_attn_block != 0;
+    set_lists(1);
+    cap(0);
+  }
+
   void build(int parser_id) {
     switch (parser_id) {
       case KVT_PARSER_RAGGED_PEQD: ragged_peqd(); break;
@@ -674,6 +775,12 @@ struct Builder {
       case KVT_PARSER_HYBRID_FI_PEQD: hybrid_peqd(true); break;
       case KVT_PARSER_HYBRID_FI_PGTD: hybrid_pgtd(true); break;
       case KVT_PARSER_HYBRID_FI_PLTD: hybrid_pltd(true); break;
+      case KVT_PARSER_KDA_PEQD: kda_state(0); break;
+      case KVT_PARSER_KDA_PGTD: kda_state(1); break;
+      case KVT_PARSER_KDA_PLTD: kda_state(-1); break;
+      case KVT_PARSER_KIMI_K3_PEQD: kimi_mla(); kda_state(0); break;
+      case KVT_PARSER_KIMI_K3_PGTD: kimi_mla(); kda_state(1); break;
+      case KVT_PARSER_KIMI_K3_PLTD: kimi_mla(); kda_state(-1); break;
       default:
         throw InvalidError("parser id not supported by this build");
     }
@@ -910,6 +1017,51 @@ void run_fill(const FillOp& f, const kvt_task& t, const Groups& sg, const Groups
   }
 }
 
+void run_mla(const MlaOp& m, const kvt_task& t, const Groups& sg, const Groups& dg, Sink& sink) {
+  const u32 *sid, *did;
+  u64 sn, dn;
+  sg.get(m.group, sid, sn);
+  dg.get(m.group, did, dn);
+  const bool last = t.reach_last_token != 0;
+  if (m.equal_tp) {
+    // whole manager blocks; an incomplete block waits for the next chunk, the last chunk
+    // sends every remaining allocated block
+    const u64 first = t.seen_tokens / m.s_mgr_tok;
+    const u64 end = last ? sn : static_cast<u32>(t.seen_tokens + t.new_tokens) / m.s_mgr_tok;
+    const u64 len = static_cast<u64>(m.s_mgr_tok) * m.tok_bytes;
+    for (u64 i = first; i < end; ++i)
+      sink.put(static_cast<u64>(id_at(sid, sn, i)) * m.s_page,
+               static_cast<u64>(id_at(did, dn, i)) * m.d_page, len);
+    return;
+  }
+  u32 pos = t.seen_tokens, rem = t.new_tokens;
+  while (rem > 0) {
+    const u32 ti = pos % m.kernel_tok;
+    const u32 k = std::min(m.kernel_tok - ti, rem);
+    if (k == m.kernel_tok || last || ti + k == m.kernel_tok)
+      sink.put(static_cast<u64>(id_at(sid, sn, pos / m.s_mgr_tok)) * m.s_page +
+                   static_cast<u64>((pos % m.s_mgr_tok) / m.kernel_tok) * m.kernel_bytes,
+               static_cast<u64>(id_at(did, dn, pos / m.d_mgr_tok)) * m.d_page +
+                   static_cast<u64>((pos % m.d_mgr_tok) / m.kernel_tok) * m.kernel_bytes,
+               m.kernel_bytes);
+    pos += k;
+    rem -= k;
+  }
+  if (!m.pad || !last) return;
+  const u64 total = static_cast<u64>(t.seen_tokens) + t.new_tokens;
+  const u64 room = dn * static_cast<u64>(m.d_mgr_tok);
+  if (total >= room) return;
+  const u64 zero = static_cast<u64>(id_at(sid, sn, 0)) * m.s_page;
+  for (u64 dpos = total; dpos < room;) {
+    const u64 tib = dpos % m.d_mgr_tok;
+    const u64 k = std::min<u64>(m.d_mgr_tok - tib, room - dpos);
+    zero_run(sink, zero,
+             static_cast<u64>(id_at(did, dn, dpos / m.d_mgr_tok)) * m.d_page + tib * m.tok_bytes,
+             k * m.tok_bytes, m.s_page);
+    dpos += k;
+  }
+}
+
 }  // namespace
 }  // namespace kvt
 
@@ -928,8 +1080,6 @@ int kvt_parser_create(int parser_id, const kvt_worker_info* src, const kvt_worke
       return fail(KVT_ERR_INVALID, "kvt_parser_create: worker_tp_rank beyond MAX_TP_SIZE");
     if (parser_id < 0 || parser_id >= KVT_PARSER_COUNT)
       return fail(KVT_ERR_UNSUPPORTED, "kvt_parser_create: unknown parser id");
-    if (parser_id >= KVT_PARSER_KDA_PEQD && parser_id <= KVT_PARSER_KIMI_K3_PLTD)
-      return fail(KVT_ERR_UNSUPPORTED, "kvt_parser_create: KDA / Kimi-K3 layouts are not built");
     std::unique_ptr<kvt_parser> p(new kvt_parser());
     kvt_parse_opts o{0, 1};
     if (opts) o = *opts;
@@ -999,6 +1149,7 @@ int kvt_parse_block(const kvt_parser* p, const kvt_task* task, kvt_block_lists* 
         case OP_STATE: run_state(op.state, sg, dg, sink); break;
         case OP_GDN: run_gdn(op.gdn, sg, dg, sink); break;
         case OP_FILL: run_fill(op.fill, *task, sg, dg, sink); break;
+        case OP_MLA: run_mla(op.mla, *task, sg, dg, sink); break;
       }
     }
     return KVT_OK;

@@ -935,6 +935,182 @@ void hybrid_fi_pltd(const kvt_worker_info& s, const kvt_worker_info& d, const kv
   }
 }
 
+
+// ---------------------------------------------------------------- KDA / Kimi-K3 (shape 8)
+// parse_block_kda.cpp:15-20 (get_kda_page_stride)
+u64 kda_stride(const kvt_worker_info& w) {
+  if (w.kda_page_stride != 0) return w.kda_page_stride;
+  if (w.n_tensors < 1) throw std::out_of_range("block_sizes.at(0)");
+  return w.block_sizes[0];
+}
+
+struct KdaLayout {
+  u64 state_len, qkv, conv, rec;
+};
+
+// parse_block_kda.cpp:22-54 (get_kda_state_layout)
+KdaLayout kda_layout(const kvt_worker_info& w) {
+  KdaLayout l;
+  l.state_len = w.kda_conv_dim_first ? shape_at(w.conv_state_shape, w.n_conv_state_shape, 2)
+                                     : shape_at(w.conv_state_shape, w.n_conv_state_shape, 1);
+  l.qkv = w.kda_conv_dim_first ? shape_at(w.conv_state_shape, w.n_conv_state_shape, 1)
+                               : shape_at(w.conv_state_shape, w.n_conv_state_shape, 2);
+  l.conv = l.state_len * l.qkv * w.gdn_conv_elem_size;
+  l.rec = shape_at(w.ssm_state_shape, w.n_ssm_state_shape, 1) *
+          shape_at(w.ssm_state_shape, w.n_ssm_state_shape, 2) *
+          shape_at(w.ssm_state_shape, w.n_ssm_state_shape, 3) * w.gdn_ssm_elem_size;
+  return l;
+}
+
+// parse_block_kda.cpp:71-129 (emit_kda_block_p_gt_d)
+void kda_emit_gt(u64 po, u64 dof, u32 gn, u32 goff, const kvt_worker_info& s, const KdaLayout& l,
+                 const Bounds& b, Runs& out) {
+  const u64 e = s.gdn_conv_elem_size;
+  if (s.kda_conv_dim_first) {
+    u64 inner = 0;
+    for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+      const u64 comp = s.gdn_conv_channel_dims[c] * l.state_len * e;
+      emit(out, b, po + inner, dof + gn * inner + goff * comp, comp);
+      inner += comp;
+    }
+  } else {
+    const u64 p_row = l.qkv * e, d_row = gn * p_row;
+    for (u64 r = 0; r < l.state_len; ++r) {
+      u64 inner = 0;
+      for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+        const u64 comp = s.gdn_conv_channel_dims[c] * e;
+        emit(out, b, po + r * p_row + inner, dof + r * d_row + gn * inner + goff * comp, comp);
+        inner += comp;
+      }
+    }
+  }
+  emit(out, b, po + l.conv, dof + gn * l.conv + goff * l.rec, l.rec);
+}
+
+// parse_block_kda.cpp:131-196 (emit_kda_block_p_lt_d)
+void kda_emit_lt(u64 po, u64 dof, u32 gn, u32 goff, const kvt_worker_info& s, const KdaLayout& l,
+                 const Bounds& b, Runs& out) {
+  const u64 e = s.gdn_conv_elem_size;
+  const u64 d_rec = l.rec / gn;
+  u64 d_conv = 0;
+  if (s.kda_conv_dim_first) {
+    u64 pin = 0, din = 0;
+    for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+      const u64 comp = (s.gdn_conv_channel_dims[c] / gn) * l.state_len * e;
+      emit(out, b, po + pin + goff * comp, dof + din, comp);
+      pin += gn * comp;
+      din += comp;
+    }
+    d_conv = din;
+  } else {
+    const u64 p_row = l.qkv * e, d_row = p_row / gn;
+    for (u64 r = 0; r < l.state_len; ++r) {
+      u64 pin = 0, din = 0;
+      for (u32 c = 0; c < s.n_gdn_conv_channel_dims; ++c) {
+        const u64 comp = (s.gdn_conv_channel_dims[c] / gn) * e;
+        emit(out, b, po + r * p_row + pin + goff * comp, dof + r * d_row + din, comp);
+        pin += gn * comp;
+        din += comp;
+      }
+    }
+    d_conv = l.conv / gn;
+  }
+  emit(out, b, po + l.conv + goff * d_rec, dof + d_conv, d_rec);
+}
+
+// parse_block_kda.cpp:213-245 (P==D), :247-289 (P>D), :291-334 (P<D)
+void kda_any(int rel, const kvt_worker_info& s, const kvt_worker_info& d, const kvt_parse_opts& o,
+             const Task& t, std::vector<Runs>& out) {
+  out.resize(1);
+  u32 gn = 1, goff = 0;
+  u64 sp = 0, dp = 0;
+  if (rel == 0) {
+    sp = kda_stride(s);
+    dp = kda_stride(d);
+    if (!t.last) return;
+  } else {
+    gn = rel > 0 ? s.engine_tp_size / d.engine_tp_size : d.engine_tp_size / s.engine_tp_size;
+    goff = (rel > 0 ? s.worker_tp_rank : d.worker_tp_rank) % gn;
+    if (!t.last) return;
+    sp = kda_stride(s);
+    dp = kda_stride(d);
+  }
+  KdaLayout l{0, 0, 0, 0};
+  if (rel != 0) l = kda_layout(s);
+  const Bounds b = make_bounds(s, d, 0, o);
+  Runs& r = out[0];
+  for (u64 g = 0; g < s.num_gdn_layers; ++g) {
+    const Ids& sg = grp(t.src, g);
+    const Ids& dg = grp(t.dst, g);
+    for (size_t i = 0; i < sg.size(); ++i) {
+      const u64 po = static_cast<u64>(sg[i]) * sp, dof = static_cast<u64>(at(dg, i)) * dp;
+      if (rel == 0) emit(r, b, po, dof, sp);
+      else if (rel > 0) kda_emit_gt(po, dof, gn, goff, s, l, b, r);
+      else kda_emit_lt(po, dof, gn, goff, s, l, b, r);
+    }
+  }
+}
+
+// parse_block_kimi_k3.cpp:9-183 (parse_replicated_mla_blocks)
+void kimi_mla(const kvt_worker_info& s, const kvt_worker_info& d, u32 valid,
+              const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  if (!((valid >> s.worker_tp_rank) & 1u)) return;
+  const u64 g = s.num_gdn_layers;
+  const Ids& sb = grp(t.src, g);
+  const Ids& db = grp(t.dst, g);
+  if (s.n_tensors < 1 || d.n_tensors < 1) throw std::out_of_range("tensor index");
+  const u64 s_logical = s.block_sizes[0], d_logical = d.block_sizes[0];
+  const u32 s_mgr = static_cast<u32>(s_logical / s.token_sizes[0]);
+  const u32 d_mgr = static_cast<u32>(d_logical / d.token_sizes[0]);
+  const u32 kn = s.attn_kernel_blk_ntpb;
+  const u64 tok = s.hybrid_attn_token_size;
+  const u64 kpage = static_cast<u64>(kn) * tok;
+  const u64 s_phys = s.kda_page_stride != 0 ? s.kda_page_stride : s_logical;
+  const u64 d_phys = d.kda_page_stride != 0 ? d.kda_page_stride : d_logical;
+  out.resize(1);
+  Runs& r = out[0];
+  const Bounds b = make_bounds(s, d, 0, o);
+  if (s.engine_tp_size == d.engine_tp_size) {
+    const u64 first = t.seen / s_mgr;
+    const u64 end = t.last ? sb.size() : static_cast<u32>(t.seen + t.fresh) / s_mgr;
+    const u64 len = static_cast<u64>(s_mgr) * tok;
+    for (u64 i = first; i < end; ++i)
+      emit(r, b, static_cast<u64>(at(sb, i)) * s_phys, static_cast<u64>(at(db, i)) * d_phys, len);
+    return;
+  }
+  u32 pos = t.seen, rem = t.fresh;
+  while (rem > 0) {
+    const u32 sbi = pos / s_mgr, dbi = pos / d_mgr;
+    const u32 ski = (pos % s_mgr) / kn, dki = (pos % d_mgr) / kn;
+    const u32 ti = pos % kn;
+    const u32 k = std::min(kn - ti, rem);
+    const bool send = k == kn || t.last || ti + k == kn;
+    if (send)
+      emit(r, b, static_cast<u64>(at(sb, sbi)) * s_phys + static_cast<u64>(ski) * kpage,
+           static_cast<u64>(at(db, dbi)) * d_phys + static_cast<u64>(dki) * kpage, kpage);
+    pos += k;
+    rem -= k;
+  }
+  if (!o.pad_last_attn_block || !t.last) return;
+  const u64 total = static_cast<u64>(t.seen) + t.fresh;
+  const u64 cap_tokens = db.size() * static_cast<u64>(d_mgr);
+  if (total >= cap_tokens) return;
+  const u64 zsrc = static_cast<u64>(at(sb, 0)) * s_phys;
+  for (u64 dpos = total; dpos < cap_tokens;) {
+    const u64 dbi = dpos / d_mgr, tib = dpos % d_mgr;
+    const u64 k = std::min<u64>(d_mgr - tib, cap_tokens - dpos);
+    zero_fill(zsrc, static_cast<u64>(at(db, dbi)) * d_phys + tib * tok, k * tok, s_phys, b, r);
+    dpos += k;
+  }
+}
+
+// parse_block_kimi_k3.cpp:187-235
+void kimi_any(int rel, const kvt_worker_info& s, const kvt_worker_info& d, u32 valid,
+              const kvt_parse_opts& o, const Task& t, std::vector<Runs>& out) {
+  kimi_mla(s, d, valid, o, t, out);
+  kda_any(rel, s, d, o, t, out);
+}
+
 std::vector<Ids> split_groups(const u32* ids, const u32* lens, u32 n) {
   std::vector<Ids> g(n);
   size_t p = 0;
@@ -968,7 +1144,13 @@ int run_parser(int id, const kvt_worker_info& s, const kvt_worker_info& d, u32 v
     case KVT_PARSER_HYBRID_FI_PEQD: hybrid_fi_peqd(s, d, o, t, out); break;
     case KVT_PARSER_HYBRID_FI_PGTD: hybrid_fi_pgtd(s, d, valid, kvt_tp_rank, o, t, out); break;
     case KVT_PARSER_HYBRID_FI_PLTD: hybrid_fi_pltd(s, d, o, t, out); break;
-    default: return KVT_ERR_UNSUPPORTED;  // KDA / Kimi-K3 parsers are not restated here
+    case KVT_PARSER_KDA_PEQD: kda_any(0, s, d, o, t, out); break;
+    case KVT_PARSER_KDA_PGTD: kda_any(1, s, d, o, t, out); break;
+    case KVT_PARSER_KDA_PLTD: kda_any(-1, s, d, o, t, out); break;
+    case KVT_PARSER_KIMI_K3_PEQD: kimi_any(0, s, d, valid, o, t, out); break;
+    case KVT_PARSER_KIMI_K3_PGTD: kimi_any(1, s, d, valid, o, t, out); break;
+    case KVT_PARSER_KIMI_K3_PLTD: kimi_any(-1, s, d, valid, o, t, out); break;
+    default: return KVT_ERR_UNSUPPORTED;
   }
   return KVT_OK;
 }

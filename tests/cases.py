@@ -238,18 +238,119 @@ def gen_hybrid(rng, parser):
                 fp8=False, tasks=tasks)
 
 
+def gen_kda(rng, parser):
+    """KDA state pages (KDA_*) and Kimi-K3 (KDA groups + one replicated MLA group)."""
+    kimi = parser.startswith("KIMI")
+    kind = parser.rsplit("_", 1)[1]
+    if kind == "PEQD":
+        p_tp = d_tp = int(rng.choice([1, 2, 4]))
+    elif kind == "PGTD":
+        d_tp = int(rng.choice([1, 2]))
+        p_tp = d_tp * int(rng.choice([2, 4]))
+    else:
+        p_tp = int(rng.choice([1, 2]))
+        d_tp = p_tp * int(rng.choice([2, 4]))
+    gn = max(p_tp, d_tp) // min(p_tp, d_tp)
+    if kind == "PLTD":
+        d_rank = int(rng.integers(0, d_tp))
+        p_rank = d_rank // gn
+    elif kind == "PGTD":
+        p_rank = int(rng.integers(0, p_tp))
+        d_rank = p_rank // gn
+    else:
+        p_rank = d_rank = int(rng.integers(0, p_tp))
+    dim_first = bool(rng.random() < 0.5)
+    state_len = int(rng.choice([2, 3, 4]))
+    narrow_ch = [int(rng.choice([2, 4, 6])) for _ in range(3)]
+    narrow_rec = (int(rng.choice([1, 2])), 2, int(rng.choice([2, 4])))
+    conv_e, rec_e = int(rng.choice([1, 2])), 4
+
+    def meta(scale):
+        ch = [c * scale for c in narrow_ch]
+        qkv = sum(ch)
+        shape = [8, qkv, state_len] if dim_first else [8, state_len, qkv]
+        rec = [8, narrow_rec[0] * scale, narrow_rec[1], narrow_rec[2]]
+        size = state_len * qkv * conv_e + rec[1] * rec[2] * rec[3] * rec_e
+        return dict(conv_state_shape=shape, ssm_state_shape=rec, gdn_conv_channel_dims=ch,
+                    gdn_conv_elem_size=conv_e, gdn_ssm_elem_size=rec_e,
+                    kda_conv_dim_first=dim_first), size
+
+    p_meta, p_size = meta(gn if kind == "PLTD" else 1)
+    d_meta, d_size = meta(gn if kind == "PGTD" else 1)
+    n_gdn = int(rng.choice([1, 2, 3]))
+    mla_tok = 16 * int(rng.choice([1, 2, 4]))
+    kernel_ntpb = int(rng.choice([2, 4]))
+    s_mgr = kernel_ntpb * int(rng.choice([1, 2]))
+    d_mgr = s_mgr if kind == "PEQD" else kernel_ntpb * int(rng.choice([1, 2, 4]))
+    # physical page must hold the KDA state and, for Kimi, the MLA prefix of a manager block
+    s_page = -(-max(p_size, s_mgr * mla_tok if kimi else 0) // 64) * 64 + 64 * int(rng.integers(0, 3))
+    d_page = -(-max(d_size, d_mgr * mla_tok if kimi else 0) // 64) * 64 + 64 * int(rng.integers(0, 3))
+    if kind == "PEQD":
+        d_page = s_page
+    use_stride = bool(rng.random() < 0.5) or kimi
+    pool_s, pool_d = int(rng.integers(16, 48)), int(rng.integers(16, 48))
+    if kimi:
+        # logical MLA blocks: block_sizes[0] = manager tokens x registered token size
+        reg_tok = mla_tok
+        s_blk, d_blk, s_tok, d_tok = s_mgr * reg_tok, d_mgr * reg_tok, reg_tok, reg_tok
+        # capacity of the registered tensor must cover pool * physical page
+        s_lnb = -(-pool_s * s_page // s_blk)
+        d_lnb = -(-pool_d * d_page // d_blk)
+    else:
+        s_blk, d_blk, s_tok, d_tok = s_page, d_page, s_page, d_page
+        s_lnb, d_lnb = pool_s, pool_d
+    common = dict(num_kv_heads=1, num_gdn_layers=n_gdn, attn_kernel_blk_ntpb=kernel_ntpb,
+                  hybrid_attn_token_size=mla_tok if kimi else 0, attn_pack_size=1)
+    src = dict(block_sizes=[s_blk], token_sizes=[s_tok], layer_num_blocks=s_lnb, tp=p_tp,
+               rank=p_rank, kda_page_stride=s_page if use_stride else 0, **common, **p_meta)
+    dst = dict(block_sizes=[d_blk], token_sizes=[d_tok], layer_num_blocks=d_lnb, tp=d_tp,
+               rank=d_rank, kda_page_stride=d_page if use_stride else 0, **common, **d_meta)
+    from checkers import oracle
+    valid = oracle().kvto_valid_ranks(p_tp, d_tp, 1)
+    tp_size = bin(valid).count("1")
+    tp_rank = bin(valid & ((1 << p_rank) - 1)).count("1")
+    tasks = []
+    for _ in range(int(rng.integers(1, 3))):
+        used_s, used_d = set(), set()
+
+        def take(pool, used, n):
+            avail = [i for i in range(pool) if i not in used]
+            got = [int(x) for x in rng.choice(avail, size=n, replace=False)]
+            used.update(got)
+            return got
+
+        sg = [take(pool_s, used_s, 1) for _ in range(n_gdn)]
+        dg = [take(pool_d, used_d, 1) for _ in range(n_gdn)]
+        steps, _, total = _token_plan(rng, s_mgr, max_blocks=4)
+        seen, new, last = _pick_steps(rng, steps)
+        if kimi:
+            extra = int(rng.choice([0, 1]))
+            n_s = -(-total // s_mgr) + extra
+            n_d = -(-total // d_mgr) + extra
+            if kind == "PEQD":
+                n_d = n_s
+            sg.append(take(pool_s, used_s, n_s))
+            dg.append(take(pool_d, used_d, n_d))
+        tasks.append([seen, new, last, sg, dg])
+    return dict(parser=parser, src=src, dst=dst, valid=int(valid), tp_size=tp_size, tp_rank=tp_rank,
+                fp8=False, tasks=tasks)
+
+
 TOKEN_WALK = ["RAGGED_PEQD", "RAGGED_PGTD", "RAGGED_PGTD_DPSK", "RAGGED_PLTD", "FLASH_PEQD",
               "FLASH_PGTD", "DPSK_PEQD", "DPSK_PGTD", "DPSK_PLTD", "FLASHINFER_PEQD",
               "FLASHINFER_PGTD"]
 HYBRID = ["HYBRID_PEQD", "HYBRID_PGTD", "HYBRID_PLTD", "HYBRID_FI_PEQD", "HYBRID_FI_PGTD",
           "HYBRID_FI_PLTD", "TURBOQUANT_PEQD", "TURBOQUANT_PGTD"]
-ALL_PARSERS = TOKEN_WALK + HYBRID
+KDA = ["KDA_PEQD", "KDA_PGTD", "KDA_PLTD", "KIMI_K3_PEQD", "KIMI_K3_PGTD", "KIMI_K3_PLTD"]
+ALL_PARSERS = TOKEN_WALK + HYBRID + KDA
 
 
 def gen_case(parser, seed):
     rng = np.random.default_rng(seed)
     if parser in TOKEN_WALK:
         c = gen_token_walk(rng, parser)
+    elif parser in KDA:
+        c = gen_kda(rng, parser)
     else:
         base = parser.replace("TURBOQUANT", "HYBRID")
         c = gen_hybrid(rng, base)

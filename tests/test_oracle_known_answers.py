@@ -150,6 +150,42 @@ def test_hybrid_flashinfer_p_gt_d_known_answer():
     assert o[:7] == exp
 
 
+# parse_block_kda_test.cpp:78-361: SD conv state {8,2,6} x 1 B, recurrent {8,1,2,2} x 4 B,
+# channel dims {2,2,2}, P tp 4 rank 1 -> D tp 2, pages of 32 B (P) and 64 B (D), block 1 -> 2
+def test_kda_p_gt_d_sd_known_answer():
+    kw = dict(num_gdn_layers=1, conv_state_shape=[8, 2, 6], ssm_state_shape=[8, 1, 2, 2],
+              gdn_conv_channel_dims=[2, 2, 2], gdn_conv_elem_size=1, gdn_ssm_elem_size=4)
+    src = make_worker_info([32], [32], 8, tp=4, rank=1, **kw)
+    dst = make_worker_info([64], [64], 8, tp=2, rank=0, **kw)
+    o = _parse("KDA_PGTD", src, dst, [TaskBuf(0, 1, True, [[1]], [[2]])])[0]
+    assert o == [(32, 130, 2), (34, 134, 2), (36, 138, 2), (38, 142, 2), (40, 146, 2),
+                 (42, 150, 2), (44, 168, 16)]
+    # nothing is sent before the request's last chunk
+    assert _parse("KDA_PGTD", src, dst, [TaskBuf(0, 1, False, [[1]], [[2]])])[0] == []
+
+
+def test_kda_layout_closed_forms():
+    # DS layout keeps each channel's history contiguous: one piece per q/k/v component
+    kw = dict(num_gdn_layers=1, conv_state_shape=[8, 6, 2], ssm_state_shape=[8, 1, 2, 2],
+              gdn_conv_channel_dims=[2, 2, 2], gdn_conv_elem_size=1, gdn_ssm_elem_size=4,
+              kda_conv_dim_first=True)
+    src = make_worker_info([32], [32], 8, tp=4, rank=1, **kw)
+    dst = make_worker_info([64], [64], 8, tp=2, rank=0, **kw)
+    o = _parse("KDA_PGTD", src, dst, [TaskBuf(0, 1, True, [[1]], [[2]])])[0]
+    assert o == [(32, 128 + 4, 4), (36, 128 + 8 + 4, 4), (40, 128 + 16 + 4, 4), (44, 168, 16)]
+    # P==D: whole pages, page stride override
+    w = make_worker_info([32], [32], 16, kda_page_stride=48, **kw)
+    o = _parse("KDA_PEQD", w, w, [TaskBuf(0, 1, True, [[3]], [[5]])])[0]
+    assert o == [(144, 240, 48)]
+    # P<D mirrors P>D: the receiver takes its slice of every component
+    kw2 = dict(kw, conv_state_shape=[8, 12, 2], ssm_state_shape=[8, 2, 2, 2],
+               gdn_conv_channel_dims=[4, 4, 4])
+    srcw = make_worker_info([64], [64], 8, tp=2, rank=0, **kw2)
+    dstn = make_worker_info([32], [32], 8, tp=4, rank=1, **kw2)
+    o = _parse("KDA_PLTD", srcw, dstn, [TaskBuf(0, 1, True, [[2]], [[1]])], valid=0b11)[0]
+    assert o == [(128 + 4, 32, 4), (128 + 8 + 4, 36, 4), (128 + 16 + 4, 40, 4), (128 + 24 + 16, 44, 16)]
+
+
 # send_stub_test.cpp:1552-1559, :2739-2802 (ComputeValidRanksTest.*) and :1803-1807
 @pytest.mark.parametrize("p,d,heads,mask", [
     (4, 2, 8, 0b1111), (8, 4, 8, 0xFF), (8, 4, -1, 0xFF), (8, 2, 2, 0b00010001),
