@@ -30,7 +30,7 @@ extern "C" {
 const char* kvt_last_error(void);
 /* sizeof() of the ABI structs as compiled, for binding self-checks:
  * which = 0 kvt_ipc_block, 1 kvt_worker_info, 2 kvt_task, 3 kvt_parse_opts,
- * 4 kvt_xform. */
+ * 4 kvt_xform, 5 kvt_wire_layout. */
 uint64_t kvt_abi_sizeof(int which);
 /* Number of usable gfx950 devices (0 when none / no driver). */
 int kvt_device_count(void);
@@ -175,6 +175,64 @@ int kvt_pack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, ui
 int kvt_unpack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, uint32_t n_layers,
                const void* packed, uint64_t layer_stride, void* stream);
 
+/* The same with caller-chosen blob positions: tensor t's blob of layer l lives at
+ * base + (l - first_layer) * layer_stride + blob_offsets[t]. Used to pack
+ * straight into a framed send buffer (blob_offsets from kvt_wire_layout) or to
+ * unpack out of a received frame. 16-byte aligned positions take the vector
+ * path; others fall back to 4-byte or byte copies. */
+int kvt_pack_at(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, uint32_t n_layers,
+                void* base, uint64_t layer_stride, const uint64_t* blob_offsets, void* stream);
+int kvt_unpack_at(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer,
+                  uint32_t n_layers, const void* base, uint64_t layer_stride,
+                  const uint64_t* blob_offsets, void* stream);
+
+/* ------------------------------------------ layer-message framing (host) */
+
+/* The per-layer messages of the staged transports:
+ *   KVT_WIRE_TCP          TCPChannel::send_data / TCPServer::handle_kv_cache_data
+ *                                               kvtransfer/src/tcp_channel.cpp:477-560, 141-261
+ *   KVT_WIRE_RDMA_STAGED  RDMAStagedChannel::send_data / RDMAStagedServer
+ *                                               kvtransfer/src/rdma_staged_channel.cpp:246-300,
+ *                                               kvtransfer/src/rdma_staged_server.cpp:379-420
+ * Byte layout: see csrc/kvt_wire.cpp. Integers are host-endian 64-bit like the
+ * reference's size_t memcpy's. */
+enum { KVT_WIRE_TCP = 0, KVT_WIRE_RDMA_STAGED = 1 };
+#define KVT_WIRE_MAGIC 0x4B564361u /* KV_CACHE_DATA_MAGIC, kvtransfer/include/copy_utils.h:32 */
+typedef struct kvt_wire_layout {
+  uint64_t total_bytes;
+  uint32_t n_tensors;
+  uint32_t reserved0;
+  uint64_t meta_offset[KVT_MAX_TENSORS]; /* where tensor t's [n][ranges] starts */
+  uint64_t blob_offset[KVT_MAX_TENSORS];
+  uint64_t blob_bytes[KVT_MAX_TENSORS];
+} kvt_wire_layout;
+/* Sizes and positions of a frame for these range lists (the total_bytes sum of
+ * register_data,                                kvtransfer/src/tcp_channel.cpp:431-446). */
+int kvt_wire_layout_of(int format, const kvt_block_lists* lists, kvt_wire_layout* out);
+/* Writes header and range metadata; the blob areas are left for the pack. */
+int kvt_wire_write_frame(int format, void* buf, uint64_t capacity, uint64_t reqid,
+                         uint64_t layer_idx, const kvt_block_lists* lists, kvt_wire_layout* out);
+/* Receiver side: checks magic, truncation and sizes the way the reference's
+ * handlers do, fills `lists` with the ranges and `out` with the blob positions.
+ * expect_tensors = 0 accepts any count. Errors: KVT_ERR_INVALID. */
+int kvt_wire_parse_frame(int format, const void* buf, uint64_t len, uint32_t expect_tensors,
+                         uint64_t* reqid, uint64_t* layer_idx, kvt_block_lists* lists,
+                         kvt_wire_layout* out);
+
+/* ------------------------------------------------- KVStore block objects */
+
+/* Range lists whose packed blob is a sequence of per-block store objects, in
+ * the order of the given block ids: the object of block b is what
+ * FileBackend saves / loads per (block hash, rank, layer),
+ * `kvcache[:, b]` for the [2, nblk, bs, h, d] layout
+ *                                               blade_kvt/hybrid_connector/file_backend.py:222-232, 269-283
+ * (K block then V block), and the contiguous block for block-major layouts.
+ * Object i of tensor t starts at i * block_sizes[t] inside that tensor's blob.
+ * Do not merge these lists. *object_bytes = sum over tensors of the block size. */
+int kvt_block_object_lists(int cache_shape, const kvt_worker_info* src, const kvt_worker_info* dst,
+                           const uint32_t* src_blocks, const uint32_t* dst_blocks, uint64_t n,
+                           kvt_block_lists* lists, uint64_t* object_bytes);
+
 /* --------------------------- drop-ins for the reference copy entry points */
 
 /* replaces launch_copy_d2h_direct_kernel()      kvtransfer/src/copy_kernels.cu:268-281
@@ -261,9 +319,14 @@ void* kvt_stager_copy_stream(kvt_stager* s);
  * `producer_stream`, then copies `bytes` from dev into the slot. */
 int kvt_stager_save(kvt_stager* s, uint32_t slot, const void* dev, uint64_t bytes,
                     void* producer_stream);
+/* Same, to byte `slot_offset` of the slot (e.g. the blob area of a frame). */
+int kvt_stager_save_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, const void* dev,
+                       uint64_t bytes, void* producer_stream);
 /* Slot -> device on the copy stream, then makes consumer_stream wait for it. */
 int kvt_stager_load(kvt_stager* s, uint32_t slot, void* dev, uint64_t bytes,
                     void* consumer_stream);
+int kvt_stager_load_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, void* dev,
+                       uint64_t bytes, void* consumer_stream);
 /* Host-blocking: the slot's last save/load has completed. */
 int kvt_stager_wait(kvt_stager* s, uint32_t slot);
 /* Measured plain pinned<->device copy rate in bytes/s (direction: KVT_COPY_*),

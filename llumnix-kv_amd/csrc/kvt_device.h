@@ -13,13 +13,18 @@ namespace kvt {
 // side), so an entry carries a single cache offset.
 struct __attribute__((aligned(16))) Chunk {
   uint64_t cache;      // byte offset in the layer tensor (source for pack, destination for unpack)
-  uint64_t packed;     // byte offset inside one layer's packed area
+  uint64_t packed;     // byte offset inside the tensor's blob of one packed layer
   uint32_t len;        // bytes, <= 4096 << sub_shift of the plan
   uint16_t tensor;     // cache tensor index within the layer
   uint16_t t0;         // layout transform only: first token of the half page covered
   uint64_t reserved;
 };
 static_assert(sizeof(Chunk) == 32, "Chunk must stay 32 bytes");
+
+// Where each cache tensor's blob starts inside one packed layer (kernel argument).
+struct BlobOffsets {
+  uint64_t off[8];
+};
 
 // Device-side constants of the HND <-> NHD page transform.
 struct XformDev {
@@ -30,11 +35,12 @@ struct XformDev {
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, hipStream_t stream);
+                              uint64_t layer_stride, const BlobOffsets& blobs, hipStream_t stream);
 hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                               uint64_t layer_stride, const XformDev& x, hipStream_t stream);
+                               uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
+                               hipStream_t stream);
 // rows = workgroups striding over the 4 KiB slices of each range
 hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                               const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,

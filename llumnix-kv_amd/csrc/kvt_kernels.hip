@@ -65,7 +65,7 @@ template <bool PACK>
 __global__ __launch_bounds__(kThreads) void copy_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint8_t* __restrict__ packed, uint64_t layer_stride) {
+    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
   const uint32_t b = xcd_remap(blockIdx.x, n_slices);
   if (b >= n_slices) return;
   const Chunk c = chunks[b >> sub_shift];
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void copy_chunks_kernel(
   const uint32_t layer = blockIdx.y;
   uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] +
                    c.cache + off;
-  uint8_t* pk = packed + layer * layer_stride + c.packed + off;
+  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
   if (PACK)
     copy_slice(pk, cache, len, threadIdx.x);
   else
@@ -90,7 +90,7 @@ template <bool PACK>
 __global__ __launch_bounds__(kThreads) void xform_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint8_t* __restrict__ packed, uint64_t layer_stride, XformDev x) {
+    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs, XformDev x) {
   const uint32_t b = xcd_remap(blockIdx.x, n_slices);
   if (b >= n_slices) return;
   const Chunk c = chunks[b >> sub_shift];
@@ -99,7 +99,8 @@ __global__ __launch_bounds__(kThreads) void xform_chunks_kernel(
   const uint32_t layer = blockIdx.y;
   u32x4* cv = reinterpret_cast<u32x4*>(
       layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache);
-  u32x4* pv = reinterpret_cast<u32x4*>(packed + layer * layer_stride + c.packed);
+  u32x4* pv =
+      reinterpret_cast<u32x4*>(packed + layer * layer_stride + blobs.off[c.tensor] + c.packed);
   // exact quotients by multiply-high (operands < 2^16); a divisor of 1 has no such constant
   const uint32_t r = x.vrow == 1 ? v : __umulhi(v, x.inv_vrow);  // packed-side row: t_local*heads + h
   const uint32_t col = v - r * x.vrow;
@@ -218,36 +219,37 @@ static uint32_t round8(uint32_t n) { return (n + 7u) & ~7u; }
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, hipStream_t stream) {
+                              uint64_t layer_stride, const BlobOffsets& blobs, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const dim3 grid(round8(n_slices), n_layers);
   if (pack)
     hipLaunchKernelGGL((copy_chunks_kernel<true>), grid, dim3(kThreads), 0, stream, chunks,
                        n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride);
+                       layer_stride, blobs);
   else
     hipLaunchKernelGGL((copy_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
                        n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride);
+                       layer_stride, blobs);
   return hipGetLastError();
 }
 
 hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                               uint64_t layer_stride, const XformDev& x, hipStream_t stream) {
+                               uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
+                               hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const dim3 grid(round8(n_slices), n_layers);
   if (pack)
     hipLaunchKernelGGL((xform_chunks_kernel<true>), grid, dim3(kThreads), 0, stream, chunks,
                        n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, x);
+                       layer_stride, blobs, x);
   else
     hipLaunchKernelGGL((xform_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
                        n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, x);
+                       layer_stride, blobs, x);
   return hipGetLastError();
 }
 

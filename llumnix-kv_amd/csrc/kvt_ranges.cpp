@@ -107,6 +107,7 @@ uint64_t kvt_abi_sizeof(int which) {
     case 2: return sizeof(kvt_task);
     case 3: return sizeof(kvt_parse_opts);
     case 4: return sizeof(kvt_xform);
+    case 5: return sizeof(kvt_wire_layout);
     default: return 0;
   }
 }

@@ -353,7 +353,7 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       for (const kvt_ipc_block& r : runs) {
         if (!p->xform) {
           for (uint64_t o = 0; o < r.length; o += chunk_bytes)
-            pieces.push_back(Piece{r.src_offset + o, r.dst_offset + o, cursor + blob + o,
+            pieces.push_back(Piece{r.src_offset + o, r.dst_offset + o, blob + o,
                                    static_cast<uint32_t>(std::min<uint64_t>(chunk_bytes, r.length - o)),
                                    static_cast<uint16_t>(t), 0});
         } else {
@@ -365,7 +365,7 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
             for (uint32_t t0 = 0; t0 < xform->ntpb; t0 += tok_per_chunk) {
               const uint32_t nt = std::min(tok_per_chunk, xform->ntpb - t0);
               pieces.push_back(Piece{r.src_offset + o, r.dst_offset + o,
-                                     cursor + blob + o + static_cast<uint64_t>(t0) * tok_bytes,
+                                     blob + o + static_cast<uint64_t>(t0) * tok_bytes,
                                      static_cast<uint32_t>(nt * tok_bytes), 0,
                                      static_cast<uint16_t>(t0)});
             }
@@ -465,7 +465,8 @@ uint64_t kvt_plan_tensor_offset(const kvt_plan* p, uint32_t t) {
 uint64_t kvt_plan_layer_bytes(const kvt_plan* p) { return p ? p->layer_bytes : 0; }
 
 static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer,
-                    uint32_t n_layers, void* packed, uint64_t layer_stride, void* stream) {
+                    uint32_t n_layers, void* packed, uint64_t layer_stride, void* stream,
+                    const uint64_t* blob_offsets = nullptr) {
   if (!p || !cache || (!packed && p->n_chunks))
     return fail(KVT_ERR_INVALID, "kvt_pack/unpack: null argument");
   if (p->device != cache->device) return fail(KVT_ERR_INVALID, "plan and cache are on different devices");
@@ -474,8 +475,13 @@ static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
   if (static_cast<uint64_t>(first_layer) + n_layers > cache->n_layers)
     return fail(KVT_ERR_OUT_OF_RANGE, "layer range exceeds the registered cache");
   if (n_layers > 65535) return fail(KVT_ERR_INVALID, "at most 65535 layers per launch");
-  if (n_layers > 1 && layer_stride < p->layer_bytes)
+  if (n_layers > 1 && !blob_offsets && layer_stride < p->layer_bytes)
     return fail(KVT_ERR_INVALID, "layer_stride smaller than one packed layer");
+  BlobOffsets blobs{};
+  for (uint32_t t = 0; t < p->n_tensors; ++t)
+    blobs.off[t] = blob_offsets ? blob_offsets[t] : p->tensor_offset[t];
+  if (p->xform && (blobs.off[0] & 15u))
+    return fail(KVT_ERR_INVALID, "layout transform needs a 16-byte aligned blob offset");
   const std::vector<uint64_t>& need = pack ? p->src_cap : p->dst_cap;
   for (uint32_t t = 0; t < p->n_tensors; ++t)
     if (cache->capacity[t] < need[t])
@@ -503,10 +509,10 @@ static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
   const hipError_t e =
       p->xform ? launch_xform_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                      first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                     layer_stride, p->xdev, s)
+                                     layer_stride, blobs, p->xdev, s)
                : launch_copy_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                     first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                    layer_stride, s);
+                                    layer_stride, blobs, s);
   if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
   if (p->buf) {
     // remember when the table is last read, so that its storage is not recycled too early
@@ -529,6 +535,22 @@ int kvt_unpack(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, 
                const void* packed, uint64_t layer_stride, void* stream) {
   return guarded([&]() {
     return run_plan(false, p, cache, first_layer, n_layers, const_cast<void*>(packed), layer_stride, stream);
+  });
+}
+
+int kvt_pack_at(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer, uint32_t n_layers,
+                void* base, uint64_t layer_stride, const uint64_t* blob_offsets, void* stream) {
+  return guarded([&]() {
+    return run_plan(true, p, cache, first_layer, n_layers, base, layer_stride, stream, blob_offsets);
+  });
+}
+
+int kvt_unpack_at(const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer,
+                  uint32_t n_layers, const void* base, uint64_t layer_stride,
+                  const uint64_t* blob_offsets, void* stream) {
+  return guarded([&]() {
+    return run_plan(false, p, cache, first_layer, n_layers, const_cast<void*>(base), layer_stride,
+                    stream, blob_offsets);
   });
 }
 
@@ -797,15 +819,21 @@ void* kvt_stager_copy_stream(kvt_stager* s) { return s ? s->copy : nullptr; }
 
 int kvt_stager_save(kvt_stager* s, uint32_t slot, const void* dev, uint64_t bytes,
                     void* producer_stream) {
+  return kvt_stager_save_at(s, slot, 0, dev, bytes, producer_stream);
+}
+
+int kvt_stager_save_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, const void* dev,
+                       uint64_t bytes, void* producer_stream) {
   return guarded([&]() -> int {
     if (!s || !dev) return fail(KVT_ERR_INVALID, "kvt_stager_save: null argument");
-    if (slot >= s->n_slots || bytes > s->slot_bytes)
+    if (slot >= s->n_slots || slot_offset > s->slot_bytes || bytes > s->slot_bytes - slot_offset)
       return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_save: slot index or size out of range");
     DeviceGuard g;
     if (int rc = g.enter(s->device)) return rc;
     KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(producer_stream)));
     KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));
-    KVT_HIP(hipMemcpyAsync(kvt_stager_slot(s, slot), dev, bytes, hipMemcpyDeviceToHost, s->copy));
+    KVT_HIP(hipMemcpyAsync(static_cast<uint8_t*>(kvt_stager_slot(s, slot)) + slot_offset, dev, bytes,
+                           hipMemcpyDeviceToHost, s->copy));
     KVT_HIP(hipEventRecord(s->slot_done[slot], s->copy));
     return KVT_OK;
   });
@@ -813,16 +841,22 @@ int kvt_stager_save(kvt_stager* s, uint32_t slot, const void* dev, uint64_t byte
 
 int kvt_stager_load(kvt_stager* s, uint32_t slot, void* dev, uint64_t bytes,
                     void* consumer_stream) {
+  return kvt_stager_load_at(s, slot, 0, dev, bytes, consumer_stream);
+}
+
+int kvt_stager_load_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, void* dev,
+                       uint64_t bytes, void* consumer_stream) {
   return guarded([&]() -> int {
     if (!s || !dev) return fail(KVT_ERR_INVALID, "kvt_stager_load: null argument");
-    if (slot >= s->n_slots || bytes > s->slot_bytes)
+    if (slot >= s->n_slots || slot_offset > s->slot_bytes || bytes > s->slot_bytes - slot_offset)
       return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_load: slot index or size out of range");
     DeviceGuard g;
     if (int rc = g.enter(s->device)) return rc;
     // the device buffer may still be read by earlier work of the consumer
     KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(consumer_stream)));
     KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));
-    KVT_HIP(hipMemcpyAsync(dev, kvt_stager_slot(s, slot), bytes, hipMemcpyHostToDevice, s->copy));
+    KVT_HIP(hipMemcpyAsync(dev, static_cast<uint8_t*>(kvt_stager_slot(s, slot)) + slot_offset, bytes,
+                           hipMemcpyHostToDevice, s->copy));
     KVT_HIP(hipEventRecord(s->slot_done[slot], s->copy));
     KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream), s->slot_done[slot], 0));
     return KVT_OK;

@@ -6,10 +6,12 @@ module only loads it and offers thin helpers used by the tests, ``bench.py`` and
 ``KvtError`` when the library or a gfx950 device is missing.
 """
 from .binding import (KvtError, LIB_PATH, BlockLists, Cache, Parser, Plan, Session, Stager,
-                      device_count, lib, select_parser, compute_valid_ranks_pd, merge_interval,
-                      validate_bounds)
+                      WireLayout, WIRE_TCP, WIRE_RDMA_STAGED, block_object_lists, device_count,
+                      lib, select_parser, compute_valid_ranks_pd, merge_interval, validate_bounds,
+                      wire_layout_of, wire_parse_frame, wire_write_frame)
 from . import ctypes_defs
 
 __all__ = ["KvtError", "LIB_PATH", "BlockLists", "Cache", "Parser", "Plan", "Session", "Stager",
            "device_count", "lib", "select_parser", "compute_valid_ranks_pd", "merge_interval",
-           "validate_bounds", "ctypes_defs"]
+           "validate_bounds", "ctypes_defs", "WireLayout", "WIRE_TCP", "WIRE_RDMA_STAGED",
+           "block_object_lists", "wire_layout_of", "wire_parse_frame", "wire_write_frame"]

@@ -15,6 +15,14 @@ _u32, _u64, _i64, _int = C.c_uint32, C.c_uint64, C.c_int64, C.c_int
 _P = C.POINTER
 
 
+class WireLayout(C.Structure):
+    _fields_ = [("total_bytes", _u64), ("n_tensors", _u32), ("reserved0", _u32),
+                ("meta_offset", _u64 * 8), ("blob_offset", _u64 * 8), ("blob_bytes", _u64 * 8)]
+
+
+WIRE_TCP, WIRE_RDMA_STAGED = 0, 1
+
+
 class Xform(C.Structure):
     _fields_ = [("kind", _u32), ("heads", _u32), ("ntpb", _u32), ("row_bytes", _u32)]
 
@@ -53,6 +61,14 @@ SIGNATURES = {
     "kvt_plan_layer_bytes": (_u64, [_vp]),
     "kvt_pack": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _vp]),
     "kvt_unpack": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _vp]),
+    "kvt_pack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
+    "kvt_unpack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
+    "kvt_wire_layout_of": (_int, [_int, _vp, _P(WireLayout)]),
+    "kvt_wire_write_frame": (_int, [_int, _vp, _u64, _u64, _u64, _vp, _P(WireLayout)]),
+    "kvt_wire_parse_frame": (_int, [_int, _vp, _u64, _u32, _P(_u64), _P(_u64), _vp,
+                                    _P(WireLayout)]),
+    "kvt_block_object_lists": (_int, [_int, _P(WorkerInfo), _P(WorkerInfo), _vp, _vp, _u64, _vp,
+                                      _P(_u64)]),
     "kvt_launch_copy_d2h_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
@@ -70,6 +86,8 @@ SIGNATURES = {
     "kvt_stager_slot": (_vp, [_vp, _u32]),
     "kvt_stager_copy_stream": (_vp, [_vp]),
     "kvt_stager_save": (_int, [_vp, _u32, _vp, _u64, _vp]),
+    "kvt_stager_save_at": (_int, [_vp, _u32, _u64, _vp, _u64, _vp]),
+    "kvt_stager_load_at": (_int, [_vp, _u32, _u64, _vp, _u64, _vp]),
     "kvt_stager_load": (_int, [_vp, _u32, _vp, _u64, _vp]),
     "kvt_stager_wait": (_int, [_vp, _u32]),
     "kvt_measure_pcie": (_int, [_int, _int, _u64, _u32, _P(C.c_double)]),
@@ -158,6 +176,39 @@ def merge_interval(runs):
     stats = (_u64 * 4)()
     check(lib().kvt_merge_interval(a.ctypes.data, len(a), C.byref(n_out), stats))
     return a[:n_out.value].copy(), tuple(stats)
+
+
+def wire_layout_of(fmt, lists):
+    lay = WireLayout()
+    check(lib().kvt_wire_layout_of(fmt, lists.h, C.byref(lay)))
+    return lay
+
+
+def wire_write_frame(fmt, buf_ptr, capacity, reqid, layer_idx, lists):
+    lay = WireLayout()
+    check(lib().kvt_wire_write_frame(fmt, buf_ptr, capacity, reqid, layer_idx, lists.h,
+                                     C.byref(lay)))
+    return lay
+
+
+def wire_parse_frame(fmt, buf_ptr, length, expect_tensors=0):
+    """-> (rc, reqid, layer_idx, BlockLists, WireLayout)"""
+    lay, reqid, layer = WireLayout(), _u64(), _u64()
+    lists = BlockLists()
+    rc = lib().kvt_wire_parse_frame(fmt, buf_ptr, length, expect_tensors, C.byref(reqid),
+                                    C.byref(layer), lists.h, C.byref(lay))
+    return rc, reqid.value, layer.value, lists, lay
+
+
+def block_object_lists(cache_shape, src, dst, src_blocks, dst_blocks, lists=None):
+    """-> (BlockLists, object_bytes)"""
+    lists = lists or BlockLists()
+    s = np.ascontiguousarray(src_blocks, dtype=np.uint32)
+    d = np.ascontiguousarray(dst_blocks, dtype=np.uint32)
+    ob = _u64()
+    check(lib().kvt_block_object_lists(cache_shape, C.byref(src), C.byref(dst), s.ctypes.data,
+                                       d.ctypes.data, len(s), lists.h, C.byref(ob)))
+    return lists, ob.value
 
 
 def validate_bounds(runs, capacity, which, scale=1):
@@ -302,6 +353,17 @@ class Plan:
         check(lib().kvt_unpack(self.h, cache.h, first_layer, n_layers, _ptr(packed), layer_stride,
                                _ptr(stream)))
 
+    def pack_at(self, cache, first_layer, n_layers, base, layer_stride, blob_offsets, stream=None):
+        offs = (_u64 * 8)(*blob_offsets)
+        check(lib().kvt_pack_at(self.h, cache.h, first_layer, n_layers, _ptr(base), layer_stride,
+                                offs, _ptr(stream)))
+
+    def unpack_at(self, cache, first_layer, n_layers, base, layer_stride, blob_offsets,
+                  stream=None):
+        offs = (_u64 * 8)(*blob_offsets)
+        check(lib().kvt_unpack_at(self.h, cache.h, first_layer, n_layers, _ptr(base), layer_stride,
+                                  offs, _ptr(stream)))
+
 
 class Session:
     def __init__(self, plan, cache, packed, layer_stride):
@@ -354,6 +416,14 @@ class Stager:
     @property
     def copy_stream(self):
         return lib().kvt_stager_copy_stream(self.h)
+
+    def save_at(self, slot, offset, dev, nbytes, producer_stream=None):
+        check(lib().kvt_stager_save_at(self.h, slot, offset, _ptr(dev), nbytes,
+                                       _ptr(producer_stream)))
+
+    def load_at(self, slot, offset, dev, nbytes, consumer_stream=None):
+        check(lib().kvt_stager_load_at(self.h, slot, offset, _ptr(dev), nbytes,
+                                       _ptr(consumer_stream)))
 
     def save(self, slot, dev, nbytes, producer_stream=None):
         check(lib().kvt_stager_save(self.h, slot, _ptr(dev), nbytes, _ptr(producer_stream)))
