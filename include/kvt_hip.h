@@ -30,7 +30,7 @@ extern "C" {
 const char* kvt_last_error(void);
 /* sizeof() of the ABI structs as compiled, for binding self-checks:
  * which = 0 kvt_ipc_block, 1 kvt_worker_info, 2 kvt_task, 3 kvt_parse_opts,
- * 4 kvt_xform, 5 kvt_wire_layout. */
+ * 4 kvt_xform, 5 kvt_wire_layout, 6 kvt_run. */
 uint64_t kvt_abi_sizeof(int which);
 /* Number of usable gfx950 devices (0 when none / no driver). */
 int kvt_device_count(void);
@@ -83,6 +83,36 @@ int kvt_block_lists_append(kvt_block_lists* l, uint32_t tensor, const kvt_ipc_bl
  * capacity overflow (parse_block_common.cpp:20-29). On error the lists keep
  * whatever was appended before the failing range, like the reference. */
 int kvt_parse_block(const kvt_parser* p, const kvt_task* task, kvt_block_lists* lists);
+
+/* ------------------------------------------- strided runs (device-side parse) */
+
+/* Per-tensor lists of kvt_run. The TP-remapping parsers (P>D, P<D) produce one
+ * range per token, per head, for K and V   kvtransfer/src/parse_block_common.cpp:81-129,
+ *                                          kvtransfer/src/parse_block_flashinfer.cpp:82-235,
+ *                                          kvtransfer/src/parse_block_qwen3_next.cpp:108-248
+ * i.e. millions of 256-512 byte ranges for a large batch. kvt_parse_block_runs
+ * emits the same sequence in closed form (one run per block segment), and a
+ * plan built from runs evaluates the token -> offset arithmetic inside the
+ * copy kernel instead of on the host. */
+typedef struct kvt_run_lists kvt_run_lists;
+int kvt_run_lists_create(kvt_run_lists** out);
+void kvt_run_lists_destroy(kvt_run_lists* l);
+void kvt_run_lists_clear(kvt_run_lists* l);
+uint32_t kvt_run_lists_num_tensors(const kvt_run_lists* l);
+int kvt_run_lists_view(const kvt_run_lists* l, uint32_t tensor, const kvt_run** data, uint64_t* n);
+/* Number of ranges / bytes the runs of one tensor expand to. */
+int kvt_run_lists_totals(const kvt_run_lists* l, uint32_t tensor, uint64_t* n_ranges,
+                         uint64_t* n_bytes);
+/* Same contract as kvt_parse_block (same ranges, same order, same errors), in
+ * run form: expanding what this appends equals what kvt_parse_block appends. */
+int kvt_parse_block_runs(const kvt_parser* p, const kvt_task* task, kvt_run_lists* lists);
+/* Appends the expansion of every run to `out` (e.g. the range metadata of a
+ * layer message for a peer that expects plain ranges). */
+int kvt_run_lists_expand(const kvt_run_lists* l, kvt_block_lists* out);
+/* The inverse, for a receiver that got plain ranges: finds the arithmetic
+ * progressions (innermost first, three levels) and appends runs whose expansion
+ * is exactly the input list. */
+int kvt_run_lists_compress(const kvt_block_lists* l, kvt_run_lists* out);
 
 /* replaces merge_interval() + the erase of zero-length entries its callers do
  *                                               kvtransfer/src/channel.cpp:53-98,
@@ -145,6 +175,27 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
                     const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
                     kvt_plan** out);
 void kvt_plan_destroy(kvt_plan* p);
+/* A plan from runs: runs whose ranges are shorter than 4 KiB and 16-byte
+ * aligned (offsets, strides, length) stay strided on the device (one table
+ * entry per <= chunk_bytes of payload, the per-token arithmetic done by the
+ * kernel); all others are expanded to plain chunks. Same pack / unpack entry
+ * points and the same packed layout as a plan made from the expanded lists.
+ * Layer base pointers, the packed buffer and blob positions given to
+ * kvt_pack_at / kvt_unpack_at must be 16-byte aligned for such a plan. */
+int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
+                         const uint64_t* dst_capacity, uint32_t chunk_bytes, kvt_plan** out);
+/* Table entries that stayed strided (0 for a plan made from plain lists). */
+uint64_t kvt_plan_num_strided_chunks(const kvt_plan* p);
+/* Inspection without a GPU: a plan created with device = KVT_DEVICE_NONE keeps
+ * its two tables on the host and cannot be launched. *chunks = 2 * n_chunks
+ * entries of 32 bytes {u64 cache, u64 packed, u32 len, u16 tensor, u16 t0,
+ * u32 shape, u32 0}: pack order first, then unpack order; *shapes = 16 record
+ * shapes of 48 bytes {u32 vlen16, u32 inv, u32 n_inner, u32 0, u64 outer[2],
+ * u64 inner[2]} ([0] source side, [1] destination side). Entry semantics: see
+ * csrc/kvt_device.h. Borrowed pointers, valid until the plan is destroyed. */
+#define KVT_DEVICE_NONE (-1)
+int kvt_plan_host_tables(const kvt_plan* p, const void** chunks, uint64_t* n_chunks,
+                         uint32_t* chunk_bytes, const void** shapes);
 /* The table upload is asynchronous; launches order themselves after it on
  * their stream. Host-blocking wait for it -- needed only before the plan is
  * used inside a stream capture (kvt_session_create does it itself). */

@@ -38,6 +38,24 @@ typedef struct kvt_ipc_block {
   uint64_t length;
 } kvt_ipc_block;
 
+/* A strided nest of equal-length ranges: n[0]*n[1]*n[2] ranges of `length`
+ * bytes; the range with indices (i0, i1, i2), i2 running fastest, is
+ *   (src_offset + sum_k i_k*src_stride[k], dst_offset + sum_k i_k*dst_stride[k], length).
+ * Expanding the runs of a list in order gives exactly the kvt_ipc_block list
+ * (same order, hence the same packed blob). A TP-remapping parser emits one run
+ * per block segment instead of one range per token (and per head). No reference
+ * counterpart: the reference materialises every range on the host
+ * (e.g. parse_block_send_gt, kvtransfer/src/parse_block_common.cpp:81-129). */
+typedef struct kvt_run {
+  uint64_t src_offset;
+  uint64_t dst_offset;
+  uint64_t length;
+  uint32_t n[3];
+  uint32_t reserved0;
+  uint64_t src_stride[3];
+  uint64_t dst_stride[3];
+} kvt_run;
+
 /* Cache shapes (values equal the reference's BLLM_KVTRANS_CACHE_SHAPE ids). */
 enum {
   KVT_SHAPE_RAGGED_FLASH = 1,          /* [nblk, bs, 2, h, d] ; also dense MLA [nblk, bs, d] */

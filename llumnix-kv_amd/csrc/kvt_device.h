@@ -17,7 +17,8 @@ struct __attribute__((aligned(16))) Chunk {
   uint32_t len;        // bytes, <= 4096 << sub_shift of the plan
   uint16_t tensor;     // cache tensor index within the layer
   uint16_t t0;         // layout transform only: first token of the half page covered
-  uint64_t reserved;
+  uint32_t shape;      // strided plans only: 1 + index into the StrideTable, 0 = contiguous
+  uint32_t reserved;
 };
 static_assert(sizeof(Chunk) == 32, "Chunk must stay 32 bytes");
 
@@ -32,6 +33,25 @@ struct XformDev {
   uint32_t inv_vrow, inv_heads;   // floor(2^32 / d) + 1: exact quotients for operands < 2^16
 };
 
+// Record shape of a strided chunk: the packed side is a dense sequence of
+// records of vlen 16-byte vectors; record r lives in the cache at
+//   chunk.cache + (r / n_inner) * outer + (r % n_inner) * inner
+// (per token: the outer step; K and V of one token: the inner step).
+struct StrideShape {
+  uint32_t vlen, inv_vlen;     // inv_vlen = floor(2^32 / vlen) + 1, exact for operands < 2^32 / vlen
+  uint32_t n_inner, reserved;
+  uint64_t outer[2], inner[2];  // [0] = source side (pack), [1] = destination side (unpack)
+};
+constexpr uint32_t kMaxShapes = 16;
+struct StrideTable {
+  StrideShape shape[kMaxShapes];
+};
+
+hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
+                                 uint32_t sub_shift, uint8_t* const* layer_ptrs,
+                                 uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
+                                 uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
+                                 const StrideTable& shapes, hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

@@ -58,4 +58,8 @@ struct kvt_block_lists {
   std::vector<kvt::RunList> tensors;
 };
 
+struct kvt_run_lists {
+  std::vector<std::vector<kvt_run>> tensors;
+};
+
 #endif  // KVT_INTERNAL_H_

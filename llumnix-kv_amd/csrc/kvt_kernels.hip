@@ -82,6 +82,50 @@ __global__ __launch_bounds__(kThreads) void copy_chunks_kernel(
     copy_slice(cache, pk, len, threadIdx.x);
 }
 
+// Gather / scatter of a table whose chunks may be strided on the cache side:
+// the token -> offset arithmetic of the TP-remapping layouts (one short range
+// per token, per head, K and V) is evaluated here, per 16-byte vector, instead
+// of being materialised as one table entry per range. Contiguous chunks
+// (shape 0) take the plain path. Everything a strided chunk touches is 16-byte
+// aligned (checked on the host).
+template <bool PACK>
+__global__ __launch_bounds__(kThreads) void strided_chunks_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs, StrideTable shapes) {
+  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
+  if (b >= n_slices) return;
+  const Chunk c = chunks[b >> sub_shift];
+  const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
+  if (off >= c.len) return;
+  const uint32_t len = min(kSlice, c.len - off);
+  const uint32_t layer = blockIdx.y;
+  uint8_t* cache =
+      layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
+  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
+  if (c.shape == 0) {
+    if (PACK)
+      copy_slice(pk, cache + off, len, threadIdx.x);
+    else
+      copy_slice(cache + off, pk, len, threadIdx.x);
+    return;
+  }
+  if (threadIdx.x >= (len >> 4)) return;
+  const StrideShape& s = shapes.shape[c.shape - 1u];
+  const uint32_t v = (off >> 4) + threadIdx.x;  // vector index inside the chunk, < 2^15
+  const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
+  const uint32_t col = v - rec * s.vlen;
+  const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
+  const uint32_t i = rec - o * s.n_inner;
+  const uint64_t at = o * s.outer[PACK ? 0 : 1] + i * s.inner[PACK ? 0 : 1] + (col << 4);
+  u32x4* cv = reinterpret_cast<u32x4*>(cache + at);
+  u32x4* pv = reinterpret_cast<u32x4*>(pk) + threadIdx.x;
+  if (PACK)
+    __builtin_nontemporal_store(__builtin_nontemporal_load(cv), pv);
+  else
+    __builtin_nontemporal_store(__builtin_nontemporal_load(pv), cv);
+}
+
 // HND <-> NHD page transform. A chunk covers tokens [t0, t0 + len/(heads*row))
 // of one K or V half page whose base is c.cache. Packed side: [token][head][row]
 // contiguous from c.packed; cache side: [head][ntpb][row]. Lane v of the chunk
@@ -231,6 +275,25 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
     hipLaunchKernelGGL((copy_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
                        n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
                        layer_stride, blobs);
+  return hipGetLastError();
+}
+
+hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
+                                 uint32_t sub_shift, uint8_t* const* layer_ptrs,
+                                 uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
+                                 uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
+                                 const StrideTable& shapes, hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  const uint32_t n_slices = n_chunks << sub_shift;
+  const dim3 grid(round8(n_slices), n_layers);
+  if (pack)
+    hipLaunchKernelGGL((strided_chunks_kernel<true>), grid, dim3(kThreads), 0, stream, chunks,
+                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
+                       layer_stride, blobs, shapes);
+  else
+    hipLaunchKernelGGL((strided_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
+                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
+                       layer_stride, blobs, shapes);
   return hipGetLastError();
 }
 

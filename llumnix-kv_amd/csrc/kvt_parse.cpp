@@ -806,15 +806,48 @@ struct Groups {
 struct Sink {
   RunList* out;
   Capacity cap;
-  void put(u64 so, u64 dof, u64 len) {
+  std::vector<kvt_run>* runs = nullptr;  // run form: every record becomes (part of) a kvt_run
+
+  void check(u64 so, u64 dof, u64 len) const {
     const u64 M = std::numeric_limits<u64>::max();
     const bool ovf = cap.scale == 0 || len > M / cap.scale;
     const u64 eff = ovf ? M : len * cap.scale;
     if (len == 0 || ovf || so > cap.src || eff > cap.src - so || dof > cap.dst ||
         len > cap.dst - dof)
       throw RangeError("KVT GPU buffer range validation failed");
-    out->push_back(kvt_ipc_block{so, dof, len});
   }
+  void put(u64 so, u64 dof, u64 len) {
+    check(so, dof, len);
+    if (runs) {
+      kvt_run r{};
+      r.src_offset = so;
+      r.dst_offset = dof;
+      r.length = len;
+      r.n[0] = r.n[1] = r.n[2] = 1;
+      runs->push_back(r);
+    } else {
+      out->push_back(kvt_ipc_block{so, dof, len});
+    }
+  }
+  // Run form only. Offsets grow with every index, so the nest is inside the
+  // buffers exactly when its last range is (an index product that overflows
+  // 64 bits cannot be inside any buffer).
+  void put_nest(kvt_run r) {
+    u64 s_max = r.src_offset, d_max = r.dst_offset;
+    for (int k = 0; k < 3; ++k) {
+      const u64 steps = r.n[k] - 1;
+      u64 ds, dd;
+      if (__builtin_mul_overflow(steps, r.src_stride[k], &ds) ||
+          __builtin_add_overflow(s_max, ds, &s_max) ||
+          __builtin_mul_overflow(steps, r.dst_stride[k], &dd) ||
+          __builtin_add_overflow(d_max, dd, &d_max))
+        throw RangeError("KVT GPU buffer range validation failed");
+    }
+    check(r.src_offset, r.dst_offset, r.length);
+    check(s_max, d_max, r.length);
+    runs->push_back(r);
+  }
+  size_t size() const { return runs ? runs->size() : out->size(); }
 };
 
 inline u32 id_at(const u32* p, u64 n, u64 i) {
@@ -834,7 +867,7 @@ void run_walk(const WalkOp& w, const kvt_task& t, const Groups& sg, const Groups
   u64 sn, dn;
   sg.get(w.s.group, sid, sn);
   dg.get(w.d.group, did, dn);
-  const size_t first = sink.out->size();
+  const size_t first = sink.size();
   u32 pos = t.seen_tokens, rem = t.new_tokens;
   const u32 c0 = w.n_loops > 0 ? w.loops[0].count : 1;
   const u32 c1 = w.n_loops > 1 ? w.loops[1].count : 1;
@@ -844,25 +877,50 @@ void run_walk(const WalkOp& w, const kvt_task& t, const Groups& sg, const Groups
     const u64 dof = side_offset(w.d, pos, did, dn);
     const u32 n_tok = w.per_token ? k : 1;
     const u64 len = w.per_token ? w.unit : static_cast<u64>(k) * w.unit;
-    for (u32 a = 0; a < c0; ++a)
-      for (u32 b = 0; b < c1; ++b) {
-        const u64 s1 = so + a * w.loops[0].s_stride + b * w.loops[1].s_stride;
-        const u64 d1 = dof + a * w.loops[0].d_stride + b * w.loops[1].d_stride;
-        for (u32 i = 0; i < n_tok; ++i) {
-          const u64 s2 = s1 + i * w.s.tok_stride, d2 = d1 + i * w.d.tok_stride;
-          sink.put(s2, d2, len);
-          if (w.kv == KV_INTERLEAVED) sink.put(s2 + w.kv_s_add, d2 + w.kv_d_add, len);
+    if (sink.runs && c1 == 1) {  // the whole segment in closed form: loop x tokens x (K, V)
+      kvt_run r{};
+      r.src_offset = so;
+      r.dst_offset = dof;
+      r.length = len;
+      r.n[0] = c0;
+      r.src_stride[0] = c0 > 1 ? w.loops[0].s_stride : 0;
+      r.dst_stride[0] = c0 > 1 ? w.loops[0].d_stride : 0;
+      r.n[1] = n_tok;
+      r.src_stride[1] = n_tok > 1 ? w.s.tok_stride : 0;
+      r.dst_stride[1] = n_tok > 1 ? w.d.tok_stride : 0;
+      r.n[2] = w.kv == KV_INTERLEAVED ? 2 : 1;
+      r.src_stride[2] = w.kv == KV_INTERLEAVED ? w.kv_s_add : 0;
+      r.dst_stride[2] = w.kv == KV_INTERLEAVED ? w.kv_d_add : 0;
+      sink.put_nest(r);
+    } else {
+      for (u32 a = 0; a < c0; ++a)
+        for (u32 b = 0; b < c1; ++b) {
+          const u64 s1 = so + a * w.loops[0].s_stride + b * w.loops[1].s_stride;
+          const u64 d1 = dof + a * w.loops[0].d_stride + b * w.loops[1].d_stride;
+          for (u32 i = 0; i < n_tok; ++i) {
+            const u64 s2 = s1 + i * w.s.tok_stride, d2 = d1 + i * w.d.tok_stride;
+            sink.put(s2, d2, len);
+            if (w.kv == KV_INTERLEAVED) sink.put(s2 + w.kv_s_add, d2 + w.kv_d_add, len);
+          }
         }
-      }
+    }
     pos += k;
     rem -= k;
   }
   if (w.kv == KV_SECOND_PASS) {
-    const size_t last = sink.out->size();
+    const size_t last = sink.size();
     for (size_t i = first; i < last; ++i) {
-      const kvt_ipc_block k = (*sink.out)[i];
-      sink.put(k.src_offset + w.kv_s_add, k.dst_offset + w.kv_d_add,
-               w.pass_len ? w.pass_len : k.length);
+      if (sink.runs) {
+        kvt_run r = (*sink.runs)[i];
+        r.src_offset += w.kv_s_add;
+        r.dst_offset += w.kv_d_add;
+        if (w.pass_len) r.length = w.pass_len;
+        sink.put_nest(r);
+      } else {
+        const kvt_ipc_block k = (*sink.out)[i];
+        sink.put(k.src_offset + w.kv_s_add, k.dst_offset + w.kv_d_add,
+                 w.pass_len ? w.pass_len : k.length);
+      }
     }
   }
 }
@@ -1062,6 +1120,33 @@ void run_mla(const MlaOp& m, const kvt_task& t, const Groups& sg, const Groups& 
   }
 }
 
+int interpret(const kvt_parser& p, const kvt_task& task, kvt_block_lists* lists,
+              kvt_run_lists* runs) {
+  const Groups sg{task.src_blocks, task.src_group_len, task.n_src_groups};
+  const Groups dg{task.dst_blocks, task.dst_group_len, task.n_dst_groups};
+  const bool last = task.reach_last_token != 0;
+  if (p.deferred_error != KVT_OK) return fail(p.deferred_error, p.deferred_msg);
+  const size_t n_lists = lists ? lists->tensors.size() : runs->tensors.size();
+  for (const Op& op : p.ops) {
+    if (op.only_last && !last) continue;
+    if (op.bad_shape) throw RangeError("state shape metadata too short");
+    u32 tensor = 0;
+    if (op.kind == OP_WALK) tensor = op.walk.tensor;
+    if (tensor >= n_lists) throw RangeError("tensor index beyond the parser's list count");
+    Sink sink{lists ? &lists->tensors[tensor] : nullptr, p.caps[tensor],
+              runs ? &runs->tensors[tensor] : nullptr};
+    switch (op.kind) {
+      case OP_WALK: run_walk(op.walk, task, sg, dg, sink); break;
+      case OP_PAGES: run_pages(op.pages, task, sg, dg, sink); break;
+      case OP_STATE: run_state(op.state, sg, dg, sink); break;
+      case OP_GDN: run_gdn(op.gdn, sg, dg, sink); break;
+      case OP_FILL: run_fill(op.fill, task, sg, dg, sink); break;
+      case OP_MLA: run_mla(op.mla, task, sg, dg, sink); break;
+    }
+  }
+  return KVT_OK;
+}
+
 }  // namespace
 }  // namespace kvt
 
@@ -1131,28 +1216,16 @@ int kvt_parse_block(const kvt_parser* p, const kvt_task* task, kvt_block_lists* 
     if (!p || !task || !lists) return fail(KVT_ERR_INVALID, "kvt_parse_block: null argument");
     if (p->silent) return KVT_OK;
     if (lists->tensors.size() != p->n_lists) lists->tensors.resize(p->n_lists);
-    const Groups sg{task->src_blocks, task->src_group_len, task->n_src_groups};
-    const Groups dg{task->dst_blocks, task->dst_group_len, task->n_dst_groups};
-    const bool last = task->reach_last_token != 0;
-    if (p->deferred_error != KVT_OK) return fail(p->deferred_error, p->deferred_msg);
-    for (const Op& op : p->ops) {
-      if (op.only_last && !last) continue;
-      if (op.bad_shape) throw RangeError("state shape metadata too short");
-      u32 tensor = 0;
-      if (op.kind == OP_WALK) tensor = op.walk.tensor;
-      if (tensor >= lists->tensors.size())
-        throw RangeError("tensor index beyond the parser's list count");
-      Sink sink{&lists->tensors[tensor], p->caps[tensor]};
-      switch (op.kind) {
-        case OP_WALK: run_walk(op.walk, *task, sg, dg, sink); break;
-        case OP_PAGES: run_pages(op.pages, *task, sg, dg, sink); break;
-        case OP_STATE: run_state(op.state, sg, dg, sink); break;
-        case OP_GDN: run_gdn(op.gdn, sg, dg, sink); break;
-        case OP_FILL: run_fill(op.fill, *task, sg, dg, sink); break;
-        case OP_MLA: run_mla(op.mla, *task, sg, dg, sink); break;
-      }
-    }
-    return KVT_OK;
+    return interpret(*p, *task, lists, nullptr);
+  });
+}
+
+int kvt_parse_block_runs(const kvt_parser* p, const kvt_task* task, kvt_run_lists* lists) {
+  return guarded([&]() -> int {
+    if (!p || !task || !lists) return fail(KVT_ERR_INVALID, "kvt_parse_block_runs: null argument");
+    if (p->silent) return KVT_OK;
+    if (lists->tensors.size() != p->n_lists) lists->tensors.resize(p->n_lists);
+    return interpret(*p, *task, nullptr, lists);
   });
 }
 

@@ -108,6 +108,7 @@ uint64_t kvt_abi_sizeof(int which) {
     case 3: return sizeof(kvt_parse_opts);
     case 4: return sizeof(kvt_xform);
     case 5: return sizeof(kvt_wire_layout);
+    case 6: return sizeof(kvt_run);
     default: return 0;
   }
 }

@@ -176,6 +176,31 @@ TablePool& table_pool() {
 constexpr uint32_t kMinChunk = 4096, kMaxAutoChunk = 32768, kMaxChunk = 1u << 19;
 constexpr uint64_t kBlobAlign = 256;
 
+
+// One table entry before sorting.
+struct Piece {
+  uint64_t src, dst, packed;
+  uint32_t len;
+  uint16_t tensor, t0;
+  uint32_t shape;
+};
+
+// Every table entry is served by chunk_bytes / 4096 workgroups, of which only
+// ceil(len / 4096) have bytes to move. Takes the largest entry size (fewest table
+// entries) that leaves at most 2 % of the launched workgroups idle. `spans` holds
+// (bytes, repetitions) of the contiguous-on-the-packed-side spans to be cut.
+uint32_t pick_chunk_bytes(const std::vector<std::pair<uint64_t, uint64_t>>& spans) {
+  for (uint32_t cand = kMaxAutoChunk; cand > kMinChunk; cand /= 2) {
+    uint64_t launched = 0, useful = 0;
+    for (const auto& sp : spans) {
+      launched += sp.second * ((sp.first + cand - 1) / cand) * (cand / kMinChunk);
+      useful += sp.second * ((sp.first + kMinChunk - 1) / kMinChunk);
+    }
+    if (launched * 100 <= useful * 102) return cand;
+  }
+  return kMinChunk;
+}
+
 }  // namespace
 }  // namespace kvt
 
@@ -187,6 +212,7 @@ struct kvt_cache {
   std::vector<uint64_t> capacity;
   std::vector<void*> host_ptrs;
   uint8_t** dev_ptrs = nullptr;
+  bool aligned16 = true;  // every layer tensor starts on a 16-byte boundary
 };
 
 struct kvt_plan {
@@ -197,6 +223,10 @@ struct kvt_plan {
   uint64_t layer_bytes = 0;
   bool xform = false;
   XformDev xdev{};
+  bool strided = false;            // some chunks carry a record shape (kvt_plan_create_runs)
+  StrideTable shapes{};
+  uint64_t n_strided = 0;
+  std::vector<Chunk> host_table;   // device == KVT_DEVICE_NONE only: the tables, kept on the host
   uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
   Chunk* dev_chunks = nullptr;     // [0, n_chunks): pack order; [n_chunks, 2 n_chunks): unpack order
   TableBuf* buf = nullptr;         // storage of dev_chunks (recycled through the table pool)
@@ -224,6 +254,71 @@ struct kvt_stager {
   hipEvent_t fence = nullptr;
 };
 
+// Sorts the pieces into the two tables and starts their upload.
+static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
+  p->n_chunks = pieces.size();
+  if ((p->n_chunks << p->sub_shift) > 0x7FFFFFF0ull)
+    return fail(KVT_ERR_INVALID, "kvt_plan_create: too many chunks for one launch");
+
+  // Two tables, each walked in ascending cache address of its own direction
+  // (tensor-major: different tensors are different allocations).
+  std::vector<Chunk> table(2 * pieces.size());
+  std::vector<uint32_t> order;
+  std::vector<uint64_t> keys(pieces.size());
+  for (int dir = 0; dir < 2; ++dir) {
+    for (size_t i = 0; i < pieces.size(); ++i) {
+      const uint64_t off = dir == 0 ? pieces[i].src : pieces[i].dst;
+      if (off >> 56) return fail(KVT_ERR_INVALID, "kvt_plan_create: offset beyond 2^56");
+      keys[i] = (static_cast<uint64_t>(pieces[i].tensor) << 56) | off;
+    }
+    stable_order_by_key(keys, order);
+    for (size_t i = 0; i < order.size(); ++i) {
+      const Piece& q = pieces[order[i]];
+      Chunk& c = table[dir * pieces.size() + i];
+      c.cache = dir == 0 ? q.src : q.dst;
+      c.packed = q.packed;
+      c.len = q.len;
+      c.tensor = q.tensor;
+      c.t0 = q.t0;
+      c.shape = q.shape;
+      c.reserved = 0;
+    }
+  }
+
+  if (p->device == KVT_DEVICE_NONE) {
+    p->host_table.swap(table);
+    return KVT_OK;
+  }
+  DeviceGuard g;
+  if (int rc = g.enter(p->device)) return rc;
+  if (!table.empty()) {
+    // Asynchronous upload: fill the pinned twin, copy on the library's upload stream; the
+    // first launch that uses the plan waits for `uploaded` on its own stream.
+    const size_t bytes = table.size() * sizeof(Chunk);
+    if (int rc = table_pool().acquire(p->device, bytes, &p->buf)) return rc;
+    std::memcpy(p->buf->host, table.data(), bytes);
+    p->dev_chunks = static_cast<Chunk*>(p->buf->dev);
+    hipStream_t up = nullptr;
+    if (int rc = table_pool().upload_stream(p->device, &up)) {
+      table_pool().release(p->buf);
+      p->buf = nullptr;
+      return rc;
+    }
+    hipError_t e = hipEventCreateWithFlags(&p->uploaded, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipMemcpyAsync(p->buf->dev, p->buf->host, bytes, hipMemcpyHostToDevice, up);
+    if (e == hipSuccess) e = hipEventRecord(p->uploaded, up);
+    if (e != hipSuccess) {
+      (void)hipStreamSynchronize(up);
+      if (p->uploaded) (void)hipEventDestroy(p->uploaded);
+      p->uploaded = nullptr;
+      table_pool().release(p->buf);
+      p->buf = nullptr;
+      return hip_fail(e, "chunk table upload");
+    }
+  }
+  return KVT_OK;
+}
+
 extern "C" {
 
 int kvt_device_count(void) { return std::max(0, usable_devices()); }
@@ -249,7 +344,10 @@ int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, u
     c->n_tensors = n_tensors;
     c->capacity.assign(capacity, capacity + n_tensors);
     c->host_ptrs.resize(n);
-    for (uint64_t i = 0; i < n; ++i) c->host_ptrs[i] = const_cast<void*>(ptrs[i]);
+    for (uint64_t i = 0; i < n; ++i) {
+      c->host_ptrs[i] = const_cast<void*>(ptrs[i]);
+      if (reinterpret_cast<uintptr_t>(ptrs[i]) & 15u) c->aligned16 = false;
+    }
     KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c->dev_ptrs), n * sizeof(void*)));
     const hipError_t e =
         hipMemcpy(c->dev_ptrs, c->host_ptrs.data(), n * sizeof(void*), hipMemcpyHostToDevice);
@@ -278,7 +376,8 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       return fail(KVT_ERR_INVALID, "kvt_plan_create: null argument");
     if (lists->tensors.empty() || lists->tensors.size() > KVT_MAX_TENSORS)
       return fail(KVT_ERR_INVALID, "kvt_plan_create: tensor count out of range");
-    if (int rc = check_device(device)) return rc;
+    if (device != KVT_DEVICE_NONE)
+      if (int rc = check_device(device)) return rc;
     if (chunk_bytes != 0 && (chunk_bytes < kMinChunk || chunk_bytes > kMaxChunk ||
                              (chunk_bytes & (chunk_bytes - 1)) != 0))
       return fail(KVT_ERR_INVALID,
@@ -309,34 +408,17 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
     }
 
     if (chunk_bytes == 0) {
-      // Every table entry is served by chunk_bytes / 4096 workgroups, of which only
-      // ceil(len / 4096) have bytes to move. Take the largest entry size (fewest table
-      // entries) that leaves at most 2 % of the launched workgroups idle.
-      chunk_bytes = kMinChunk;
-      for (uint32_t cand = kMaxAutoChunk; cand > kMinChunk; cand /= 2) {
-        uint64_t launched = 0, useful = 0;
-        for (const RunList& runs : lists->tensors)
-          for (const kvt_ipc_block& r : runs) {
-            const uint64_t len = p->xform ? half : r.length;
-            const uint64_t reps = p->xform ? r.length / std::max<uint64_t>(half, 1) : 1;
-            launched += reps * ((len + cand - 1) / cand) * (cand / kMinChunk);
-            useful += reps * ((len + kMinChunk - 1) / kMinChunk);
-          }
-        if (launched * 100 <= useful * 102) {
-          chunk_bytes = cand;
-          break;
-        }
-      }
+      std::vector<std::pair<uint64_t, uint64_t>> spans;
+      for (const RunList& runs : lists->tensors)
+        for (const kvt_ipc_block& r : runs)
+          spans.emplace_back(p->xform ? half : r.length,
+                             p->xform ? r.length / std::max<uint64_t>(half, 1) : 1);
+      chunk_bytes = pick_chunk_bytes(spans);
     }
     if (p->xform)  // a chunk holds whole tokens
       while (chunk_bytes < tok_bytes) chunk_bytes *= 2;
     while ((kMinChunk << p->sub_shift) < chunk_bytes) ++p->sub_shift;
 
-    struct Piece {
-      uint64_t src, dst, packed;
-      uint32_t len;
-      uint16_t tensor, t0;
-    };
     std::vector<Piece> pieces;
     uint64_t cursor = 0;
     for (uint32_t t = 0; t < p->n_tensors; ++t) {
@@ -355,7 +437,7 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
           for (uint64_t o = 0; o < r.length; o += chunk_bytes)
             pieces.push_back(Piece{r.src_offset + o, r.dst_offset + o, blob + o,
                                    static_cast<uint32_t>(std::min<uint64_t>(chunk_bytes, r.length - o)),
-                                   static_cast<uint16_t>(t), 0});
+                                   static_cast<uint16_t>(t), 0, 0});
         } else {
           const uint64_t page = 2 * half;
           if (r.src_offset % page || r.dst_offset % page || r.length % page)
@@ -367,7 +449,7 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
               pieces.push_back(Piece{r.src_offset + o, r.dst_offset + o,
                                      blob + o + static_cast<uint64_t>(t0) * tok_bytes,
                                      static_cast<uint32_t>(nt * tok_bytes), 0,
-                                     static_cast<uint16_t>(t0)});
+                                     static_cast<uint16_t>(t0), 0});
             }
         }
         blob += r.length;
@@ -376,61 +458,178 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       cursor += blob;
     }
     p->layer_bytes = round_up(cursor, kBlobAlign);
-    p->n_chunks = pieces.size();
-    if ((p->n_chunks << p->sub_shift) > 0x7FFFFFF0ull)
-      return fail(KVT_ERR_INVALID, "kvt_plan_create: too many chunks for one launch");
-
-    // Two tables, each walked in ascending cache address of its own direction
-    // (tensor-major: different tensors are different allocations).
-    std::vector<Chunk> table(2 * pieces.size());
-    std::vector<uint32_t> order;
-    std::vector<uint64_t> keys(pieces.size());
-    for (int dir = 0; dir < 2; ++dir) {
-      for (size_t i = 0; i < pieces.size(); ++i) {
-        const uint64_t off = dir == 0 ? pieces[i].src : pieces[i].dst;
-        if (off >> 56) return fail(KVT_ERR_INVALID, "kvt_plan_create: offset beyond 2^56");
-        keys[i] = (static_cast<uint64_t>(pieces[i].tensor) << 56) | off;
-      }
-      stable_order_by_key(keys, order);
-      for (size_t i = 0; i < order.size(); ++i) {
-        const Piece& q = pieces[order[i]];
-        Chunk& c = table[dir * pieces.size() + i];
-        c.cache = dir == 0 ? q.src : q.dst;
-        c.packed = q.packed;
-        c.len = q.len;
-        c.tensor = q.tensor;
-        c.t0 = q.t0;
-        c.reserved = 0;
-      }
-    }
-
-    DeviceGuard g;
-    if (int rc = g.enter(device)) return rc;
-    if (!table.empty()) {
-      // Asynchronous upload: fill the pinned twin, copy on the library's upload stream; the
-      // first launch that uses the plan waits for `uploaded` on its own stream.
-      const size_t bytes = table.size() * sizeof(Chunk);
-      if (int rc = table_pool().acquire(device, bytes, &p->buf)) return rc;
-      std::memcpy(p->buf->host, table.data(), bytes);
-      p->dev_chunks = static_cast<Chunk*>(p->buf->dev);
-      hipStream_t up = nullptr;
-      if (int rc = table_pool().upload_stream(device, &up)) {
-        table_pool().release(p->buf);
-        return rc;
-      }
-      hipError_t e = hipEventCreateWithFlags(&p->uploaded, hipEventDisableTiming);
-      if (e == hipSuccess) e = hipMemcpyAsync(p->buf->dev, p->buf->host, bytes, hipMemcpyHostToDevice, up);
-      if (e == hipSuccess) e = hipEventRecord(p->uploaded, up);
-      if (e != hipSuccess) {
-        (void)hipStreamSynchronize(up);
-        if (p->uploaded) (void)hipEventDestroy(p->uploaded);
-        table_pool().release(p->buf);
-        return hip_fail(e, "chunk table upload");
-      }
-    }
+    if (int rc = finish_plan(p.get(), pieces)) return rc;
     *out = p.release();
     return KVT_OK;
   });
+}
+
+int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
+                         const uint64_t* dst_capacity, uint32_t chunk_bytes, kvt_plan** out) {
+  return guarded([&]() -> int {
+    if (!lists || !src_capacity || !dst_capacity || !out)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create_runs: null argument");
+    if (lists->tensors.empty() || lists->tensors.size() > KVT_MAX_TENSORS)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create_runs: tensor count out of range");
+    if (device != KVT_DEVICE_NONE)
+      if (int rc = check_device(device)) return rc;
+    if (chunk_bytes != 0 && (chunk_bytes < kMinChunk || chunk_bytes > kMaxChunk ||
+                             (chunk_bytes & (chunk_bytes - 1)) != 0))
+      return fail(KVT_ERR_INVALID,
+                  "kvt_plan_create_runs: chunk_bytes must be a power of two in [4096, 524288]");
+
+    std::unique_ptr<kvt_plan> p(new kvt_plan());
+    p->device = device;
+    p->n_tensors = static_cast<uint32_t>(lists->tensors.size());
+    p->src_cap.assign(src_capacity, src_capacity + p->n_tensors);
+    p->dst_cap.assign(dst_capacity, dst_capacity + p->n_tensors);
+
+    // A span is contiguous on the packed side: either one plain range, or the
+    // records of one outermost iteration of a run that stays strided.
+    struct Span {
+      uint64_t src, dst, packed, bytes;
+      uint32_t group;  // strided: bytes of one outer step (cut only there); 0 = plain
+      uint32_t shape;
+      uint64_t s_outer, d_outer;
+      uint16_t tensor;
+    };
+    std::vector<Span> spans;
+    uint32_t n_shapes = 0, max_group = 0;
+    uint64_t cursor = 0;
+    for (uint32_t t = 0; t < p->n_tensors; ++t) {
+      cursor = round_up(cursor, kBlobAlign);
+      p->tensor_offset.push_back(cursor);
+      uint64_t blob = 0;
+      const std::vector<kvt_run>& runs = lists->tensors[t];
+      for (size_t ri = 0; ri < runs.size(); ++ri) {
+        const kvt_run& r = runs[ri];
+        // bounds: offsets grow with every index, so the last range decides
+        uint64_t s_max = r.src_offset, d_max = r.dst_offset, count = 1;
+        bool bad = r.length == 0 || r.n[0] == 0 || r.n[1] == 0 || r.n[2] == 0;
+        for (int k = 0; k < 3 && !bad; ++k) {
+          uint64_t ds, dd;
+          bad = __builtin_mul_overflow(static_cast<uint64_t>(r.n[k] - 1), r.src_stride[k], &ds) ||
+                __builtin_add_overflow(s_max, ds, &s_max) ||
+                __builtin_mul_overflow(static_cast<uint64_t>(r.n[k] - 1), r.dst_stride[k], &dd) ||
+                __builtin_add_overflow(d_max, dd, &d_max) ||
+                __builtin_mul_overflow(count, static_cast<uint64_t>(r.n[k]), &count);
+        }
+        uint64_t total = 0;
+        bad = bad || __builtin_mul_overflow(count, r.length, &total) ||
+              s_max > p->src_cap[t] || r.length > p->src_cap[t] - s_max ||
+              d_max > p->dst_cap[t] || r.length > p->dst_cap[t] - d_max;
+        if (bad)
+          return fail(KVT_ERR_OUT_OF_RANGE, "kvt_plan_create_runs: run " + std::to_string(ri) +
+                                                " of tensor " + std::to_string(t) +
+                                                " exceeds the stated capacity");
+        // effective levels (n > 1), outermost first
+        int lv[3], n_lv = 0;
+        for (int k = 0; k < 3; ++k)
+          if (r.n[k] > 1) lv[n_lv++] = k;
+        bool strided = n_lv > 0 && r.length < kMinChunk && ((r.length | r.src_offset | r.dst_offset | blob) & 15u) == 0;
+        for (int k = 0; k < n_lv && strided; ++k)
+          strided = ((r.src_stride[lv[k]] | r.dst_stride[lv[k]]) & 15u) == 0;
+        // kernel nest: (outer, inner) = the last two effective levels; an earlier one is cut here
+        const int in_k = n_lv >= 2 ? lv[n_lv - 1] : -1;
+        const int out_k = n_lv >= 2 ? lv[n_lv - 2] : (n_lv == 1 ? lv[0] : -1);
+        const int top_k = n_lv == 3 ? lv[0] : -1;
+        const uint64_t n_in = in_k >= 0 ? r.n[in_k] : 1;
+        strided = strided && n_in * r.length <= kMaxChunk / 2;
+        uint32_t shape = 0;
+        if (strided) {
+          StrideShape sh{};
+          sh.vlen = static_cast<uint32_t>(r.length >> 4);
+          sh.inv_vlen = static_cast<uint32_t>((1ull << 32) / sh.vlen) + 1u;
+          sh.n_inner = static_cast<uint32_t>(n_in);
+          sh.outer[0] = r.src_stride[out_k];
+          sh.outer[1] = r.dst_stride[out_k];
+          sh.inner[0] = in_k >= 0 ? r.src_stride[in_k] : 0;
+          sh.inner[1] = in_k >= 0 ? r.dst_stride[in_k] : 0;
+          for (uint32_t i = 0; i < n_shapes && !shape; ++i)
+            if (std::memcmp(&p->shapes.shape[i], &sh, sizeof(sh)) == 0) shape = i + 1;
+          if (!shape && n_shapes < kMaxShapes) {
+            p->shapes.shape[n_shapes] = sh;
+            shape = ++n_shapes;
+          }
+          strided = shape != 0;  // shape table full: expand this run
+        }
+        if (strided) {
+          const uint32_t group = static_cast<uint32_t>(n_in * r.length);
+          max_group = std::max(max_group, group);
+          const uint64_t sub_bytes = static_cast<uint64_t>(r.n[out_k]) * group;
+          const uint32_t n_top = top_k >= 0 ? r.n[top_k] : 1;
+          for (uint32_t a = 0; a < n_top; ++a) {
+            spans.push_back(Span{r.src_offset + (top_k >= 0 ? a * r.src_stride[top_k] : 0),
+                                 r.dst_offset + (top_k >= 0 ? a * r.dst_stride[top_k] : 0), blob,
+                                 sub_bytes, group, shape, r.src_stride[out_k], r.dst_stride[out_k],
+                                 static_cast<uint16_t>(t)});
+            blob += sub_bytes;
+          }
+        } else {
+          for (uint32_t a = 0; a < r.n[0]; ++a)
+            for (uint32_t b = 0; b < r.n[1]; ++b)
+              for (uint32_t c = 0; c < r.n[2]; ++c) {
+                spans.push_back(Span{
+                    r.src_offset + a * r.src_stride[0] + b * r.src_stride[1] + c * r.src_stride[2],
+                    r.dst_offset + a * r.dst_stride[0] + b * r.dst_stride[1] + c * r.dst_stride[2],
+                    blob, r.length, 0, 0, 0, 0, static_cast<uint16_t>(t)});
+                blob += r.length;
+              }
+        }
+      }
+      p->tensor_bytes.push_back(blob);
+      cursor += blob;
+    }
+    p->layer_bytes = round_up(cursor, kBlobAlign);
+    p->strided = n_shapes > 0;
+
+    if (chunk_bytes == 0) {
+      std::vector<std::pair<uint64_t, uint64_t>> sized;
+      sized.reserve(spans.size());
+      for (const Span& sp : spans) sized.emplace_back(sp.bytes, 1);
+      chunk_bytes = pick_chunk_bytes(sized);
+    }
+    while (chunk_bytes < max_group) chunk_bytes *= 2;  // a chunk holds whole outer steps
+    while ((kMinChunk << p->sub_shift) < chunk_bytes) ++p->sub_shift;
+
+    std::vector<Piece> pieces;
+    for (const Span& sp : spans) {
+      if (sp.group == 0) {
+        for (uint64_t o = 0; o < sp.bytes; o += chunk_bytes)
+          pieces.push_back(Piece{sp.src + o, sp.dst + o, sp.packed + o,
+                                 static_cast<uint32_t>(std::min<uint64_t>(chunk_bytes, sp.bytes - o)),
+                                 sp.tensor, 0, 0});
+      } else {
+        const uint64_t steps_per = chunk_bytes / sp.group;
+        const uint64_t per = steps_per * sp.group;
+        for (uint64_t o = 0, step = 0; o < sp.bytes; o += per, step += steps_per) {
+          pieces.push_back(Piece{sp.src + step * sp.s_outer, sp.dst + step * sp.d_outer,
+                                 sp.packed + o,
+                                 static_cast<uint32_t>(std::min<uint64_t>(per, sp.bytes - o)),
+                                 sp.tensor, 0, sp.shape});
+          ++p->n_strided;
+        }
+      }
+    }
+    if (int rc = finish_plan(p.get(), pieces)) return rc;
+    *out = p.release();
+    return KVT_OK;
+  });
+}
+
+uint64_t kvt_plan_num_strided_chunks(const kvt_plan* p) { return p ? p->n_strided : 0; }
+
+int kvt_plan_host_tables(const kvt_plan* p, const void** chunks, uint64_t* n_chunks,
+                         uint32_t* chunk_bytes, const void** shapes) {
+  if (!p || !chunks || !n_chunks || !chunk_bytes || !shapes)
+    return fail(KVT_ERR_INVALID, "kvt_plan_host_tables: null argument");
+  if (p->device != KVT_DEVICE_NONE)
+    return fail(KVT_ERR_INVALID, "kvt_plan_host_tables: the plan lives on a device");
+  *chunks = p->host_table.data();
+  *n_chunks = p->n_chunks;
+  *chunk_bytes = kMinChunk << p->sub_shift;
+  *shapes = &p->shapes;
+  return KVT_OK;
 }
 
 void kvt_plan_destroy(kvt_plan* p) {
@@ -469,6 +668,7 @@ static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
                     const uint64_t* blob_offsets = nullptr) {
   if (!p || !cache || (!packed && p->n_chunks))
     return fail(KVT_ERR_INVALID, "kvt_pack/unpack: null argument");
+  if (p->device == KVT_DEVICE_NONE) return fail(KVT_ERR_INVALID, "a host-only plan cannot be launched");
   if (p->device != cache->device) return fail(KVT_ERR_INVALID, "plan and cache are on different devices");
   if (p->n_tensors != cache->n_tensors)
     return fail(KVT_ERR_INVALID, "plan and cache disagree on tensors per layer");
@@ -506,7 +706,20 @@ static int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
   }
   const Chunk* table = p->dev_chunks + (pack ? 0 : p->n_chunks);
   const uint32_t n = static_cast<uint32_t>(p->n_chunks);
+  if (p->strided) {
+    if ((reinterpret_cast<uintptr_t>(packed) | layer_stride) & 15u)
+      return fail(KVT_ERR_INVALID, "a strided plan needs a 16-byte aligned packed buffer and stride");
+    for (uint32_t t = 0; t < p->n_tensors; ++t)
+      if (blobs.off[t] & 15u)
+        return fail(KVT_ERR_INVALID, "a strided plan needs 16-byte aligned blob offsets");
+    if (!cache->aligned16)
+      return fail(KVT_ERR_INVALID, "a strided plan needs 16-byte aligned layer tensors");
+  }
   const hipError_t e =
+      p->strided ? launch_strided_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs,
+                                         p->n_tensors, first_layer, n_layers,
+                                         static_cast<uint8_t*>(packed), layer_stride, blobs,
+                                         p->shapes, s) :
       p->xform ? launch_xform_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                      first_layer, n_layers, static_cast<uint8_t*>(packed),
                                      layer_stride, blobs, p->xdev, s)

@@ -61,6 +61,18 @@ SIGNATURES = {
     "kvt_plan_layer_bytes": (_u64, [_vp]),
     "kvt_pack": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _vp]),
     "kvt_unpack": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _vp]),
+    "kvt_run_lists_create": (_int, [_P(_vp)]),
+    "kvt_run_lists_destroy": (None, [_vp]),
+    "kvt_run_lists_clear": (None, [_vp]),
+    "kvt_run_lists_num_tensors": (_u32, [_vp]),
+    "kvt_run_lists_view": (_int, [_vp, _u32, _P(_vp), _P(_u64)]),
+    "kvt_run_lists_totals": (_int, [_vp, _u32, _P(_u64), _P(_u64)]),
+    "kvt_parse_block_runs": (_int, [_vp, _P(Task), _vp]),
+    "kvt_run_lists_expand": (_int, [_vp, _vp]),
+    "kvt_run_lists_compress": (_int, [_vp, _vp]),
+    "kvt_plan_create_runs": (_int, [_int, _vp, _P(_u64), _P(_u64), _u32, _P(_vp)]),
+    "kvt_plan_num_strided_chunks": (_u64, [_vp]),
+    "kvt_plan_host_tables": (_int, [_vp, _P(_vp), _P(_u64), _P(_u32), _P(_vp)]),
     "kvt_pack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
     "kvt_unpack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
     "kvt_wire_layout_of": (_int, [_int, _vp, _P(WireLayout)]),
@@ -259,6 +271,62 @@ class BlockLists:
         return [self.tensor(t) for t in range(self.num_tensors())]
 
 
+class RunLists:
+    """Per-tensor lists of strided runs (kvt_run, 11 uint64 words each)."""
+
+    def __init__(self):
+        self.h = _vp()
+        check(lib().kvt_run_lists_create(C.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().kvt_run_lists_destroy(self.h)
+            self.h = _vp()
+
+    __del__ = close
+
+    def clear(self):
+        lib().kvt_run_lists_clear(self.h)
+
+    def num_tensors(self):
+        return lib().kvt_run_lists_num_tensors(self.h)
+
+    def tensor(self, t):
+        """-> structured copy of tensor t's runs"""
+        data, n = _vp(), _u64()
+        check(lib().kvt_run_lists_view(self.h, t, C.byref(data), C.byref(n)))
+        if n.value == 0:
+            return np.zeros(0, dtype=RUN_DTYPE)
+        buf = (C.c_uint8 * (n.value * RUN_DTYPE.itemsize)).from_address(data.value)
+        return np.frombuffer(buf, dtype=RUN_DTYPE).copy()
+
+    def totals(self, t):
+        """-> (ranges, bytes) the runs of tensor t expand to"""
+        a, b = _u64(), _u64()
+        check(lib().kvt_run_lists_totals(self.h, t, C.byref(a), C.byref(b)))
+        return a.value, b.value
+
+    def expand(self, lists=None):
+        lists = lists or BlockLists()
+        check(lib().kvt_run_lists_expand(self.h, lists.h))
+        return lists
+
+    @staticmethod
+    def compress(lists):
+        out = RunLists()
+        check(lib().kvt_run_lists_compress(lists.h, out.h))
+        return out
+
+
+CHUNK_DTYPE = np.dtype([("cache", "<u8"), ("packed", "<u8"), ("len", "<u4"), ("tensor", "<u2"),
+                        ("t0", "<u2"), ("shape", "<u4"), ("reserved", "<u4")])
+SHAPE_DTYPE = np.dtype([("vlen", "<u4"), ("inv_vlen", "<u4"), ("n_inner", "<u4"),
+                        ("reserved", "<u4"), ("outer", "<u8", 2), ("inner", "<u8", 2)])
+RUN_DTYPE = np.dtype([("src_offset", "<u8"), ("dst_offset", "<u8"), ("length", "<u8"),
+                      ("n", "<u4", 3), ("reserved0", "<u4"), ("src_stride", "<u8", 3),
+                      ("dst_stride", "<u8", 3)])
+
+
 class Parser:
     def __init__(self, parser_id, src, dst, valid, tp_size, tp_rank, fp8=False, pad=True):
         self.h = _vp()
@@ -276,6 +344,10 @@ class Parser:
     def parse(self, task_struct, lists):
         """Appends one task's ranges; returns the KVT_* code (0 = ok)."""
         return lib().kvt_parse_block(self.h, C.byref(task_struct), lists.h)
+
+    def parse_runs(self, task_struct, run_lists):
+        """Same ranges in run form (one run per block segment)."""
+        return lib().kvt_parse_block_runs(self.h, C.byref(task_struct), run_lists.h)
 
 
 def _ptr(x):
@@ -319,7 +391,31 @@ class Plan:
         if xform is not None:
             xf = C.byref(Xform(1, *xform))
         self.h = _vp()
+        if isinstance(lists, RunLists):
+            if xform is not None:
+                raise ValueError("no layout transform for a plan made from runs")
+            check(lib().kvt_plan_create_runs(device, lists.h, sc, dc, chunk_bytes,
+                                             C.byref(self.h)))
+            return
         check(lib().kvt_plan_create(device, lists.h, sc, dc, xf, chunk_bytes, C.byref(self.h)))
+
+    @property
+    def num_strided_chunks(self):
+        return lib().kvt_plan_num_strided_chunks(self.h)
+
+    def host_tables(self):
+        """Host-only plans (device=-1): -> (pack table, unpack table, chunk_bytes, shapes)."""
+        chunks, shapes, n, cb = _vp(), _vp(), _u64(), _u32()
+        check(lib().kvt_plan_host_tables(self.h, C.byref(chunks), C.byref(n), C.byref(cb),
+                                         C.byref(shapes)))
+        if n.value:
+            buf = (C.c_uint8 * (2 * n.value * CHUNK_DTYPE.itemsize)).from_address(chunks.value)
+            table = np.frombuffer(buf, dtype=CHUNK_DTYPE).copy()
+        else:
+            table = np.zeros(0, dtype=CHUNK_DTYPE)
+        sbuf = (C.c_uint8 * (16 * SHAPE_DTYPE.itemsize)).from_address(shapes.value)
+        return (table[:n.value], table[n.value:], cb.value,
+                np.frombuffer(sbuf, dtype=SHAPE_DTYPE).copy())
 
     def close(self):
         if self.h:

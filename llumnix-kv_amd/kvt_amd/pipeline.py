@@ -28,3 +28,24 @@ def build_plan(workload, device=0, chunk_bytes=0):
     plan = binding.Plan(device, lists, workload.capacities("src"), workload.capacities("dst"),
                         xform=workload.xform, chunk_bytes=chunk_bytes)
     return plan, lists
+
+
+def parse_batch_runs(cache_shape, src, dst, task_bufs, fp8=False, pad=True):
+    """-> (RunLists, tp_kind): the same ranges in closed form (one run per block segment).
+    Runs are never merged; for P==D use parse_batch()."""
+    valid, tp_size, tp_rank, parser_id, tp_kind = binding.select_parser(cache_shape, src, dst)
+    parser = binding.Parser(parser_id, src, dst, valid, tp_size, tp_rank, fp8=fp8, pad=pad)
+    runs = binding.RunLists()
+    for t in task_bufs:
+        binding.check(parser.parse_runs(t.struct, runs))
+    parser.close()
+    return runs, tp_kind
+
+
+def build_plan_runs(workload, device=0, chunk_bytes=0):
+    """Workload -> (Plan whose per-token arithmetic runs on the device, RunLists)."""
+    src, dst = workload.worker_infos()
+    runs, _ = parse_batch_runs(workload.cache_shape, src, dst, workload.task_bufs())
+    plan = binding.Plan(device, runs, workload.capacities("src"), workload.capacities("dst"),
+                        chunk_bytes=chunk_bytes)
+    return plan, runs

@@ -10,7 +10,7 @@ from dataclasses import dataclass, field
 import numpy as np
 
 from .ctypes_defs import (PARSER, SHAPE_DPSK_V32_SPARSE_MLA, SHAPE_FLASH, SHAPE_FLASHINFER,
-                          SHAPE_QWEN3_NEXT_FLASH, TaskBuf, make_worker_info)
+                          SHAPE_QWEN3_NEXT_FLASH, SHAPE_RAGGED_FLASH, TaskBuf, make_worker_info)
 
 
 @dataclass
@@ -154,6 +154,36 @@ def qwen3next_gdn(n_layers=36, slots=256, n_req=128, seed=20256):
     tasks = [[0, 1, True, [[int(s)]], [[int(d)]]] for s, d in zip(perm_s, perm_d)]
     return Workload("qwen3-next GDN state %dreq" % n_req, SHAPE_QWEN3_NEXT_FLASH, "HYBRID_PEQD",
                     n_layers, info, dict(info), tasks, elem_dtype="f32", seed=seed)
+
+
+def tp_split(layout="flash", p_tp=2, d_tp=1, rank=0, n_layers=32, src_pool=16384,
+             dst_pool=24576, n_req=64, min_tok=1024, max_tok=8192, total_heads=8, head_dim=128,
+             ntpb=16, seed=20257):
+    """A TP-remapping batch (prefill TP != decode TP): every token's K and V rows are split
+    between / gathered from several ranks, i.e. one short range per token (and per head for
+    the HND page layout). layout = "flash" ([2, nblk, bs, h, d]), "hnd" ([nblk, 2, h, bs, d])
+    or "ragged" ([nblk, bs, 2, h, d], the only one with a P<D parser); bf16. `rank` is the sending rank when p_tp > d_tp, the receiving rank otherwise."""
+    rng = np.random.default_rng(seed)
+    row = head_dim * 2
+    pT = 2 * (total_heads // p_tp) * row
+    dT = 2 * (total_heads // d_tp) * row
+    lens = rng.integers(min_tok, max_tok + 1, size=n_req)
+    src, dst = _tables(rng, n_req, lens, ntpb, src_pool, dst_pool)
+    gn = max(p_tp, d_tp) // min(p_tp, d_tp)
+    p_rank, d_rank = (rank, rank // gn) if p_tp > d_tp else (rank // gn, rank)
+    s_info = dict(block_sizes=[pT * ntpb], token_sizes=[pT], layer_num_blocks=src_pool, tp=p_tp,
+                  rank=p_rank, num_kv_heads=total_heads, num_layers=n_layers)
+    d_info = dict(block_sizes=[dT * ntpb], token_sizes=[dT], layer_num_blocks=dst_pool, tp=d_tp,
+                  rank=d_rank, num_kv_heads=total_heads, num_layers=n_layers)
+    tasks = [[0, int(n), True, [s], [d]] for n, s, d in zip(lens, src, dst)]
+    kind = "PGTD" if p_tp > d_tp else "PLTD"
+    shape, fam = {"flash": (SHAPE_FLASH, "FLASH"), "hnd": (SHAPE_FLASHINFER, "FLASHINFER"),
+                  "ragged": (SHAPE_RAGGED_FLASH, "RAGGED")}[layout]
+    if kind == "PLTD" and layout != "ragged":
+        raise ValueError("the reference has a P<D parser only for the ragged layout")
+    return Workload("%s TP%d->TP%d %dreq x %d-%d tok" % (layout, p_tp, d_tp, n_req, min_tok, max_tok),
+                    shape, "%s_%s" % (fam, kind), n_layers, s_info, d_info, tasks, seed=seed,
+                    notes=dict(tokens=int(lens.sum())))
 
 
 def parser_id(w):

@@ -1,0 +1,137 @@
+"""GPU parity of plans built from strided runs (the per-token / per-head offset
+arithmetic of the TP-remapping parsers evaluated inside the copy kernel) against
+the CPU oracle's pack / unpack of the oracle's own per-token range lists.
+Bit-exact. Needs a real MI355X."""
+import numpy as np
+import pytest
+
+import cases
+import checkers
+import kvt_amd
+from kvt_amd import pipeline, workloads
+from test_gpu_pack import _dev_bytes, _host, _make_caches
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _oracle_ranges(w):
+    src, dst = w.worker_infos()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, src, dst)
+    assert rc == 0 and kind != 0          # never merged
+    rc, outs = checkers.oracle_parse(pid, src, dst, valid, tps, tpr, w.task_bufs())
+    assert rc == 0
+    return outs
+
+
+def _check(w, plan, o_lists, seed, expect_strided):
+    if expect_strided is not None:
+        assert (plan.num_strided_chunks > 0) == expect_strided
+    src_layers = _make_caches(w, "src", seed)
+    dst_layers = _make_caches(w, "dst", seed + 1, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, w.n_layers, packed, stride)
+    torch.cuda.synchronize()
+    packed_h = _host(packed)
+    for l in range(w.n_layers):
+        for t in range(w.n_tensors):
+            blob = checkers.oracle_pack(_host(src_layers[l][t]), o_lists[t])
+            off = l * stride + plan.tensor_offset(t)
+            assert plan.tensor_bytes(t) == len(blob)
+            assert np.array_equal(packed_h[off:off + len(blob)], blob), (l, t)
+    plan.unpack(dc, 0, w.n_layers, packed, stride)
+    torch.cuda.synchronize()
+    for l in range(w.n_layers):
+        for t in range(w.n_tensors):
+            exp = np.full(w.capacities("dst")[t], 0xA5, dtype=np.uint8)
+            off = l * stride + plan.tensor_offset(t)
+            checkers.oracle_unpack(exp, o_lists[t], packed_h[off:off + plan.tensor_bytes(t)])
+            assert np.array_equal(_host(dst_layers[l][t]), exp), (l, t)
+
+
+SPLITS = [("flash", 2, 1, 1, True), ("flash", 4, 1, 2, True), ("ragged", 1, 2, 1, True),
+          ("ragged", 4, 2, 3, True), ("ragged", 1, 4, 0, True), ("hnd", 2, 1, 1, None)]   # hnd: whole-segment head rows (plain), short tails strided
+
+
+@pytest.mark.parametrize("layout,p_tp,d_tp,rank,strided", SPLITS)
+@pytest.mark.parametrize("chunk", [0, 4096, 65536])
+def test_tp_split_batches_through_a_run_plan(layout, p_tp, d_tp, rank, strided, chunk):
+    w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=3, src_pool=300, dst_pool=400,
+                           n_req=5, min_tok=30, max_tok=900)
+    plan, runs = pipeline.build_plan_runs(w, 0, chunk)
+    o_lists = _oracle_ranges(w)
+    assert np.array_equal(runs.expand().tensor(0), o_lists[0])
+    assert len(runs.tensor(0)) < len(o_lists[0])
+    _check(w, plan, o_lists, 51, strided)
+
+
+def test_receiver_compresses_plain_ranges_then_unpacks_strided():
+    w = workloads.tp_split("flash", 2, 1, 0, n_layers=2, src_pool=200, dst_pool=300, n_req=4,
+                           min_tok=100, max_tok=700)
+    o_lists = _oracle_ranges(w)
+    lists = kvt_amd.BlockLists()
+    lists.append(0, o_lists[0])                      # as taken off a layer message
+    runs = kvt_amd.RunLists.compress(lists)
+    plan = kvt_amd.Plan(0, runs, w.capacities("src"), w.capacities("dst"))
+    _check(w, plan, o_lists, 61, True)
+    plain = kvt_amd.Plan(0, lists, w.capacities("src"), w.capacities("dst"))
+    assert plan.layer_bytes == plain.layer_bytes and plan.num_chunks * 3 < plain.num_chunks
+
+
+PER_TOKEN = ["RAGGED_PGTD", "RAGGED_PLTD", "FLASH_PGTD", "DPSK_PGTD", "DPSK_PLTD",
+             "FLASHINFER_PGTD", "HYBRID_PGTD", "HYBRID_PLTD", "HYBRID_FI_PGTD", "HYBRID_FI_PLTD",
+             "KDA_PGTD", "KIMI_K3_PLTD", "TURBOQUANT_PGTD"]
+
+
+@pytest.mark.parametrize("parser", PER_TOKEN)
+def test_pack_of_random_cases_of_every_remapping_parser(parser):
+    """Gather only: the random cases may repeat destination blocks."""
+    done = 0
+    for seed in range(900, 1100):
+        case = cases.gen_case(parser, seed)
+        pid, src, dst, valid, tps, tpr, tasks = cases.materialise(case)
+        rc, outs = checkers.oracle_parse(pid, src, dst, valid, tps, tpr, tasks)
+        if rc != 0 or not any(len(o) for o in outs) or any(len(o) == 0 for o in outs):
+            continue
+        parser_h = kvt_amd.Parser(pid, src, dst, valid, tps, tpr)
+        runs = kvt_amd.RunLists()
+        for t in tasks:
+            assert parser_h.parse_runs(t.struct, runs) == 0
+        n_t = runs.num_tensors()
+        s_cap = [int(src.block_sizes[t]) * int(src.layer_num_blocks) for t in range(n_t)]
+        d_cap = [int(dst.block_sizes[t]) * int(dst.layer_num_blocks) for t in range(n_t)]
+        plan = kvt_amd.Plan(0, runs, s_cap, d_cap)
+        layers = [[_dev_bytes((c + 3) // 4 * 4, seed * 10 + t, "u8") for t, c in enumerate(s_cap)]]
+        cache = kvt_amd.Cache(0, layers, s_cap)
+        packed = torch.zeros(max(plan.layer_bytes, 16), dtype=torch.uint8, device="cuda")
+        plan.pack(cache, 0, 1, packed, plan.layer_bytes)
+        torch.cuda.synchronize()
+        packed_h = _host(packed)
+        for t in range(n_t):
+            blob = checkers.oracle_pack(_host(layers[0][t]), outs[t])
+            off = plan.tensor_offset(t)
+            assert np.array_equal(packed_h[off:off + len(blob)], blob), (case["name"], t)
+        done += 1
+        if done == 12:
+            break
+    assert done >= 4
+
+
+def test_strided_plan_refuses_misaligned_blob_positions():
+    w = workloads.tp_split("flash", 2, 1, 0, n_layers=1, src_pool=64, dst_pool=64, n_req=1,
+                           min_tok=100, max_tok=100)
+    plan, _ = pipeline.build_plan_runs(w, 0)
+    assert plan.num_strided_chunks > 0
+    layers = _make_caches(w, "src", 5)
+    sc = kvt_amd.Cache(0, layers, w.capacities("src"))
+    out = torch.zeros(plan.layer_bytes + 64, dtype=torch.uint8, device="cuda")
+    with pytest.raises(kvt_amd.KvtError):
+        plan.pack_at(sc, 0, 1, out, 0, [4] + [0] * 7)
+    plan.pack_at(sc, 0, 1, out, 0, [32] + [0] * 7)
+    torch.cuda.synchronize()
+    blob = checkers.oracle_pack(_host(layers[0][0]), _oracle_ranges(w)[0])
+    assert np.array_equal(_host(out)[32:32 + len(blob)], blob)

@@ -1,0 +1,182 @@
+"""Copy-plan tables checked without a GPU: a host-only plan (device = -1)
+exposes the two chunk tables the kernels walk; a numpy emulation of the kernels'
+addressing (same formulas as csrc/kvt_kernels.hip, with bounds asserted on
+every access) must reproduce the CPU oracle's pack / unpack. Guards the table
+builder -- above all that no entry can make a kernel touch memory outside the
+registered tensors or the packed layer."""
+import numpy as np
+import pytest
+
+import cases
+import checkers
+import kvt_amd
+from kvt_amd import pipeline, workloads
+
+
+def emulate(table, chunk_bytes, shapes, caches, tensor_offset, packed, pack):
+    side = 0 if pack else 1
+    touched = [np.zeros(len(c), dtype=bool) for c in caches]
+    for c in table:
+        n = int(c["len"])
+        t = int(c["tensor"])
+        assert 0 < n <= chunk_bytes
+        pk0 = tensor_offset[t] + int(c["packed"])
+        assert pk0 + n <= len(packed)
+        if c["shape"] == 0:
+            idx = int(c["cache"]) + np.arange(n, dtype=np.int64)
+        else:
+            s = shapes[int(c["shape"]) - 1]
+            vlen, inv, n_inner = int(s["vlen"]), int(s["inv_vlen"]), int(s["n_inner"])
+            assert n % 16 == 0 and vlen > 0 and n_inner > 0
+            assert int(c["cache"]) % 16 == 0 and pk0 % 16 == 0
+            v = np.arange(n // 16, dtype=np.uint64)
+            rec = v if vlen == 1 else (v * np.uint64(inv)) >> np.uint64(32)   # __umulhi
+            assert np.array_equal(rec, v // np.uint64(vlen))                   # the reciprocal is exact
+            col = v - rec * np.uint64(vlen)
+            o, i = rec // np.uint64(n_inner), rec % np.uint64(n_inner)
+            at = (o * np.uint64(int(s["outer"][side])) + i * np.uint64(int(s["inner"][side]))
+                  + col * np.uint64(16)).astype(np.int64) + int(c["cache"])
+            assert (at % 16 == 0).all()
+            idx = (at[:, None] + np.arange(16, dtype=np.int64)[None, :]).reshape(-1)
+        assert idx.min() >= 0 and idx.max() < len(caches[t]), "access outside the cache tensor"
+        if pack:
+            packed[pk0:pk0 + n] = caches[t][idx]
+        else:
+            assert not touched[t][idx].any(), "two table entries write the same bytes"
+            touched[t][idx] = True
+            caches[t][idx] = packed[pk0:pk0 + n]
+
+
+def _host_plan(lists_or_runs, s_cap, d_cap, chunk):
+    return kvt_amd.Plan(-1, lists_or_runs, s_cap, d_cap, chunk_bytes=chunk)
+
+
+def _check_tables(plan, o_lists, s_cap, d_cap, seed, unpack=True):
+    pack_t, unpack_t, cb, shapes = plan.host_tables()
+    n_t = len(o_lists)
+    rng = np.random.default_rng(seed)
+    src = [rng.integers(0, 256, c, dtype=np.uint8) for c in s_cap]
+    offs = [plan.tensor_offset(t) for t in range(n_t)]
+    packed = np.zeros(plan.layer_bytes, dtype=np.uint8)
+    emulate(pack_t, cb, shapes, src, offs, packed, True)
+    for t in range(n_t):
+        blob = checkers.oracle_pack(src[t], o_lists[t])
+        assert plan.tensor_bytes(t) == len(blob)
+        assert np.array_equal(packed[offs[t]:offs[t] + len(blob)], blob), t
+    # both tables hold the same entries up to order
+    assert sorted(pack_t["packed"].tolist()) == sorted(unpack_t["packed"].tolist())
+    for t in range(n_t):           # each table ascends in its own cache offset, tensor-major
+        for tab in (pack_t, unpack_t):
+            sel = tab[tab["tensor"] == t]["cache"]
+            assert (np.diff(sel.astype(np.int64)) >= 0).all()
+    if unpack:
+        dst = [np.full(c, 0xA5, dtype=np.uint8) for c in d_cap]
+        emulate(unpack_t, cb, shapes, dst, offs, packed, False)
+        for t in range(n_t):
+            exp = np.full(d_cap[t], 0xA5, dtype=np.uint8)
+            checkers.oracle_unpack(exp, o_lists[t], packed[offs[t]:offs[t] + plan.tensor_bytes(t)])
+            assert np.array_equal(dst[t], exp), t
+
+
+def _oracle_ranges(w):
+    src, dst = w.worker_infos()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, src, dst)
+    rc, outs = checkers.oracle_parse(pid, src, dst, valid, tps, tpr, w.task_bufs())
+    assert rc == 0
+    if kind == 0:
+        outs = [checkers.oracle_merge(o)[0] for o in outs]
+    return outs
+
+
+@pytest.mark.parametrize("chunk", [0, 4096, 16384, 524288])
+@pytest.mark.parametrize("layout,p_tp,d_tp,rank", [("flash", 2, 1, 1), ("flash", 4, 1, 2),
+                                                   ("ragged", 1, 2, 1), ("ragged", 4, 2, 3),
+                                                   ("ragged", 1, 4, 0), ("hnd", 2, 1, 1)])
+def test_run_plan_tables_for_tp_split_batches(layout, p_tp, d_tp, rank, chunk):
+    w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=1, src_pool=40, dst_pool=60,
+                           n_req=4, min_tok=5, max_tok=150, total_heads=4, head_dim=32)
+    src, dst = w.worker_infos()
+    runs, _ = pipeline.parse_batch_runs(w.cache_shape, src, dst, w.task_bufs())
+    plan = _host_plan(runs, w.capacities("src"), w.capacities("dst"), chunk)
+    assert plan.num_strided_chunks > 0       # (the short head rows make "hnd" strided here too)
+    _check_tables(plan, _oracle_ranges(w), w.capacities("src"), w.capacities("dst"), 7)
+
+
+@pytest.mark.parametrize("parser", cases.ALL_PARSERS)
+def test_run_plan_tables_for_random_cases_of_every_parser(parser):
+    done = 0
+    for seed in range(1200, 1320):
+        case = cases.gen_case(parser, seed)
+        pid, src, dst, valid, tps, tpr, tasks = cases.materialise(case)
+        rc, outs = checkers.oracle_parse(pid, src, dst, valid, tps, tpr, tasks)
+        if rc != 0 or not outs or any(len(o) == 0 for o in outs):
+            continue
+        parser_h = kvt_amd.Parser(pid, src, dst, valid, tps, tpr)
+        runs = kvt_amd.RunLists()
+        for t in tasks:
+            assert parser_h.parse_runs(t.struct, runs) == 0
+        n_t = runs.num_tensors()
+        s_cap = [int(src.block_sizes[t]) * int(src.layer_num_blocks) for t in range(n_t)]
+        d_cap = [int(dst.block_sizes[t]) * int(dst.layer_num_blocks) for t in range(n_t)]
+        if max(s_cap + d_cap) > (64 << 20):
+            continue
+        plan = _host_plan(runs, s_cap, d_cap, [0, 4096, 32768][seed % 3])
+        # the random cases may repeat destination blocks: gather only
+        _check_tables(plan, outs, s_cap, d_cap, seed, unpack=False)
+        # compressed plain lists give a second, independently built table
+        lists = kvt_amd.BlockLists()
+        for t, o in enumerate(outs):
+            lists.append(t, o)
+        plan2 = _host_plan(kvt_amd.RunLists.compress(lists), s_cap, d_cap, 0)
+        _check_tables(plan2, outs, s_cap, d_cap, seed, unpack=False)
+        done += 1
+    assert done >= 10
+
+
+@pytest.mark.parametrize("chunk", [0, 4096, 65536])
+def test_plain_plan_tables_for_merged_batches(chunk):
+    for w in (workloads.llama8b_batch(n_layers=1, src_pool=64, dst_pool=96, n_req=5, min_tok=10,
+                                      max_tok=200),
+              workloads.deepseek_mla(n_layers=1, pool=48, n_req=3, tokens=700)):
+        src, dst = w.worker_infos()
+        lists, _ = pipeline.parse_batch(w.cache_shape, src, dst, w.task_bufs())
+        plan = _host_plan(lists, w.capacities("src"), w.capacities("dst"), chunk)
+        assert plan.num_strided_chunks == 0
+        _check_tables(plan, _oracle_ranges(w), w.capacities("src"), w.capacities("dst"), 9)
+
+
+def test_hand_made_runs_three_levels_and_fallbacks():
+    R = kvt_amd.RunLists()
+    B = kvt_amd.BlockLists()
+    rows = []
+    # heads x tokens x (K,V): 3 x 5 x 2 records of 32 bytes
+    for h in range(3):
+        for tok in range(5):
+            for kv in range(2):
+                rows.append((64 + h * 2048 + tok * 64 + kv * 1024, 128 + h * 4096 + tok * 256 + kv * 128, 32))
+    rows += [(8192, 16384, 8000)]                       # long plain range
+    rows += [(20001 + 48 * i, 30000 + 100 * i, 20) for i in range(6)]   # misaligned: expanded
+    B.append(0, rows)
+    R = kvt_amd.RunLists.compress(B)
+    assert R.tensor(0)[0]["n"].tolist() == [3, 5, 2]
+    cap = [1 << 16]
+    for chunk in (0, 4096, 8192):
+        plan = _host_plan(R, cap, cap, chunk)
+        assert plan.num_strided_chunks == 3             # one per head
+        _check_tables(plan, [np.asarray(rows, np.uint64)], cap, cap, 3)
+
+
+def test_run_plan_rejects_runs_beyond_capacity():
+    B = kvt_amd.BlockLists()
+    B.append(0, [(0 + 64 * i, 0 + 64 * i, 32) for i in range(8)])
+    R = kvt_amd.RunLists.compress(B)
+    assert len(R.tensor(0)) == 1
+    kvt_amd.Plan(-1, R, [480], [480]).close()
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.Plan(-1, R, [479], [480])
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.Plan(-1, R, [480], [479])
+    with pytest.raises(kvt_amd.KvtError):              # a host-only plan cannot be launched
+        kvt_amd.lib().kvt_pack.restype
+        p = kvt_amd.Plan(-1, R, [480], [480])
+        kvt_amd.binding.check(kvt_amd.lib().kvt_pack(p.h, None, 0, 1, None, 0, None))
