@@ -57,6 +57,14 @@ def build_workload(cfg, scale):
                                  pool=max(512, int(36864 * scale)), n_req=max(2, int(128 * scale))),
                 W.qwen3next_gdn(n_layers=max(2, int(36 * scale)), slots=max(4, int(256 * scale)),
                                 n_req=max(2, int(128 * scale)))]
+    if cfg in (6, 7):
+        # TP-remapping batches (not among the baseline configurations): config 2's batch with
+        # the sender on TP2 and the receiver on TP1 (6), or TP1 -> TP2 on the ragged layout (7)
+        layout, p_tp, d_tp = ("flash", 2, 1) if cfg == 6 else ("ragged", 1, 2)
+        return [W.tp_split(layout, p_tp, d_tp, 0, n_layers=max(2, int(32 * scale)),
+                           src_pool=max(1024, int(16384 * scale)),
+                           dst_pool=max(1536, int(24576 * scale)), n_req=max(2, int(64 * scale)),
+                           min_tok=max(64, int(1024 * scale)), max_tok=max(128, int(8192 * scale)))]
     raise SystemExit("unknown --config %r" % cfg)
 
 
@@ -105,6 +113,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, help="BASELINE.json configs[] index + 1")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")
     ap.add_argument("--chunk-bytes", type=int, default=0)
+    ap.add_argument("--plan", choices=["ranges", "runs"], default="ranges",
+                    help="runs: ParseBlock in closed form (strided runs), the per-token offset "
+                         "arithmetic done by the copy kernel")
     ap.add_argument("--cpu-layers", type=int, default=4, help="layers in the CPU baseline sample")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
@@ -153,6 +164,10 @@ def main():
     def prepare(i):
         """host part of a step for workload i: ParseBlock + merge + plan upload"""
         w = wls[i]
+        if args.plan == "runs":
+            runs, _ = pipeline.parse_batch_runs(w.cache_shape, infos[i][0], infos[i][1], tasks[i])
+            return kvt.Plan(0, runs, w.capacities("src"), w.capacities("dst"),
+                            chunk_bytes=args.chunk_bytes), runs
         lists, _ = pipeline.parse_batch(w.cache_shape, infos[i][0], infos[i][1], tasks[i])
         plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
                         chunk_bytes=args.chunk_bytes)
@@ -240,15 +255,18 @@ def main():
         "config": {"workload": "; ".join(w.name for w in wls), "baseline_config": args.config,
                    "scale": args.scale, "layers": [w.n_layers for w in wls],
                    "requests": [len(w.tasks) for w in wls], "payload_bytes_per_step": P,
-                   "chunk_bytes": args.chunk_bytes or 32768},
+                   "chunk_bytes": args.chunk_bytes or "auto", "plan": args.plan,
+                   "table_entries_per_layer": [p.num_chunks for p, _ in first]},
         "frac_hbm_peak": round(value * 1e9 / HBM_PEAK, 4),
         "pack_ms": round(pack_avg, 4),
         "unpack_ms": round(unpack_avg, 4),
         "pack_gbps": round(achieved, 1),
         "unpack_gbps": round(2.0 * P / (unpack_avg * 1e-3) / 1e9, 1),
         "host_parse_plan_ms": round(statistics.mean(host_ms), 4),
-        "roofline": {"bound": "hbm", "kernel": "copy_chunks_kernel<pack>" if not wls[0].xform
-                     else "xform_chunks_kernel<pack>",
+        "roofline": {"bound": "hbm",
+                     "kernel": "strided_chunks_kernel<pack>" if first[0][0].num_strided_chunks
+                     else ("copy_chunks_kernel<pack>" if not wls[0].xform
+                           else "xform_chunks_kernel<pack>"),
                      "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                      "traffic": MEASURED_PACK_TRAFFIC.get((args.config, args.scale,
