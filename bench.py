@@ -116,6 +116,9 @@ def main():
     ap.add_argument("--plan", choices=["ranges", "runs"], default="ranges",
                     help="runs: ParseBlock in closed form (strided runs), the per-token offset "
                          "arithmetic done by the copy kernel")
+    ap.add_argument("--sequential", action="store_true",
+                    help="config 5 only: pack everything, then unpack everything, instead of the "
+                         "mixed mode (half of the requests packing while the other half unpacks)")
     ap.add_argument("--cpu-layers", type=int, default=4, help="layers in the CPU baseline sample")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
@@ -152,11 +155,26 @@ def main():
                           "gbps_read_plus_write": round(2 * n / dt / 1e9, 1)}))
         return
 
-    wls = build_workload(args.config, args.scale)
+    full_wls = build_workload(args.config, args.scale)
     t_init = time.time()
-    sides = [DeviceSide(torch, kvt, w, 7 + i) for i, w in enumerate(wls)]
+    full_sides = [DeviceSide(torch, kvt, w, 7 + i) for i, w in enumerate(full_wls)]
     torch.cuda.synchronize()
     log("caches resident in %.1fs" % (time.time() - t_init))
+    mixed = args.config == 5 and not args.sequential
+    if mixed:
+        # halves A and B of every workload's requests, on the same caches; a step is
+        # (pack A || unpack B) then (pack B || unpack A): every request still goes both ways
+        import dataclasses
+        wls, sides = [], []
+        for half in (0, 1):
+            for w, sd in zip(full_wls, full_sides):
+                h = len(w.tasks) // 2
+                part = w.tasks[:h] if half == 0 else w.tasks[h:]
+                wls.append(dataclasses.replace(w, tasks=part, name=w.name + " [half %s]" % "AB"[half]))
+                sides.append(sd)
+        n_half = len(full_wls)
+    else:
+        wls, sides = full_wls, full_sides
 
     infos = [w.worker_infos() for w in wls]
     tasks = [w.task_bufs() for w in wls]
@@ -191,7 +209,42 @@ def main():
         assert lib.kvt_event_create(C.byref(e)) == 0, lib.kvt_last_error()
         return e
 
+    s2 = torch.cuda.Stream()
+    sh2 = s2.cuda_stream
+
+    def launch_mixed(plans, evs):
+        def go(i, pack, stream_handle):
+            plan = plans[i][0]
+            fn = plan.pack if pack else plan.unpack
+            fn(sides[i].src_cache if pack else sides[i].dst_cache, 0, wls[i].n_layers, packed[i],
+               strides[i], stream_handle)
+        A, B = range(0, n_half), range(n_half, 2 * n_half)
+        lib.kvt_event_record(evs[0], sh)
+        start = torch.cuda.Event()
+        start.record(stream)
+        s2.wait_event(start)
+        for i in A:
+            go(i, True, sh)            # pack A          | stream 1
+        for i in B:
+            go(i, False, sh2)          # unpack B        | stream 2 (B was packed by the previous step)
+        a_packed, b_unpacked = torch.cuda.Event(), torch.cuda.Event()
+        a_packed.record(stream)
+        b_unpacked.record(s2)
+        lib.kvt_event_record(evs[1], sh)
+        stream.wait_event(b_unpacked)  # pack B overwrites what unpack B read
+        s2.wait_event(a_packed)        # unpack A needs pack A
+        for i in B:
+            go(i, True, sh)
+        for i in A:
+            go(i, False, sh2)
+        done2 = torch.cuda.Event()
+        done2.record(s2)
+        stream.wait_event(done2)
+        lib.kvt_event_record(evs[2], sh)
+
     def launch(plans, evs):
+        if mixed:
+            return launch_mixed(plans, evs)
         lib.kvt_event_record(evs[0], sh)
         for i, (plan, _) in enumerate(plans):
             plan.pack(sides[i].src_cache, 0, wls[i].n_layers, packed[i], strides[i], sh)
@@ -200,6 +253,9 @@ def main():
             plan.unpack(sides[i].dst_cache, 0, wls[i].n_layers, packed[i], strides[i], sh)
         lib.kvt_event_record(evs[2], sh)
 
+    if mixed:   # the first mixed step unpacks half B: give it packed data
+        for i in range(n_half, 2 * n_half):
+            first[i][0].pack(sides[i].src_cache, 0, wls[i].n_layers, packed[i], strides[i], sh)
     keep = [first]
     plans = first
     for _ in range(args.warmup):
@@ -236,6 +292,9 @@ def main():
     pack_avg, unpack_avg = statistics.mean(pack_ms), statistics.mean(unpack_ms)
     value = 4.0 * P / (ms_per_step * 1e-3) / 1e9
     achieved = 2.0 * P / (pack_avg * 1e-3) / 1e9
+    if mixed:   # the two event intervals are the two phases; both directions run in each
+        pack_avg = unpack_avg = (pack_avg + unpack_avg) / 2
+        achieved = 2.0 * P / (pack_avg * 1e-3) / 1e9
     log("pack %.3f ms  unpack %.3f ms  host %.3f ms/step  wall %.3f ms/step" %
         (pack_avg, unpack_avg, statistics.mean(host_ms), ms_per_step))
 
@@ -263,6 +322,8 @@ def main():
         "pack_gbps": round(achieved, 1),
         "unpack_gbps": round(2.0 * P / (unpack_avg * 1e-3) / 1e9, 1),
         "host_parse_plan_ms": round(statistics.mean(host_ms), 4),
+        "mode": ("mixed: (pack A || unpack B) then (pack B || unpack A) on two streams; pack_ms = "
+                 "unpack_ms = mean phase time") if mixed else "sequential: pack all, then unpack all",
         "roofline": {"bound": "hbm",
                      "kernel": "strided_chunks_kernel<pack>" if first[0][0].num_strided_chunks
                      else ("copy_chunks_kernel<pack>" if not wls[0].xform
@@ -276,9 +337,10 @@ def main():
     # ---------------------------------------------------------------- parity spot check + CPU leg
     if not args.skip_cpu:
         import checkers
-        w, side = wls[0], sides[0]
+        w, side = full_wls[0], full_sides[0]      # (mixed mode: both halves of the requests)
         L = max(1, min(args.cpu_layers, w.n_layers))
-        s_info, d_info = infos[0]
+        s_info, d_info = w.worker_infos()
+        cpu_tasks = w.task_bufs()
         rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, s_info, d_info)
         assert rc == 0
         olib = checkers.oracle()
@@ -290,7 +352,7 @@ def main():
 
         def cpu_pass():
             t_a = time.perf_counter()
-            rc, outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, tasks[0])
+            rc, outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
             assert rc == 0
             if kind == 0:
                 outs = [checkers.oracle_merge(o)[0] for o in outs]
@@ -313,7 +375,7 @@ def main():
         outs, blobs = reps[-1][1], reps[-1][2]
         parity = True
         if w.xform is None:
-            for l in range(L):
+            for l in range(L if not mixed else 0):   # (mixed: the packed buffers are per half)
                 for t in range(w.n_tensors):
                     off = l * stride + plan0.tensor_offset(t)
                     parity &= bool(np.array_equal(gpu_packed[off:off + len(blobs[l][t])],
@@ -371,11 +433,46 @@ def main():
         out["latency_p50_us"] = round(statistics.median(lat), 2)
         out["latency_note"] = "per request: one pack launch covering all %d layers, GPU time" % w.n_layers
 
+        # the reference-shaped launchers (one launch per layer, ranges as three int64 arrays
+        # resident on the device) and the converting bf16 -> fp8 gather
+        if w.xform is None and args.plan == "ranges" and w.elem_dtype == "bf16":
+            runs0 = first[0][1].tensor(0).astype(np.int64)
+            so = torch.from_numpy(np.ascontiguousarray(runs0[:, 0])).cuda()
+            ln = torch.from_numpy(np.ascontiguousarray(runs0[:, 2])).cuda()
+            do = torch.from_numpy(np.concatenate([[0], np.cumsum(runs0[:, 2])[:-1]])).cuda()
+            ln_e = ln // 2
+            do_e = do // 2
+            nb = int(runs0[:, 2].sum())
+            a, b = new_event(), new_event()
+            res = {}
+            for name, fn, offs, lens, moved in (
+                    ("launch_copy_d2h_direct", lib.kvt_launch_copy_d2h_direct, do, ln, 2 * nb),
+                    ("launch_copy_d2h_bf16_to_fp8", lib.kvt_launch_copy_d2h_bf16_to_fp8, do_e,
+                     ln_e, nb + nb // 2)):
+                for rep in range(2):
+                    lib.kvt_event_record(a, sh)
+                    for l in range(w.n_layers):
+                        rc = fn(side.src[l][0].data_ptr(), packed[0].data_ptr() + l * strides[0],
+                                so.data_ptr(), offs.data_ptr(), lens.data_ptr(), len(runs0), 0, 0,
+                                sh)
+                        assert rc == 0, lib.kvt_last_error()
+                    lib.kvt_event_record(b, sh)
+                lib.kvt_event_synchronize(b)
+                res[name + "_gbps"] = round(moved * w.n_layers / (ev_ms(lib, a, b) * 1e-3) / 1e9, 1)
+            res["note"] = ("%d launches of %d ranges each; GB/s = bytes read + bytes written; the "
+                           "fp8 gather reads 2 bytes and writes 1 per element" %
+                           (w.n_layers, len(runs0)))
+            out["reference_shaped_launchers"] = res
+
         # pinned-host staging of packed layers, double buffered against the pack kernel
+        # Small layers are grouped so that one transfer is at least 256 MiB (a copy has a fixed
+        # start-up cost of some tens of microseconds; config 1's layers are 2 MiB).
         plan = first[0][0]
-        nbytes = plan.layer_bytes
-        Ls = min(w.n_layers, 8)
-        if nbytes > 0 and nbytes < (3 << 30):
+        lbytes = plan.layer_bytes
+        if 0 < lbytes < (3 << 30):
+            group = max(1, min(w.n_layers, -(-(256 << 20) // lbytes)))
+            n_groups = max(1, min(8, w.n_layers // group))
+            nbytes = group * lbytes
             ceil = {}
             for name, d in (("d2h", 1), ("h2d", 0)):
                 r = C.c_double()
@@ -384,34 +481,39 @@ def main():
             stg = kvt.Stager(0, nbytes, 2)
             bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
             ps = torch.cuda.Stream()
-            for phase in ("warm", "timed"):
+            d2h_t, h2d_t = [], []
+            for phase in range(4):          # first phase warms up
                 torch.cuda.synchronize()
                 a = time.perf_counter()
-                for l in range(Ls):
-                    slot = l % 2
-                    if l >= 2:
+                for g in range(n_groups):
+                    slot = g % 2
+                    if g >= 2:
                         stg.wait(slot)
-                    plan.pack(side.src_cache, l, 1, bufs[slot], nbytes, ps.cuda_stream)
+                    plan.pack(side.src_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
                     stg.save(slot, bufs[slot], nbytes, ps.cuda_stream)
                 stg.wait(0)
-                stg.wait(1)
-                d2h_s = time.perf_counter() - a
-            for phase in ("warm", "timed"):
+                if n_groups > 1:
+                    stg.wait(1)
+                d2h_t.append(time.perf_counter() - a)
+            for phase in range(4):
                 torch.cuda.synchronize()
                 a = time.perf_counter()
-                for l in range(Ls):
-                    slot = l % 2
+                for g in range(n_groups):
+                    slot = g % 2
                     stg.load(slot, bufs[slot], nbytes, ps.cuda_stream)
-                    plan.unpack(side.dst_cache, l, 1, bufs[slot], nbytes, ps.cuda_stream)
+                    plan.unpack(side.dst_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
                 ps.synchronize()
-                h2d_s = time.perf_counter() - a
-            pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * Ls
+                h2d_t.append(time.perf_counter() - a)
+            d2h_s, h2d_s = statistics.median(d2h_t[1:]), statistics.median(h2d_t[1:])
+            pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * group * n_groups
             out["staging"] = {
                 "save_gbps": round(pay / d2h_s / 1e9, 2), "load_gbps": round(pay / h2d_s / 1e9, 2),
                 "pcie_d2h_gbps": round(ceil["d2h"] / 1e9, 2), "pcie_h2d_gbps": round(ceil["h2d"] / 1e9, 2),
                 "save_frac_of_pcie": round(pay / d2h_s / ceil["d2h"], 4),
                 "load_frac_of_pcie": round(pay / h2d_s / ceil["h2d"], 4),
-                "sample": "%d layers x %.1f MiB through 2 pinned slots" % (Ls, nbytes / 2**20),
+                "sample": "%d transfers of %d layer(s) = %.1f MiB each through 2 pinned slots, "
+                          "pack / unpack of the group in one launch; median of 3 passes" %
+                          (n_groups, group, nbytes / 2**20),
             }
             stg.close()
 

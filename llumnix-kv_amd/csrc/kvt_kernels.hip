@@ -178,30 +178,31 @@ __global__ __launch_bounds__(kThreads) void copy_ranges_kernel(
 
 // bf16 -> fp8 E4M3 (OCP "fn" variant: no infinities, 0x7F = NaN), round to
 // nearest even, finite values and infinities saturate to +-448 (0x7E), NaN
-// stays NaN. Integer-only so that every bit pattern is reproducible.
-__device__ __forceinline__ uint32_t bf16_to_e4m3(uint32_t bits) {
-  const uint32_t sign = (bits >> 8) & 0x80u;
-  const uint32_t e = (bits >> 7) & 0xFFu;
-  const uint32_t m = bits & 0x7Fu;
-  if (e == 0xFFu) return sign | (m ? 0x7Fu : 0x7Eu);
-  // below 2^-10, half of the smallest subnormal 2^-9 (the tie at 2^-10 itself goes to even = 0 below)
-  if (e < 117u) return sign;
-  const uint32_t sig = 0x80u | m;  // 1.mmmmmmm, value = sig * 2^(e - 134)
-  const bool normal = e >= 121u;   // >= 2^-6: keep 1+3 bits; else subnormal in units of 2^-9
-  const uint32_t shift = normal ? 4u : 125u - e;
-  const uint32_t base = normal ? ((e - 121u) << 3) : 0u;  // exponent field minus the leading one in q
-  uint32_t q = sig >> shift;
-  const uint32_t rem = sig & ((1u << shift) - 1u);
-  const uint32_t half = 1u << (shift - 1u);
-  q += (rem > half || (rem == half && (q & 1u))) ? 1u : 0u;
-  uint32_t code = base + q;
-  code = code > 0x7Eu ? 0x7Eu : code;
-  return sign | code;
+// stays NaN (sign kept). `pair` holds two bf16; the two fp8 bytes go to the low
+// (HIGH = false) or high half of `acc`. The matrix-core conversion instruction
+// of gfx950 rounds exactly like the integer definition (checked for all 65 536
+// bit patterns by the tests); its overflow result depends on a mode bit, so the
+// operands are clamped to +-448 first, and NaNs, which the clamp would turn
+// into 448, are patched afterwards.
+template <bool HIGH>
+__device__ __forceinline__ uint32_t bf16x2_to_e4m3(uint32_t pair, uint32_t acc) {
+  const float a = __uint_as_float(pair << 16);
+  const float b = __uint_as_float(pair & 0xFFFF0000u);
+  uint32_t r = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(a, -448.0f, 448.0f),
+                                               __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f), acc, HIGH);
+  constexpr uint32_t sh = HIGH ? 16u : 0u;
+  if (a != a) r = (r & ~(0xFFu << sh)) | ((((pair >> 8) & 0x80u) | 0x7Fu) << sh);
+  if (b != b) r = (r & ~(0xFF00u << sh)) | ((((pair >> 24) & 0x80u) | 0x7Fu) << (sh + 8u));
+  return r;
 }
 
 __device__ __forceinline__ uint32_t cvt4(uint32_t lo, uint32_t hi) {
-  return bf16_to_e4m3(lo & 0xFFFFu) | (bf16_to_e4m3(lo >> 16) << 8) |
-         (bf16_to_e4m3(hi & 0xFFFFu) << 16) | (bf16_to_e4m3(hi >> 16) << 24);
+  return bf16x2_to_e4m3<true>(hi, bf16x2_to_e4m3<false>(lo, 0u));
+}
+
+// One element (stragglers of a range).
+__device__ __forceinline__ uint32_t bf16_to_e4m3(uint32_t bits) {
+  return bf16x2_to_e4m3<false>(bits & 0xFFFFu, 0u) & 0xFFu;
 }
 
 // Converting gather: range i = lens[i] bf16 elements at src_base + src_off[i]
