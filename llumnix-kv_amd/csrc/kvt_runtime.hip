@@ -260,30 +260,33 @@ static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
   if ((p->n_chunks << p->sub_shift) > 0x7FFFFFF0ull)
     return fail(KVT_ERR_INVALID, "kvt_plan_create: too many chunks for one launch");
 
-  // Two tables, each walked in ascending cache address of its own direction
-  // (tensor-major: different tensors are different allocations).
+  // Two tables. What matters most to HBM throughput is that the WRITES of a launch
+  // ascend: the unpack table is sorted by destination offset (tensor-major: different
+  // tensors are different allocations); the pack table keeps generation order, which is
+  // ascending packed offset (for a merged list that is ascending source offset as well).
+  // Measured on MI355X: pack of an unmerged batch 5.88 -> 6.27 TB/s against sorting the
+  // pack table by source offset; unpack +6 % against leaving it unsorted.
   std::vector<Chunk> table(2 * pieces.size());
+  auto fill = [](Chunk& c, const Piece& q, uint64_t cache) {
+    c.cache = cache;
+    c.packed = q.packed;
+    c.len = q.len;
+    c.tensor = q.tensor;
+    c.t0 = q.t0;
+    c.shape = q.shape;
+    c.reserved = 0;
+  };
   std::vector<uint32_t> order;
   std::vector<uint64_t> keys(pieces.size());
-  for (int dir = 0; dir < 2; ++dir) {
-    for (size_t i = 0; i < pieces.size(); ++i) {
-      const uint64_t off = dir == 0 ? pieces[i].src : pieces[i].dst;
-      if (off >> 56) return fail(KVT_ERR_INVALID, "kvt_plan_create: offset beyond 2^56");
-      keys[i] = (static_cast<uint64_t>(pieces[i].tensor) << 56) | off;
-    }
-    stable_order_by_key(keys, order);
-    for (size_t i = 0; i < order.size(); ++i) {
-      const Piece& q = pieces[order[i]];
-      Chunk& c = table[dir * pieces.size() + i];
-      c.cache = dir == 0 ? q.src : q.dst;
-      c.packed = q.packed;
-      c.len = q.len;
-      c.tensor = q.tensor;
-      c.t0 = q.t0;
-      c.shape = q.shape;
-      c.reserved = 0;
-    }
+  for (size_t i = 0; i < pieces.size(); ++i) {
+    if ((pieces[i].src | pieces[i].dst) >> 56)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create: offset beyond 2^56");
+    fill(table[i], pieces[i], pieces[i].src);
+    keys[i] = (static_cast<uint64_t>(pieces[i].tensor) << 56) | pieces[i].dst;
   }
+  stable_order_by_key(keys, order);
+  for (size_t i = 0; i < order.size(); ++i)
+    fill(table[pieces.size() + i], pieces[order[i]], pieces[order[i]].dst);
 
   if (p->device == KVT_DEVICE_NONE) {
     p->host_table.swap(table);

@@ -65,10 +65,11 @@ def _check_tables(plan, o_lists, s_cap, d_cap, seed, unpack=True):
         assert np.array_equal(packed[offs[t]:offs[t] + len(blob)], blob), t
     # both tables hold the same entries up to order
     assert sorted(pack_t["packed"].tolist()) == sorted(unpack_t["packed"].tolist())
-    for t in range(n_t):           # each table ascends in its own cache offset, tensor-major
-        for tab in (pack_t, unpack_t):
-            sel = tab[tab["tensor"] == t]["cache"]
-            assert (np.diff(sel.astype(np.int64)) >= 0).all()
+    for t in range(n_t):   # writes ascend: packed offset in the pack table, destination in the other
+        sel = pack_t[pack_t["tensor"] == t]["packed"]
+        assert (np.diff(sel.astype(np.int64)) > 0).all()
+        sel = unpack_t[unpack_t["tensor"] == t]["cache"]
+        assert (np.diff(sel.astype(np.int64)) >= 0).all()
     if unpack:
         dst = [np.full(c, 0xA5, dtype=np.uint8) for c in d_cap]
         emulate(unpack_t, cb, shapes, dst, offs, packed, False)
