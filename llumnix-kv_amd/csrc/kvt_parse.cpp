@@ -531,6 +531,8 @@ struct Builder {
             u32 d_kb, u64 d_seg_bytes, u64 d_tok_stride, u64 unit, u64 d_base, u64 d_half,
             u32 heads, u64 d_head_stride) {
     need(d_blk_tok > 0 && s_kb > 0 && d_kb > 0, "tokens per block must be positive");
+    // the fills emit one record per token of a block
+    need(d_blk_tok <= (1u << 16), "more than 65536 tokens per block");
     FillOp& f = push(OP_FILL, true).fill;
     f.kind = kind;
     f.group = group;
@@ -965,6 +967,9 @@ void run_state(const StateOp& st, const Groups& sg, const Groups& dg, Sink& sink
 }
 
 void run_gdn(const GdnOp& g, const Groups& sg, const Groups& dg, Sink& sink) {
+  // conv rows = convolution width - 1 (a handful); the trip count below comes straight from
+  // caller metadata, so refuse values that can only be garbage instead of spinning on them
+  if (g.rows > (1u << 16)) throw RangeError("state shape metadata implausible: conv rows");
   for (u32 grp = 0; grp < g.n_groups; ++grp) {
     const u32 *sid, *did;
     u64 sn, dn;
@@ -982,6 +987,11 @@ void run_gdn(const GdnOp& g, const Groups& sg, const Groups& dg, Sink& sink) {
 }
 
 void zero_run(Sink& sink, u64 zero_src, u64 dof, u64 len, u64 max_piece) {
+  // A fill is cut into pieces no longer than the (all-zero) source page. Real geometries need
+  // a handful of pieces; a page of a few bytes against a huge fill is malformed metadata and
+  // would otherwise emit billions of ranges.
+  if (max_piece == 0 || len / max_piece > (1u << 20))
+    throw RangeError("zero fill: source page too small for the range to fill");
   for (u64 done = 0; done < len;) {
     const u64 n = std::min(max_piece, len - done);
     sink.put(zero_src, dof + done, n);
@@ -1165,6 +1175,13 @@ int kvt_parser_create(int parser_id, const kvt_worker_info* src, const kvt_worke
       return fail(KVT_ERR_INVALID, "kvt_parser_create: worker_tp_rank beyond MAX_TP_SIZE");
     if (parser_id < 0 || parser_id >= KVT_PARSER_COUNT)
       return fail(KVT_ERR_UNSUPPORTED, "kvt_parser_create: unknown parser id");
+    if (src->engine_tp_size == 0 || dst->engine_tp_size == 0)
+      return fail(KVT_ERR_INVALID, "kvt_parser_create: engine_tp_size must be positive");
+    if (src->n_conv_state_shape > KVT_MAX_SHAPE_DIMS || src->n_ssm_state_shape > KVT_MAX_SHAPE_DIMS ||
+        src->n_ple_conv_state_shape > KVT_MAX_SHAPE_DIMS ||
+        src->n_gdn_conv_channel_dims > KVT_MAX_CHANNEL_DIMS ||
+        src->n_ple_conv_channel_dims > KVT_MAX_CHANNEL_DIMS)
+      return fail(KVT_ERR_INVALID, "kvt_parser_create: shape metadata count beyond the array size");
     std::unique_ptr<kvt_parser> p(new kvt_parser());
     kvt_parse_opts o{0, 1};
     if (opts) o = *opts;
