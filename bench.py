@@ -24,8 +24,10 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 
 # HBM bytes moved by ONE pack launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (each counter scaled by what it reads for the plain copy kernel of known size); see
-# profiles/copy_chunks_kernel_config2_hbm_traffic.md. Keyed by (config, scale, chunk_bytes).
-MEASURED_PACK_TRAFFIC = {(2, 1.0, 0): 70.966e9}
+# profiles/copy_chunks_kernel_config2_hbm_traffic.md and
+# profiles/strided_and_xform_kernels_hbm_traffic.md. Keyed by (config, scale, chunk_bytes, plan).
+MEASURED_PACK_TRAFFIC = {(2, 1.0, 0, "ranges"): 70.966e9, (3, 1.0, 0, "ranges"): 85.892e9,
+                         (6, 1.0, 0, "runs"): 40.879e9}
 
 
 def log(*a):
@@ -331,7 +333,7 @@ def main():
                      "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                      "traffic": MEASURED_PACK_TRAFFIC.get((args.config, args.scale,
-                                                           args.chunk_bytes))},
+                                                           args.chunk_bytes, args.plan))},
     }
 
     # ---------------------------------------------------------------- parity spot check + CPU leg
