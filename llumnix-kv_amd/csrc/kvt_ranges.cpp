@@ -32,20 +32,31 @@ void stable_order_by_key(const std::vector<uint64_t>& keys, std::vector<uint32_t
   const uint64_t varying = all_or ^ all_and;  // bits that differ somewhere
   constexpr int kBits = 11;
   constexpr size_t kBuckets = size_t(1) << kBits;
-  std::vector<uint32_t> tmp(n);
-  std::vector<uint32_t> count(kBuckets);
+  // (key, index) pairs move together, so every pass streams through memory; the scratch
+  // arrays are kept per thread (a plan is built per batch: no fresh pages every time)
+  static thread_local std::vector<uint64_t> ka, kb;
+  static thread_local std::vector<uint32_t> ib;
+  ka.assign(keys.begin(), keys.end());
+  kb.resize(n);
+  ib.resize(n);
+  uint32_t count[kBuckets];
   for (int shift = 0; shift < 64; shift += kBits) {
     if (((varying >> shift) & (kBuckets - 1)) == 0) continue;
-    std::fill(count.begin(), count.end(), 0u);
-    for (size_t i = 0; i < n; ++i) ++count[(keys[order[i]] >> shift) & (kBuckets - 1)];
+    std::fill(count, count + kBuckets, 0u);
+    for (size_t i = 0; i < n; ++i) ++count[(ka[i] >> shift) & (kBuckets - 1)];
     uint32_t run = 0;
-    for (size_t b = 0; b < kBuckets; ++b) {
-      const uint32_t c = count[b];
-      count[b] = run;
+    for (size_t k = 0; k < kBuckets; ++k) {
+      const uint32_t c = count[k];
+      count[k] = run;
       run += c;
     }
-    for (size_t i = 0; i < n; ++i) tmp[count[(keys[order[i]] >> shift) & (kBuckets - 1)]++] = order[i];
-    order.swap(tmp);
+    for (size_t i = 0; i < n; ++i) {
+      const uint32_t at = count[(ka[i] >> shift) & (kBuckets - 1)]++;
+      kb[at] = ka[i];
+      ib[at] = order[i];
+    }
+    ka.swap(kb);
+    order.swap(ib);
   }
 }
 
@@ -54,16 +65,18 @@ void stable_order_by_key(const std::vector<uint64_t>& keys, std::vector<uint32_t
 static void merge_runs(RunList& v, uint64_t stats[4]) {
   if (v.size() > 0xFFFFFFF0ull) throw InvalidError("range list too long");
   {
-    std::vector<uint64_t> keys(v.size());
+    static thread_local std::vector<uint64_t> keys;
+    static thread_local std::vector<uint32_t> order;
+    static thread_local RunList sorted;
+    keys.resize(v.size());
     for (size_t i = 0; i < v.size(); ++i) keys[i] = v[i].src_offset;
-    std::vector<uint32_t> order;
     stable_order_by_key(keys, order);
     bool identity = true;
     for (size_t i = 0; i < order.size() && identity; ++i) identity = order[i] == i;
     if (!identity) {
-      RunList sorted(v.size());
+      sorted.resize(v.size());
       for (size_t i = 0; i < v.size(); ++i) sorted[i] = v[order[i]];
-      v.swap(sorted);
+      v.swap(sorted);   // the caller's old storage becomes next call's scratch
     }
   }
   size_t w = 0;  // index of the run being grown

@@ -266,7 +266,6 @@ static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
   // ascending packed offset (for a merged list that is ascending source offset as well).
   // Measured on MI355X: pack of an unmerged batch 5.88 -> 6.27 TB/s against sorting the
   // pack table by source offset; unpack +6 % against leaving it unsorted.
-  std::vector<Chunk> table(2 * pieces.size());
   auto fill = [](Chunk& c, const Piece& q, uint64_t cache) {
     c.cache = cache;
     c.packed = q.packed;
@@ -276,30 +275,35 @@ static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
     c.shape = q.shape;
     c.reserved = 0;
   };
-  std::vector<uint32_t> order;
-  std::vector<uint64_t> keys(pieces.size());
-  for (size_t i = 0; i < pieces.size(); ++i) {
+  static thread_local std::vector<uint32_t> order;
+  static thread_local std::vector<uint64_t> keys;
+  const size_t n = pieces.size();
+  keys.resize(n);
+  for (size_t i = 0; i < n; ++i) {
     if ((pieces[i].src | pieces[i].dst) >> 56)
       return fail(KVT_ERR_INVALID, "kvt_plan_create: offset beyond 2^56");
-    fill(table[i], pieces[i], pieces[i].src);
     keys[i] = (static_cast<uint64_t>(pieces[i].tensor) << 56) | pieces[i].dst;
   }
   stable_order_by_key(keys, order);
-  for (size_t i = 0; i < order.size(); ++i)
-    fill(table[pieces.size() + i], pieces[order[i]], pieces[order[i]].dst);
+  auto build = [&](Chunk* table) {
+    for (size_t i = 0; i < n; ++i) fill(table[i], pieces[i], pieces[i].src);
+    for (size_t i = 0; i < n; ++i) fill(table[n + i], pieces[order[i]], pieces[order[i]].dst);
+  };
 
   if (p->device == KVT_DEVICE_NONE) {
-    p->host_table.swap(table);
+    p->host_table.resize(2 * n);
+    build(p->host_table.data());
     return KVT_OK;
   }
   DeviceGuard g;
   if (int rc = g.enter(p->device)) return rc;
-  if (!table.empty()) {
-    // Asynchronous upload: fill the pinned twin, copy on the library's upload stream; the
-    // first launch that uses the plan waits for `uploaded` on its own stream.
-    const size_t bytes = table.size() * sizeof(Chunk);
+  if (n != 0) {
+    // Asynchronous upload: the tables are written straight into the pinned twin and copied
+    // on the library's upload stream; the first launch that uses the plan waits for
+    // `uploaded` on its own stream.
+    const size_t bytes = 2 * n * sizeof(Chunk);
     if (int rc = table_pool().acquire(p->device, bytes, &p->buf)) return rc;
-    std::memcpy(p->buf->host, table.data(), bytes);
+    build(static_cast<Chunk*>(p->buf->host));
     p->dev_chunks = static_cast<Chunk*>(p->buf->dev);
     hipStream_t up = nullptr;
     if (int rc = table_pool().upload_stream(p->device, &up)) {
@@ -422,7 +426,10 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       while (chunk_bytes < tok_bytes) chunk_bytes *= 2;
     while ((kMinChunk << p->sub_shift) < chunk_bytes) ++p->sub_shift;
 
-    std::vector<Piece> pieces;
+    // scratch kept per thread: a plan is built per batch, fresh pages every time would cost
+    // more than filling them
+    static thread_local std::vector<Piece> pieces;
+    pieces.clear();
     uint64_t cursor = 0;
     for (uint32_t t = 0; t < p->n_tensors; ++t) {
       cursor = round_up(cursor, kBlobAlign);
@@ -595,7 +602,10 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
     while (chunk_bytes < max_group) chunk_bytes *= 2;  // a chunk holds whole outer steps
     while ((kMinChunk << p->sub_shift) < chunk_bytes) ++p->sub_shift;
 
-    std::vector<Piece> pieces;
+    // scratch kept per thread: a plan is built per batch, fresh pages every time would cost
+    // more than filling them
+    static thread_local std::vector<Piece> pieces;
+    pieces.clear();
     for (const Span& sp : spans) {
       if (sp.group == 0) {
         for (uint64_t o = 0; o < sp.bytes; o += chunk_bytes)
