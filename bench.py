@@ -7,7 +7,8 @@ ONE unpack launch (all layers). Inputs (caches, block tables) are resident
 before the timed region. Steps are issued the way a serving loop issues them:
 the host prepares step k+1 while the GPU still runs step k.
 
-Prints one JSON line; see DESIGN.md for the meaning of every field.
+Prints one JSON line: the whole-job rate plus `roofline` (dominant kernel against the HBM
+peak) and `cpu_baseline` (the CPU oracle on a bounded sample of the same batch).
 """
 import argparse
 import ctypes as C
@@ -130,7 +131,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         raise SystemExit("bench.py: this build measures ONE MI355X; the path has no inter-GPU "
-                         "part, so --gpus N with N > 1 is not supported (see DESIGN.md, sharding).")
+                         "part, so --gpus N with N > 1 is not supported.")
 
     import numpy as np
     import torch

@@ -25,6 +25,11 @@
 //     textbook permutation in numpy (einsum/transpose) and round trip.
 //   * bf16->fp8: all 65536 bit patterns against torch's float8_e4m3fn cast
 //     (finite values) and the saturating rule of the reference kernel.
+//   * PARITY UNPINNED: parsing with pad_last_attn_block = 0 (no zero fill of the
+//     last destination block). The reference reads that switch through a helper
+//     that maps "0" to the default 1 (kvtransfer/src/envcfg.cpp:13-25), so the
+//     compiled reference cannot produce such vectors; the branch is restated from
+//     the source text only.
 #include <algorithm>
 #include <atomic>
 #include <cstdint>
