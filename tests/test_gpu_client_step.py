@@ -1,0 +1,82 @@
+"""The reference's end-to-end test of this path, replayed on the library:
+KVTransferClientTest.TestKernelSyncAndDataTransfer
+(kvtransfer/tests/client_step_test.cu:103-206). Two layers of 128 blocks x 16 KiB
+are produced by kernels on a compute stream, each followed by an event; one
+request (64 tokens, source blocks 0..3 -> destination blocks 4..7) is sent
+layer by layer through a channel into *host* layers; every destination block of
+layer 0 must sum to 10 x block_size and of layer 1 to 20 x block_size. The
+reference plugs in a FakeChannel that copies range by range; here the channel is
+kvt_amd.channel.LoopbackChannel (one pack + one unpack launch per layer, gated
+on the layer's event on a side stream). Needs a real MI355X."""
+import numpy as np
+import pytest
+
+import kvt_amd
+from kvt_amd import pipeline
+from kvt_amd.channel import LoopbackChannel
+from kvt_amd.ctypes_defs import SHAPE_RAGGED_FLASH, TaskBuf, make_worker_info
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+KB = 1024
+
+
+def test_kernel_sync_and_data_transfer():
+    num_layers, block_size, nblk = 2, 16 * KB, 128
+    data_size = nblk * block_size
+    stream = torch.cuda.Stream()
+    layers = [torch.zeros(data_size, dtype=torch.uint8, device="cuda") for _ in range(num_layers)]
+    host_layers = [torch.zeros(data_size, dtype=torch.uint8, pin_memory=True)
+                   for _ in range(num_layers)]
+    info = dict(block_sizes=[block_size], token_sizes=[KB], layer_num_blocks=nblk, tp=1, rank=0,
+                num_layers=num_layers)
+    src_info, dst_info = make_worker_info(**info), make_worker_info(**info)
+    dst_blocks = [4, 5, 6, 7]
+    # submit_req_send("0", 0, REQ, seen=0, new=16*4, last=true, {{0,1,2,3}}, dst_blocks)
+    task = TaskBuf(0, 16 * 4, True, [[0, 1, 2, 3]], [dst_blocks])
+    lists, tp_kind = pipeline.parse_batch(SHAPE_RAGGED_FLASH, src_info, dst_info, [task])
+
+    src_cache = kvt_amd.Cache(0, [[l] for l in layers], [data_size])
+    dst_cache = kvt_amd.Cache(0, [[h] for h in host_layers], [data_size])
+    ch = LoopbackChannel(0, src_cache, dst_cache, [data_size], [data_size])
+    ch.connect(dst_info)
+    assert ch.is_active()
+    ch.register_data(lists, tp_kind, num_layers,
+                     lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+    with torch.cuda.stream(stream):
+        layers[0].fill_(10)                       # mock layer 0
+        ch.send_data(0, stream.cuda_stream)       # event record + notify_event_record
+        layers[1].fill_(20)                       # mock layer 1
+        ch.send_data(1, stream.cuda_stream)
+    stream.synchronize()
+    metrics = ch.flush()
+    assert "layers_sent=2," in metrics and "sb_size_total=%d," % (4 * block_size) in metrics
+
+    for layer, val in ((0, 10), (1, 20)):
+        host = host_layers[layer].numpy()
+        for bid in dst_blocks:
+            blk = host[bid * block_size:(bid + 1) * block_size]
+            assert int(blk.astype(np.uint32).sum()) == val * block_size
+        untouched = np.delete(host.reshape(nblk, block_size), dst_blocks, axis=0)
+        assert not untouched.any()
+    ch.close()
+    assert not ch.is_active()
+
+
+def test_channel_rejects_metadata_beyond_the_destination():
+    block_size, nblk = 16 * KB, 8
+    info = dict(block_sizes=[block_size], token_sizes=[KB], layer_num_blocks=nblk, tp=1, rank=0)
+    src_info, dst_info = make_worker_info(**info), make_worker_info(**info)
+    lists, tp_kind = pipeline.parse_batch(SHAPE_RAGGED_FLASH, src_info, dst_info,
+                                          [TaskBuf(0, 32, True, [[0, 1]], [[6, 7]])])
+    layer = torch.zeros(nblk * block_size, dtype=torch.uint8, device="cuda")
+    small = torch.zeros(7 * block_size, dtype=torch.uint8, device="cuda")   # receiver has 7 blocks
+    sc = kvt_amd.Cache(0, [[layer]], [nblk * block_size])
+    dc = kvt_amd.Cache(0, [[small]], [7 * block_size])
+    ch = LoopbackChannel(0, sc, dc, [nblk * block_size], [7 * block_size])
+    ch.connect(dst_info)
+    with pytest.raises(kvt_amd.KvtError):
+        ch.register_data(lists, tp_kind, 1, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+    ch.close()
