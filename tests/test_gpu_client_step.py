@@ -80,3 +80,49 @@ def test_channel_rejects_metadata_beyond_the_destination():
     with pytest.raises(kvt_amd.KvtError):
         ch.register_data(lists, tp_kind, 1, lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
     ch.close()
+
+
+def test_cuda_kernel_sync_over_four_steps():
+    """StepTest.TestCudaKernelSync (kvtransfer/tests/step_sync_test.cu:18-104): four steps,
+    each filling layer 0 with step+1 and layer 1 with step+2 on a non-blocking stream; a
+    consumer thread waits for each layer and must see the step's value in every byte. The
+    reference's consumer blocks in Step::wait_layer_ready and copies the layer; here it blocks
+    in kvt_session_wait_layer and reads the layer's packed copy."""
+    import threading
+
+    num_layers, data_size = 2, 128 * (1 << 14)
+    stream = torch.cuda.Stream()
+    layers = [torch.zeros(data_size, dtype=torch.uint8, device="cuda") for _ in range(num_layers)]
+    lists = kvt_amd.BlockLists()
+    lists.append(0, [(0, 0, data_size)])
+    plan = kvt_amd.Plan(0, lists, [data_size], [data_size])
+    cache = kvt_amd.Cache(0, [[l] for l in layers], [data_size])
+    packed = torch.zeros(num_layers * plan.layer_bytes, dtype=torch.uint8, device="cuda")
+    for step in range(4):
+        session = kvt_amd.Session(plan, cache, packed, plan.layer_bytes)
+        seen, errors = {}, []
+
+        def consumer():
+            try:
+                for layer in range(num_layers):
+                    session.wait_layer(layer)
+                    got = packed[layer * plan.layer_bytes:][:data_size].cpu().numpy()
+                    seen[layer] = (int(got[:128].max()), int(got[:128].min()),
+                                   int(got.astype(np.uint64).sum()))
+            except Exception as e:
+                errors.append(e)
+
+        with torch.cuda.stream(stream):
+            layers[0].fill_(step + 1)
+            session.save_layer(0, stream.cuda_stream)
+            layers[1].fill_(step + 2)
+            session.save_layer(1, stream.cuda_stream)
+        t = threading.Thread(target=consumer)     # started after the launches: wait_layer
+        t.start()                                 # needs the layer's done event to be recorded
+        stream.synchronize()
+        t.join()
+        assert not errors, errors
+        for layer in range(num_layers):
+            val = step + 1 + layer
+            assert seen[layer] == (val, val, val * data_size), (step, layer, seen[layer])
+        session.close()
