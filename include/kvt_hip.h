@@ -345,7 +345,9 @@ void kvt_session_destroy(kvt_session* s);
  * already queued on compute_stream has run. Never blocks the host. */
 int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream);
 /* Host-blocking wait until layer's packed bytes are complete (what the
- * transport thread calls before send_data(layer)); not capturable. */
+ * transport thread calls before send_data(layer), Step::wait_layer_ready in the
+ * reference, kvtransfer/src/step.cpp:49-69). May be called from another thread
+ * before save_layer(layer): it then waits for that call first. Not capturable. */
 int kvt_session_wait_layer(kvt_session* s, uint32_t layer);
 /* Makes `stream` wait for every pack issued so far (joins the side stream
  * back; required before ending a capture that included save_layer calls). */

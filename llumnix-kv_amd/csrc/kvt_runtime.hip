@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <condition_variable>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -242,6 +243,11 @@ struct kvt_session {
   hipStream_t side = nullptr;
   std::vector<hipEvent_t> ready, done;
   hipEvent_t last_done = nullptr;
+  // which layers' packs have been issued (wait_layer may be called, from another thread,
+  // before the forward pass reaches the layer)
+  std::mutex mu;
+  std::condition_variable issued_cv;
+  std::vector<uint8_t> issued;
 };
 
 struct kvt_stager {
@@ -943,6 +949,7 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
     KVT_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));
     s->ready.resize(cache->n_layers);
     s->done.resize(cache->n_layers);
+    s->issued.assign(cache->n_layers, 0);
     for (uint32_t l = 0; l < cache->n_layers; ++l) {
       KVT_HIP(hipEventCreateWithFlags(&s->ready[l], hipEventDisableTiming));
       KVT_HIP(hipEventCreateWithFlags(&s->done[l], hipEventDisableTiming));
@@ -976,7 +983,12 @@ int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream)
     uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
     if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
     KVT_HIP(hipEventRecord(s->done[layer], s->side));
-    s->last_done = s->done[layer];
+    {
+      std::lock_guard<std::mutex> lock(s->mu);
+      s->last_done = s->done[layer];
+      s->issued[layer] = 1;
+    }
+    s->issued_cv.notify_all();
     return KVT_OK;
   });
 }
@@ -985,6 +997,10 @@ int kvt_session_wait_layer(kvt_session* s, uint32_t layer) {
   return guarded([&]() -> int {
     if (!s) return fail(KVT_ERR_INVALID, "kvt_session_wait_layer: null session");
     if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    {
+      std::unique_lock<std::mutex> lock(s->mu);
+      s->issued_cv.wait(lock, [&] { return s->issued[layer] != 0; });
+    }
     KVT_HIP(hipEventSynchronize(s->done[layer]));
     return KVT_OK;
   });

@@ -112,13 +112,13 @@ def test_cuda_kernel_sync_over_four_steps():
             except Exception as e:
                 errors.append(e)
 
+        t = threading.Thread(target=consumer)     # waits before the layers are even launched
+        t.start()
         with torch.cuda.stream(stream):
             layers[0].fill_(step + 1)
             session.save_layer(0, stream.cuda_stream)
             layers[1].fill_(step + 2)
             session.save_layer(1, stream.cuda_stream)
-        t = threading.Thread(target=consumer)     # started after the launches: wait_layer
-        t.start()                                 # needs the layer's done event to be recorded
         stream.synchronize()
         t.join()
         assert not errors, errors
