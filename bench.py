@@ -465,6 +465,36 @@ def main():
             res["note"] = ("%d launches of %d ranges each; GB/s = bytes read + bytes written; the "
                            "fp8 gather reads 2 bytes and writes 1 per element" %
                            (w.n_layers, len(runs0)))
+            # the reference's host entry point, called the way TCPChannel::send_data /
+            # handle_kv_cache_data call it: pinned host buffer on the contiguous side, metadata
+            # uploaded per call through the caller's two 8192-range buffers
+            if nb <= (2 << 30):
+                pin = torch.empty(nb, dtype=torch.uint8, pin_memory=True)
+                meta_n = 3 * 8192
+                dev_meta = torch.zeros(meta_n, dtype=torch.int64, device="cuda")
+                host_meta = torch.zeros(meta_n, dtype=torch.int64).pin_memory()
+                zeros = np.zeros(len(runs0), dtype=np.uint64)
+                kb_send = np.ascontiguousarray(np.stack(
+                    [zeros, runs0[:, 0].astype(np.uint64), runs0[:, 2].astype(np.uint64)], axis=1))
+                kb_recv = np.ascontiguousarray(first[0][1].tensor(0))
+                Lh = min(4, w.n_layers)
+                for name, direction, blocks, tensors in (
+                        ("handle_data_d2h_pinned_gbps", 1, kb_send, side.src),
+                        ("handle_data_h2d_pinned_gbps", 0, kb_recv, side.dst)):
+                    for rep in range(2):
+                        torch.cuda.synchronize()
+                        t_a = time.perf_counter()
+                        for l in range(Lh):
+                            rc = lib.kvt_copy_handle_data_with_kernel(
+                                pin.data_ptr(), tensors[l][0].data_ptr(), blocks.ctypes.data,
+                                len(blocks), nb, direction, 0, sh, dev_meta.data_ptr(),
+                                host_meta.data_ptr(), 8192)
+                            assert rc == 0, lib.kvt_last_error()
+                            stream.synchronize()     # the reference syncs after every tensor
+                        dt = time.perf_counter() - t_a
+                    res[name] = round(nb * Lh / dt / 1e9, 2)
+                res["handle_data_note"] = ("%d layers, one call per layer incl. metadata upload and "
+                                           "stream sync; GB/s = payload bytes over PCIe" % Lh)
             out["reference_shaped_launchers"] = res
 
         # pinned-host staging of packed layers, double buffered against the pack kernel
