@@ -1,0 +1,155 @@
+// The reference's copy entry points, same calling conventions: range lists as
+// three int64 device arrays, or kvt_ipc_block lists with caller-owned metadata
+// buffers.
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "kvt_runtime.h"
+
+using namespace kvt;
+
+extern "C" {
+
+// ------------------------------------------- reference-shaped entry points
+
+static int range_launch_shape(int64_t n, int num_wg, int* wgs) {
+  if (n > 0x7FFFFFFFll) return fail(KVT_ERR_INVALID, "too many ranges");
+  int w = num_wg > 0 ? num_wg : static_cast<int>(std::min<int64_t>(n, 1 << 20));
+  *wgs = std::max(1, w);
+  return KVT_OK;
+}
+
+static int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so,
+                         const int64_t* dof, const int64_t* len, int64_t n, int num_wg,
+                         int threads_per_wg, void* stream) {
+  (void)threads_per_wg;  // workgroups are always 256 lanes (4 wavefronts)
+  if (n == 0) return KVT_OK;
+  if (n < 0 || !src || !dst || !so || !dof || !len)
+    return fail(KVT_ERR_INVALID, "launch_copy: bad argument");
+  if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+  int wgs = 0;
+  if (int rc = range_launch_shape(n, num_wg, &wgs)) return rc;
+  // The range lengths live on the device; eight workgroups stride over each range's slices.
+  const int rows = 8;
+  const hipStream_t s = static_cast<hipStream_t>(stream);
+  const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, s)
+                               : launch_copy_ranges(src, dst, so, dof, len, n, wgs, rows, s);
+  if (e != hipSuccess) return hip_fail(e, "range copy launch");
+  return KVT_OK;
+}
+
+int kvt_launch_copy_d2h_direct(const void* gpu_src_base, void* dst, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(false, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+int kvt_launch_copy_h2d_direct(const void* src, void* gpu_dst_base, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(false, src, gpu_dst_base, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
+                                    const int64_t* src_offsets, const int64_t* dst_offsets,
+                                    const int64_t* lengths, int64_t n, int num_wg,
+                                    int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(true, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+// Shared body of the two "handle data" entry points. `halve`: converting
+// gather (contiguous side advances by length / 2, lengths passed to the kernel
+// are element counts).
+static int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks,
+                       uint64_t n, uint64_t tensor_data_size, int direction, bool halve,
+                       int device, void* stream, int64_t* dev_meta, int64_t* host_meta,
+                       int64_t max_block_num) {
+  if (n == 0) return KVT_OK;
+  if (!tensor_buf || !layer_gpu_ptr || !blocks || !dev_meta || !host_meta)
+    return fail(KVT_ERR_INVALID, "copy_handle_data: null argument");
+  if (direction != KVT_COPY_H2D && direction != KVT_COPY_D2H)
+    return fail(KVT_ERR_INVALID, "copy_handle_data: bad direction");
+  if (int rc = check_device(device)) return rc;
+  if (max_block_num <= 0) max_block_num = 8192;
+  uint64_t total = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    if (blocks[i].length == 0) return fail(KVT_ERR_INVALID, "copy_handle_data: zero-length range");
+    if (halve && (blocks[i].length & 1)) return fail(KVT_ERR_INVALID, "odd bf16 byte length");
+    total += blocks[i].length;
+  }
+  if (total != tensor_data_size)
+    return fail(KVT_ERR_INVALID, "copy_handle_data: tensor_data_size != sum of range lengths");
+  DeviceGuard g;
+  if (int rc = g.enter(device)) return rc;
+  const hipStream_t s = static_cast<hipStream_t>(stream);
+  uint64_t host_cursor = 0;
+  for (uint64_t first = 0; first < n; first += static_cast<uint64_t>(max_block_num)) {
+    const uint64_t m = std::min<uint64_t>(static_cast<uint64_t>(max_block_num), n - first);
+    int64_t* contig = host_meta;
+    int64_t* gpu = host_meta + m;
+    int64_t* lens = host_meta + 2 * m;
+    uint64_t longest = 0;
+    for (uint64_t i = 0; i < m; ++i) {
+      const kvt_ipc_block& b = blocks[first + i];
+      contig[i] = static_cast<int64_t>(host_cursor);
+      gpu[i] = static_cast<int64_t>(b.dst_offset);
+      lens[i] = static_cast<int64_t>(halve ? b.length / 2 : b.length);
+      host_cursor += halve ? b.length / 2 : b.length;
+      longest = std::max<uint64_t>(longest, b.length);
+    }
+    KVT_HIP(hipMemcpyAsync(dev_meta, host_meta, 3 * m * sizeof(int64_t), hipMemcpyHostToDevice, s));
+    const int64_t* d_contig = dev_meta;
+    const int64_t* d_gpu = dev_meta + m;
+    const int64_t* d_lens = dev_meta + 2 * m;
+    const int wgs = static_cast<int>(m);
+    // one workgroup per 4 KiB slice of the longest range (bounded; longer ranges are strided)
+    const uint64_t unit = halve ? 8192 : 4096;
+    const int rows = static_cast<int>(std::min<uint64_t>(std::max<uint64_t>(1, (longest + unit - 1) / unit), 512));
+    hipError_t e;
+    if (halve)
+      e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
+                                static_cast<int64_t>(m), wgs, rows, s);
+    else if (direction == KVT_COPY_D2H)
+      e = launch_copy_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
+                             static_cast<int64_t>(m), wgs, rows, s);
+    else
+      e = launch_copy_ranges(tensor_buf, layer_gpu_ptr, d_contig, d_gpu, d_lens,
+                             static_cast<int64_t>(m), wgs, rows, s);
+    if (e != hipSuccess) return hip_fail(e, "copy_handle_data launch");
+    // the metadata buffers are reused by the next batch
+    if (first + m < n) KVT_HIP(hipStreamSynchronize(s));
+  }
+  return KVT_OK;
+}
+
+int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
+                                     const kvt_ipc_block* blocks, uint64_t n,
+                                     uint64_t tensor_data_size, int direction, int device,
+                                     void* stream, int64_t* dev_meta, int64_t* host_meta,
+                                     int64_t max_block_num) {
+  return guarded([&]() {
+    return handle_data(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction, false,
+                       device, stream, dev_meta, host_meta, max_block_num);
+  });
+}
+
+int kvt_copy_d2h_bf16_to_fp8(void* tensor_buf, const void* layer_gpu_ptr,
+                             const kvt_ipc_block* blocks, uint64_t n, uint64_t tensor_data_size,
+                             int device, void* stream, int64_t* dev_meta, int64_t* host_meta,
+                             int64_t max_block_num) {
+  return guarded([&]() {
+    return handle_data(tensor_buf, const_cast<void*>(layer_gpu_ptr), blocks, n, tensor_data_size,
+                       KVT_COPY_D2H, true, device, stream, dev_meta, host_meta, max_block_num);
+  });
+}
+}  // extern "C"

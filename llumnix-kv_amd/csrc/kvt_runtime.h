@@ -1,0 +1,188 @@
+// Internal declarations shared by the HIP translation units of libkvt_hip
+// (device selection, the chunk-table pool, registered caches and copy plans).
+#ifndef KVT_RUNTIME_H_
+#define KVT_RUNTIME_H_
+
+#include <hip/hip_runtime.h>
+
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "kvt_device.h"
+#include "kvt_internal.h"
+
+namespace kvt {
+
+int hip_fail(hipError_t e, const char* what);
+
+#define KVT_HIP(call)                                  \
+  do {                                                 \
+    const hipError_t _e = (call);                      \
+    if (_e != hipSuccess) return hip_fail(_e, #call);  \
+  } while (0)
+
+// Number of devices, or 0. Only gfx950 parts are accepted: the code objects in
+// this library are built for that target alone.
+int usable_devices();
+// KVT_OK, or KVT_ERR_NO_DEVICE / KVT_ERR_INVALID with the message set.
+int check_device(int device);
+
+struct DeviceGuard {
+  int prev = -1;
+  bool switched = false;
+  int enter(int device) {
+    if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+    if (prev != device) {
+      const hipError_t e = hipSetDevice(device);
+      if (e != hipSuccess) return hip_fail(e, "hipSetDevice");
+      switched = true;
+    }
+    return KVT_OK;
+  }
+  ~DeviceGuard() {
+    if (switched && prev >= 0) (void)hipSetDevice(prev);
+  }
+};
+
+inline uint64_t round_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+// Chunk tables are uploaded once per batch and die with the batch. hipMalloc /
+// hipFree per batch would stall (hipFree waits for the whole device), so table
+// storage is recycled: a buffer = device memory + a pinned host twin of the same
+// size + an event that marks its last use on the GPU. A released buffer is handed
+// out again only once that event has completed.
+struct TableBuf {
+  int device = -1;
+  size_t cap = 0;
+  void* dev = nullptr;
+  void* host = nullptr;          // pinned staging for the asynchronous upload
+  hipEvent_t last_use = nullptr; // recorded after every launch that reads `dev`
+  bool used = false;             // last_use has been recorded at least once
+  bool captured = false;         // read by a kernel recorded into a hipGraph
+};
+
+class TablePool {
+ public:
+  int acquire(int device, size_t bytes, TableBuf** out) {
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      size_t best = idle_.size();
+      for (size_t i = 0; i < idle_.size(); ++i) {
+        TableBuf* b = idle_[i];
+        if (b->device != device || b->cap < bytes) continue;
+        if (b->used && hipEventQuery(b->last_use) != hipSuccess) {
+          (void)hipGetLastError();
+          continue;  // still being read by a queued kernel
+        }
+        if (best == idle_.size() || b->cap < idle_[best]->cap) best = i;
+      }
+      if (best != idle_.size()) {
+        *out = idle_[best];
+        idle_.erase(idle_.begin() + best);
+        (*out)->used = false;
+        return KVT_OK;
+      }
+    }
+    std::unique_ptr<TableBuf> b(new TableBuf());
+    b->device = device;
+    b->cap = 65536;
+    while (b->cap < bytes) b->cap *= 2;
+    KVT_HIP(hipMalloc(&b->dev, b->cap));
+    hipError_t e = hipHostMalloc(&b->host, b->cap, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&b->last_use, hipEventDisableTiming);
+    if (e != hipSuccess) {
+      destroy(b.get());
+      return hip_fail(e, "table buffer allocation");
+    }
+    *out = b.release();
+    return KVT_OK;
+  }
+
+  void release(TableBuf* b) {
+    if (!b) return;
+    if (b->captured) {  // a graph may replay the kernel later: never recycle, free for good
+      destroy(b);
+      delete b;
+      return;
+    }
+    std::lock_guard<std::mutex> lock(mu_);
+    if (idle_.size() >= 64) {
+      TableBuf* victim = idle_.front();
+      idle_.erase(idle_.begin());
+      if (victim->used) (void)hipEventSynchronize(victim->last_use);
+      destroy(victim);
+      delete victim;
+    }
+    idle_.push_back(b);
+  }
+
+  // One upload stream per device, created on first use.
+  int upload_stream(int device, hipStream_t* out) {
+    std::lock_guard<std::mutex> lock(mu_);
+    if (device >= static_cast<int>(streams_.size())) streams_.resize(device + 1, nullptr);
+    if (!streams_[device]) KVT_HIP(hipStreamCreateWithFlags(&streams_[device], hipStreamNonBlocking));
+    *out = streams_[device];
+    return KVT_OK;
+  }
+
+ private:
+  static void destroy(TableBuf* b) {
+    if (b->dev) (void)hipFree(b->dev);
+    if (b->host) (void)hipHostFree(b->host);
+    if (b->last_use) (void)hipEventDestroy(b->last_use);
+    b->dev = b->host = nullptr;
+    b->last_use = nullptr;
+  }
+  std::mutex mu_;
+  std::vector<TableBuf*> idle_;
+  std::vector<hipStream_t> streams_;
+};
+
+TablePool& table_pool();
+
+constexpr uint32_t kMinChunk = 4096, kMaxAutoChunk = 32768, kMaxChunk = 1u << 19;
+constexpr uint64_t kBlobAlign = 256;
+
+}  // namespace kvt
+
+struct kvt_cache {
+  int device = 0;
+  uint32_t n_layers = 0, n_tensors = 0;
+  std::vector<uint64_t> capacity;
+  std::vector<void*> host_ptrs;
+  uint8_t** dev_ptrs = nullptr;
+  bool aligned16 = true;  // every layer tensor starts on a 16-byte boundary
+};
+
+struct kvt_plan {
+  int device = 0;
+  uint32_t n_tensors = 0;
+  uint64_t n_chunks = 0;
+  std::vector<uint64_t> tensor_bytes, tensor_offset, src_cap, dst_cap;
+  uint64_t layer_bytes = 0;
+  bool xform = false;
+  kvt::XformDev xdev{};
+  bool strided = false;            // some chunks carry a record shape (kvt_plan_create_runs)
+  kvt::StrideTable shapes{};
+  uint64_t n_strided = 0;
+  std::vector<kvt::Chunk> host_table;   // device == KVT_DEVICE_NONE only: the tables, kept on the host
+  uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
+  kvt::Chunk* dev_chunks = nullptr;     // [0, n_chunks): pack order; [n_chunks, 2 n_chunks): unpack order
+  kvt::TableBuf* buf = nullptr;         // storage of dev_chunks (recycled through the table pool)
+  hipEvent_t uploaded = nullptr;   // completes when the table has reached the device
+  mutable bool upload_seen = false;  // a launch has already observed `uploaded` as complete
+};
+
+namespace kvt {
+
+// Launches the pack (gather) or unpack (scatter) of layers [first_layer, first_layer +
+// n_layers) of a plan. blob_offsets = nullptr: the plan's own blob positions.
+int run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer,
+             uint32_t n_layers, void* packed, uint64_t layer_stride, void* stream,
+             const uint64_t* blob_offsets = nullptr);
+
+}  // namespace kvt
+
+#endif  // KVT_RUNTIME_H_

@@ -1,0 +1,273 @@
+// Per-layer gating sessions (event -> side stream -> pack -> done event) and
+// pinned-host staging of packed layers.
+#include <condition_variable>
+#include <cstring>
+#include <memory>
+
+#include "kvt_runtime.h"
+
+using namespace kvt;
+
+struct kvt_session {
+  const kvt_plan* plan = nullptr;
+  const kvt_cache* cache = nullptr;
+  void* packed = nullptr;
+  uint64_t layer_stride = 0;
+  hipStream_t side = nullptr;
+  std::vector<hipEvent_t> ready, done;
+  hipEvent_t last_done = nullptr;
+  // which layers' packs have been issued (wait_layer may be called, from another thread,
+  // before the forward pass reaches the layer)
+  std::mutex mu;
+  std::condition_variable issued_cv;
+  std::vector<uint8_t> issued;
+};
+
+struct kvt_stager {
+  int device = 0;
+  uint64_t slot_bytes = 0;
+  uint32_t n_slots = 0;
+  uint8_t* pinned = nullptr;
+  hipStream_t copy = nullptr;
+  std::vector<hipEvent_t> slot_done;
+  hipEvent_t fence = nullptr;
+};
+extern "C" {
+
+// ----------------------------------------------------------------- session
+
+int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packed,
+                       uint64_t layer_stride, kvt_session** out) {
+  return guarded([&]() -> int {
+    if (!plan || !cache || !packed || !out)
+      return fail(KVT_ERR_INVALID, "kvt_session_create: null argument");
+    if (layer_stride < plan->layer_bytes)
+      return fail(KVT_ERR_INVALID, "kvt_session_create: layer_stride smaller than one packed layer");
+    if (int rc = check_device(plan->device)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(plan->device)) return rc;
+    if (int rc = kvt_plan_ready(plan)) return rc;  // save_layer may run inside a stream capture
+    std::unique_ptr<kvt_session> s(new kvt_session());
+    s->plan = plan;
+    s->cache = cache;
+    s->packed = packed;
+    s->layer_stride = layer_stride;
+    KVT_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));
+    s->ready.resize(cache->n_layers);
+    s->done.resize(cache->n_layers);
+    s->issued.assign(cache->n_layers, 0);
+    for (uint32_t l = 0; l < cache->n_layers; ++l) {
+      KVT_HIP(hipEventCreateWithFlags(&s->ready[l], hipEventDisableTiming));
+      KVT_HIP(hipEventCreateWithFlags(&s->done[l], hipEventDisableTiming));
+    }
+    *out = s.release();
+    return KVT_OK;
+  });
+}
+
+void kvt_session_destroy(kvt_session* s) {
+  if (!s) return;
+  if (s->side) {
+    (void)hipStreamSynchronize(s->side);
+    (void)hipStreamDestroy(s->side);
+  }
+  for (hipEvent_t e : s->ready)
+    if (e) (void)hipEventDestroy(e);
+  for (hipEvent_t e : s->done)
+    if (e) (void)hipEventDestroy(e);
+  delete s;
+}
+
+int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_save_layer: null session");
+    if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    DeviceGuard g;
+    if (int rc = g.enter(s->plan->device)) return rc;
+    KVT_HIP(hipEventRecord(s->ready[layer], static_cast<hipStream_t>(compute_stream)));
+    KVT_HIP(hipStreamWaitEvent(s->side, s->ready[layer], 0));
+    uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
+    if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
+    KVT_HIP(hipEventRecord(s->done[layer], s->side));
+    {
+      std::lock_guard<std::mutex> lock(s->mu);
+      s->last_done = s->done[layer];
+      s->issued[layer] = 1;
+    }
+    s->issued_cv.notify_all();
+    return KVT_OK;
+  });
+}
+
+int kvt_session_wait_layer(kvt_session* s, uint32_t layer) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_wait_layer: null session");
+    if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    {
+      std::unique_lock<std::mutex> lock(s->mu);
+      s->issued_cv.wait(lock, [&] { return s->issued[layer] != 0; });
+    }
+    KVT_HIP(hipEventSynchronize(s->done[layer]));
+    return KVT_OK;
+  });
+}
+
+int kvt_session_join(kvt_session* s, void* stream) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_join: null session");
+    if (s->last_done) KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), s->last_done, 0));
+    return KVT_OK;
+  });
+}
+
+void* kvt_session_side_stream(kvt_session* s) { return s ? s->side : nullptr; }
+
+// ------------------------------------------------------------------ stager
+
+int kvt_stager_create(int device, uint64_t slot_bytes, uint32_t n_slots, kvt_stager** out) {
+  return guarded([&]() -> int {
+    if (!out || slot_bytes == 0 || n_slots < 2)
+      return fail(KVT_ERR_INVALID, "kvt_stager_create: need >= 2 slots of > 0 bytes");
+    if (int rc = check_device(device)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    std::unique_ptr<kvt_stager> s(new kvt_stager());
+    s->device = device;
+    s->slot_bytes = round_up(slot_bytes, 4096);
+    s->n_slots = n_slots;
+    KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&s->pinned), s->slot_bytes * n_slots,
+                          hipHostMallocDefault));
+    KVT_HIP(hipStreamCreateWithFlags(&s->copy, hipStreamNonBlocking));
+    s->slot_done.resize(n_slots);
+    for (uint32_t i = 0; i < n_slots; ++i)
+      KVT_HIP(hipEventCreateWithFlags(&s->slot_done[i], hipEventDisableTiming));
+    KVT_HIP(hipEventCreateWithFlags(&s->fence, hipEventDisableTiming));
+    *out = s.release();
+    return KVT_OK;
+  });
+}
+
+void kvt_stager_destroy(kvt_stager* s) {
+  if (!s) return;
+  if (s->copy) {
+    (void)hipStreamSynchronize(s->copy);
+    (void)hipStreamDestroy(s->copy);
+  }
+  for (hipEvent_t e : s->slot_done)
+    if (e) (void)hipEventDestroy(e);
+  if (s->fence) (void)hipEventDestroy(s->fence);
+  if (s->pinned) (void)hipHostFree(s->pinned);
+  delete s;
+}
+
+void* kvt_stager_slot(kvt_stager* s, uint32_t slot) {
+  return (s && slot < s->n_slots) ? s->pinned + static_cast<uint64_t>(slot) * s->slot_bytes : nullptr;
+}
+void* kvt_stager_copy_stream(kvt_stager* s) { return s ? s->copy : nullptr; }
+
+int kvt_stager_save(kvt_stager* s, uint32_t slot, const void* dev, uint64_t bytes,
+                    void* producer_stream) {
+  return kvt_stager_save_at(s, slot, 0, dev, bytes, producer_stream);
+}
+
+int kvt_stager_save_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, const void* dev,
+                       uint64_t bytes, void* producer_stream) {
+  return guarded([&]() -> int {
+    if (!s || !dev) return fail(KVT_ERR_INVALID, "kvt_stager_save: null argument");
+    if (slot >= s->n_slots || slot_offset > s->slot_bytes || bytes > s->slot_bytes - slot_offset)
+      return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_save: slot index or size out of range");
+    DeviceGuard g;
+    if (int rc = g.enter(s->device)) return rc;
+    KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(producer_stream)));
+    KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));
+    KVT_HIP(hipMemcpyAsync(static_cast<uint8_t*>(kvt_stager_slot(s, slot)) + slot_offset, dev, bytes,
+                           hipMemcpyDeviceToHost, s->copy));
+    KVT_HIP(hipEventRecord(s->slot_done[slot], s->copy));
+    return KVT_OK;
+  });
+}
+
+int kvt_stager_load(kvt_stager* s, uint32_t slot, void* dev, uint64_t bytes,
+                    void* consumer_stream) {
+  return kvt_stager_load_at(s, slot, 0, dev, bytes, consumer_stream);
+}
+
+int kvt_stager_load_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, void* dev,
+                       uint64_t bytes, void* consumer_stream) {
+  return guarded([&]() -> int {
+    if (!s || !dev) return fail(KVT_ERR_INVALID, "kvt_stager_load: null argument");
+    if (slot >= s->n_slots || slot_offset > s->slot_bytes || bytes > s->slot_bytes - slot_offset)
+      return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_load: slot index or size out of range");
+    DeviceGuard g;
+    if (int rc = g.enter(s->device)) return rc;
+    // the device buffer may still be read by earlier work of the consumer
+    KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(consumer_stream)));
+    KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));
+    KVT_HIP(hipMemcpyAsync(dev, static_cast<uint8_t*>(kvt_stager_slot(s, slot)) + slot_offset, bytes,
+                           hipMemcpyHostToDevice, s->copy));
+    KVT_HIP(hipEventRecord(s->slot_done[slot], s->copy));
+    KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(consumer_stream), s->slot_done[slot], 0));
+    return KVT_OK;
+  });
+}
+
+int kvt_stager_wait(kvt_stager* s, uint32_t slot) {
+  return guarded([&]() -> int {
+    if (!s || slot >= s->n_slots) return fail(KVT_ERR_INVALID, "kvt_stager_wait: bad argument");
+    KVT_HIP(hipEventSynchronize(s->slot_done[slot]));
+    return KVT_OK;
+  });
+}
+
+int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats,
+                     double* bytes_per_s) {
+  return guarded([&]() -> int {
+    if (!bytes_per_s || bytes == 0 || repeats == 0)
+      return fail(KVT_ERR_INVALID, "kvt_measure_pcie: bad argument");
+    if (int rc = check_device(device)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    void *host = nullptr, *dev = nullptr;
+    hipStream_t st = nullptr;
+    hipEvent_t a = nullptr, b = nullptr;
+    int rc = KVT_OK;
+    auto cleanup = [&]() {
+      if (a) (void)hipEventDestroy(a);
+      if (b) (void)hipEventDestroy(b);
+      if (st) (void)hipStreamDestroy(st);
+      if (dev) (void)hipFree(dev);
+      if (host) (void)hipHostFree(host);
+    };
+#define KVT_TRY(call)                         \
+  do {                                        \
+    const hipError_t _e = (call);             \
+    if (_e != hipSuccess) {                   \
+      rc = hip_fail(_e, #call);               \
+      cleanup();                              \
+      return rc;                              \
+    }                                         \
+  } while (0)
+    KVT_TRY(hipHostMalloc(&host, bytes, hipHostMallocDefault));
+    KVT_TRY(hipMalloc(&dev, bytes));
+    std::memset(host, 0x5a, bytes);
+    KVT_TRY(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    KVT_TRY(hipEventCreate(&a));
+    KVT_TRY(hipEventCreate(&b));
+    const bool d2h = direction == KVT_COPY_D2H;
+    KVT_TRY(hipMemcpyAsync(d2h ? host : dev, d2h ? dev : host, bytes,
+                           d2h ? hipMemcpyDeviceToHost : hipMemcpyHostToDevice, st));
+    KVT_TRY(hipEventRecord(a, st));
+    for (uint32_t i = 0; i < repeats; ++i)
+      KVT_TRY(hipMemcpyAsync(d2h ? host : dev, d2h ? dev : host, bytes,
+                             d2h ? hipMemcpyDeviceToHost : hipMemcpyHostToDevice, st));
+    KVT_TRY(hipEventRecord(b, st));
+    KVT_TRY(hipEventSynchronize(b));
+    float ms = 0;
+    KVT_TRY(hipEventElapsedTime(&ms, a, b));
+#undef KVT_TRY
+    *bytes_per_s = static_cast<double>(bytes) * repeats / (ms * 1e-3);
+    cleanup();
+    return KVT_OK;
+  });
+}
+}  // extern "C"
