@@ -9,7 +9,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "llumnix-kv_amd", "csrc")
-HOST_SOURCES = ["kvt_parse.cpp", "kvt_ranges.cpp", "kvt_wire.cpp", "kvt_runs.cpp"]
+HOST_SOURCES = ["kvt_parse.cpp", "kvt_parse_build.cpp", "kvt_ranges.cpp", "kvt_wire.cpp", "kvt_runs.cpp"]
 
 
 def test_host_entry_points_under_sanitizers(tmp_path):
