@@ -284,6 +284,12 @@ int kvt_block_object_lists(int cache_shape, const kvt_worker_info* src, const kv
                            const uint32_t* src_blocks, const uint32_t* dst_blocks, uint64_t n,
                            kvt_block_lists* lists, uint64_t* object_bytes);
 
+/* The store's block ids -> the engine's kernel-block ids when one store block
+ * spans `factor` kernel blocks: out[i] = ids[i / factor] * factor + i % factor
+ * for i < n * factor (VineyardKVSBackend._enlarge_list,
+ *                                               blade_kvt/hybrid_connector/kvsbackend.py:207-214). */
+int kvt_enlarge_block_ids(const uint32_t* ids, uint64_t n, uint32_t factor, uint32_t* out);
+
 /* --------------------------- drop-ins for the reference copy entry points */
 
 /* replaces launch_copy_d2h_direct_kernel()      kvtransfer/src/copy_kernels.cu:268-281

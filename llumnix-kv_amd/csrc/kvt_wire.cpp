@@ -217,4 +217,16 @@ int kvt_block_object_lists(int cache_shape, const kvt_worker_info* src, const kv
   });
 }
 
+int kvt_enlarge_block_ids(const uint32_t* ids, uint64_t n, uint32_t factor, uint32_t* out) {
+  if ((!ids && n) || (!out && n) || factor == 0)
+    return fail(KVT_ERR_INVALID, "kvt_enlarge_block_ids: bad argument");
+  for (uint64_t i = 0; i < n; ++i) {
+    const uint64_t first = static_cast<uint64_t>(ids[i]) * factor;
+    if (first + factor - 1 > 0xFFFFFFFFull)
+      return fail(KVT_ERR_OVERFLOW, "kvt_enlarge_block_ids: block id does not fit 32 bits");
+    for (uint32_t k = 0; k < factor; ++k) out[i * factor + k] = static_cast<uint32_t>(first + k);
+  }
+  return KVT_OK;
+}
+
 }  // extern "C"

@@ -81,6 +81,7 @@ SIGNATURES = {
                                     _P(WireLayout)]),
     "kvt_block_object_lists": (_int, [_int, _P(WorkerInfo), _P(WorkerInfo), _vp, _vp, _u64, _vp,
                                       _P(_u64)]),
+    "kvt_enlarge_block_ids": (_int, [_vp, _u64, _u32, _vp]),
     "kvt_launch_copy_d2h_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
@@ -221,6 +222,13 @@ def block_object_lists(cache_shape, src, dst, src_blocks, dst_blocks, lists=None
     check(lib().kvt_block_object_lists(cache_shape, C.byref(src), C.byref(dst), s.ctypes.data,
                                        d.ctypes.data, len(s), lists.h, C.byref(ob)))
     return lists, ob.value
+
+
+def enlarge_block_ids(ids, factor):
+    a = np.ascontiguousarray(ids, dtype=np.uint32)
+    out = np.empty(len(a) * factor, dtype=np.uint32)
+    check(lib().kvt_enlarge_block_ids(a.ctypes.data, len(a), factor, out.ctypes.data))
+    return out
 
 
 def validate_bounds(runs, capacity, which, scale=1):

@@ -255,3 +255,17 @@ def test_block_objects_of_block_major_layouts_and_errors():
     with pytest.raises(kvt_amd.KvtError):
         kvt_amd.block_object_lists(kvt_amd.ctypes_defs.SHAPE_FLASHINFER, _info([B0], 10),
                                    _info([B0 * 2], 20), [1], [0])
+
+
+def test_enlarge_block_ids_is_the_kvsbackend_formula():
+    """res[i] = lst[i // n] * n + (i % n)   (kvsbackend.py:207-214)"""
+    rng = np.random.default_rng(8)
+    for n in (1, 2, 3, 8):
+        lst = rng.integers(0, 1 << 20, 37).tolist()
+        want = [lst[i // n] * n + (i % n) for i in range(len(lst) * n)]
+        assert binding.enlarge_block_ids(lst, n).tolist() == want
+    assert len(binding.enlarge_block_ids([], 4)) == 0
+    with pytest.raises(kvt_amd.KvtError):
+        binding.enlarge_block_ids([1 << 31], 4)          # does not fit 32 bits
+    with pytest.raises(kvt_amd.KvtError):
+        binding.enlarge_block_ids([1], 0)
