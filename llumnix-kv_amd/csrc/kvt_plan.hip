@@ -484,9 +484,8 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
     // remember when the table is last read, so that its storage is not recycled too early
     if (capturing) {
       p->buf->captured = true;
-    } else {
-      KVT_HIP(hipEventRecord(p->buf->last_use, s));
-      p->buf->used = true;
+    } else if (int rc = p->buf->mark_use(s)) {
+      return rc;
     }
   }
   return KVT_OK;

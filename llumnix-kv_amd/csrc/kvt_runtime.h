@@ -51,16 +51,65 @@ inline uint64_t round_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 // Chunk tables are uploaded once per batch and die with the batch. hipMalloc /
 // hipFree per batch would stall (hipFree waits for the whole device), so table
 // storage is recycled: a buffer = device memory + a pinned host twin of the same
-// size + an event that marks its last use on the GPU. A released buffer is handed
-// out again only once that event has completed.
+// size + one event per stream that has launched kernels reading it, marking the
+// last such launch. A released buffer is handed out again only once all of them
+// have completed.
 struct TableBuf {
+  struct Use {
+    hipStream_t stream;
+    hipEvent_t done;
+    bool recorded;
+  };
   int device = -1;
   size_t cap = 0;
   void* dev = nullptr;
-  void* host = nullptr;          // pinned staging for the asynchronous upload
-  hipEvent_t last_use = nullptr; // recorded after every launch that reads `dev`
-  bool used = false;             // last_use has been recorded at least once
-  bool captured = false;         // read by a kernel recorded into a hipGraph
+  void* host = nullptr;   // pinned staging for the asynchronous upload
+  std::mutex mu;          // a plan may be launched from several threads
+  std::vector<Use> uses;  // events are kept across recycling (streams repeat)
+  bool captured = false;  // read by a kernel recorded into a hipGraph
+
+  // Call after every launch on `stream` that reads `dev`.
+  int mark_use(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(mu);
+    Use* u = nullptr;
+    for (Use& x : uses)
+      if (x.stream == stream) u = &x;
+    if (!u) {
+      if (uses.size() >= 16) {  // many streams: retire the oldest entry instead of growing
+        if (uses.front().recorded) KVT_HIP(hipEventSynchronize(uses.front().done));
+        uses.front().recorded = false;
+        uses.front().stream = stream;
+        u = &uses.front();
+      } else {
+        hipEvent_t ev = nullptr;
+        KVT_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        uses.push_back(Use{stream, ev, false});
+        u = &uses.back();
+      }
+    }
+    KVT_HIP(hipEventRecord(u->done, stream));
+    u->recorded = true;
+    return KVT_OK;
+  }
+  // No queued kernel reads the table any more.
+  bool idle() {
+    std::lock_guard<std::mutex> lock(mu);
+    for (const Use& x : uses)
+      if (x.recorded && hipEventQuery(x.done) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+    return true;
+  }
+  void wait_idle() {
+    std::lock_guard<std::mutex> lock(mu);
+    for (const Use& x : uses)
+      if (x.recorded) (void)hipEventSynchronize(x.done);
+  }
+  void forget_uses() {
+    std::lock_guard<std::mutex> lock(mu);
+    for (Use& x : uses) x.recorded = false;
+  }
 };
 
 class TablePool {
@@ -72,16 +121,13 @@ class TablePool {
       for (size_t i = 0; i < idle_.size(); ++i) {
         TableBuf* b = idle_[i];
         if (b->device != device || b->cap < bytes) continue;
-        if (b->used && hipEventQuery(b->last_use) != hipSuccess) {
-          (void)hipGetLastError();
-          continue;  // still being read by a queued kernel
-        }
+        if (!b->idle()) continue;  // still being read by a queued kernel
         if (best == idle_.size() || b->cap < idle_[best]->cap) best = i;
       }
       if (best != idle_.size()) {
         *out = idle_[best];
         idle_.erase(idle_.begin() + best);
-        (*out)->used = false;
+        (*out)->forget_uses();
         return KVT_OK;
       }
     }
@@ -90,8 +136,7 @@ class TablePool {
     b->cap = 65536;
     while (b->cap < bytes) b->cap *= 2;
     KVT_HIP(hipMalloc(&b->dev, b->cap));
-    hipError_t e = hipHostMalloc(&b->host, b->cap, hipHostMallocDefault);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&b->last_use, hipEventDisableTiming);
+    const hipError_t e = hipHostMalloc(&b->host, b->cap, hipHostMallocDefault);
     if (e != hipSuccess) {
       destroy(b.get());
       return hip_fail(e, "table buffer allocation");
@@ -111,7 +156,7 @@ class TablePool {
     if (idle_.size() >= 64) {
       TableBuf* victim = idle_.front();
       idle_.erase(idle_.begin());
-      if (victim->used) (void)hipEventSynchronize(victim->last_use);
+      victim->wait_idle();
       destroy(victim);
       delete victim;
     }
@@ -131,9 +176,9 @@ class TablePool {
   static void destroy(TableBuf* b) {
     if (b->dev) (void)hipFree(b->dev);
     if (b->host) (void)hipHostFree(b->host);
-    if (b->last_use) (void)hipEventDestroy(b->last_use);
+    for (TableBuf::Use& u : b->uses) (void)hipEventDestroy(u.done);
+    b->uses.clear();
     b->dev = b->host = nullptr;
-    b->last_use = nullptr;
   }
   std::mutex mu_;
   std::vector<TableBuf*> idle_;

@@ -503,3 +503,47 @@ def test_copy_linear():
     assert kvt_amd.lib().kvt_copy_linear(b.data_ptr(), a.data_ptr(), a.numel(), None) == 0
     torch.cuda.synchronize()
     assert torch.equal(a, b)
+
+
+def test_plan_used_on_two_streams_then_destroyed_while_launches_are_queued():
+    """The chunk table of a destroyed plan goes back to a pool; it must not be handed to the
+    next plan while a kernel queued on ANY stream still reads it."""
+    w = workloads.llama8b_batch(n_layers=24, src_pool=2048, dst_pool=3072, n_req=12, min_tok=500,
+                                max_tok=2500)
+    w2 = workloads.llama8b_batch(n_layers=24, src_pool=2048, dst_pool=3072, n_req=12, min_tok=500,
+                                 max_tok=2500, seed=99)
+    o_lists = _oracle_lists(w)
+    src_layers = _make_caches(w, "src", 71)
+    dst_layers = _make_caches(w, "dst", 72, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    plan, _ = pipeline.build_plan(w, 0)
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    junk = torch.zeros(w.n_layers * stride * 2, dtype=torch.uint8, device="cuda")
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    plan.pack(sc, 0, w.n_layers, packed, stride, a.cuda_stream)
+    done = torch.cuda.Event()
+    done.record(a)
+    b.wait_event(done)
+    # keep stream a busy with a second, independent launch of the same plan, then use the
+    # plan on stream b as well and drop it at once
+    plan.pack(sc, 0, w.n_layers, junk, stride, a.cuda_stream)
+    plan.unpack(dc, 0, w.n_layers, packed, stride, b.cuda_stream)
+    plan.close()
+    others = []
+    for _ in range(4):       # same table size: the pool would hand the same storage out again
+        p2, _ = pipeline.build_plan(w2, 0)
+        p2.ready()
+        others.append(p2)
+    torch.cuda.synchronize()
+    packed_h, junk_h = _host(packed), _host(junk)
+    for l in range(w.n_layers):
+        blob = checkers.oracle_pack(_host(src_layers[l][0]), o_lists[0])
+        assert np.array_equal(packed_h[l * stride:l * stride + len(blob)], blob), l
+        assert np.array_equal(junk_h[l * stride:l * stride + len(blob)], blob), l
+        exp = np.full(w.capacities("dst")[0], 0xA5, dtype=np.uint8)
+        checkers.oracle_unpack(exp, o_lists[0], blob)
+        assert np.array_equal(_host(dst_layers[l][0]), exp), l
+    for p2 in others:
+        p2.close()
