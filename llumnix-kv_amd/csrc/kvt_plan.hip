@@ -277,10 +277,15 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
         bool strided = n_lv > 0 && r.length < kMinChunk && ((r.length | r.src_offset | r.dst_offset | blob) & 15u) == 0;
         for (int k = 0; k < n_lv && strided; ++k)
           strided = ((r.src_stride[lv[k]] | r.dst_stride[lv[k]]) & 15u) == 0;
-        // kernel nest: (outer, inner) = the last two effective levels; an earlier one is cut here
-        const int in_k = n_lv >= 2 ? lv[n_lv - 1] : -1;
-        const int out_k = n_lv >= 2 ? lv[n_lv - 2] : (n_lv == 1 ? lv[0] : -1);
-        const int top_k = n_lv == 3 ? lv[0] : -1;
+        // Kernel nest: the innermost effective level alone when it already spans a slice
+        // (folding more levels into the kernel would only multiply record shapes: outer
+        // strides between blocks are arbitrary), else the innermost two (K and V of a token
+        // inside a token walk). The remaining outer levels are unrolled here.
+        const int last = n_lv > 0 ? lv[n_lv - 1] : -1;
+        const bool two = n_lv >= 2 && static_cast<uint64_t>(r.n[last]) * r.length < kMinChunk;
+        const int in_k = two ? last : -1;
+        const int out_k = two ? lv[n_lv - 2] : last;
+        const int n_host = n_lv - (two ? 2 : 1);          // levels unrolled on the host: 0..2
         const uint64_t n_in = in_k >= 0 ? r.n[in_k] : 1;
         strided = strided && n_in * r.length <= kMaxChunk / 2;
         uint32_t shape = 0;
@@ -305,14 +310,17 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
           const uint32_t group = static_cast<uint32_t>(n_in * r.length);
           max_group = std::max(max_group, group);
           const uint64_t sub_bytes = static_cast<uint64_t>(r.n[out_k]) * group;
-          const uint32_t n_top = top_k >= 0 ? r.n[top_k] : 1;
-          for (uint32_t a = 0; a < n_top; ++a) {
-            spans.push_back(Span{r.src_offset + (top_k >= 0 ? a * r.src_stride[top_k] : 0),
-                                 r.dst_offset + (top_k >= 0 ? a * r.dst_stride[top_k] : 0), blob,
-                                 sub_bytes, group, shape, r.src_stride[out_k], r.dst_stride[out_k],
-                                 static_cast<uint16_t>(t)});
-            blob += sub_bytes;
-          }
+          const int h0 = n_host >= 1 ? lv[0] : -1, h1 = n_host >= 2 ? lv[1] : -1;
+          const uint32_t c0 = h0 >= 0 ? r.n[h0] : 1, c1 = h1 >= 0 ? r.n[h1] : 1;
+          for (uint32_t a = 0; a < c0; ++a)
+            for (uint32_t b = 0; b < c1; ++b) {
+              const uint64_t so = (h0 >= 0 ? a * r.src_stride[h0] : 0) + (h1 >= 0 ? b * r.src_stride[h1] : 0);
+              const uint64_t dof = (h0 >= 0 ? a * r.dst_stride[h0] : 0) + (h1 >= 0 ? b * r.dst_stride[h1] : 0);
+              spans.push_back(Span{r.src_offset + so, r.dst_offset + dof, blob, sub_bytes, group,
+                                   shape, r.src_stride[out_k], r.dst_stride[out_k],
+                                   static_cast<uint16_t>(t)});
+              blob += sub_bytes;
+            }
         } else {
           for (uint32_t a = 0; a < r.n[0]; ++a)
             for (uint32_t b = 0; b < r.n[1]; ++b)

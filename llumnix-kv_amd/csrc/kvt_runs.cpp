@@ -49,6 +49,41 @@ void fold_level(std::vector<kvt_run>& items, int k) {
   items.resize(w);
 }
 
+// The innermost pass straight from the plain ranges: same rule as fold_level(items, 2),
+// without first materialising one 88-byte item per range (a TP-remapping batch has
+// hundreds of thousands of ranges, sixteen or more per run).
+void fold_ranges(const RunList& v, std::vector<kvt_run>& items) {
+  const size_t n = v.size();
+  for (size_t i = 0; i < n;) {
+    kvt_run cur{};
+    cur.src_offset = v[i].src_offset;
+    cur.dst_offset = v[i].dst_offset;
+    cur.length = v[i].length;
+    cur.n[0] = cur.n[1] = cur.n[2] = 1;
+    size_t j = i + 1;
+    if (j < n && v[j].length == cur.length && v[j].src_offset >= cur.src_offset &&
+        v[j].dst_offset >= cur.dst_offset) {
+      const uint64_t ds = v[j].src_offset - cur.src_offset;
+      const uint64_t dd = v[j].dst_offset - cur.dst_offset;
+      uint64_t count = 1;
+      while (j < n && count < 0xFFFFFFFFull && v[j].length == cur.length &&
+             v[j].src_offset >= v[j - 1].src_offset && v[j].dst_offset >= v[j - 1].dst_offset &&
+             v[j].src_offset - v[j - 1].src_offset == ds &&
+             v[j].dst_offset - v[j - 1].dst_offset == dd) {
+        ++count;
+        ++j;
+      }
+      if (count > 1) {
+        cur.n[2] = static_cast<uint32_t>(count);
+        cur.src_stride[2] = ds;
+        cur.dst_stride[2] = dd;
+      }
+    }
+    items.push_back(cur);
+    i = j;
+  }
+}
+
 }  // namespace
 }  // namespace kvt
 
@@ -119,16 +154,8 @@ int kvt_run_lists_compress(const kvt_block_lists* l, kvt_run_lists* out) {
     std::vector<kvt_run> items;
     for (size_t t = 0; t < l->tensors.size(); ++t) {
       items.clear();
-      items.reserve(l->tensors[t].size());
-      for (const kvt_ipc_block& b : l->tensors[t]) {
-        kvt_run r{};
-        r.src_offset = b.src_offset;
-        r.dst_offset = b.dst_offset;
-        r.length = b.length;
-        r.n[0] = r.n[1] = r.n[2] = 1;
-        items.push_back(r);
-      }
-      for (int k = 2; k >= 0; --k) fold_level(items, k);
+      fold_ranges(l->tensors[t], items);
+      for (int k = 1; k >= 0; --k) fold_level(items, k);
       out->tensors[t].insert(out->tensors[t].end(), items.begin(), items.end());
     }
     return KVT_OK;
