@@ -46,7 +46,11 @@ class LoopbackChannel:
             rc, bad = binding.validate_bounds(lists.tensor(t), self.dst_capacity[t], 1)
             if rc != 0:
                 raise binding.KvtError(rc, "rejected invalid copy metadata (range %d)" % bad)
-        self.plan = binding.Plan(self.device, lists, self.src_capacity, self.dst_capacity)
+        if tp_kind == TP_PEQD:
+            source = lists
+        else:   # per-token ranges of a TP remap: fold them back into strided runs
+            source = binding.RunLists.compress(lists)
+        self.plan = binding.Plan(self.device, source, self.src_capacity, self.dst_capacity)
         self.stride = self.plan.layer_bytes
         self._buf = alloc(max(1, n_layers * self.stride))
         self.session = binding.Session(self.plan, self.src_cache, self._buf, self.stride)

@@ -126,3 +126,35 @@ def test_cuda_kernel_sync_over_four_steps():
             val = step + 1 + layer
             assert seen[layer] == (val, val, val * data_size), (step, layer, seen[layer])
         session.close()
+
+
+def test_channel_with_a_tp_remapping_destination():
+    """Same flow with the sender on TP2 and the receiver on TP1: the channel folds the
+    per-token ranges into strided runs before planning."""
+    import checkers
+    from kvt_amd import workloads
+    from test_gpu_pack import _host, _make_caches
+    w = workloads.tp_split("flash", 2, 1, 1, n_layers=2, src_pool=200, dst_pool=300, n_req=3,
+                           min_tok=40, max_tok=600)
+    src_info, dst_info = w.worker_infos()
+    lists, tp_kind = pipeline.parse_batch(w.cache_shape, src_info, dst_info, w.task_bufs())
+    assert tp_kind != 0
+    expect = lists.tensor(0)
+    src_layers = _make_caches(w, "src", 81)
+    dst_layers = _make_caches(w, "dst", 82, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    ch = LoopbackChannel(0, sc, dc, w.capacities("src"), w.capacities("dst"))
+    ch.connect(dst_info)
+    ch.register_data(lists, tp_kind, w.n_layers,
+                     lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+    assert ch.plan.num_strided_chunks > 0
+    for l in range(w.n_layers):
+        ch.send_data(l, None)
+    ch.flush()
+    for l in range(w.n_layers):
+        exp = np.full(w.capacities("dst")[0], 0xA5, dtype=np.uint8)
+        blob = checkers.oracle_pack(_host(src_layers[l][0]), expect)
+        checkers.oracle_unpack(exp, expect, blob)
+        assert np.array_equal(_host(dst_layers[l][0]), exp), l
+    ch.close()
