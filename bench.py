@@ -60,10 +60,11 @@ def build_workload(cfg, scale):
                                  pool=max(512, int(36864 * scale)), n_req=max(2, int(128 * scale))),
                 W.qwen3next_gdn(n_layers=max(2, int(36 * scale)), slots=max(4, int(256 * scale)),
                                 n_req=max(2, int(128 * scale)))]
-    if cfg in (6, 7):
+    if cfg in (6, 7, 8):
         # TP-remapping batches (not among the baseline configurations): config 2's batch with
-        # the sender on TP2 and the receiver on TP1 (6), or TP1 -> TP2 on the ragged layout (7)
-        layout, p_tp, d_tp = ("flash", 2, 1) if cfg == 6 else ("ragged", 1, 2)
+        # the sender on TP2 and the receiver on TP1 (6), TP1 -> TP2 on the ragged layout (7),
+        # TP2 -> TP1 on FlashInfer HND pages (8: per-head rows, whole segments of 4 KiB)
+        layout, p_tp, d_tp = {6: ("flash", 2, 1), 7: ("ragged", 1, 2), 8: ("hnd", 2, 1)}[cfg]
         return [W.tp_split(layout, p_tp, d_tp, 0, n_layers=max(2, int(32 * scale)),
                            src_pool=max(1024, int(16384 * scale)),
                            dst_pool=max(1536, int(24576 * scale)), n_req=max(2, int(64 * scale)),
