@@ -437,6 +437,26 @@ def main():
         out["latency_p50_us"] = round(statistics.median(lat), 2)
         out["latency_note"] = "per request: one pack launch covering all %d layers, GPU time" % w.n_layers
 
+        # layer-by-layer operation (the serving pattern: every layer is packed as soon as the
+        # forward pass has produced it): one event-gated launch per layer on the side stream
+        if w.xform is None:
+            plan0 = first[0][0]
+            sess = kvt.Session(plan0, side.src_cache, packed[0], strides[0])
+            a, b = new_event(), new_event()
+            for rep in range(2):
+                lib.kvt_event_record(a, sh)
+                for l in range(w.n_layers):
+                    sess.save_layer(l, sh)
+                sess.join(sh)
+                lib.kvt_event_record(b, sh)
+            lib.kvt_event_synchronize(b)
+            ms = ev_ms(lib, a, b)
+            pay0 = sum(plan0.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
+            out["per_layer_session"] = {"pack_ms_all_layers": round(ms, 4),
+                                        "pack_gbps": round(2.0 * pay0 / (ms * 1e-3) / 1e9, 1),
+                                        "launches": w.n_layers}
+            sess.close()
+
         # the reference-shaped launchers (one launch per layer, ranges as three int64 arrays
         # resident on the device) and the converting bf16 -> fp8 gather
         if w.xform is None and args.plan == "ranges" and w.elem_dtype == "bf16":
