@@ -455,6 +455,23 @@ def main():
             out["per_layer_session"] = {"pack_ms_all_layers": round(ms, 4),
                                         "pack_gbps": round(2.0 * pay0 / (ms * 1e-3) / 1e9, 1),
                                         "launches": w.n_layers}
+            # the same sequence captured once into a hipGraph and replayed
+            gs = torch.cuda.Stream()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(gs):
+                with torch.cuda.graph(graph, stream=gs):
+                    for l in range(w.n_layers):
+                        sess.save_layer(l, gs.cuda_stream)
+                    sess.join(gs.cuda_stream)
+            for rep in range(2):
+                torch.cuda.synchronize()
+                t_a = time.perf_counter()
+                for _ in range(5):
+                    graph.replay()
+                torch.cuda.synchronize()
+                g_ms = (time.perf_counter() - t_a) / 5 * 1e3
+            out["per_layer_session"]["graph_replay_ms_all_layers"] = round(g_ms, 4)
+            del graph
             sess.close()
 
         # the reference-shaped launchers (one launch per layer, ranges as three int64 arrays
