@@ -9,20 +9,17 @@
 
 using namespace kvt;
 
-extern "C" {
+namespace {
 
-// ------------------------------------------- reference-shaped entry points
-
-static int range_launch_shape(int64_t n, int num_wg, int* wgs) {
+int range_launch_shape(int64_t n, int num_wg, int* wgs) {
   if (n > 0x7FFFFFFFll) return fail(KVT_ERR_INVALID, "too many ranges");
   int w = num_wg > 0 ? num_wg : static_cast<int>(std::min<int64_t>(n, 1 << 20));
   *wgs = std::max(1, w);
   return KVT_OK;
 }
 
-static int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so,
-                         const int64_t* dof, const int64_t* len, int64_t n, int num_wg,
-                         int threads_per_wg, void* stream) {
+int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, const int64_t* dof,
+                  const int64_t* len, int64_t n, int num_wg, int threads_per_wg, void* stream) {
   (void)threads_per_wg;  // workgroups are always 256 lanes (4 wavefronts)
   if (n == 0) return KVT_OK;
   if (n < 0 || !src || !dst || !so || !dof || !len)
@@ -39,41 +36,12 @@ static int launch_ranges(bool convert, const void* src, void* dst, const int64_t
   return KVT_OK;
 }
 
-int kvt_launch_copy_d2h_direct(const void* gpu_src_base, void* dst, const int64_t* src_offsets,
-                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
-                               int num_wg, int threads_per_wg, void* stream) {
-  return guarded([&]() {
-    return launch_ranges(false, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
-                         threads_per_wg, stream);
-  });
-}
-
-int kvt_launch_copy_h2d_direct(const void* src, void* gpu_dst_base, const int64_t* src_offsets,
-                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
-                               int num_wg, int threads_per_wg, void* stream) {
-  return guarded([&]() {
-    return launch_ranges(false, src, gpu_dst_base, src_offsets, dst_offsets, lengths, n, num_wg,
-                         threads_per_wg, stream);
-  });
-}
-
-int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
-                                    const int64_t* src_offsets, const int64_t* dst_offsets,
-                                    const int64_t* lengths, int64_t n, int num_wg,
-                                    int threads_per_wg, void* stream) {
-  return guarded([&]() {
-    return launch_ranges(true, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
-                         threads_per_wg, stream);
-  });
-}
-
 // Shared body of the two "handle data" entry points. `halve`: converting
 // gather (contiguous side advances by length / 2, lengths passed to the kernel
 // are element counts).
-static int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks,
-                       uint64_t n, uint64_t tensor_data_size, int direction, bool halve,
-                       int device, void* stream, int64_t* dev_meta, int64_t* host_meta,
-                       int64_t max_block_num) {
+int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks, uint64_t n,
+                uint64_t tensor_data_size, int direction, bool halve, int device, void* stream,
+                int64_t* dev_meta, int64_t* host_meta, int64_t max_block_num) {
   if (n == 0) return KVT_OK;
   if (!tensor_buf || !layer_gpu_ptr || !blocks || !dev_meta || !host_meta)
     return fail(KVT_ERR_INVALID, "copy_handle_data: null argument");
@@ -132,6 +100,38 @@ static int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
   return KVT_OK;
 }
 
+}  // namespace
+
+extern "C" {
+
+int kvt_launch_copy_d2h_direct(const void* gpu_src_base, void* dst, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(false, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+int kvt_launch_copy_h2d_direct(const void* src, void* gpu_dst_base, const int64_t* src_offsets,
+                               const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
+                               int num_wg, int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(false, src, gpu_dst_base, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
+int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
+                                    const int64_t* src_offsets, const int64_t* dst_offsets,
+                                    const int64_t* lengths, int64_t n, int num_wg,
+                                    int threads_per_wg, void* stream) {
+  return guarded([&]() {
+    return launch_ranges(true, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
+                         threads_per_wg, stream);
+  });
+}
+
 int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
                                      const kvt_ipc_block* blocks, uint64_t n,
                                      uint64_t tensor_data_size, int direction, int device,
@@ -152,4 +152,5 @@ int kvt_copy_d2h_bf16_to_fp8(void* tensor_buf, const void* layer_gpu_ptr,
                        KVT_COPY_D2H, true, device, stream, dev_meta, host_meta, max_block_num);
   });
 }
+
 }  // extern "C"
