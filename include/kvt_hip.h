@@ -12,6 +12,10 @@
  *     base address, exactly like IpcBlock offsets in the reference.
  *   - every GPU entry point fails with KVT_ERR_NO_DEVICE when no gfx950 device
  *     is usable; there is no CPU fallback inside this library.
+ *   - threads: parsers, caches and plans are immutable once created and may be
+ *     used from any number of threads at once (a plan may be launched on several
+ *     streams); list containers (kvt_block_lists, kvt_run_lists), sessions and
+ *     stagers belong to one thread at a time unless stated otherwise.
  *
  * Each declaration cites the reference interface it replaces (paths relative
  * to the reference checkout).
@@ -358,7 +362,8 @@ int kvt_session_wait_layer(kvt_session* s, uint32_t layer);
 /* Makes `stream` wait for every pack issued so far (joins the side stream
  * back; required before ending a capture that included save_layer calls). */
 int kvt_session_join(kvt_session* s, void* stream);
-/* hipStream_t of the side stream (for tests / profiling). */
+/* hipStream_t of the side stream (for tests / profiling). Threads: save_layer /
+ * join from the thread that drives the forward pass, wait_layer from any thread. */
 void* kvt_session_side_stream(kvt_session* s);
 
 /* ------------------------------------ pinned-host staging (KVStore path) */
@@ -368,7 +373,9 @@ void* kvt_session_side_stream(kvt_session* s);
  * the unpack of L). Stands where the reference's KVStore backends hand packed
  * layers to a host-side store                   blade_kvt/hybrid_connector/kvsbackend.py:268-357,
  *                                               blade_kvt/hybrid_connector/file_backend.py:222-283.
- * slot_bytes bounds one transfer; n_slots >= 2. */
+ * slot_bytes bounds one transfer; n_slots >= 2. One stager serves one caller
+ * thread at a time (save / load calls of different threads must not overlap);
+ * a saving and a loading side each take their own stager. */
 typedef struct kvt_stager kvt_stager;
 int kvt_stager_create(int device, uint64_t slot_bytes, uint32_t n_slots, kvt_stager** out);
 void kvt_stager_destroy(kvt_stager* s);

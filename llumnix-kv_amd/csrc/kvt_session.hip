@@ -32,6 +32,7 @@ struct kvt_stager {
   std::vector<hipEvent_t> slot_done;
   hipEvent_t fence = nullptr;
 };
+
 extern "C" {
 
 // ----------------------------------------------------------------- session
@@ -47,7 +48,8 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
     DeviceGuard g;
     if (int rc = g.enter(plan->device)) return rc;
     if (int rc = kvt_plan_ready(plan)) return rc;  // save_layer may run inside a stream capture
-    std::unique_ptr<kvt_session> s(new kvt_session());
+    // destroyed through kvt_session_destroy on any early return: stream and events included
+    std::unique_ptr<kvt_session, void (*)(kvt_session*)> s(new kvt_session(), kvt_session_destroy);
     s->plan = plan;
     s->cache = cache;
     s->packed = packed;
@@ -131,7 +133,7 @@ int kvt_stager_create(int device, uint64_t slot_bytes, uint32_t n_slots, kvt_sta
     if (int rc = check_device(device)) return rc;
     DeviceGuard g;
     if (int rc = g.enter(device)) return rc;
-    std::unique_ptr<kvt_stager> s(new kvt_stager());
+    std::unique_ptr<kvt_stager, void (*)(kvt_stager*)> s(new kvt_stager(), kvt_stager_destroy);
     s->device = device;
     s->slot_bytes = round_up(slot_bytes, 4096);
     s->n_slots = n_slots;
@@ -270,4 +272,5 @@ int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats
     return KVT_OK;
   });
 }
+
 }  // extern "C"
