@@ -102,6 +102,20 @@ class DeviceSide:
         self.dst_cache = kvt.Cache(0, self.dst, w.capacities("dst"))
 
 
+class stdout_to_stderr:
+    """The compiled reference announces every environment variable it reads on stdout
+    (kvtransfer/src/envcfg.cpp:15); this file's stdout carries exactly one JSON line."""
+
+    def __enter__(self):
+        sys.stdout.flush()
+        self.saved = os.dup(1)
+        os.dup2(2, 1)
+
+    def __exit__(self, *exc):
+        os.dup2(self.saved, 1)
+        os.close(self.saved)
+
+
 def ev_ms(lib, a, b):
     ms = C.c_float()
     rc = lib.kvt_event_elapsed_ms(a, b, C.byref(ms))
@@ -399,6 +413,37 @@ def main():
                       (L, w.n_layers, len(w.tasks), parse_s * 1e3, pack_s * 1e3, unpack_s * 1e3),
             "host_cores_available": os.cpu_count(),
         }
+        # ParseBlock alone for the whole batch: the reference's own functions (compiled from its
+        # sources into oracle/_ref where that was possible), the oracle, and the product
+        pb = {}
+        if checkers.ref() is not None and not w.xform:
+            tt = []
+            with stdout_to_stderr():
+                for _ in range(5):
+                    a = time.perf_counter()
+                    rc, _outs = checkers.ref_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
+                    tt.append(time.perf_counter() - a)
+                    assert rc == 0
+            pb["reference_ms"] = round(sorted(tt)[2] * 1e3, 3)
+        tt = []
+        for _ in range(5):
+            a = time.perf_counter()
+            rc, _outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
+            tt.append(time.perf_counter() - a)
+        pb["oracle_ms"] = round(sorted(tt)[2] * 1e3, 3)
+        parser = kvt.Parser(pid, s_info, d_info, valid, tps, tpr)
+        tt = []
+        for _ in range(5):
+            lst = kvt.BlockLists()
+            a = time.perf_counter()
+            for t in cpu_tasks:
+                parser.parse(t.struct, lst)
+            tt.append(time.perf_counter() - a)
+            lst.close()
+        pb["product_ms"] = round(sorted(tt)[2] * 1e3, 3)
+        pb["note"] = "%d requests, median of 5, one thread; output copies included" % len(cpu_tasks)
+        out["cpu_baseline"]["parse_block"] = pb
+
         # all host cores, threads striding over layers (not the reference's threading model)
         nthr = min(16, os.cpu_count() or 1, L)
         if nthr > 1 and w.xform is None and w.n_tensors == 1:
