@@ -104,6 +104,9 @@ void kvt_run_lists_destroy(kvt_run_lists* l);
 void kvt_run_lists_clear(kvt_run_lists* l);
 uint32_t kvt_run_lists_num_tensors(const kvt_run_lists* l);
 int kvt_run_lists_view(const kvt_run_lists* l, uint32_t tensor, const kvt_run** data, uint64_t* n);
+/* Appends runs that arrived from elsewhere (e.g. a peer that sends runs instead
+ * of plain ranges). Runs with a zero count or length are refused. */
+int kvt_run_lists_append(kvt_run_lists* l, uint32_t tensor, const kvt_run* runs, uint64_t n);
 /* Number of ranges / bytes the runs of one tensor expand to. */
 int kvt_run_lists_totals(const kvt_run_lists* l, uint32_t tensor, uint64_t* n_ranges,
                          uint64_t* n_bytes);

@@ -112,6 +112,20 @@ int kvt_run_lists_view(const kvt_run_lists* l, uint32_t tensor, const kvt_run** 
   return KVT_OK;
 }
 
+int kvt_run_lists_append(kvt_run_lists* l, uint32_t tensor, const kvt_run* runs, uint64_t n) {
+  return guarded([&]() -> int {
+    if (!l || (!runs && n)) return fail(KVT_ERR_INVALID, "kvt_run_lists_append: null argument");
+    if (tensor >= KVT_MAX_TENSORS)
+      return fail(KVT_ERR_OUT_OF_RANGE, "kvt_run_lists_append: tensor index out of range");
+    for (uint64_t i = 0; i < n; ++i)
+      if (runs[i].length == 0 || runs[i].n[0] == 0 || runs[i].n[1] == 0 || runs[i].n[2] == 0)
+        return fail(KVT_ERR_INVALID, "kvt_run_lists_append: empty run");
+    if (l->tensors.size() <= tensor) l->tensors.resize(tensor + 1);
+    l->tensors[tensor].insert(l->tensors[tensor].end(), runs, runs + n);
+    return KVT_OK;
+  });
+}
+
 int kvt_run_lists_totals(const kvt_run_lists* l, uint32_t tensor, uint64_t* n_ranges,
                          uint64_t* n_bytes) {
   if (!l) return fail(KVT_ERR_INVALID, "kvt_run_lists_totals: null argument");

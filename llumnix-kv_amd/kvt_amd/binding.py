@@ -66,6 +66,7 @@ SIGNATURES = {
     "kvt_run_lists_clear": (None, [_vp]),
     "kvt_run_lists_num_tensors": (_u32, [_vp]),
     "kvt_run_lists_view": (_int, [_vp, _u32, _P(_vp), _P(_u64)]),
+    "kvt_run_lists_append": (_int, [_vp, _u32, _vp, _u64]),
     "kvt_run_lists_totals": (_int, [_vp, _u32, _P(_u64), _P(_u64)]),
     "kvt_parse_block_runs": (_int, [_vp, _P(Task), _vp]),
     "kvt_run_lists_expand": (_int, [_vp, _vp]),
@@ -307,6 +308,11 @@ class RunLists:
             return np.zeros(0, dtype=RUN_DTYPE)
         buf = (C.c_uint8 * (n.value * RUN_DTYPE.itemsize)).from_address(data.value)
         return np.frombuffer(buf, dtype=RUN_DTYPE).copy()
+
+    def append(self, t, runs):
+        """runs: structured array of RUN_DTYPE"""
+        a = np.ascontiguousarray(runs, dtype=RUN_DTYPE)
+        check(lib().kvt_run_lists_append(self.h, t, a.ctypes.data, len(a)))
 
     def totals(self, t):
         """-> (ranges, bytes) the runs of tensor t expand to"""

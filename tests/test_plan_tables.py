@@ -181,3 +181,48 @@ def test_run_plan_rejects_runs_beyond_capacity():
         kvt_amd.lib().kvt_pack.restype
         p = kvt_amd.Plan(-1, R, [480], [480])
         kvt_amd.binding.check(kvt_amd.lib().kvt_pack(p.h, None, 0, 1, None, 0, None))
+
+
+@pytest.mark.parametrize("seed", range(25))
+def test_run_plan_tables_for_random_synthetic_runs(seed):
+    """Runs that no parser would emit: odd lengths, zero strides on the source side,
+    three full levels, lengths around the 4 KiB limit, many distinct shapes (more than the
+    16 the kernel takes by value: the rest must fall back to plain chunks)."""
+    rng = np.random.default_rng(seed)
+    cap = 1 << 22
+    runs = np.zeros(int(rng.integers(1, 40)), dtype=kvt_amd.binding.RUN_DTYPE)
+    d_cursor = 0
+    for r in runs:
+        length = int(rng.choice([16, 48, 256, 1000, 1024, 4080, 4096, 5000, 20]))
+        n = [int(rng.integers(1, 4)), int(rng.integers(1, 9)), int(rng.integers(1, 4))]
+        unit = 16 if rng.random() < 0.8 else 4
+        # destination: dense nest laid out from a running cursor, so that ranges never overlap
+        d2 = (length + unit - 1) // unit * unit + unit * int(rng.integers(0, 3))
+        d1 = d2 * n[2] + unit * int(rng.integers(0, 3))
+        d0 = d1 * n[1] + unit * int(rng.integers(0, 3))
+        r["length"], r["n"] = length, n
+        r["dst_offset"] = d_cursor
+        r["dst_stride"] = [d0, d1, d2]
+        d_cursor += d0 * n[0] + 64
+        # source: anything inside the buffer, repeats allowed (strides may be zero)
+        s_str = [unit * int(rng.integers(0, 600)), unit * int(rng.integers(0, 80)),
+                 unit * int(rng.integers(0, 40))]
+        span = sum(s * (k - 1) for s, k in zip(s_str, n)) + length
+        r["src_offset"] = unit * int(rng.integers(0, (cap - span) // unit))
+        r["src_stride"] = s_str
+    assert d_cursor < cap
+    R = kvt_amd.RunLists()
+    R.append(0, runs)
+    expect = R.expand().tensor(0)
+    from test_runs import numpy_expand
+    assert np.array_equal(expect, numpy_expand(runs))
+    for chunk in (0, 4096, 65536):
+        plan = _host_plan(R, [cap], [cap], chunk)
+        _check_tables(plan, [expect], [cap], [cap], seed)
+
+
+def test_run_lists_append_refuses_empty_runs():
+    bad = np.zeros(1, dtype=kvt_amd.binding.RUN_DTYPE)
+    bad["length"], bad["n"] = 16, [[1, 0, 1]]
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.RunLists().append(0, bad)
