@@ -135,3 +135,27 @@ def test_strided_plan_refuses_misaligned_blob_positions():
     torch.cuda.synchronize()
     blob = checkers.oracle_pack(_host(layers[0][0]), _oracle_ranges(w)[0])
     assert np.array_equal(_host(out)[32:32 + len(blob)], blob)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_synthetic_runs_on_the_gpu(seed):
+    """Runs no parser would emit (odd lengths, zero source strides, three levels, more record
+    shapes than the kernel takes): gather and scatter against the oracle on the expanded list."""
+    cap = 1 << 22
+    runs = cases.gen_synthetic_runs(seed, cap, kvt_amd.binding.RUN_DTYPE)
+    R = kvt_amd.RunLists()
+    R.append(0, runs)
+    expect = R.expand().tensor(0)
+    plan = kvt_amd.Plan(0, R, [cap], [cap], chunk_bytes=[0, 4096, 65536][seed % 3])
+    src = _dev_bytes(cap, 700 + seed, "u8")
+    dst = torch.full((cap,), 0xA5, dtype=torch.uint8, device="cuda")
+    sc, dc = kvt_amd.Cache(0, [[src]], [cap]), kvt_amd.Cache(0, [[dst]], [cap])
+    packed = torch.zeros(max(plan.layer_bytes, 16), dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, 1, packed, plan.layer_bytes)
+    plan.unpack(dc, 0, 1, packed, plan.layer_bytes)
+    torch.cuda.synchronize()
+    blob = checkers.oracle_pack(_host(src), expect)
+    assert np.array_equal(_host(packed)[:len(blob)], blob)
+    exp = np.full(cap, 0xA5, dtype=np.uint8)
+    checkers.oracle_unpack(exp, expect, blob)
+    assert np.array_equal(_host(dst), exp)

@@ -188,29 +188,8 @@ def test_run_plan_tables_for_random_synthetic_runs(seed):
     """Runs that no parser would emit: odd lengths, zero strides on the source side,
     three full levels, lengths around the 4 KiB limit, many distinct shapes (more than the
     16 the kernel takes by value: the rest must fall back to plain chunks)."""
-    rng = np.random.default_rng(seed)
     cap = 1 << 22
-    runs = np.zeros(int(rng.integers(1, 40)), dtype=kvt_amd.binding.RUN_DTYPE)
-    d_cursor = 0
-    for r in runs:
-        length = int(rng.choice([16, 48, 256, 1000, 1024, 4080, 4096, 5000, 20]))
-        n = [int(rng.integers(1, 4)), int(rng.integers(1, 9)), int(rng.integers(1, 4))]
-        unit = 16 if rng.random() < 0.8 else 4
-        # destination: dense nest laid out from a running cursor, so that ranges never overlap
-        d2 = (length + unit - 1) // unit * unit + unit * int(rng.integers(0, 3))
-        d1 = d2 * n[2] + unit * int(rng.integers(0, 3))
-        d0 = d1 * n[1] + unit * int(rng.integers(0, 3))
-        r["length"], r["n"] = length, n
-        r["dst_offset"] = d_cursor
-        r["dst_stride"] = [d0, d1, d2]
-        d_cursor += d0 * n[0] + 64
-        # source: anything inside the buffer, repeats allowed (strides may be zero)
-        s_str = [unit * int(rng.integers(0, 600)), unit * int(rng.integers(0, 80)),
-                 unit * int(rng.integers(0, 40))]
-        span = sum(s * (k - 1) for s, k in zip(s_str, n)) + length
-        r["src_offset"] = unit * int(rng.integers(0, (cap - span) // unit))
-        r["src_stride"] = s_str
-    assert d_cursor < cap
+    runs = cases.gen_synthetic_runs(seed, cap, kvt_amd.binding.RUN_DTYPE)
     R = kvt_amd.RunLists()
     R.append(0, runs)
     expect = R.expand().tensor(0)
