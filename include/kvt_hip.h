@@ -187,8 +187,10 @@ void kvt_plan_destroy(kvt_plan* p);
  * entry per <= chunk_bytes of payload, the per-token arithmetic done by the
  * kernel); all others are expanded to plain chunks. Same pack / unpack entry
  * points and the same packed layout as a plan made from the expanded lists.
- * Layer base pointers, the packed buffer and blob positions given to
- * kvt_pack_at / kvt_unpack_at must be 16-byte aligned for such a plan. */
+ * With 16-byte aligned layer base pointers, packed buffer, layer stride and blob
+ * positions a strided entry moves one 16-byte vector per lane; 4-byte alignment
+ * (a blob inside a layer message) is served by a slower word-wise path; anything
+ * less is refused with KVT_ERR_INVALID. */
 int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
                          const uint64_t* dst_capacity, uint32_t chunk_bytes, kvt_plan** out);
 /* Table entries that stayed strided (0 for a plan made from plain lists). */
@@ -197,7 +199,7 @@ uint64_t kvt_plan_num_strided_chunks(const kvt_plan* p);
  * its two tables on the host and cannot be launched. *chunks = 2 * n_chunks
  * entries of 32 bytes {u64 cache, u64 packed, u32 len, u16 tensor, u16 t0,
  * u32 shape, u32 0}: pack order first, then unpack order; *shapes = 16 record
- * shapes of 48 bytes {u32 vlen16, u32 inv, u32 n_inner, u32 0, u64 outer[2],
+ * shapes of 48 bytes {u32 vlen16, u32 inv, u32 n_inner, u32 inv_words, u64 outer[2],
  * u64 inner[2]} ([0] source side, [1] destination side). Entry semantics: see
  * csrc/kvt_device.h. Borrowed pointers, valid until the plan is destroyed. */
 #define KVT_DEVICE_NONE (-1)

@@ -39,7 +39,8 @@ struct XformDev {
 // (per token: the outer step; K and V of one token: the inner step).
 struct StrideShape {
   uint32_t vlen, inv_vlen;     // inv_vlen = floor(2^32 / vlen) + 1, exact for operands < 2^32 / vlen
-  uint32_t n_inner, reserved;
+  uint32_t n_inner;
+  uint32_t inv_wlen;           // the same reciprocal for the record length in 4-byte words (4 * vlen)
   uint64_t outer[2], inner[2];  // [0] = source side (pack), [1] = destination side (unpack)
 };
 constexpr uint32_t kMaxShapes = 16;
@@ -51,7 +52,7 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, hipStream_t stream);
+                                 const StrideTable& shapes, bool words, hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

@@ -86,9 +86,12 @@ __global__ __launch_bounds__(kThreads) void copy_chunks_kernel(
 // the token -> offset arithmetic of the TP-remapping layouts (one short range
 // per token, per head, K and V) is evaluated here, per 16-byte vector, instead
 // of being materialised as one table entry per range. Contiguous chunks
-// (shape 0) take the plain path. Everything a strided chunk touches is 16-byte
-// aligned (checked on the host).
-template <bool PACK>
+// (shape 0) take the plain path. Cache offsets, strides and record lengths of
+// strided chunks are multiples of 16 by construction; WORDS = false additionally
+// needs 16-byte aligned base pointers and blob positions (one vector per lane),
+// WORDS = true moves 4-byte words instead (a blob inside a received layer
+// message sits at 4 or 12 modulo 16; that path is PCIe-bound anyway).
+template <bool PACK, bool WORDS>
 __global__ __launch_bounds__(kThreads) void strided_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
@@ -110,20 +113,37 @@ __global__ __launch_bounds__(kThreads) void strided_chunks_kernel(
       copy_slice(cache + off, pk, len, threadIdx.x);
     return;
   }
-  if (threadIdx.x >= (len >> 4)) return;
   const StrideShape& s = shapes.shape[c.shape - 1u];
-  const uint32_t v = (off >> 4) + threadIdx.x;  // vector index inside the chunk, < 2^15
-  const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
-  const uint32_t col = v - rec * s.vlen;
-  const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
-  const uint32_t i = rec - o * s.n_inner;
-  const uint64_t at = o * s.outer[PACK ? 0 : 1] + i * s.inner[PACK ? 0 : 1] + (col << 4);
-  u32x4* cv = reinterpret_cast<u32x4*>(cache + at);
-  u32x4* pv = reinterpret_cast<u32x4*>(pk) + threadIdx.x;
-  if (PACK)
-    __builtin_nontemporal_store(__builtin_nontemporal_load(cv), pv);
-  else
-    __builtin_nontemporal_store(__builtin_nontemporal_load(pv), cv);
+  const uint64_t outer = s.outer[PACK ? 0 : 1], inner = s.inner[PACK ? 0 : 1];
+  if (!WORDS) {
+    if (threadIdx.x >= (len >> 4)) return;
+    const uint32_t v = (off >> 4) + threadIdx.x;  // vector index inside the chunk, < 2^15
+    const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
+    const uint32_t col = v - rec * s.vlen;
+    const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
+    const uint32_t i = rec - o * s.n_inner;
+    u32x4* cv = reinterpret_cast<u32x4*>(cache + o * outer + i * inner + (col << 4));
+    u32x4* pv = reinterpret_cast<u32x4*>(pk) + threadIdx.x;
+    if (PACK)
+      __builtin_nontemporal_store(__builtin_nontemporal_load(cv), pv);
+    else
+      __builtin_nontemporal_store(__builtin_nontemporal_load(pv), cv);
+  } else {
+    const uint32_t wlen = s.vlen << 2;  // record length in words, < 1024
+    for (uint32_t t = threadIdx.x; t < (len >> 2); t += kThreads) {
+      const uint32_t w = (off >> 2) + t;          // word index inside the chunk, < 2^17
+      const uint32_t rec = __umulhi(w, s.inv_wlen);
+      const uint32_t col = w - rec * wlen;
+      const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
+      const uint32_t i = rec - o * s.n_inner;
+      uint32_t* cw = reinterpret_cast<uint32_t*>(cache + o * outer + i * inner + (col << 2));
+      uint32_t* pw = reinterpret_cast<uint32_t*>(pk) + t;
+      if (PACK)
+        *pw = *cw;
+      else
+        *cw = *pw;
+    }
+  }
 }
 
 // HND <-> NHD page transform. A chunk covers tokens [t0, t0 + len/(heads*row))
@@ -283,18 +303,19 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, hipStream_t stream) {
+                                 const StrideTable& shapes, bool words, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const dim3 grid(round8(n_slices), n_layers);
-  if (pack)
-    hipLaunchKernelGGL((strided_chunks_kernel<true>), grid, dim3(kThreads), 0, stream, chunks,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs, shapes);
-  else
-    hipLaunchKernelGGL((strided_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs, shapes);
+#define KVT_LAUNCH_STRIDED(P, W)                                                                \
+  hipLaunchKernelGGL((strided_chunks_kernel<P, W>), grid, dim3(kThreads), 0, stream, chunks,   \
+                     n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,           \
+                     layer_stride, blobs, shapes)
+  if (pack && !words) KVT_LAUNCH_STRIDED(true, false);
+  else if (pack) KVT_LAUNCH_STRIDED(true, true);
+  else if (!words) KVT_LAUNCH_STRIDED(false, false);
+  else KVT_LAUNCH_STRIDED(false, true);
+#undef KVT_LAUNCH_STRIDED
   return hipGetLastError();
 }
 

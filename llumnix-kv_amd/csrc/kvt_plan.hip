@@ -294,6 +294,7 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
           sh.vlen = static_cast<uint32_t>(r.length >> 4);
           sh.inv_vlen = static_cast<uint32_t>((1ull << 32) / sh.vlen) + 1u;
           sh.n_inner = static_cast<uint32_t>(n_in);
+          sh.inv_wlen = static_cast<uint32_t>((1ull << 32) / (4u * sh.vlen)) + 1u;
           sh.outer[0] = r.src_stride[out_k];
           sh.outer[1] = r.dst_stride[out_k];
           sh.inner[0] = in_k >= 0 ? r.src_stride[in_k] : 0;
@@ -467,20 +468,21 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   }
   const Chunk* table = p->dev_chunks + (pack ? 0 : p->n_chunks);
   const uint32_t n = static_cast<uint32_t>(p->n_chunks);
+  bool words = false;  // strided chunks moved as 4-byte words instead of 16-byte vectors
   if (p->strided) {
-    if ((reinterpret_cast<uintptr_t>(packed) | layer_stride) & 15u)
-      return fail(KVT_ERR_INVALID, "a strided plan needs a 16-byte aligned packed buffer and stride");
-    for (uint32_t t = 0; t < p->n_tensors; ++t)
-      if (blobs.off[t] & 15u)
-        return fail(KVT_ERR_INVALID, "a strided plan needs 16-byte aligned blob offsets");
-    if (!cache->aligned16)
-      return fail(KVT_ERR_INVALID, "a strided plan needs 16-byte aligned layer tensors");
+    uint64_t mis = reinterpret_cast<uintptr_t>(packed) | layer_stride | (cache->aligned16 ? 0 : 4);
+    for (uint32_t t = 0; t < p->n_tensors; ++t) mis |= blobs.off[t];
+    if ((mis & 3u) || !cache->aligned4)
+      return fail(KVT_ERR_INVALID,
+                  "a strided plan needs 4-byte aligned layer tensors, packed buffer, stride and "
+                  "blob offsets (16-byte aligned ones take the fast path)");
+    words = (mis & 15u) != 0;
   }
   const hipError_t e =
       p->strided ? launch_strided_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                          p->n_tensors, first_layer, n_layers,
                                          static_cast<uint8_t*>(packed), layer_stride, blobs,
-                                         p->shapes, s) :
+                                         p->shapes, words, s) :
       p->xform ? launch_xform_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                      first_layer, n_layers, static_cast<uint8_t*>(packed),
                                      layer_stride, blobs, p->xdev, s)

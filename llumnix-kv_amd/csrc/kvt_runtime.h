@@ -199,6 +199,7 @@ struct kvt_cache {
   std::vector<void*> host_ptrs;
   uint8_t** dev_ptrs = nullptr;
   bool aligned16 = true;  // every layer tensor starts on a 16-byte boundary
+  bool aligned4 = true;   // ... on a 4-byte boundary
 };
 
 struct kvt_plan {

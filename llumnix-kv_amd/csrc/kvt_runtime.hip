@@ -78,6 +78,7 @@ int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, u
     for (uint64_t i = 0; i < n; ++i) {
       c->host_ptrs[i] = const_cast<void*>(ptrs[i]);
       if (reinterpret_cast<uintptr_t>(ptrs[i]) & 15u) c->aligned16 = false;
+      if (reinterpret_cast<uintptr_t>(ptrs[i]) & 3u) c->aligned4 = false;
     }
     KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c->dev_ptrs), n * sizeof(void*)));
     const hipError_t e =

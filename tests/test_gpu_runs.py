@@ -121,20 +121,36 @@ def test_pack_of_random_cases_of_every_remapping_parser(parser):
     assert done >= 4
 
 
-def test_strided_plan_refuses_misaligned_blob_positions():
-    w = workloads.tp_split("flash", 2, 1, 0, n_layers=1, src_pool=64, dst_pool=64, n_req=1,
-                           min_tok=100, max_tok=100)
+def test_strided_plan_with_word_aligned_and_misaligned_blob_positions():
+    """16-byte aligned positions: one vector per lane; 4-byte aligned ones (a blob inside a
+    layer message): word-wise path, same bytes; anything else is refused."""
+    w = workloads.tp_split("flash", 2, 1, 0, n_layers=2, src_pool=64, dst_pool=64, n_req=2,
+                           min_tok=100, max_tok=300)
     plan, _ = pipeline.build_plan_runs(w, 0)
     assert plan.num_strided_chunks > 0
+    o_runs = _oracle_ranges(w)[0]
     layers = _make_caches(w, "src", 5)
     sc = kvt_amd.Cache(0, layers, w.capacities("src"))
+    for off, stride_pad in ((32, 0), (4, 0), (12, 4), (44, 8)):
+        stride = plan.layer_bytes + 64 + stride_pad
+        out = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+        plan.pack_at(sc, 0, w.n_layers, out, stride, [off] + [0] * 7)
+        dst_layers = _make_caches(w, "dst", 6, fill=False)
+        dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+        plan.unpack_at(dc, 0, w.n_layers, out, stride, [off] + [0] * 7)
+        torch.cuda.synchronize()
+        out_h = _host(out)
+        for l in range(w.n_layers):
+            blob = checkers.oracle_pack(_host(layers[l][0]), o_runs)
+            assert np.array_equal(out_h[l * stride + off: l * stride + off + len(blob)], blob), (off, l)
+            exp = np.full(w.capacities("dst")[0], 0xA5, dtype=np.uint8)
+            checkers.oracle_unpack(exp, o_runs, blob)
+            assert np.array_equal(_host(dst_layers[l][0]), exp), (off, l)
     out = torch.zeros(plan.layer_bytes + 64, dtype=torch.uint8, device="cuda")
     with pytest.raises(kvt_amd.KvtError):
-        plan.pack_at(sc, 0, 1, out, 0, [4] + [0] * 7)
-    plan.pack_at(sc, 0, 1, out, 0, [32] + [0] * 7)
-    torch.cuda.synchronize()
-    blob = checkers.oracle_pack(_host(layers[0][0]), _oracle_ranges(w)[0])
-    assert np.array_equal(_host(out)[32:32 + len(blob)], blob)
+        plan.pack_at(sc, 0, 1, out, 0, [1] + [0] * 7)
+    with pytest.raises(kvt_amd.KvtError):
+        plan.pack_at(sc, 0, 1, out.data_ptr() + 2, 0, [0] * 8)
 
 
 @pytest.mark.parametrize("seed", range(8))

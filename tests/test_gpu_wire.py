@@ -180,3 +180,52 @@ def test_block_objects_save_and_load_equal_kvcache_colon_blkid():
         exp = torch.zeros_like(kv[l])
         exp[:, torch.as_tensor(dst_ids, device="cuda")] = kv[l][:, torch.as_tensor(src_ids, device="cuda")]
         assert torch.equal(new[l].view(torch.int16), exp.view(torch.int16)), l
+
+
+def test_framed_layers_of_a_tp_remapping_batch_with_run_plans():
+    """Sender: ParseBlock in run form, frame metadata = the expanded ranges, blob packed by the
+    strided kernel straight into the pinned frame. Receiver: ranges off the frame folded back
+    into runs, unpack straight out of the frame (blob at 4 or 12 modulo 16: word-wise path)."""
+    w = workloads.tp_split("flash", 2, 1, 1, n_layers=2, src_pool=160, dst_pool=240, n_req=3,
+                           min_tok=60, max_tok=500)
+    src, dst = w.worker_infos()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, src, dst)
+    rc, outs = checkers.oracle_parse(pid, src, dst, valid, tps, tpr, w.task_bufs())
+    assert rc == 0 and kind != 0
+    o_runs = outs[0]
+    plan, runs = pipeline.build_plan_runs(w, 0)
+    lists = runs.expand()
+    assert np.array_equal(lists.tensor(0), o_runs)
+    src_layers = _make_caches(w, "src", 91)
+    dst_layers = _make_caches(w, "dst", 92, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    lay = binding.wire_layout_of(WIRE_RDMA_STAGED, lists)
+    assert lay.blob_offset[0] % 16 in (4, 12)
+    stager = kvt_amd.Stager(0, lay.total_bytes, 2)
+    stream = torch.cuda.Stream()
+    for l in range(w.n_layers):
+        slot = l % 2
+        binding.wire_write_frame(WIRE_RDMA_STAGED, stager.slot_ptr(slot), stager.slot_bytes, 7, l,
+                                 lists)
+        plan.pack_at(sc, l, 1, stager.slot_ptr(slot), 0, list(lay.blob_offset), stream.cuda_stream)
+        stream.synchronize()
+        frame = stager.slot_array(slot, lay.total_bytes).tobytes()
+        blob = checkers.oracle_pack(_host(src_layers[l][0]), o_runs)
+        assert frame == wo.staged_write(7, l, [tuple(int(v) for v in r) for r in o_runs],
+                                        blob.tobytes())
+        # receiver
+        rc, reqid, layer, rlists, rlay = binding.wire_parse_frame(
+            WIRE_RDMA_STAGED, stager.slot_ptr(slot), lay.total_bytes, 1)
+        assert rc == 0 and (reqid, layer) == (7, l)
+        rplan = kvt_amd.Plan(0, kvt_amd.RunLists.compress(rlists), [2**64 - 1],
+                             w.capacities("dst"))
+        assert rplan.num_strided_chunks > 0
+        rplan.unpack_at(dc, l, 1, stager.slot_ptr(slot), 0, list(rlay.blob_offset),
+                        stream.cuda_stream)
+        stream.synchronize()
+        exp = np.full(w.capacities("dst")[0], 0xA5, dtype=np.uint8)
+        checkers.oracle_unpack(exp, o_runs, blob)
+        assert np.array_equal(_host(dst_layers[l][0]), exp), l
+        rplan.close()
+    stager.close()

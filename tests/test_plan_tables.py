@@ -32,6 +32,9 @@ def emulate(table, chunk_bytes, shapes, caches, tensor_offset, packed, pack):
             v = np.arange(n // 16, dtype=np.uint64)
             rec = v if vlen == 1 else (v * np.uint64(inv)) >> np.uint64(32)   # __umulhi
             assert np.array_equal(rec, v // np.uint64(vlen))                   # the reciprocal is exact
+            w = np.arange(n // 4, dtype=np.uint64)                             # word-wise path
+            assert np.array_equal((w * np.uint64(int(s["inv_wlen"]))) >> np.uint64(32),
+                                  w // np.uint64(4 * vlen))
             col = v - rec * np.uint64(vlen)
             o, i = rec // np.uint64(n_inner), rec % np.uint64(n_inner)
             at = (o * np.uint64(int(s["outer"][side])) + i * np.uint64(int(s["inner"][side]))
