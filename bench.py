@@ -17,6 +17,7 @@ import os
 import statistics
 import sys
 import time
+import types
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path[:0] = [os.path.join(ROOT, "llumnix-kv_amd"), os.path.join(ROOT, "tests")]
@@ -121,6 +122,317 @@ def ev_ms(lib, a, b):
     rc = lib.kvt_event_elapsed_ms(a, b, C.byref(ms))
     assert rc == 0, lib.kvt_last_error()
     return ms.value
+
+def leg_cpu(c, out):
+    """Parity spot check of the GPU results and the CPU baseline (oracle) on a bounded sample."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    wls, sides, infos, tasks, first = c.wls, c.sides, c.infos, c.tasks, c.first
+    strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
+    full_wls, full_sides, mixed = c.full_wls, c.full_sides, c.mixed
+    import checkers
+    w, side = full_wls[0], full_sides[0]      # (mixed mode: both halves of the requests)
+    L = max(1, min(args.cpu_layers, w.n_layers))
+    s_info, d_info = w.worker_infos()
+    cpu_tasks = w.task_bufs()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, s_info, d_info)
+    assert rc == 0
+    olib = checkers.oracle()
+    host_src = [[t.cpu().numpy() for t in side.src[l]] for l in range(L)]
+    host_dst = [[np.zeros(c, dtype=np.uint8) for c in w.capacities("dst")] for _ in range(L)]
+    stride = strides[0]
+    gpu_packed = packed[0][:L * stride].cpu().numpy()
+    plan0 = first[0][0]
+
+    def cpu_pass():
+        t_a = time.perf_counter()
+        rc, outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
+        assert rc == 0
+        if kind == 0:
+            outs = [checkers.oracle_merge(o)[0] for o in outs]
+        t_b = time.perf_counter()
+        blobs = []
+        for l in range(L):
+            blobs.append([checkers.oracle_pack(host_src[l][t], outs[t])
+                          for t in range(w.n_tensors)])
+        t_c = time.perf_counter()
+        if w.xform is None:
+            for l in range(L):
+                for t in range(w.n_tensors):
+                    checkers.oracle_unpack(host_dst[l][t], outs[t], blobs[l][t])
+        t_d = time.perf_counter()
+        return (t_b - t_a, t_c - t_b, t_d - t_c), outs, blobs
+
+    reps = [cpu_pass() for _ in range(3)]
+    times = sorted(r[0] for r in reps)
+    parse_s, pack_s, unpack_s = times[1]
+    outs, blobs = reps[-1][1], reps[-1][2]
+    parity = True
+    if w.xform is None:
+        for l in range(L if not mixed else 0):   # (mixed: the packed buffers are per half)
+            for t in range(w.n_tensors):
+                off = l * stride + plan0.tensor_offset(t)
+                parity &= bool(np.array_equal(gpu_packed[off:off + len(blobs[l][t])],
+                                              blobs[l][t]))
+        gpu_dst = [[x.cpu().numpy() for x in side.dst[l]] for l in range(L)]
+        for l in range(L):
+            for t in range(w.n_tensors):
+                parity &= bool(np.array_equal(gpu_dst[l][t], host_dst[l][t]))
+    P_s = sum(int(o[:, 2].sum()) for o in outs) * L
+    total_s = parse_s + pack_s + unpack_s
+    out["parity_vs_oracle"] = parity if w.xform is None else "n/a (transposing pack is checked in tests/)"
+    out["cpu_baseline"] = {
+        "value": round(4.0 * P_s / total_s / 1e9, 2), "unit": "GB/s", "cores": 1,
+        "kind": "port",
+        "sample": "%d of %d layers of the same batch (%d requests): ParseBlock+merge %.1f ms, "
+                  "pack %.1f ms, unpack %.1f ms; median of 3" %
+                  (L, w.n_layers, len(w.tasks), parse_s * 1e3, pack_s * 1e3, unpack_s * 1e3),
+        "host_cores_available": os.cpu_count(),
+    }
+    # ParseBlock alone for the whole batch: the reference's own functions (compiled from its
+    # sources into oracle/_ref where that was possible), the oracle, and the product
+    pb = {}
+    if checkers.ref() is not None and not w.xform:
+        tt = []
+        with stdout_to_stderr():
+            for _ in range(5):
+                a = time.perf_counter()
+                rc, _outs = checkers.ref_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
+                tt.append(time.perf_counter() - a)
+                assert rc == 0
+        pb["reference_ms"] = round(sorted(tt)[2] * 1e3, 3)
+    tt = []
+    for _ in range(5):
+        a = time.perf_counter()
+        rc, _outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
+        tt.append(time.perf_counter() - a)
+    pb["oracle_ms"] = round(sorted(tt)[2] * 1e3, 3)
+    parser = kvt.Parser(pid, s_info, d_info, valid, tps, tpr)
+    tt = []
+    for _ in range(5):
+        lst = kvt.BlockLists()
+        a = time.perf_counter()
+        for t in cpu_tasks:
+            parser.parse(t.struct, lst)
+        tt.append(time.perf_counter() - a)
+        lst.close()
+    pb["product_ms"] = round(sorted(tt)[2] * 1e3, 3)
+    pb["note"] = "%d requests, median of 5, one thread; output copies included" % len(cpu_tasks)
+    out["cpu_baseline"]["parse_block"] = pb
+
+    # all host cores, threads striding over layers (not the reference's threading model)
+    nthr = min(16, os.cpu_count() or 1, L)
+    if nthr > 1 and w.xform is None and w.n_tensors == 1:
+        ptrs = (C.c_void_p * L)(*[host_src[l][0].ctypes.data for l in range(L)])
+        runs0 = np.ascontiguousarray(outs[0])
+        tb = int(runs0[:, 2].sum())
+        blob = np.empty(L * tb, dtype=np.uint8)
+        tt = []
+        for _ in range(3):
+            a = time.perf_counter()
+            olib.kvto_pack_layers(ptrs, L, runs0.ctypes.data, len(runs0), blob.ctypes.data, tb,
+                                  nthr)
+            tt.append(time.perf_counter() - a)
+        out["cpu_baseline_threads"] = {"pack_gbps": round(2.0 * tb * L / sorted(tt)[1] / 1e9, 2),
+                                       "cores": nthr}
+    log("cpu baseline done, parity:", out.get("parity_vs_oracle"))
+    del host_src, host_dst, gpu_packed
+
+
+def leg_latency(c, out):
+    """GPU time of one pack launch per request (all layers of the request)."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    wls, sides, infos, tasks, first = c.wls, c.sides, c.infos, c.tasks, c.first
+    strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
+    w, side = wls[0], sides[0]
+    lat = []
+    reqs = list(range(len(w.tasks)))
+    for r in reqs:
+        lists, _ = pipeline.parse_batch(w.cache_shape, infos[0][0], infos[0][1], [tasks[0][r]])
+        plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
+                        chunk_bytes=args.chunk_bytes)
+        c.keep.append(plan)
+        a, b = new_event(), new_event()
+        for rep in range(2):   # second run is the measurement
+            lib.kvt_event_record(a, sh)
+            plan.pack(side.src_cache, 0, w.n_layers, packed[0], plan.layer_bytes, sh)
+            lib.kvt_event_record(b, sh)
+        lib.kvt_event_synchronize(b)
+        lat.append(ev_ms(lib, a, b) * 1e3)
+    out["latency_p50_us"] = round(statistics.median(lat), 2)
+    out["latency_note"] = "per request: one pack launch covering all %d layers, GPU time" % w.n_layers
+
+
+def leg_session(c, out):
+    """Layer-by-layer packing through an event-gated session, eager and replayed from a hipGraph."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    wls, sides, infos, tasks, first = c.wls, c.sides, c.infos, c.tasks, c.first
+    strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
+    w, side = wls[0], sides[0]
+    # layer-by-layer operation (the serving pattern: every layer is packed as soon as the
+    # forward pass has produced it): one event-gated launch per layer on the side stream
+    if w.xform is None:
+        plan0 = first[0][0]
+        sess = kvt.Session(plan0, side.src_cache, packed[0], strides[0])
+        a, b = new_event(), new_event()
+        for rep in range(2):
+            lib.kvt_event_record(a, sh)
+            for l in range(w.n_layers):
+                sess.save_layer(l, sh)
+            sess.join(sh)
+            lib.kvt_event_record(b, sh)
+        lib.kvt_event_synchronize(b)
+        ms = ev_ms(lib, a, b)
+        pay0 = sum(plan0.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
+        out["per_layer_session"] = {"pack_ms_all_layers": round(ms, 4),
+                                    "pack_gbps": round(2.0 * pay0 / (ms * 1e-3) / 1e9, 1),
+                                    "launches": w.n_layers}
+        # the same sequence captured once into a hipGraph and replayed
+        gs = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(gs):
+            with torch.cuda.graph(graph, stream=gs):
+                for l in range(w.n_layers):
+                    sess.save_layer(l, gs.cuda_stream)
+                sess.join(gs.cuda_stream)
+        for rep in range(2):
+            torch.cuda.synchronize()
+            t_a = time.perf_counter()
+            for _ in range(5):
+                graph.replay()
+            torch.cuda.synchronize()
+            g_ms = (time.perf_counter() - t_a) / 5 * 1e3
+        out["per_layer_session"]["graph_replay_ms_all_layers"] = round(g_ms, 4)
+        del graph
+        sess.close()
+
+
+def leg_launchers(c, out):
+    """The reference-shaped entry points on the same ranges."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    wls, sides, infos, tasks, first = c.wls, c.sides, c.infos, c.tasks, c.first
+    strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
+    w, side = wls[0], sides[0]
+    # the reference-shaped launchers (one launch per layer, ranges as three int64 arrays
+    # resident on the device) and the converting bf16 -> fp8 gather
+    if w.xform is None and args.plan == "ranges" and w.elem_dtype == "bf16":
+        runs0 = first[0][1].tensor(0).astype(np.int64)
+        so = torch.from_numpy(np.ascontiguousarray(runs0[:, 0])).cuda()
+        ln = torch.from_numpy(np.ascontiguousarray(runs0[:, 2])).cuda()
+        do = torch.from_numpy(np.concatenate([[0], np.cumsum(runs0[:, 2])[:-1]])).cuda()
+        ln_e = ln // 2
+        do_e = do // 2
+        nb = int(runs0[:, 2].sum())
+        a, b = new_event(), new_event()
+        res = {}
+        for name, fn, offs, lens, moved in (
+                ("launch_copy_d2h_direct", lib.kvt_launch_copy_d2h_direct, do, ln, 2 * nb),
+                ("launch_copy_d2h_bf16_to_fp8", lib.kvt_launch_copy_d2h_bf16_to_fp8, do_e,
+                 ln_e, nb + nb // 2)):
+            for rep in range(2):
+                lib.kvt_event_record(a, sh)
+                for l in range(w.n_layers):
+                    rc = fn(side.src[l][0].data_ptr(), packed[0].data_ptr() + l * strides[0],
+                            so.data_ptr(), offs.data_ptr(), lens.data_ptr(), len(runs0), 0, 0,
+                            sh)
+                    assert rc == 0, lib.kvt_last_error()
+                lib.kvt_event_record(b, sh)
+            lib.kvt_event_synchronize(b)
+            res[name + "_gbps"] = round(moved * w.n_layers / (ev_ms(lib, a, b) * 1e-3) / 1e9, 1)
+        res["note"] = ("%d launches of %d ranges each; GB/s = bytes read + bytes written; the "
+                       "fp8 gather reads 2 bytes and writes 1 per element" %
+                       (w.n_layers, len(runs0)))
+        # the reference's host entry point, called the way TCPChannel::send_data /
+        # handle_kv_cache_data call it: pinned host buffer on the contiguous side, metadata
+        # uploaded per call through the caller's two 8192-range buffers
+        if nb <= (2 << 30):
+            pin = torch.empty(nb, dtype=torch.uint8, pin_memory=True)
+            meta_n = 3 * 8192
+            dev_meta = torch.zeros(meta_n, dtype=torch.int64, device="cuda")
+            host_meta = torch.zeros(meta_n, dtype=torch.int64).pin_memory()
+            zeros = np.zeros(len(runs0), dtype=np.uint64)
+            kb_send = np.ascontiguousarray(np.stack(
+                [zeros, runs0[:, 0].astype(np.uint64), runs0[:, 2].astype(np.uint64)], axis=1))
+            kb_recv = np.ascontiguousarray(first[0][1].tensor(0))
+            Lh = min(4, w.n_layers)
+            for name, direction, blocks, tensors in (
+                    ("handle_data_d2h_pinned_gbps", 1, kb_send, side.src),
+                    ("handle_data_h2d_pinned_gbps", 0, kb_recv, side.dst)):
+                for rep in range(2):
+                    torch.cuda.synchronize()
+                    t_a = time.perf_counter()
+                    for l in range(Lh):
+                        rc = lib.kvt_copy_handle_data_with_kernel(
+                            pin.data_ptr(), tensors[l][0].data_ptr(), blocks.ctypes.data,
+                            len(blocks), nb, direction, 0, sh, dev_meta.data_ptr(),
+                            host_meta.data_ptr(), 8192)
+                        assert rc == 0, lib.kvt_last_error()
+                        stream.synchronize()     # the reference syncs after every tensor
+                    dt = time.perf_counter() - t_a
+                res[name] = round(nb * Lh / dt / 1e9, 2)
+            res["handle_data_note"] = ("%d layers, one call per layer incl. metadata upload and "
+                                       "stream sync; GB/s = payload bytes over PCIe" % Lh)
+        out["reference_shaped_launchers"] = res
+
+    # pinned-host staging of packed layers, double buffered against the pack kernel
+
+
+def leg_staging(c, out):
+    """Packed layers through pinned host memory, double buffered against the kernels."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    wls, sides, infos, tasks, first = c.wls, c.sides, c.infos, c.tasks, c.first
+    strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
+    w, side = wls[0], sides[0]
+    # Small layers are grouped so that one transfer is at least 256 MiB (a copy has a fixed
+    # start-up cost of some tens of microseconds; config 1's layers are 2 MiB).
+    plan = first[0][0]
+    lbytes = plan.layer_bytes
+    if 0 < lbytes < (3 << 30):
+        group = max(1, min(w.n_layers, -(-(256 << 20) // lbytes)))
+        n_groups = max(1, min(8, w.n_layers // group))
+        nbytes = group * lbytes
+        ceil = {}
+        for name, d in (("d2h", 1), ("h2d", 0)):
+            r = C.c_double()
+            assert lib.kvt_measure_pcie(0, d, min(nbytes, 1 << 30), 5, C.byref(r)) == 0
+            ceil[name] = r.value
+        stg = kvt.Stager(0, nbytes, 2)
+        bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
+        ps = torch.cuda.Stream()
+        d2h_t, h2d_t = [], []
+        for phase in range(4):          # first phase warms up
+            torch.cuda.synchronize()
+            a = time.perf_counter()
+            for g in range(n_groups):
+                slot = g % 2
+                if g >= 2:
+                    stg.wait(slot)
+                plan.pack(side.src_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
+                stg.save(slot, bufs[slot], nbytes, ps.cuda_stream)
+            stg.wait(0)
+            if n_groups > 1:
+                stg.wait(1)
+            d2h_t.append(time.perf_counter() - a)
+        for phase in range(4):
+            torch.cuda.synchronize()
+            a = time.perf_counter()
+            for g in range(n_groups):
+                slot = g % 2
+                stg.load(slot, bufs[slot], nbytes, ps.cuda_stream)
+                plan.unpack(side.dst_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
+            ps.synchronize()
+            h2d_t.append(time.perf_counter() - a)
+        d2h_s, h2d_s = statistics.median(d2h_t[1:]), statistics.median(h2d_t[1:])
+        pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * group * n_groups
+        out["staging"] = {
+            "save_gbps": round(pay / d2h_s / 1e9, 2), "load_gbps": round(pay / h2d_s / 1e9, 2),
+            "pcie_d2h_gbps": round(ceil["d2h"] / 1e9, 2), "pcie_h2d_gbps": round(ceil["h2d"] / 1e9, 2),
+            "save_frac_of_pcie": round(pay / d2h_s / ceil["d2h"], 4),
+            "load_frac_of_pcie": round(pay / h2d_s / ceil["h2d"], 4),
+            "sample": "%d transfers of %d layer(s) = %.1f MiB each through 2 pinned slots, "
+                      "pack / unpack of the group in one launch; median of 3 passes" %
+                      (n_groups, group, nbytes / 2**20),
+        }
+        stg.close()
 
 
 def main():
@@ -351,287 +663,15 @@ def main():
                      "traffic": MEASURED_PACK_TRAFFIC.get((args.config, args.scale,
                                                            args.chunk_bytes, args.plan))},
     }
-
-    # ---------------------------------------------------------------- parity spot check + CPU leg
+    c = types.SimpleNamespace(torch=torch, np=np, kvt=kvt, lib=lib, args=args, pipeline=pipeline,
+                              wls=wls, sides=sides, full_wls=full_wls, full_sides=full_sides,
+                              mixed=mixed, infos=infos, tasks=tasks, first=first, strides=strides,
+                              packed=packed, stream=stream, sh=sh, new_event=new_event, keep=keep)
     if not args.skip_cpu:
-        import checkers
-        w, side = full_wls[0], full_sides[0]      # (mixed mode: both halves of the requests)
-        L = max(1, min(args.cpu_layers, w.n_layers))
-        s_info, d_info = w.worker_infos()
-        cpu_tasks = w.task_bufs()
-        rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, s_info, d_info)
-        assert rc == 0
-        olib = checkers.oracle()
-        host_src = [[t.cpu().numpy() for t in side.src[l]] for l in range(L)]
-        host_dst = [[np.zeros(c, dtype=np.uint8) for c in w.capacities("dst")] for _ in range(L)]
-        stride = strides[0]
-        gpu_packed = packed[0][:L * stride].cpu().numpy()
-        plan0 = first[0][0]
-
-        def cpu_pass():
-            t_a = time.perf_counter()
-            rc, outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
-            assert rc == 0
-            if kind == 0:
-                outs = [checkers.oracle_merge(o)[0] for o in outs]
-            t_b = time.perf_counter()
-            blobs = []
-            for l in range(L):
-                blobs.append([checkers.oracle_pack(host_src[l][t], outs[t])
-                              for t in range(w.n_tensors)])
-            t_c = time.perf_counter()
-            if w.xform is None:
-                for l in range(L):
-                    for t in range(w.n_tensors):
-                        checkers.oracle_unpack(host_dst[l][t], outs[t], blobs[l][t])
-            t_d = time.perf_counter()
-            return (t_b - t_a, t_c - t_b, t_d - t_c), outs, blobs
-
-        reps = [cpu_pass() for _ in range(3)]
-        times = sorted(r[0] for r in reps)
-        parse_s, pack_s, unpack_s = times[1]
-        outs, blobs = reps[-1][1], reps[-1][2]
-        parity = True
-        if w.xform is None:
-            for l in range(L if not mixed else 0):   # (mixed: the packed buffers are per half)
-                for t in range(w.n_tensors):
-                    off = l * stride + plan0.tensor_offset(t)
-                    parity &= bool(np.array_equal(gpu_packed[off:off + len(blobs[l][t])],
-                                                  blobs[l][t]))
-            gpu_dst = [[x.cpu().numpy() for x in side.dst[l]] for l in range(L)]
-            for l in range(L):
-                for t in range(w.n_tensors):
-                    parity &= bool(np.array_equal(gpu_dst[l][t], host_dst[l][t]))
-        P_s = sum(int(o[:, 2].sum()) for o in outs) * L
-        total_s = parse_s + pack_s + unpack_s
-        out["parity_vs_oracle"] = parity if w.xform is None else "n/a (transposing pack is checked in tests/)"
-        out["cpu_baseline"] = {
-            "value": round(4.0 * P_s / total_s / 1e9, 2), "unit": "GB/s", "cores": 1,
-            "kind": "port",
-            "sample": "%d of %d layers of the same batch (%d requests): ParseBlock+merge %.1f ms, "
-                      "pack %.1f ms, unpack %.1f ms; median of 3" %
-                      (L, w.n_layers, len(w.tasks), parse_s * 1e3, pack_s * 1e3, unpack_s * 1e3),
-            "host_cores_available": os.cpu_count(),
-        }
-        # ParseBlock alone for the whole batch: the reference's own functions (compiled from its
-        # sources into oracle/_ref where that was possible), the oracle, and the product
-        pb = {}
-        if checkers.ref() is not None and not w.xform:
-            tt = []
-            with stdout_to_stderr():
-                for _ in range(5):
-                    a = time.perf_counter()
-                    rc, _outs = checkers.ref_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
-                    tt.append(time.perf_counter() - a)
-                    assert rc == 0
-            pb["reference_ms"] = round(sorted(tt)[2] * 1e3, 3)
-        tt = []
-        for _ in range(5):
-            a = time.perf_counter()
-            rc, _outs = checkers.oracle_parse(pid, s_info, d_info, valid, tps, tpr, cpu_tasks)
-            tt.append(time.perf_counter() - a)
-        pb["oracle_ms"] = round(sorted(tt)[2] * 1e3, 3)
-        parser = kvt.Parser(pid, s_info, d_info, valid, tps, tpr)
-        tt = []
-        for _ in range(5):
-            lst = kvt.BlockLists()
-            a = time.perf_counter()
-            for t in cpu_tasks:
-                parser.parse(t.struct, lst)
-            tt.append(time.perf_counter() - a)
-            lst.close()
-        pb["product_ms"] = round(sorted(tt)[2] * 1e3, 3)
-        pb["note"] = "%d requests, median of 5, one thread; output copies included" % len(cpu_tasks)
-        out["cpu_baseline"]["parse_block"] = pb
-
-        # all host cores, threads striding over layers (not the reference's threading model)
-        nthr = min(16, os.cpu_count() or 1, L)
-        if nthr > 1 and w.xform is None and w.n_tensors == 1:
-            ptrs = (C.c_void_p * L)(*[host_src[l][0].ctypes.data for l in range(L)])
-            runs0 = np.ascontiguousarray(outs[0])
-            tb = int(runs0[:, 2].sum())
-            blob = np.empty(L * tb, dtype=np.uint8)
-            tt = []
-            for _ in range(3):
-                a = time.perf_counter()
-                olib.kvto_pack_layers(ptrs, L, runs0.ctypes.data, len(runs0), blob.ctypes.data, tb,
-                                      nthr)
-                tt.append(time.perf_counter() - a)
-            out["cpu_baseline_threads"] = {"pack_gbps": round(2.0 * tb * L / sorted(tt)[1] / 1e9, 2),
-                                           "cores": nthr}
-        log("cpu baseline done, parity:", out.get("parity_vs_oracle"))
-        del host_src, host_dst, gpu_packed
-
-    # ---------------------------------------------------------------- per-request latency, staging
+        leg_cpu(c, out)
     if not args.skip_extras:
-        w, side = wls[0], sides[0]
-        lat = []
-        reqs = list(range(len(w.tasks)))
-        for r in reqs:
-            lists, _ = pipeline.parse_batch(w.cache_shape, infos[0][0], infos[0][1], [tasks[0][r]])
-            plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
-                            chunk_bytes=args.chunk_bytes)
-            keep.append(plan)
-            a, b = new_event(), new_event()
-            for rep in range(2):   # second run is the measurement
-                lib.kvt_event_record(a, sh)
-                plan.pack(side.src_cache, 0, w.n_layers, packed[0], plan.layer_bytes, sh)
-                lib.kvt_event_record(b, sh)
-            lib.kvt_event_synchronize(b)
-            lat.append(ev_ms(lib, a, b) * 1e3)
-        out["latency_p50_us"] = round(statistics.median(lat), 2)
-        out["latency_note"] = "per request: one pack launch covering all %d layers, GPU time" % w.n_layers
-
-        # layer-by-layer operation (the serving pattern: every layer is packed as soon as the
-        # forward pass has produced it): one event-gated launch per layer on the side stream
-        if w.xform is None:
-            plan0 = first[0][0]
-            sess = kvt.Session(plan0, side.src_cache, packed[0], strides[0])
-            a, b = new_event(), new_event()
-            for rep in range(2):
-                lib.kvt_event_record(a, sh)
-                for l in range(w.n_layers):
-                    sess.save_layer(l, sh)
-                sess.join(sh)
-                lib.kvt_event_record(b, sh)
-            lib.kvt_event_synchronize(b)
-            ms = ev_ms(lib, a, b)
-            pay0 = sum(plan0.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
-            out["per_layer_session"] = {"pack_ms_all_layers": round(ms, 4),
-                                        "pack_gbps": round(2.0 * pay0 / (ms * 1e-3) / 1e9, 1),
-                                        "launches": w.n_layers}
-            # the same sequence captured once into a hipGraph and replayed
-            gs = torch.cuda.Stream()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.stream(gs):
-                with torch.cuda.graph(graph, stream=gs):
-                    for l in range(w.n_layers):
-                        sess.save_layer(l, gs.cuda_stream)
-                    sess.join(gs.cuda_stream)
-            for rep in range(2):
-                torch.cuda.synchronize()
-                t_a = time.perf_counter()
-                for _ in range(5):
-                    graph.replay()
-                torch.cuda.synchronize()
-                g_ms = (time.perf_counter() - t_a) / 5 * 1e3
-            out["per_layer_session"]["graph_replay_ms_all_layers"] = round(g_ms, 4)
-            del graph
-            sess.close()
-
-        # the reference-shaped launchers (one launch per layer, ranges as three int64 arrays
-        # resident on the device) and the converting bf16 -> fp8 gather
-        if w.xform is None and args.plan == "ranges" and w.elem_dtype == "bf16":
-            runs0 = first[0][1].tensor(0).astype(np.int64)
-            so = torch.from_numpy(np.ascontiguousarray(runs0[:, 0])).cuda()
-            ln = torch.from_numpy(np.ascontiguousarray(runs0[:, 2])).cuda()
-            do = torch.from_numpy(np.concatenate([[0], np.cumsum(runs0[:, 2])[:-1]])).cuda()
-            ln_e = ln // 2
-            do_e = do // 2
-            nb = int(runs0[:, 2].sum())
-            a, b = new_event(), new_event()
-            res = {}
-            for name, fn, offs, lens, moved in (
-                    ("launch_copy_d2h_direct", lib.kvt_launch_copy_d2h_direct, do, ln, 2 * nb),
-                    ("launch_copy_d2h_bf16_to_fp8", lib.kvt_launch_copy_d2h_bf16_to_fp8, do_e,
-                     ln_e, nb + nb // 2)):
-                for rep in range(2):
-                    lib.kvt_event_record(a, sh)
-                    for l in range(w.n_layers):
-                        rc = fn(side.src[l][0].data_ptr(), packed[0].data_ptr() + l * strides[0],
-                                so.data_ptr(), offs.data_ptr(), lens.data_ptr(), len(runs0), 0, 0,
-                                sh)
-                        assert rc == 0, lib.kvt_last_error()
-                    lib.kvt_event_record(b, sh)
-                lib.kvt_event_synchronize(b)
-                res[name + "_gbps"] = round(moved * w.n_layers / (ev_ms(lib, a, b) * 1e-3) / 1e9, 1)
-            res["note"] = ("%d launches of %d ranges each; GB/s = bytes read + bytes written; the "
-                           "fp8 gather reads 2 bytes and writes 1 per element" %
-                           (w.n_layers, len(runs0)))
-            # the reference's host entry point, called the way TCPChannel::send_data /
-            # handle_kv_cache_data call it: pinned host buffer on the contiguous side, metadata
-            # uploaded per call through the caller's two 8192-range buffers
-            if nb <= (2 << 30):
-                pin = torch.empty(nb, dtype=torch.uint8, pin_memory=True)
-                meta_n = 3 * 8192
-                dev_meta = torch.zeros(meta_n, dtype=torch.int64, device="cuda")
-                host_meta = torch.zeros(meta_n, dtype=torch.int64).pin_memory()
-                zeros = np.zeros(len(runs0), dtype=np.uint64)
-                kb_send = np.ascontiguousarray(np.stack(
-                    [zeros, runs0[:, 0].astype(np.uint64), runs0[:, 2].astype(np.uint64)], axis=1))
-                kb_recv = np.ascontiguousarray(first[0][1].tensor(0))
-                Lh = min(4, w.n_layers)
-                for name, direction, blocks, tensors in (
-                        ("handle_data_d2h_pinned_gbps", 1, kb_send, side.src),
-                        ("handle_data_h2d_pinned_gbps", 0, kb_recv, side.dst)):
-                    for rep in range(2):
-                        torch.cuda.synchronize()
-                        t_a = time.perf_counter()
-                        for l in range(Lh):
-                            rc = lib.kvt_copy_handle_data_with_kernel(
-                                pin.data_ptr(), tensors[l][0].data_ptr(), blocks.ctypes.data,
-                                len(blocks), nb, direction, 0, sh, dev_meta.data_ptr(),
-                                host_meta.data_ptr(), 8192)
-                            assert rc == 0, lib.kvt_last_error()
-                            stream.synchronize()     # the reference syncs after every tensor
-                        dt = time.perf_counter() - t_a
-                    res[name] = round(nb * Lh / dt / 1e9, 2)
-                res["handle_data_note"] = ("%d layers, one call per layer incl. metadata upload and "
-                                           "stream sync; GB/s = payload bytes over PCIe" % Lh)
-            out["reference_shaped_launchers"] = res
-
-        # pinned-host staging of packed layers, double buffered against the pack kernel
-        # Small layers are grouped so that one transfer is at least 256 MiB (a copy has a fixed
-        # start-up cost of some tens of microseconds; config 1's layers are 2 MiB).
-        plan = first[0][0]
-        lbytes = plan.layer_bytes
-        if 0 < lbytes < (3 << 30):
-            group = max(1, min(w.n_layers, -(-(256 << 20) // lbytes)))
-            n_groups = max(1, min(8, w.n_layers // group))
-            nbytes = group * lbytes
-            ceil = {}
-            for name, d in (("d2h", 1), ("h2d", 0)):
-                r = C.c_double()
-                assert lib.kvt_measure_pcie(0, d, min(nbytes, 1 << 30), 5, C.byref(r)) == 0
-                ceil[name] = r.value
-            stg = kvt.Stager(0, nbytes, 2)
-            bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
-            ps = torch.cuda.Stream()
-            d2h_t, h2d_t = [], []
-            for phase in range(4):          # first phase warms up
-                torch.cuda.synchronize()
-                a = time.perf_counter()
-                for g in range(n_groups):
-                    slot = g % 2
-                    if g >= 2:
-                        stg.wait(slot)
-                    plan.pack(side.src_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
-                    stg.save(slot, bufs[slot], nbytes, ps.cuda_stream)
-                stg.wait(0)
-                if n_groups > 1:
-                    stg.wait(1)
-                d2h_t.append(time.perf_counter() - a)
-            for phase in range(4):
-                torch.cuda.synchronize()
-                a = time.perf_counter()
-                for g in range(n_groups):
-                    slot = g % 2
-                    stg.load(slot, bufs[slot], nbytes, ps.cuda_stream)
-                    plan.unpack(side.dst_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
-                ps.synchronize()
-                h2d_t.append(time.perf_counter() - a)
-            d2h_s, h2d_s = statistics.median(d2h_t[1:]), statistics.median(h2d_t[1:])
-            pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * group * n_groups
-            out["staging"] = {
-                "save_gbps": round(pay / d2h_s / 1e9, 2), "load_gbps": round(pay / h2d_s / 1e9, 2),
-                "pcie_d2h_gbps": round(ceil["d2h"] / 1e9, 2), "pcie_h2d_gbps": round(ceil["h2d"] / 1e9, 2),
-                "save_frac_of_pcie": round(pay / d2h_s / ceil["d2h"], 4),
-                "load_frac_of_pcie": round(pay / h2d_s / ceil["h2d"], 4),
-                "sample": "%d transfers of %d layer(s) = %.1f MiB each through 2 pinned slots, "
-                          "pack / unpack of the group in one launch; median of 3 passes" %
-                          (n_groups, group, nbytes / 2**20),
-            }
-            stg.close()
+        for leg in (leg_latency, leg_session, leg_launchers, leg_staging):
+            leg(c, out)
 
     print(json.dumps(out), flush=True)
 
