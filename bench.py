@@ -270,40 +270,39 @@ def leg_session(c, out):
     w, side = wls[0], sides[0]
     # layer-by-layer operation (the serving pattern: every layer is packed as soon as the
     # forward pass has produced it): one event-gated launch per layer on the side stream
-    if w.xform is None:
-        plan0 = first[0][0]
-        sess = kvt.Session(plan0, side.src_cache, packed[0], strides[0])
-        a, b = new_event(), new_event()
-        for rep in range(2):
-            lib.kvt_event_record(a, sh)
+    plan0 = first[0][0]
+    sess = kvt.Session(plan0, side.src_cache, packed[0], strides[0])
+    a, b = new_event(), new_event()
+    for rep in range(2):
+        lib.kvt_event_record(a, sh)
+        for l in range(w.n_layers):
+            sess.save_layer(l, sh)
+        sess.join(sh)
+        lib.kvt_event_record(b, sh)
+    lib.kvt_event_synchronize(b)
+    ms = ev_ms(lib, a, b)
+    pay0 = sum(plan0.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
+    out["per_layer_session"] = {"pack_ms_all_layers": round(ms, 4),
+                                "pack_gbps": round(2.0 * pay0 / (ms * 1e-3) / 1e9, 1),
+                                "launches": w.n_layers}
+    # the same sequence captured once into a hipGraph and replayed
+    gs = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(gs):
+        with torch.cuda.graph(graph, stream=gs):
             for l in range(w.n_layers):
-                sess.save_layer(l, sh)
-            sess.join(sh)
-            lib.kvt_event_record(b, sh)
-        lib.kvt_event_synchronize(b)
-        ms = ev_ms(lib, a, b)
-        pay0 = sum(plan0.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
-        out["per_layer_session"] = {"pack_ms_all_layers": round(ms, 4),
-                                    "pack_gbps": round(2.0 * pay0 / (ms * 1e-3) / 1e9, 1),
-                                    "launches": w.n_layers}
-        # the same sequence captured once into a hipGraph and replayed
-        gs = torch.cuda.Stream()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(gs):
-            with torch.cuda.graph(graph, stream=gs):
-                for l in range(w.n_layers):
-                    sess.save_layer(l, gs.cuda_stream)
-                sess.join(gs.cuda_stream)
-        for rep in range(2):
-            torch.cuda.synchronize()
-            t_a = time.perf_counter()
-            for _ in range(5):
-                graph.replay()
-            torch.cuda.synchronize()
-            g_ms = (time.perf_counter() - t_a) / 5 * 1e3
-        out["per_layer_session"]["graph_replay_ms_all_layers"] = round(g_ms, 4)
-        del graph
-        sess.close()
+                sess.save_layer(l, gs.cuda_stream)
+            sess.join(gs.cuda_stream)
+    for rep in range(2):
+        torch.cuda.synchronize()
+        t_a = time.perf_counter()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        g_ms = (time.perf_counter() - t_a) / 5 * 1e3
+    out["per_layer_session"]["graph_replay_ms_all_layers"] = round(g_ms, 4)
+    del graph
+    sess.close()
 
 
 def leg_launchers(c, out):
