@@ -334,6 +334,20 @@ int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
                                      uint64_t tensor_data_size, int direction, int device,
                                      void* stream, int64_t* dev_meta, int64_t* host_meta,
                                      int64_t max_block_num);
+/* replaces copy_handle_data_kernel_direct()     kvtransfer/include/copy_kernels.h:24-57,
+ *                                               kvtransfer/src/copy_kernels.cpp:363-439
+ * One batch, no internal synchronisation: the three device arrays (n int64 each)
+ * and host_meta (3 n int64, pinned) belong to the caller and must stay untouched
+ * until the stream has run the copy. With use_explicit_host_offsets the
+ * contiguous-side offset of range i is blocks[i].src_offset instead of the
+ * running sum. Unlike the reference (which only asserts), ranges that leave
+ * the contiguous buffer are refused with KVT_ERR_OUT_OF_RANGE. */
+int kvt_copy_handle_data_kernel_direct(void* tensor_buf, void* layer_gpu_ptr,
+                                       const kvt_ipc_block* blocks, uint64_t n,
+                                       uint64_t tensor_data_size, int direction, int device,
+                                       void* stream, int64_t* src_offsets_dev,
+                                       int64_t* dst_offsets_dev, int64_t* lengths_dev,
+                                       int64_t* host_meta, int use_explicit_host_offsets);
 /* replaces copy_d2h_bf16_to_fp8()               kvtransfer/include/copy_kernels.h:112-121,
  *                                               kvtransfer/src/copy_kernels.cpp:833-959
  * blocks[i].length = bf16 bytes at the source; the contiguous side receives

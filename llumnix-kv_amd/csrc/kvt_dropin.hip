@@ -100,6 +100,52 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
   return KVT_OK;
 }
 
+// Single batch with separate device arrays (copy_handle_data_kernel_direct).
+int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks,
+                       uint64_t n, uint64_t tensor_data_size, int direction, int device,
+                       void* stream, int64_t* src_dev, int64_t* dst_dev, int64_t* len_dev,
+                       int64_t* host_meta, bool explicit_host_offsets) {
+  if (n == 0) return KVT_OK;
+  if (!tensor_buf || !layer_gpu_ptr || !blocks || !src_dev || !dst_dev || !len_dev || !host_meta)
+    return fail(KVT_ERR_INVALID, "copy_handle_data_kernel_direct: null argument");
+  if (direction != KVT_COPY_H2D && direction != KVT_COPY_D2H)
+    return fail(KVT_ERR_INVALID, "copy_handle_data_kernel_direct: bad direction");
+  if (n > 0x7FFFFFFFull) return fail(KVT_ERR_INVALID, "too many ranges");
+  if (int rc = check_device(device)) return rc;
+  uint64_t cursor = 0, longest = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    const kvt_ipc_block& b = blocks[i];
+    const uint64_t host_off = explicit_host_offsets ? b.src_offset : cursor;
+    if (b.length == 0 || host_off > tensor_data_size || b.length > tensor_data_size - host_off)
+      return fail(KVT_ERR_OUT_OF_RANGE,
+                  "copy_handle_data_kernel_direct: range outside the contiguous buffer");
+    host_meta[i] = static_cast<int64_t>(host_off);
+    host_meta[n + i] = static_cast<int64_t>(b.dst_offset);
+    host_meta[2 * n + i] = static_cast<int64_t>(b.length);
+    cursor += b.length;
+    longest = std::max<uint64_t>(longest, b.length);
+  }
+  if (!explicit_host_offsets && cursor != tensor_data_size)
+    return fail(KVT_ERR_INVALID,
+                "copy_handle_data_kernel_direct: tensor_data_size != sum of range lengths");
+  DeviceGuard g;
+  if (int rc = g.enter(device)) return rc;
+  const hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t bytes = n * sizeof(int64_t);
+  KVT_HIP(hipMemcpyAsync(src_dev, host_meta, bytes, hipMemcpyHostToDevice, s));
+  KVT_HIP(hipMemcpyAsync(dst_dev, host_meta + n, bytes, hipMemcpyHostToDevice, s));
+  KVT_HIP(hipMemcpyAsync(len_dev, host_meta + 2 * n, bytes, hipMemcpyHostToDevice, s));
+  const int rows = static_cast<int>(std::min<uint64_t>(std::max<uint64_t>(1, (longest + 4095) / 4096), 512));
+  const hipError_t e =
+      direction == KVT_COPY_D2H
+          ? launch_copy_ranges(layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
+                               static_cast<int64_t>(n), static_cast<int>(n), rows, s)
+          : launch_copy_ranges(tensor_buf, layer_gpu_ptr, src_dev, dst_dev, len_dev,
+                               static_cast<int64_t>(n), static_cast<int>(n), rows, s);
+  if (e != hipSuccess) return hip_fail(e, "copy_handle_data_kernel_direct launch");
+  return KVT_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -140,6 +186,19 @@ int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
   return guarded([&]() {
     return handle_data(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction, false,
                        device, stream, dev_meta, host_meta, max_block_num);
+  });
+}
+
+int kvt_copy_handle_data_kernel_direct(void* tensor_buf, void* layer_gpu_ptr,
+                                       const kvt_ipc_block* blocks, uint64_t n,
+                                       uint64_t tensor_data_size, int direction, int device,
+                                       void* stream, int64_t* src_offsets_dev,
+                                       int64_t* dst_offsets_dev, int64_t* lengths_dev,
+                                       int64_t* host_meta, int use_explicit_host_offsets) {
+  return guarded([&]() {
+    return handle_data_direct(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction,
+                              device, stream, src_offsets_dev, dst_offsets_dev, lengths_dev,
+                              host_meta, use_explicit_host_offsets != 0);
   });
 }
 

@@ -547,3 +547,58 @@ def test_plan_used_on_two_streams_then_destroyed_while_launches_are_queued():
         assert np.array_equal(_host(dst_layers[l][0]), exp), l
     for p2 in others:
         p2.close()
+
+
+@pytest.mark.parametrize("explicit", [False, True])
+def test_copy_handle_data_kernel_direct(explicit):
+    """copy_handle_data_kernel_direct (copy_kernels.cpp:363-439): single batch, separate device
+    arrays; the contiguous-side offset is the running sum, or blocks[i].src_offset when
+    use_explicit_host_offsets is set."""
+    rng = np.random.default_rng(12)
+    cap, n = 1 << 20, 40
+    lens = rng.integers(1, 6000, n).astype(np.uint64)
+    gpu_off = (np.cumsum(lens + rng.integers(0, 5000, n).astype(np.uint64)) - lens).astype(np.uint64)
+    assert int(gpu_off[-1] + lens[-1]) <= cap
+    total = int(lens.sum())
+    if explicit:      # contiguous side in shuffled order, with gaps
+        order = rng.permutation(n)
+        host_off = np.zeros(n, dtype=np.uint64)
+        cur = 0
+        for i in order:
+            host_off[i] = cur
+            cur += int(lens[i]) + int(rng.integers(0, 64))
+        size = cur
+    else:
+        host_off = (np.cumsum(lens) - lens).astype(np.uint64)
+        size = total
+    blocks = np.ascontiguousarray(np.stack([host_off if explicit else np.zeros(n, np.uint64),
+                                            gpu_off, lens], axis=1))
+    layer = _dev_bytes(cap, 44, "u8")
+    pinned = torch.zeros(size, dtype=torch.uint8).pin_memory()
+    dev = [torch.zeros(n, dtype=torch.int64, device="cuda") for _ in range(3)]
+    host_meta = torch.zeros(3 * n, dtype=torch.int64).pin_memory()
+    lib = kvt_amd.lib()
+    st = torch.cuda.Stream()
+
+    def call(buf, gpu, direction, data_size=size):
+        return lib.kvt_copy_handle_data_kernel_direct(
+            buf.data_ptr(), gpu.data_ptr(), blocks.ctypes.data, n, data_size, direction, 0,
+            st.cuda_stream, dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(),
+            host_meta.data_ptr(), 1 if explicit else 0)
+
+    assert call(pinned, layer, 1) == 0, lib.kvt_last_error()
+    st.synchronize()
+    layer_h, got = _host(layer), pinned.numpy()
+    for i in range(n):
+        a, b, m = int(host_off[i]), int(gpu_off[i]), int(lens[i])
+        assert np.array_equal(got[a:a + m], layer_h[b:b + m]), i
+    dst = torch.full((cap,), 0x33, dtype=torch.uint8, device="cuda")
+    assert call(pinned, dst, 0) == 0, lib.kvt_last_error()
+    st.synchronize()
+    exp = np.full(cap, 0x33, dtype=np.uint8)
+    for i in range(n):
+        b, m = int(gpu_off[i]), int(lens[i])
+        exp[b:b + m] = layer_h[b:b + m]
+    assert np.array_equal(_host(dst), exp)
+    # a range that leaves the contiguous buffer is refused before anything is launched
+    assert call(pinned, dst, 0, data_size=int((host_off + lens).max()) - 1) != 0
