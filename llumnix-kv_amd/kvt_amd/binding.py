@@ -164,6 +164,14 @@ def lib():
     return _lib
 
 
+def _quiet_close(obj):
+    """__del__ hook: at interpreter shutdown the module globals may already be gone."""
+    try:
+        obj.close()
+    except Exception:
+        pass
+
+
 def check(rc):
     if rc != 0:
         raise KvtError(rc, (lib().kvt_last_error() or b"").decode())
@@ -253,7 +261,7 @@ class BlockLists:
             lib().kvt_block_lists_destroy(self.h)
             self.h = _vp()
 
-    __del__ = close
+    __del__ = _quiet_close
 
     def clear(self):
         lib().kvt_block_lists_clear(self.h)
@@ -294,7 +302,7 @@ class RunLists:
             lib().kvt_run_lists_destroy(self.h)
             self.h = _vp()
 
-    __del__ = close
+    __del__ = _quiet_close
 
     def clear(self):
         lib().kvt_run_lists_clear(self.h)
@@ -355,7 +363,7 @@ class Parser:
             lib().kvt_parser_destroy(self.h)
             self.h = _vp()
 
-    __del__ = close
+    __del__ = _quiet_close
 
     def parse(self, task_struct, lists):
         """Appends one task's ranges; returns the KVT_* code (0 = ok)."""
@@ -395,7 +403,7 @@ class Cache:
             lib().kvt_cache_destroy(self.h)
             self.h = _vp()
 
-    __del__ = close
+    __del__ = _quiet_close
 
 
 class Plan:
@@ -438,7 +446,7 @@ class Plan:
             lib().kvt_plan_destroy(self.h)
             self.h = _vp()
 
-    __del__ = close
+    __del__ = _quiet_close
 
     def ready(self):
         check(lib().kvt_plan_ready(self.h))
@@ -489,7 +497,7 @@ class Session:
             lib().kvt_session_destroy(self.h)
             self.h = _vp()
 
-    __del__ = close
+    __del__ = _quiet_close
 
     def save_layer(self, layer, compute_stream=None):
         check(lib().kvt_session_save_layer(self.h, layer, _ptr(compute_stream)))
@@ -516,7 +524,7 @@ class Stager:
             lib().kvt_stager_destroy(self.h)
             self.h = _vp()
 
-    __del__ = close
+    __del__ = _quiet_close
 
     def slot_ptr(self, slot):
         return lib().kvt_stager_slot(self.h, slot)
