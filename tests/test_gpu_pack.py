@@ -602,3 +602,53 @@ def test_copy_handle_data_kernel_direct(explicit):
     assert np.array_equal(_host(dst), exp)
     # a range that leaves the contiguous buffer is refused before anything is launched
     assert call(pinned, dst, 0, data_size=int((host_off + lens).max()) - 1) != 0
+
+
+def test_random_range_lists_sweep():
+    """80 seeded batches of arbitrary ranges: 1-3 tensors, 1-3 layers, lengths from 1 byte to
+    70 000, alignments 1 / 4 / 16 / 256, shuffled list order, every chunk size, packed buffer
+    at a 16-, 4- or 1-byte aligned address."""
+    for seed in range(80):
+        rng = np.random.default_rng(10_000 + seed)
+        n_t, n_layers = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        caps_s = [int(rng.integers(1 << 14, 1 << 20)) for _ in range(n_t)]
+        caps_d = [int(rng.integers(1 << 14, 1 << 20)) for _ in range(n_t)]
+        lists, all_runs = kvt_amd.BlockLists(), []
+        for t in range(n_t):
+            runs, d = [], 0
+            align = int(rng.choice([1, 4, 16, 256]))
+            while len(runs) <= 60:
+                ln = int(rng.choice([1, 3, 16, 100, 4096, 5000, 40000, 70000]))
+                ln = max(align, ln // align * align)
+                gap = int(rng.integers(0, 4)) * align
+                if d + gap + ln > caps_d[t] or ln > caps_s[t]:
+                    break
+                s = int(rng.integers(0, (caps_s[t] - ln) // align + 1)) * align
+                runs.append((s, d + gap, ln))
+                d += gap + ln
+            runs = [runs[i] for i in rng.permutation(len(runs))] or [(0, 0, align)]
+            lists.append(t, runs)
+            all_runs.append(np.asarray(runs, np.uint64))
+        chunk = int(rng.choice([0, 4096, 8192, 65536, 524288]))
+        plan = kvt_amd.Plan(0, lists, caps_s, caps_d, chunk_bytes=chunk)
+        src = [[_dev_bytes((c + 3) // 4 * 4, seed * 64 + l * 8 + t, "u8")[:c] for t, c in enumerate(caps_s)]
+               for l in range(n_layers)]
+        dst = [[torch.full((c,), 0xA5, device="cuda", dtype=torch.uint8) for c in caps_d]
+               for _ in range(n_layers)]
+        sc, dc = kvt_amd.Cache(0, src, caps_s), kvt_amd.Cache(0, dst, caps_d)
+        pad = int(rng.choice([0, 0, 4, 1]))
+        stride = plan.layer_bytes + 256
+        packed = torch.zeros(n_layers * stride + 64, dtype=torch.uint8, device="cuda")
+        plan.pack(sc, 0, n_layers, packed.data_ptr() + pad, stride)
+        plan.unpack(dc, 0, n_layers, packed.data_ptr() + pad, stride)
+        torch.cuda.synchronize()
+        ph = _host(packed)[pad:]
+        for l in range(n_layers):
+            for t in range(n_t):
+                blob = checkers.oracle_pack(_host(src[l][t]), all_runs[t])
+                off = l * stride + plan.tensor_offset(t)
+                assert np.array_equal(ph[off:off + len(blob)], blob), (seed, l, t, chunk, pad)
+                exp = np.full(caps_d[t], 0xA5, dtype=np.uint8)
+                checkers.oracle_unpack(exp, all_runs[t], blob)
+                assert np.array_equal(_host(dst[l][t]), exp), (seed, l, t, chunk, pad)
+        plan.close()
