@@ -652,3 +652,25 @@ def test_random_range_lists_sweep():
                 checkers.oracle_unpack(exp, all_runs[t], blob)
                 assert np.array_equal(_host(dst[l][t]), exp), (seed, l, t, chunk, pad)
         plan.close()
+
+
+def test_transposing_pack_random_geometry_sweep():
+    """30 seeded page geometries (heads 1-9, 1-70 tokens per page, rows of 16-1024 bytes, so
+    also token rows longer than a slice) through the HND <-> NHD transform, each checked against
+    the oracle's permutation, numpy's transpose and the round trip."""
+    for seed in range(30):
+        rng = np.random.default_rng(500 + seed)
+        heads, ntpb = int(rng.integers(1, 10)), int(rng.integers(1, 71))
+        row = 16 * int(rng.choice([1, 2, 3, 8, 16, 31, 64]))
+        pool = int(rng.integers(6, 30))
+        w = workloads.llama70b_flashinfer(n_layers=int(rng.integers(1, 3)), pool=pool, n_req=2,
+                                          tokens=16)      # (tables are replaced below)
+        T = 2 * heads * row
+        for info in (w.src_info, w.dst_info):
+            info["block_sizes"], info["token_sizes"], info["num_kv_heads"] = [T * ntpb], [T], heads
+        src_ids = rng.permutation(pool)[:4]
+        dst_ids = rng.permutation(pool)[:4]
+        w.tasks = [[0, 2 * ntpb, True, [[int(x) for x in src_ids[2 * i:2 * i + 2]]],
+                    [[int(x) for x in dst_ids[2 * i:2 * i + 2]]]] for i in range(2)]
+        w.xform = (heads, ntpb, row)
+        _transposing(w, seed=seed + 40)
