@@ -109,6 +109,7 @@ static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
   }
   return KVT_OK;
 }
+
 extern "C" {
 
 // -------------------------------------------------------------------- plan
