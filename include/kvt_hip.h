@@ -293,6 +293,22 @@ int kvt_block_object_lists(int cache_shape, const kvt_worker_info* src, const kv
                            const uint32_t* src_blocks, const uint32_t* dst_blocks, uint64_t n,
                            kvt_block_lists* lists, uint64_t* object_bytes);
 
+/* A plan whose packed side holds one object per block SPANNING ALL LAYERS, for a
+ * store that keeps a block under one key (MooncakeKVSBackend saves whole blocks,
+ * all layers at once, when the last layer is done,
+ *                                               blade_kvt/hybrid_connector/mooncake_kvsbackend.py:382-437).
+ * `lists` = kvt_block_object_lists output (one cache tensor per layer), object_bytes
+ * = its *object_bytes, object_stride >= n_layers * object_bytes. Packed with
+ * layer_stride = object_bytes, block i's object is
+ *   [layer 0 part][layer 1 part]... at base + i * object_stride,
+ * each part being the per-layer object described above. (The store library is
+ * third-party and not part of the reference checkout; the order of the parts
+ * inside an object is this library's choice.) kvt_plan_layer_bytes() = the span
+ * of one layer's parts: (n_objects - 1) * object_stride + object_bytes. */
+int kvt_plan_create_objects(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
+                            const uint64_t* dst_capacity, uint64_t object_bytes,
+                            uint64_t object_stride, uint32_t chunk_bytes, kvt_plan** out);
+
 /* The store's block ids -> the engine's kernel-block ids when one store block
  * spans `factor` kernel blocks: out[i] = ids[i / factor] * factor + i % factor
  * for i < n * factor (VineyardKVSBackend._enlarge_list,

@@ -110,14 +110,13 @@ static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
   return KVT_OK;
 }
 
-extern "C" {
-
-// -------------------------------------------------------------------- plan
-
-int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
-                    const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
-                    kvt_plan** out) {
-  return guarded([&]() -> int {
+// Plan from plain range lists. object_bytes != 0: the packed side is a sequence of objects of
+// object_bytes each, object i placed at i * object_stride (room for the same object of other
+// layers behind it); every object must consist of whole ranges.
+static int create_plan(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
+                       const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
+                       uint64_t object_bytes, uint64_t object_stride, kvt_plan** out) {
+  {
     if (!lists || !src_capacity || !dst_capacity || !out)
       return fail(KVT_ERR_INVALID, "kvt_plan_create: null argument");
     if (lists->tensors.empty() || lists->tensors.size() > KVT_MAX_TENSORS)
@@ -207,9 +206,53 @@ int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* sr
       cursor += blob;
     }
     p->layer_bytes = round_up(cursor, kBlobAlign);
+    if (object_bytes != 0) {
+      // spread the objects: [object 0 of this layer | room for the other layers][object 1 ...
+      const uint64_t n_objects = p->tensor_bytes[0] / object_bytes;
+      for (Piece& q : pieces) {
+        const uint64_t obj = q.packed / object_bytes, in = q.packed % object_bytes;
+        if (in + q.len > object_bytes)
+          return fail(KVT_ERR_INVALID, "kvt_plan_create_objects: a range straddles two objects");
+        q.packed = obj * object_stride + in;
+      }
+      p->tensor_bytes[0] = n_objects == 0 ? 0 : (n_objects - 1) * object_stride + object_bytes;
+      p->layer_bytes = p->tensor_bytes[0];
+      p->min_layer_stride = object_bytes;
+    } else {
+      p->min_layer_stride = p->layer_bytes;
+    }
     if (int rc = finish_plan(p.get(), pieces)) return rc;
     *out = p.release();
     return KVT_OK;
+  }
+}
+
+extern "C" {
+
+// -------------------------------------------------------------------- plan
+
+int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
+                    const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
+                    kvt_plan** out) {
+  return guarded([&]() -> int {
+    return create_plan(device, lists, src_capacity, dst_capacity, xform, chunk_bytes, 0, 0, out);
+  });
+}
+
+int kvt_plan_create_objects(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
+                            const uint64_t* dst_capacity, uint64_t object_bytes,
+                            uint64_t object_stride, uint32_t chunk_bytes, kvt_plan** out) {
+  return guarded([&]() -> int {
+    if (!lists || lists->tensors.size() != 1)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create_objects: exactly one cache tensor per layer");
+    if (object_bytes == 0 || object_stride < object_bytes)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create_objects: object_stride < object_bytes");
+    uint64_t total = 0;
+    for (const kvt_ipc_block& r : lists->tensors[0]) total += r.length;
+    if (total % object_bytes != 0)
+      return fail(KVT_ERR_INVALID, "kvt_plan_create_objects: ranges do not add up to whole objects");
+    return create_plan(device, lists, src_capacity, dst_capacity, nullptr, chunk_bytes,
+                       object_bytes, object_stride, out);
   });
 }
 
@@ -339,6 +382,7 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
       cursor += blob;
     }
     p->layer_bytes = round_up(cursor, kBlobAlign);
+    p->min_layer_stride = p->layer_bytes;
     p->strided = n_shapes > 0;
 
     if (chunk_bytes == 0) {
@@ -438,7 +482,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   if (static_cast<uint64_t>(first_layer) + n_layers > cache->n_layers)
     return fail(KVT_ERR_OUT_OF_RANGE, "layer range exceeds the registered cache");
   if (n_layers > 65535) return fail(KVT_ERR_INVALID, "at most 65535 layers per launch");
-  if (n_layers > 1 && !blob_offsets && layer_stride < p->layer_bytes)
+  if (n_layers > 1 && !blob_offsets && layer_stride < p->min_layer_stride)
     return fail(KVT_ERR_INVALID, "layer_stride smaller than one packed layer");
   BlobOffsets blobs{};
   for (uint32_t t = 0; t < p->n_tensors; ++t)

@@ -208,6 +208,7 @@ struct kvt_plan {
   uint64_t n_chunks = 0;
   std::vector<uint64_t> tensor_bytes, tensor_offset, src_cap, dst_cap;
   uint64_t layer_bytes = 0;
+  uint64_t min_layer_stride = 0;   // smallest layer_stride a multi-layer launch accepts
   bool xform = false;
   kvt::XformDev xdev{};
   bool strided = false;            // some chunks carry a record shape (kvt_plan_create_runs)

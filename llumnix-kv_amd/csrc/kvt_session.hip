@@ -42,7 +42,7 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
   return guarded([&]() -> int {
     if (!plan || !cache || !packed || !out)
       return fail(KVT_ERR_INVALID, "kvt_session_create: null argument");
-    if (layer_stride < plan->layer_bytes)
+    if (layer_stride < plan->min_layer_stride)
       return fail(KVT_ERR_INVALID, "kvt_session_create: layer_stride smaller than one packed layer");
     if (int rc = check_device(plan->device)) return rc;
     DeviceGuard g;

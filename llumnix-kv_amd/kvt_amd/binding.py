@@ -73,6 +73,7 @@ SIGNATURES = {
     "kvt_run_lists_compress": (_int, [_vp, _vp]),
     "kvt_plan_create_runs": (_int, [_int, _vp, _P(_u64), _P(_u64), _u32, _P(_vp)]),
     "kvt_plan_num_strided_chunks": (_u64, [_vp]),
+    "kvt_plan_create_objects": (_int, [_int, _vp, _P(_u64), _P(_u64), _u64, _u64, _u32, _P(_vp)]),
     "kvt_plan_host_tables": (_int, [_vp, _P(_vp), _P(_u64), _P(_u32), _P(_vp)]),
     "kvt_pack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
     "kvt_unpack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
@@ -407,7 +408,9 @@ class Cache:
 
 
 class Plan:
-    def __init__(self, device, lists, src_capacity, dst_capacity, xform=None, chunk_bytes=0):
+    def __init__(self, device, lists, src_capacity, dst_capacity, xform=None, chunk_bytes=0,
+                 objects=None):
+        """objects = (object_bytes, object_stride): per-block objects spanning all layers."""
         n = lists.num_tensors()
         sc = (_u64 * max(1, n))(*src_capacity)
         dc = (_u64 * max(1, n))(*dst_capacity)
@@ -415,6 +418,10 @@ class Plan:
         if xform is not None:
             xf = C.byref(Xform(1, *xform))
         self.h = _vp()
+        if objects is not None:
+            check(lib().kvt_plan_create_objects(device, lists.h, sc, dc, objects[0], objects[1],
+                                                chunk_bytes, C.byref(self.h)))
+            return
         if isinstance(lists, RunLists):
             if xform is not None:
                 raise ValueError("no layout transform for a plan made from runs")

@@ -229,3 +229,41 @@ def test_framed_layers_of_a_tp_remapping_batch_with_run_plans():
         assert np.array_equal(_host(dst_layers[l][0]), exp), l
         rplan.close()
     stager.close()
+
+
+def test_per_block_objects_spanning_all_layers():
+    """One pack launch builds, for every block, one object holding that block of all layers
+    ([layer][K block][V block]); checked against torch.stack of kvcache[:, b] per layer, and
+    loaded back into other blocks of a second cache."""
+    n_layers, nblk, bs, h, d = 4, 24, 16, 2, 64
+    g = torch.Generator(device="cuda")
+    g.manual_seed(123)
+    kv = [torch.randn((2, nblk, bs, h, d), generator=g, device="cuda").to(torch.bfloat16)
+          for _ in range(n_layers)]
+    new = [torch.zeros_like(k) for k in kv]
+    B = 2 * bs * h * d * 2
+    rng = np.random.default_rng(9)
+    src_ids, dst_ids = rng.permutation(nblk)[:7], rng.permutation(nblk)[:7]
+    info = kvt_amd.ctypes_defs.make_worker_info(block_sizes=[B], token_sizes=[B // bs],
+                                                layer_num_blocks=nblk, num_layers=n_layers)
+    lists, ob = kvt_amd.block_object_lists(kvt_amd.ctypes_defs.SHAPE_FLASH, info, info, src_ids,
+                                           dst_ids)
+    assert ob == B
+    stride = n_layers * ob
+    plan = kvt_amd.Plan(0, lists, [B * nblk], [B * nblk], objects=(ob, stride))
+    sc = kvt_amd.Cache(0, [[k.view(torch.uint8).reshape(-1)] for k in kv], [B * nblk])
+    dc = kvt_amd.Cache(0, [[k.view(torch.uint8).reshape(-1)] for k in new], [B * nblk])
+    objs = torch.zeros((len(src_ids), stride), dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, n_layers, objs, ob)             # layer_stride = one layer's part
+    torch.cuda.synchronize()
+    for i, b in enumerate(src_ids):
+        want = torch.stack([kv[l][:, int(b)] for l in range(n_layers)]).contiguous()
+        assert torch.equal(objs[i], want.view(torch.uint8).reshape(-1)), i
+    plan.unpack(dc, 0, n_layers, objs, ob)
+    torch.cuda.synchronize()
+    s_idx = torch.as_tensor(src_ids, device="cuda")
+    d_idx = torch.as_tensor(dst_ids, device="cuda")
+    for l in range(n_layers):
+        exp = torch.zeros_like(kv[l])
+        exp[:, d_idx] = kv[l][:, s_idx]
+        assert torch.equal(new[l].view(torch.int16), exp.view(torch.int16)), l

@@ -269,3 +269,25 @@ def test_enlarge_block_ids_is_the_kvsbackend_formula():
         binding.enlarge_block_ids([1 << 31], 4)          # does not fit 32 bits
     with pytest.raises(kvt_amd.KvtError):
         binding.enlarge_block_ids([1], 0)
+
+
+def test_object_plan_tables_place_every_block_under_one_object():
+    """Host-only plan: packed position of block i's part = i * object_stride (+ the offset
+    inside the part), so that packing layer l with layer_stride = object_bytes builds
+    [layer 0 part][layer 1 part]... per block."""
+    B, nblk, L = 4096, 12, 3
+    lists, ob = kvt_amd.block_object_lists(kvt_amd.ctypes_defs.SHAPE_FLASH, _info([B], nblk),
+                                           _info([B], nblk), [5, 1, 9], [0, 2, 4])
+    plan = kvt_amd.Plan(-1, lists, [B * nblk], [B * nblk], objects=(ob, L * ob))
+    pack_t, unpack_t, cb, shapes = plan.host_tables()
+    assert plan.layer_bytes == 2 * L * ob + ob
+    got = sorted((int(c["packed"]), int(c["cache"]), int(c["len"])) for c in pack_t)
+    half = B // 2
+    want = []
+    for i, b in enumerate([5, 1, 9]):
+        want += [(i * L * ob, b * half, half), (i * L * ob + half, nblk * half + b * half, half)]
+    assert got == sorted(want)
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.Plan(-1, lists, [B * nblk], [B * nblk], objects=(ob, ob - 1))
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.Plan(-1, lists, [B * nblk], [B * nblk], objects=(ob + 16, 8 * ob))
