@@ -375,6 +375,64 @@ def leg_launchers(c, out):
     # pinned-host staging of packed layers, double buffered against the pack kernel
 
 
+def leg_store_objects(c, out):
+    """KVStore block objects (one per block and layer, or one per block over all layers):
+    pack rate in HBM and save rate through the pinned stager."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    wls, sides, new_event, sh = c.wls, c.sides, c.new_event, c.sh
+    w, side = wls[0], sides[0]
+    from kvt_amd.ctypes_defs import SHAPE_FLASH
+    if w.cache_shape != SHAPE_FLASH or w.xform is not None:
+        return
+    s_info, d_info = w.worker_infos()
+    ids = sorted({b for t in w.tasks for b in t[3][0]})[:4096]
+    rng = np.random.default_rng(1)
+    dst_ids = rng.permutation(w.dst_info["layer_num_blocks"])[:len(ids)]
+    lists, ob = kvt.block_object_lists(w.cache_shape, s_info, d_info, ids, dst_ids)
+    L = w.n_layers
+    res = {"blocks": len(ids), "object_bytes_per_layer": ob, "layers": L}
+    for name, objects in (("per_block_and_layer", None), ("per_block_all_layers", (ob, L * ob))):
+        plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), objects=objects)
+        stride = ob if objects else plan.layer_bytes
+        buf = torch.empty(len(ids) * ob * L, dtype=torch.uint8, device="cuda")
+        a, b = new_event(), new_event()
+        for rep in range(2):
+            lib.kvt_event_record(a, sh)
+            plan.pack(side.src_cache, 0, L, buf, stride, sh)
+            lib.kvt_event_record(b, sh)
+        lib.kvt_event_synchronize(b)
+        res[name + "_pack_gbps"] = round(2.0 * len(ids) * ob * L / (ev_ms(lib, a, b) * 1e-3) / 1e9, 1)
+        plan.close()
+        del buf
+    # save: per-layer object arrays through two pinned slots, several layers per transfer
+    plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"))
+    lbytes = plan.layer_bytes
+    group = max(1, min(L, -(-(256 << 20) // lbytes)))
+    n_groups = max(1, min(6, L // group))
+    stg = kvt.Stager(0, group * lbytes, 2)
+    bufs = [torch.empty(group * lbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    ps = torch.cuda.Stream()
+    times = []
+    for phase in range(3):
+        torch.cuda.synchronize()
+        t_a = time.perf_counter()
+        for g in range(n_groups):
+            slot = g % 2
+            if g >= 2:
+                stg.wait(slot)
+            plan.pack(side.src_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
+            stg.save(slot, bufs[slot], group * lbytes, ps.cuda_stream)
+        stg.wait(0)
+        if n_groups > 1:
+            stg.wait(1)
+        times.append(time.perf_counter() - t_a)
+    res["save_gbps"] = round(n_groups * group * len(ids) * ob / min(times[1:]) / 1e9, 2)
+    res["save_note"] = "%d transfers of %d layer(s) x %d objects" % (n_groups, group, len(ids))
+    stg.close()
+    plan.close()
+    out["kvstore_objects"] = res
+
+
 def leg_staging(c, out):
     """Packed layers through pinned host memory, double buffered against the kernels."""
     torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
@@ -669,7 +727,7 @@ def main():
     if not args.skip_cpu:
         leg_cpu(c, out)
     if not args.skip_extras:
-        for leg in (leg_latency, leg_session, leg_launchers, leg_staging):
+        for leg in (leg_latency, leg_session, leg_launchers, leg_store_objects, leg_staging):
             leg(c, out)
 
     print(json.dumps(out), flush=True)
