@@ -375,6 +375,72 @@ def leg_launchers(c, out):
     # pinned-host staging of packed layers, double buffered against the pack kernel
 
 
+def leg_frames(c, out):
+    """Layer messages (TCP frame format) built around the GPU's output and consumed again:
+    header + range metadata written by the host, blobs packed in HBM and placed by DMA;
+    receiver parses the frame, DMAs the blobs back and unpacks."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    wls, sides, first = c.wls, c.sides, c.first
+    from kvt_amd import binding
+    w, side = wls[0], sides[0]
+    if w.xform is not None or args.plan != "ranges":
+        return
+    plan, lists = first[0]
+    lay = binding.wire_layout_of(binding.WIRE_TCP, lists)
+    if lay.total_bytes > (3 << 30):
+        return
+    L = min(w.n_layers, 6)
+    stg = kvt.Stager(0, lay.total_bytes, 2)
+    dev = [torch.empty(plan.layer_bytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    ps = torch.cuda.Stream()
+    payload = sum(lay.blob_bytes[t] for t in range(w.n_tensors))
+    host_write, host_parse, send_t, recv_t = [], [], [], []
+    for phase in range(4):
+        torch.cuda.synchronize()
+        t_a = time.perf_counter()
+        for l in range(L):
+            slot = l % 2
+            if l >= 2:
+                stg.wait(slot)
+            h0 = time.perf_counter()
+            binding.wire_write_frame(binding.WIRE_TCP, stg.slot_ptr(slot), stg.slot_bytes, 1, l, lists)
+            host_write.append(time.perf_counter() - h0)
+            plan.pack(side.src_cache, l, 1, dev[slot], plan.layer_bytes, ps.cuda_stream)
+            for t in range(w.n_tensors):
+                stg.save_at(slot, lay.blob_offset[t], dev[slot].data_ptr() + plan.tensor_offset(t),
+                            lay.blob_bytes[t], ps.cuda_stream)
+        stg.wait(0)
+        if L > 1:
+            stg.wait(1)
+        send_t.append(time.perf_counter() - t_a)
+    # receiver: the last two frames are still in the slots; consume them repeatedly
+    for phase in range(4):
+        torch.cuda.synchronize()
+        t_a = time.perf_counter()
+        for l in range(L):
+            slot = l % 2
+            h0 = time.perf_counter()
+            rc, reqid, layer, rlists, rlay = binding.wire_parse_frame(
+                binding.WIRE_TCP, stg.slot_ptr(slot), lay.total_bytes, w.n_tensors)
+            host_parse.append(time.perf_counter() - h0)
+            assert rc == 0
+            rlists.close()
+            for t in range(w.n_tensors):
+                stg.load_at(slot, rlay.blob_offset[t], dev[slot].data_ptr() + plan.tensor_offset(t),
+                            rlay.blob_bytes[t], ps.cuda_stream)
+            plan.unpack(side.dst_cache, int(layer), 1, dev[slot], plan.layer_bytes, ps.cuda_stream)
+        ps.synchronize()
+        recv_t.append(time.perf_counter() - t_a)
+    out["layer_frames"] = {
+        "frame_bytes": int(lay.total_bytes), "metadata_bytes": int(lay.total_bytes - payload),
+        "send_gbps": round(L * payload / min(send_t[1:]) / 1e9, 2),
+        "recv_gbps": round(L * payload / min(recv_t[1:]) / 1e9, 2),
+        "host_write_frame_us": round(statistics.median(host_write) * 1e6, 1),
+        "host_parse_frame_us": round(statistics.median(host_parse) * 1e6, 1),
+        "note": "%d layer messages through 2 pinned slots; GB/s = payload over PCIe" % L}
+    stg.close()
+
+
 def leg_store_objects(c, out):
     """KVStore block objects (one per block and layer, or one per block over all layers):
     pack rate in HBM and save rate through the pinned stager."""
@@ -727,7 +793,8 @@ def main():
     if not args.skip_cpu:
         leg_cpu(c, out)
     if not args.skip_extras:
-        for leg in (leg_latency, leg_session, leg_launchers, leg_store_objects, leg_staging):
+        for leg in (leg_latency, leg_session, leg_launchers, leg_frames, leg_store_objects,
+                    leg_staging):
             leg(c, out)
 
     print(json.dumps(out), flush=True)
