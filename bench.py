@@ -448,7 +448,8 @@ def leg_store_objects(c, out):
     wls, sides, new_event, sh = c.wls, c.sides, c.new_event, c.sh
     w, side = wls[0], sides[0]
     from kvt_amd.ctypes_defs import SHAPE_FLASH
-    if w.cache_shape != SHAPE_FLASH or w.xform is not None:
+    if (w.cache_shape != SHAPE_FLASH or w.xform is not None or
+            w.src_info["block_sizes"] != w.dst_info["block_sizes"]):
         return
     s_info, d_info = w.worker_infos()
     ids = sorted({b for t in w.tasks for b in t[3][0]})[:4096]
