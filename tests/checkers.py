@@ -69,6 +69,8 @@ def ref():
             lib.kvtref_parse.argtypes = _PARSE_HEAD + _PARSE_TAIL
             lib.kvtref_parse.restype = C.c_int
             lib.kvtref_free.argtypes = [C.c_void_p]
+            lib.kvtref_plan_parse.argtypes = _PARSE_HEAD + _PARSE_TAIL + [C.POINTER(C.c_int)]
+            lib.kvtref_plan_parse.restype = C.c_int
         _cache["r"] = lib
     return _cache["r"]
 
@@ -83,13 +85,13 @@ def _collect(free, outs, n_out, n_tensors, cap):
     return res
 
 
-def _run(fn, free, head, tasks, extra):
+def _run(fn, free, head, tasks, extra, tail=()):
     cap = 8
     outs = (C.POINTER(IpcBlock) * cap)()
     n_out = (C.c_uint64 * cap)()
     n_t = C.c_uint32(0)
     arr = task_array(tasks)
-    rc = fn(*head, *extra, arr, len(tasks), cap, outs, n_out, C.byref(n_t))
+    rc = fn(*head, *extra, arr, len(tasks), cap, outs, n_out, C.byref(n_t), *tail)
     if rc != 0:
         return rc, []
     return rc, _collect(free, outs, n_out, n_t.value, cap)
@@ -107,6 +109,16 @@ def ref_parse(parser_id, src, dst, valid, tp_size, tp_rank, tasks):
     lib = ref()
     head = (parser_id, C.byref(src), C.byref(dst), valid, tp_size, tp_rank)
     return _run(lib.kvtref_parse, lib.kvtref_free, head, tasks, ())
+
+
+def ref_plan_parse(cache_shape, src, dst, valid, tp_size, tp_rank, tasks):
+    """The reference's descriptor-driven generator (cache_transfer_spec.cpp) on the same
+    inputs -> (rc, per-tensor arrays, TPKind)."""
+    lib = ref()
+    kind = C.c_int(-1)
+    head = (cache_shape, C.byref(src), C.byref(dst), valid, tp_size, tp_rank)
+    rc, out = _run(lib.kvtref_plan_parse, lib.kvtref_free, head, tasks, (), (C.byref(kind),))
+    return rc, out, kind.value
 
 
 def oracle_select(shape, src, dst):
