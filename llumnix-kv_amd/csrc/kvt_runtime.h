@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <memory>
 #include <mutex>
 #include <string>
@@ -219,7 +220,8 @@ struct kvt_plan {
   kvt::Chunk* dev_chunks = nullptr;     // [0, n_chunks): pack order; [n_chunks, 2 n_chunks): unpack order
   kvt::TableBuf* buf = nullptr;         // storage of dev_chunks (recycled through the table pool)
   hipEvent_t uploaded = nullptr;   // completes when the table has reached the device
-  mutable bool upload_seen = false;  // a launch has already observed `uploaded` as complete
+  // a launch has already observed `uploaded` as complete (several threads may launch one plan)
+  mutable std::atomic<bool> upload_seen{false};
 };
 
 namespace kvt {

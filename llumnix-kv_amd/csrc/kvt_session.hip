@@ -117,7 +117,12 @@ int kvt_session_wait_layer(kvt_session* s, uint32_t layer) {
 int kvt_session_join(kvt_session* s, void* stream) {
   return guarded([&]() -> int {
     if (!s) return fail(KVT_ERR_INVALID, "kvt_session_join: null session");
-    if (s->last_done) KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), s->last_done, 0));
+    hipEvent_t last = nullptr;
+    {
+      std::lock_guard<std::mutex> lock(s->mu);
+      last = s->last_done;
+    }
+    if (last) KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), last, 0));
     return KVT_OK;
   });
 }
