@@ -138,3 +138,37 @@ def test_int64_launcher_arrays_beyond_4_gib():
     lut = torch.from_numpy(table).cuda()
     bits = gathered.view(torch.int16).to(torch.int32) & 0xFFFF
     assert torch.equal(out8, lut[bits.long()])
+
+
+def test_transposing_pack_with_a_6_gib_page_pool():
+    # HND pages -> NHD blob and back; page bases beyond 2^32
+    w = workloads.llama70b_flashinfer(n_layers=1, pool=98304, n_req=3, tokens=2048)
+    heads, ntpb, row = w.xform
+    cap = w.capacities("src")[0]
+    assert cap == 6 * GIB
+    plan, lists = pipeline.build_plan(w, 0)
+    runs = _oracle_lists(w)[0]
+    assert np.array_equal(lists.tensor(0), runs)
+    assert (runs[:, 0] >= 2**32).sum() > 20 and (runs[:, 1] >= 2**32).sum() > 20
+    B = 2 * heads * ntpb * row
+    nblk = cap // B
+    s_ids = torch.from_numpy(np.concatenate(
+        [np.arange(r[0] // B, (r[0] + r[2]) // B) for r in runs]).astype(np.int64)).cuda()
+    d_ids = torch.from_numpy(np.concatenate(
+        [np.arange(r[1] // B, (r[1] + r[2]) // B) for r in runs]).astype(np.int64)).cuda()
+    assert len(torch.unique(d_ids)) == len(d_ids)
+    src = _random_bytes(cap, 15)
+    dst = torch.full((cap,), 0xA5, device="cuda", dtype=torch.uint8)
+    sc, dc = kvt_amd.Cache(0, [[src]], [cap]), kvt_amd.Cache(0, [[dst]], [cap])
+    stride = plan.layer_bytes
+    assert stride == len(s_ids) * B
+    packed = torch.zeros(stride, dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, 1, packed, stride)
+    plan.unpack(dc, 0, 1, packed, stride)
+    torch.cuda.synchronize()
+    picked = src.view(nblk, 2, heads, ntpb, row).index_select(0, s_ids)
+    want = picked.permute(0, 1, 3, 2, 4).contiguous()
+    assert torch.equal(packed, want.view(-1))
+    exp = torch.full_like(dst, 0xA5).view(nblk, 2, heads, ntpb, row)
+    exp.index_copy_(0, d_ids, picked)
+    assert torch.equal(dst.view(nblk, 2, heads, ntpb, row), exp)
