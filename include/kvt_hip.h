@@ -389,6 +389,13 @@ void kvt_session_destroy(kvt_session* s);
 /* save_kv_layer hook: layer `layer` of the cache is complete once the work
  * already queued on compute_stream has run. Never blocks the host. */
 int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream);
+/* The same for a caller that owns the per-layer events, as the reference's Python side does:
+ * it creates one event per layer, hands their handles to the library at init and records
+ * event[layer] itself after the layer's KV is written (blade_kvt/kv_transfer_impl.py:287-291,
+ * 320-327; consumed by CudaEventBarrier::wait, kvtransfer/src/context.cpp:18-20).
+ * `ready_event` is that hipEvent_t (torch.cuda.Event.cuda_event), already recorded on the
+ * compute stream; the side stream waits for it, the host never does. */
+int kvt_session_save_layer_event(kvt_session* s, uint32_t layer, void* ready_event);
 /* Host-blocking wait until layer's packed bytes are complete (what the
  * transport thread calls before send_data(layer), Step::wait_layer_ready in the
  * reference, kvtransfer/src/step.cpp:49-69). May be called from another thread

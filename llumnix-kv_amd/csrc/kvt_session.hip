@@ -80,6 +80,21 @@ void kvt_session_destroy(kvt_session* s) {
   delete s;
 }
 
+// The pack of `layer` on the side stream, gated by `ready` (already recorded).
+static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
+  KVT_HIP(hipStreamWaitEvent(s->side, ready, 0));
+  uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
+  if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
+  KVT_HIP(hipEventRecord(s->done[layer], s->side));
+  {
+    std::lock_guard<std::mutex> lock(s->mu);
+    s->last_done = s->done[layer];
+    s->issued[layer] = 1;
+  }
+  s->issued_cv.notify_all();
+  return KVT_OK;
+}
+
 int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream) {
   return guarded([&]() -> int {
     if (!s) return fail(KVT_ERR_INVALID, "kvt_session_save_layer: null session");
@@ -87,17 +102,18 @@ int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream)
     DeviceGuard g;
     if (int rc = g.enter(s->plan->device)) return rc;
     KVT_HIP(hipEventRecord(s->ready[layer], static_cast<hipStream_t>(compute_stream)));
-    KVT_HIP(hipStreamWaitEvent(s->side, s->ready[layer], 0));
-    uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
-    if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
-    KVT_HIP(hipEventRecord(s->done[layer], s->side));
-    {
-      std::lock_guard<std::mutex> lock(s->mu);
-      s->last_done = s->done[layer];
-      s->issued[layer] = 1;
-    }
-    s->issued_cv.notify_all();
-    return KVT_OK;
+    return issue_layer(s, layer, s->ready[layer]);
+  });
+}
+
+int kvt_session_save_layer_event(kvt_session* s, uint32_t layer, void* ready_event) {
+  return guarded([&]() -> int {
+    if (!s || !ready_event)
+      return fail(KVT_ERR_INVALID, "kvt_session_save_layer_event: null argument");
+    if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    DeviceGuard g;
+    if (int rc = g.enter(s->plan->device)) return rc;
+    return issue_layer(s, layer, static_cast<hipEvent_t>(ready_event));
   });
 }
 

@@ -95,6 +95,7 @@ SIGNATURES = {
     "kvt_session_create": (_int, [_vp, _vp, _vp, _u64, _P(_vp)]),
     "kvt_session_destroy": (None, [_vp]),
     "kvt_session_save_layer": (_int, [_vp, _u32, _vp]),
+    "kvt_session_save_layer_event": (_int, [_vp, _u32, _vp]),
     "kvt_session_wait_layer": (_int, [_vp, _u32]),
     "kvt_session_join": (_int, [_vp, _vp]),
     "kvt_session_side_stream": (_vp, [_vp]),
@@ -508,6 +509,12 @@ class Session:
 
     def save_layer(self, layer, compute_stream=None):
         check(lib().kvt_session_save_layer(self.h, layer, _ptr(compute_stream)))
+
+    def save_layer_event(self, layer, ready_event):
+        """ready_event: a hipEvent_t handle the caller has recorded (an int, e.g.
+        torch.cuda.Event.cuda_event), or the torch event itself."""
+        handle = getattr(ready_event, "cuda_event", ready_event)
+        check(lib().kvt_session_save_layer_event(self.h, layer, handle))
 
     def wait_layer(self, layer):
         check(lib().kvt_session_wait_layer(self.h, layer))

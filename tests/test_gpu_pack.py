@@ -403,6 +403,40 @@ def test_per_layer_session_on_side_stream():
     sess.close()
 
 
+def test_per_layer_session_gated_by_the_callers_own_events():
+    """The reference's arrangement (blade_kvt/kv_transfer_impl.py:287-291, 320-327): the
+    engine owns one event per layer, created once, and re-records event[layer] in every
+    step; the library only ever sees the handles."""
+    w = workloads.llama8b_batch(n_layers=5, src_pool=256, dst_pool=256, n_req=3, min_tok=200,
+                                max_tok=900)
+    plan, lists = pipeline.build_plan(w, 0)
+    cap = w.capacities("src")[0]
+    layers = [[torch.zeros(cap, dtype=torch.uint8, device="cuda")] for _ in range(w.n_layers)]
+    cache = kvt_amd.Cache(0, layers, w.capacities("src"))
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    events = [torch.cuda.Event() for _ in range(w.n_layers)]
+    compute = torch.cuda.Stream()
+    for step in range(2):                          # the same events serve every step
+        sess = kvt_amd.Session(plan, cache, packed, stride)
+        fresh = [_dev_bytes(cap, 70 + 10 * step + l) for l in range(w.n_layers)]
+        with torch.cuda.stream(compute):
+            for l in range(w.n_layers):
+                layers[l][0].copy_(fresh[l])
+                events[l].record(compute)
+                sess.save_layer_event(l, events[l].cuda_event if l % 2 else events[l])
+        for l in range(w.n_layers):
+            sess.wait_layer(l)
+            blob = checkers.oracle_pack(_host(fresh[l]), lists.tensor(0))
+            got = packed[l * stride:l * stride + len(blob)].cpu().numpy()
+            assert np.array_equal(got, blob), (step, l)
+        sess.join(compute.cuda_stream)
+        compute.synchronize()
+        sess.close()
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.Session(plan, cache, packed, stride).save_layer_event(0, None)
+
+
 def test_session_inside_hip_graph_replays():
     w = workloads.llama8b_single(n_layers=4, pool=64, tokens=200)
     plan, lists = pipeline.build_plan(w, 0)
