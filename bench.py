@@ -61,6 +61,12 @@ def build_workload(cfg, scale):
                                  pool=max(512, int(36864 * scale)), n_req=max(2, int(128 * scale))),
                 W.qwen3next_gdn(n_layers=max(2, int(36 * scale)), slots=max(4, int(256 * scale)),
                                 n_req=max(2, int(128 * scale)))]
+    if cfg == 9:
+        # config 5 in the reference's own arrangement: one tensor per full-attention layer with
+        # uniform 2 MiB pages shared by attention and the GDN states in front of it
+        return [W.qwen3next_uniform_pages(n_layers=max(2, int(12 * scale)),
+                                          pool=max(16, int(1024 * scale)),
+                                          n_req=max(2, int(128 * scale)))]
     if cfg in (6, 7, 8):
         # TP-remapping batches (not among the baseline configurations): config 2's batch with
         # the sender on TP2 and the receiver on TP1 (6), TP1 -> TP2 on the ragged layout (7),
@@ -564,7 +570,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", type=int, default=2, help="BASELINE.json configs[] index + 1")
+    ap.add_argument("--config", type=int, default=2, help="1-5: BASELINE.json configs[] index + 1; 6-8: TP-remapping batches; "
+                         "9: config 5 with the reference's uniform 2 MiB pages")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")
     ap.add_argument("--chunk-bytes", type=int, default=0)
     ap.add_argument("--plan", choices=["ranges", "runs"], default="ranges",

@@ -28,10 +28,11 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
   int wgs = 0;
   if (int rc = range_launch_shape(n, num_wg, &wgs)) return rc;
   // The range lengths live on the device, so the grid cannot be sized to them: `rows`
-  // workgroups stride over the 4 KiB slices of each range. Workgroups that find nothing to do
-  // are not free (35 000 ranges: 6.1 TB/s with 2 rows, 5.9 with 8, 4.1 with 32), so a long
-  // list gets 2 rows and only a short one more (enough to fill the device when its ranges
-  // are long).
+  // workgroups stride over the 4 KiB slices of each range. One slice per workgroup is the
+  // fastest shape, but workgroups that find nothing to do are not free (35 000 ranges of 8
+  // slices: 6.0 TB/s with 1 row, 6.3 with 2, 6.45 with 4, 6.5 with 8, 4.5 with 16, 2.2 with
+  // 64), so a long list gets 2 rows (at most half idle even for one-slice ranges) and only a
+  // short one more (enough to fill the device when its ranges are long).
   const int rows = static_cast<int>(std::max<int64_t>(2, std::min<int64_t>(64, (8192 + n - 1) / n)));
   const hipStream_t s = static_cast<hipStream_t>(stream);
   const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, s)

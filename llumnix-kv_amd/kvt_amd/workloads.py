@@ -156,6 +156,36 @@ def qwen3next_gdn(n_layers=36, slots=256, n_req=128, seed=20256):
                     n_layers, info, dict(info), tasks, elem_dtype="f32", seed=seed)
 
 
+def qwen3next_uniform_pages(n_layers=12, pool=1024, n_req=128, tokens=4096, n_gdn=3, seed=20258):
+    """Config 5 the way the reference itself lays a hybrid model out: ONE cache tensor per
+    full-attention layer, shared with the n_gdn linear-attention layers in front of it, with
+    one uniform page size (kvtbackend.py:994-1000). The page must hold a 2 MiB GDN state
+    (32 x 128 x 128 fp32), so an attention page holds 1024 tokens of 2 KV heads x 256 bf16.
+    Block groups per request: [gdn_0, .., gdn_{n-1}, attn]; a request sends its attention pages
+    and, with its last token, one state page per GDN layer
+    (parse_block_qwen3_next.cpp:865-955)."""
+    rng = np.random.default_rng(seed)
+    T, page = 2 * 2 * 256 * 2, 32 * 128 * 128 * 4
+    ntpb = page // T
+    n_attn = (tokens + ntpb - 1) // ntpb
+    per_req = n_gdn + n_attn
+    if per_req * n_req > pool:
+        raise ValueError("pool too small for disjoint tables: %d > %d" % (per_req * n_req, pool))
+    sperm, dperm = rng.permutation(pool), rng.permutation(pool)
+    tasks = []
+    for r in range(n_req):
+        s = [int(x) for x in sperm[r * per_req:(r + 1) * per_req]]
+        d = [int(x) for x in dperm[r * per_req:(r + 1) * per_req]]
+        sg = [[s[g]] for g in range(n_gdn)] + [s[n_gdn:]]
+        dg = [[d[g]] for g in range(n_gdn)] + [d[n_gdn:]]
+        tasks.append([0, tokens, True, sg, dg])
+    info = dict(block_sizes=[page], token_sizes=[T], layer_num_blocks=pool, num_kv_heads=2,
+                num_layers=n_layers, num_gdn_layers=n_gdn)
+    return Workload("qwen3-next hybrid, uniform 2 MiB pages %dreq x %d tok" % (n_req, tokens),
+                    SHAPE_QWEN3_NEXT_FLASH, "HYBRID_PEQD", n_layers, info, dict(info), tasks,
+                    seed=seed)
+
+
 def tp_split(layout="flash", p_tp=2, d_tp=1, rank=0, n_layers=32, src_pool=16384,
              dst_pool=24576, n_req=64, min_tok=1024, max_tok=8192, total_heads=8, head_dim=128,
              ntpb=16, seed=20257):

@@ -126,6 +126,24 @@ def test_config5_attention_pages_and_gdn_states():
     _check_pack_unpack(workloads.qwen3next_gdn(n_layers=2, slots=12, n_req=5), chunk_bytes=65536)
 
 
+def test_config5_reference_layout_uniform_pages_shared_by_attention_and_gdn():
+    w = workloads.qwen3next_uniform_pages(n_layers=2, pool=40, n_req=5)
+    lists = _oracle_lists(w)[0]
+    assert len(lists) <= 5 * 7 and int(lists[:, 2].sum()) == 5 * 7 * (2 << 20)
+    _check_pack_unpack(w)
+    # a chunked prefill: the first step ends inside the second attention page and sends
+    # page 0 only; the step that reaches the last token sends the rest and the GDN states
+    first, last = [list(t) for t in w.tasks[:1]], [list(t) for t in w.tasks[:1]]
+    first[0][:3] = [0, 1500, False]
+    last[0][:3] = [1500, 4096 - 1500, True]
+    w.tasks = first
+    assert len(_oracle_lists(w)[0]) == 1
+    _check_pack_unpack(w, seed=3)
+    w.tasks = last
+    assert int(_oracle_lists(w)[0][:, 2].sum()) == 6 * (2 << 20)
+    _check_pack_unpack(w, seed=4)
+
+
 def test_chunked_prefill_steps_and_ragged_tail():
     # two chunked-prefill steps of one request + a second request, ragged last block
     w = workloads.llama8b_single(n_layers=2, pool=64, tokens=100)
