@@ -143,7 +143,12 @@ int kvt_validate_ipc_block_bounds(const kvt_ipc_block* blocks, uint64_t n, uint6
  * (flattened by _flatten_cache,                 blade_kvt/hybrid_connector/kvtbackend.py:594-629).
  * ptrs is a host array of n_layers * n_tensors device pointers
  * (ptrs[layer * n_tensors + tensor]); capacity[t] is tensor t's size in bytes
- * (block_sizes[t] * layer_num_blocks). The table is copied to the device once. */
+ * (block_sizes[t] * layer_num_blocks). The table is copied to the device once.
+ * Every pointer is checked against what the runtime knows about it: memory the
+ * device cannot address is refused (KVT_ERR_INVALID), and so is a capacity that
+ * reaches beyond the device allocation holding the pointer
+ * (KVT_ERR_OUT_OF_RANGE) -- a kernel running off a tensor is a GPU memory
+ * fault, not an error code. */
 typedef struct kvt_cache kvt_cache;
 int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, uint32_t n_tensors,
                        const uint64_t* capacity, kvt_cache** out);

@@ -41,6 +41,14 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
   return KVT_OK;
 }
 
+// Workgroups per range when the lengths are known on the host: the mean number of slices
+// per range (bounded). Equal lengths then get exactly one slice per workgroup, the fastest
+// shape; in a mixed list the few long ranges are strided over by their `rows` workgroups
+// instead of every short range paying for idle ones.
+int rows_for(uint64_t slices, uint64_t n_ranges) {
+  return static_cast<int>(std::min<uint64_t>(std::max<uint64_t>(1, (slices + n_ranges - 1) / n_ranges), 512));
+}
+
 // Shared body of the two "handle data" entry points. `halve`: converting
 // gather (contiguous side advances by length / 2, lengths passed to the kernel
 // are element counts).
@@ -71,23 +79,22 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     int64_t* contig = host_meta;
     int64_t* gpu = host_meta + m;
     int64_t* lens = host_meta + 2 * m;
-    uint64_t longest = 0;
+    const uint64_t unit = halve ? 8192 : 4096;  // source bytes of one workgroup's slice
+    uint64_t slices = 0;
     for (uint64_t i = 0; i < m; ++i) {
       const kvt_ipc_block& b = blocks[first + i];
       contig[i] = static_cast<int64_t>(host_cursor);
       gpu[i] = static_cast<int64_t>(b.dst_offset);
       lens[i] = static_cast<int64_t>(halve ? b.length / 2 : b.length);
       host_cursor += halve ? b.length / 2 : b.length;
-      longest = std::max<uint64_t>(longest, b.length);
+      slices += (b.length + unit - 1) / unit;
     }
     KVT_HIP(hipMemcpyAsync(dev_meta, host_meta, 3 * m * sizeof(int64_t), hipMemcpyHostToDevice, s));
     const int64_t* d_contig = dev_meta;
     const int64_t* d_gpu = dev_meta + m;
     const int64_t* d_lens = dev_meta + 2 * m;
     const int wgs = static_cast<int>(m);
-    // one workgroup per 4 KiB slice of the longest range (bounded; longer ranges are strided)
-    const uint64_t unit = halve ? 8192 : 4096;
-    const int rows = static_cast<int>(std::min<uint64_t>(std::max<uint64_t>(1, (longest + unit - 1) / unit), 512));
+    const int rows = rows_for(slices, m);
     hipError_t e;
     if (halve)
       e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
@@ -117,7 +124,7 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
     return fail(KVT_ERR_INVALID, "copy_handle_data_kernel_direct: bad direction");
   if (n > 0x7FFFFFFFull) return fail(KVT_ERR_INVALID, "too many ranges");
   if (int rc = check_device(device)) return rc;
-  uint64_t cursor = 0, longest = 0;
+  uint64_t cursor = 0, slices = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const kvt_ipc_block& b = blocks[i];
     const uint64_t host_off = explicit_host_offsets ? b.src_offset : cursor;
@@ -128,7 +135,7 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
     host_meta[n + i] = static_cast<int64_t>(b.dst_offset);
     host_meta[2 * n + i] = static_cast<int64_t>(b.length);
     cursor += b.length;
-    longest = std::max<uint64_t>(longest, b.length);
+    slices += (b.length + 4095) / 4096;
   }
   if (!explicit_host_offsets && cursor != tensor_data_size)
     return fail(KVT_ERR_INVALID,
@@ -140,7 +147,7 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
   KVT_HIP(hipMemcpyAsync(src_dev, host_meta, bytes, hipMemcpyHostToDevice, s));
   KVT_HIP(hipMemcpyAsync(dst_dev, host_meta + n, bytes, hipMemcpyHostToDevice, s));
   KVT_HIP(hipMemcpyAsync(len_dev, host_meta + 2 * n, bytes, hipMemcpyHostToDevice, s));
-  const int rows = static_cast<int>(std::min<uint64_t>(std::max<uint64_t>(1, (longest + 4095) / 4096), 512));
+  const int rows = rows_for(slices, n);
   const hipError_t e =
       direction == KVT_COPY_D2H
           ? launch_copy_ranges(layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,

@@ -261,6 +261,21 @@ def test_plan_refuses_ranges_beyond_capacity_and_small_caches():
     torch.cuda.synchronize()
 
 
+def test_cache_registration_checks_what_the_runtime_knows_about_the_memory():
+    big = torch.zeros(64 << 20, dtype=torch.uint8, device="cuda")      # an allocation of its own
+    kvt_amd.Cache(0, [[big]], [64 << 20]).close()
+    kvt_amd.Cache(0, [[big[4096:]]], [(64 << 20) - 4096]).close()      # interior pointers are fine
+    with pytest.raises(kvt_amd.KvtError) as e:
+        kvt_amd.Cache(0, [[big]], [(64 << 20) + (1 << 30)])             # runs off the allocation
+    assert e.value.code == 1 and "beyond the device allocation" in str(e.value)
+    host = np.zeros(1 << 16, dtype=np.uint8)
+    with pytest.raises(kvt_amd.KvtError) as e:
+        kvt_amd.Cache(0, [[host]], [1 << 16])                           # pageable host memory
+    assert "cannot address" in str(e.value) or "can address" in str(e.value)
+    pinned = torch.zeros(1 << 16, dtype=torch.uint8).pin_memory()
+    kvt_amd.Cache(0, [[pinned]], [1 << 16]).close()                     # pinned host memory is legal
+
+
 def test_empty_plan_is_a_no_op():
     lists = kvt_amd.BlockLists()
     lists.append(0, np.zeros((0, 3), dtype=np.uint64))
