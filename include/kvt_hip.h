@@ -12,6 +12,13 @@
  *     base address, exactly like IpcBlock offsets in the reference.
  *   - every GPU entry point fails with KVT_ERR_NO_DEVICE when no gfx950 device
  *     is usable; there is no CPU fallback inside this library.
+ *   - buffers handed to a launch whose extent the host knows (layer tensors at
+ *     registration, the packed buffer of kvt_pack / kvt_unpack, both sides of
+ *     the copy_handle_data calls, stager transfers) are checked against what the
+ *     runtime knows about the pointer: memory the device cannot address gives
+ *     KVT_ERR_INVALID, an extent beyond the allocation holding the pointer
+ *     KVT_ERR_OUT_OF_RANGE, instead of a GPU memory fault. Not checked inside a
+ *     stream capture, nor where offsets live on the device (kvt_launch_copy_*).
  *   - threads: parsers, caches and plans are immutable once created and may be
  *     used from any number of threads at once (a plan may be launched on several
  *     streams); list containers (kvt_block_lists, kvt_run_lists), sessions and

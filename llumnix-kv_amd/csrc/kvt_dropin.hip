@@ -62,16 +62,22 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     return fail(KVT_ERR_INVALID, "copy_handle_data: bad direction");
   if (int rc = check_device(device)) return rc;
   if (max_block_num <= 0) max_block_num = 8192;
-  uint64_t total = 0;
+  uint64_t total = 0, layer_extent = 0;
   for (uint64_t i = 0; i < n; ++i) {
     if (blocks[i].length == 0) return fail(KVT_ERR_INVALID, "copy_handle_data: zero-length range");
     if (halve && (blocks[i].length & 1)) return fail(KVT_ERR_INVALID, "odd bf16 byte length");
     total += blocks[i].length;
+    layer_extent = std::max(layer_extent, blocks[i].dst_offset + blocks[i].length);
   }
   if (total != tensor_data_size)
     return fail(KVT_ERR_INVALID, "copy_handle_data: tensor_data_size != sum of range lengths");
   DeviceGuard g;
   if (int rc = g.enter(device)) return rc;
+  if (int rc = check_device_span(tensor_buf, halve ? total / 2 : total,
+                                 "copy_handle_data: the contiguous buffer"))
+    return rc;
+  if (int rc = check_device_span(layer_gpu_ptr, layer_extent, "copy_handle_data: the layer tensor"))
+    return rc;
   const hipStream_t s = static_cast<hipStream_t>(stream);
   uint64_t host_cursor = 0;
   for (uint64_t first = 0; first < n; first += static_cast<uint64_t>(max_block_num)) {
@@ -124,9 +130,10 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
     return fail(KVT_ERR_INVALID, "copy_handle_data_kernel_direct: bad direction");
   if (n > 0x7FFFFFFFull) return fail(KVT_ERR_INVALID, "too many ranges");
   if (int rc = check_device(device)) return rc;
-  uint64_t cursor = 0, slices = 0;
+  uint64_t cursor = 0, slices = 0, layer_extent = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const kvt_ipc_block& b = blocks[i];
+    layer_extent = std::max(layer_extent, b.dst_offset + b.length);
     const uint64_t host_off = explicit_host_offsets ? b.src_offset : cursor;
     if (b.length == 0 || host_off > tensor_data_size || b.length > tensor_data_size - host_off)
       return fail(KVT_ERR_OUT_OF_RANGE,
@@ -142,6 +149,12 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
                 "copy_handle_data_kernel_direct: tensor_data_size != sum of range lengths");
   DeviceGuard g;
   if (int rc = g.enter(device)) return rc;
+  if (int rc = check_device_span(tensor_buf, tensor_data_size,
+                                 "copy_handle_data_kernel_direct: the contiguous buffer"))
+    return rc;
+  if (int rc = check_device_span(layer_gpu_ptr, layer_extent,
+                                 "copy_handle_data_kernel_direct: the layer tensor"))
+    return rc;
   const hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t bytes = n * sizeof(int64_t);
   KVT_HIP(hipMemcpyAsync(src_dev, host_meta, bytes, hipMemcpyHostToDevice, s));

@@ -511,6 +511,15 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       KVT_HIP(hipStreamWaitEvent(s, p->uploaded, 0));
     }
   }
+  if (!capturing && p->n_chunks != 0 && n_layers != 0) {
+    uint64_t extent = 0;
+    for (uint32_t t = 0; t < p->n_tensors; ++t)
+      extent = std::max(extent, blobs.off[t] + p->tensor_bytes[t]);
+    extent += static_cast<uint64_t>(n_layers - 1) * layer_stride;
+    if (int rc = check_device_span(packed, extent, pack ? "kvt_pack: the packed buffer"
+                                                        : "kvt_unpack: the packed buffer"))
+      return rc;
+  }
   const Chunk* table = p->dev_chunks + (pack ? 0 : p->n_chunks);
   const uint32_t n = static_cast<uint32_t>(p->n_chunks);
   bool words = false;  // strided chunks moved as 4-byte words instead of 16-byte vectors

@@ -41,6 +41,47 @@ int check_device(int device) {
   return KVT_OK;
 }
 
+// A kernel that runs past a buffer takes a GPU memory fault, which can cost the whole
+// process (and more) instead of an error code. What the runtime knows about a pointer is
+// therefore checked on the host before a launch uses it: it must be memory the device can
+// address, and where the runtime can name the allocation around it, [ptr, ptr + bytes) must
+// lie inside. A framework's caching allocator hands out pieces of larger allocations, so this
+// catches an extent that overshoots the underlying allocation, not one that overshoots the
+// tensor. Spans that passed are remembered per thread (a serving loop reuses its buffers),
+// so the steady state costs a few comparisons and no runtime call.
+int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) {
+  if (bytes == 0) return KVT_OK;
+  struct Span {
+    uintptr_t lo = 0, hi = 0;
+  };
+  static thread_local Span seen[8];
+  static thread_local unsigned next = 0;
+  const uintptr_t p = reinterpret_cast<uintptr_t>(ptr);
+  for (const Span& s : seen)
+    if (p >= s.lo && p < s.hi && bytes <= s.hi - p) return KVT_OK;
+  hipPointerAttribute_t attr{};
+  if (hipPointerGetAttributes(&attr, ptr) != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(KVT_ERR_INVALID, what + " is not memory the device can address");
+  }
+  if (attr.type == hipMemoryTypeUnregistered)
+    return fail(KVT_ERR_INVALID, what + " is plain host memory the device cannot address");
+  hipDeviceptr_t base = nullptr;
+  size_t size = 0;
+  if (hipMemGetAddressRange(&base, &size, const_cast<void*>(ptr)) != hipSuccess) {
+    (void)hipGetLastError();  // pinned host memory, virtual-memory mappings: nothing to compare
+    return KVT_OK;
+  }
+  const uintptr_t lo = reinterpret_cast<uintptr_t>(base);
+  if (p < lo || p - lo > size || bytes > size - (p - lo))
+    return fail(KVT_ERR_OUT_OF_RANGE,
+                what + ": " + std::to_string(bytes) +
+                    " bytes reach beyond the allocation that holds the pointer (" +
+                    std::to_string(p < lo || p - lo > size ? 0 : size - (p - lo)) + " bytes left)");
+  seen[next++ % 8] = Span{lo, lo + size};
+  return KVT_OK;
+}
+
 TablePool& table_pool() {
   static TablePool* pool = new TablePool();  // intentionally leaked: outlives static destruction
   return *pool;
@@ -55,38 +96,6 @@ extern "C" {
 int kvt_device_count(void) { return std::max(0, usable_devices()); }
 
 // ------------------------------------------------------------------- cache
-
-// A kernel that runs past a layer tensor takes a GPU memory fault, which can cost the whole
-// process (and more) instead of an error code. What the runtime knows about the pointer is
-// checked here, once, at registration: it must be memory the device can address, and where
-// the runtime can name the allocation around it, [ptr, ptr + capacity) must lie inside. A
-// framework's caching allocator hands out pieces of larger allocations, so this catches a
-// capacity that overshoots the underlying allocation, not one that overshoots the tensor.
-static int check_layer_memory(const void* ptr, uint64_t capacity, uint64_t layer, uint64_t tensor) {
-  const std::string where = "kvt_cache_register: layer " + std::to_string(layer) + " tensor " +
-                            std::to_string(tensor);
-  hipPointerAttribute_t attr{};
-  if (hipPointerGetAttributes(&attr, ptr) != hipSuccess) {
-    (void)hipGetLastError();
-    return fail(KVT_ERR_INVALID, where + " is not memory the device can address");
-  }
-  if (attr.type == hipMemoryTypeUnregistered)
-    return fail(KVT_ERR_INVALID, where + " is plain host memory the device cannot address");
-  if (attr.type == hipMemoryTypeHost) return KVT_OK;  // pinned host memory: legal, if slow
-  hipDeviceptr_t base = nullptr;
-  size_t size = 0;
-  if (hipMemGetAddressRange(&base, &size, const_cast<void*>(ptr)) != hipSuccess) {
-    (void)hipGetLastError();  // e.g. virtual-memory mappings: nothing to compare against
-    return KVT_OK;
-  }
-  const uintptr_t lo = reinterpret_cast<uintptr_t>(base), p = reinterpret_cast<uintptr_t>(ptr);
-  if (p < lo || p - lo > size || capacity > size - (p - lo))
-    return fail(KVT_ERR_OUT_OF_RANGE,
-                where + ": capacity " + std::to_string(capacity) +
-                    " reaches beyond the device allocation that holds the pointer (" +
-                    std::to_string(size - (p - lo)) + " bytes left)");
-  return KVT_OK;
-}
 
 int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, uint32_t n_tensors,
                        const uint64_t* capacity, kvt_cache** out) {
@@ -111,7 +120,9 @@ int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, u
       c->host_ptrs[i] = const_cast<void*>(ptrs[i]);
       if (reinterpret_cast<uintptr_t>(ptrs[i]) & 15u) c->aligned16 = false;
       if (reinterpret_cast<uintptr_t>(ptrs[i]) & 3u) c->aligned4 = false;
-      if (int rc = check_layer_memory(ptrs[i], capacity[i % n_tensors], i / n_tensors, i % n_tensors))
+      if (int rc = check_device_span(ptrs[i], capacity[i % n_tensors],
+                                     "kvt_cache_register: layer " + std::to_string(i / n_tensors) +
+                                         " tensor " + std::to_string(i % n_tensors)))
         return rc;
     }
     KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c->dev_ptrs), n * sizeof(void*)));

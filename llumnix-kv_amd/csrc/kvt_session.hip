@@ -201,6 +201,7 @@ int kvt_stager_save_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, const
       return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_save: slot index or size out of range");
     DeviceGuard g;
     if (int rc = g.enter(s->device)) return rc;
+    if (int rc = check_device_span(dev, bytes, "kvt_stager_save: the device buffer")) return rc;
     KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(producer_stream)));
     KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));
     KVT_HIP(hipMemcpyAsync(static_cast<uint8_t*>(kvt_stager_slot(s, slot)) + slot_offset, dev, bytes,
@@ -223,6 +224,7 @@ int kvt_stager_load_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, void*
       return fail(KVT_ERR_OUT_OF_RANGE, "kvt_stager_load: slot index or size out of range");
     DeviceGuard g;
     if (int rc = g.enter(s->device)) return rc;
+    if (int rc = check_device_span(dev, bytes, "kvt_stager_load: the device buffer")) return rc;
     // the device buffer may still be read by earlier work of the consumer
     KVT_HIP(hipEventRecord(s->fence, static_cast<hipStream_t>(consumer_stream)));
     KVT_HIP(hipStreamWaitEvent(s->copy, s->fence, 0));

@@ -266,14 +266,28 @@ def test_cache_registration_checks_what_the_runtime_knows_about_the_memory():
     kvt_amd.Cache(0, [[big]], [64 << 20]).close()
     kvt_amd.Cache(0, [[big[4096:]]], [(64 << 20) - 4096]).close()      # interior pointers are fine
     with pytest.raises(kvt_amd.KvtError) as e:
-        kvt_amd.Cache(0, [[big]], [(64 << 20) + (1 << 30)])             # runs off the allocation
-    assert e.value.code == 1 and "beyond the device allocation" in str(e.value)
+        kvt_amd.Cache(0, [[big]], [1 << 44])      # runs off any allocation (torch may have carved
+        #                                             `big` out of a larger cached segment)
+    assert e.value.code == 1 and "beyond the allocation" in str(e.value)
     host = np.zeros(1 << 16, dtype=np.uint8)
     with pytest.raises(kvt_amd.KvtError) as e:
         kvt_amd.Cache(0, [[host]], [1 << 16])                           # pageable host memory
     assert "cannot address" in str(e.value) or "can address" in str(e.value)
     pinned = torch.zeros(1 << 16, dtype=torch.uint8).pin_memory()
     kvt_amd.Cache(0, [[pinned]], [1 << 16]).close()                     # pinned host memory is legal
+    # the packed buffer of a launch gets the same treatment
+    lists = kvt_amd.BlockLists()
+    lists.append(0, [(0, 0, 32 << 20)])
+    plan = kvt_amd.Plan(0, lists, [64 << 20], [64 << 20])
+    cache = kvt_amd.Cache(0, [[big], [big]], [64 << 20])
+    packed = torch.zeros(48 << 20, dtype=torch.uint8, device="cuda")    # room for one layer only
+    plan.pack(cache, 0, 1, packed, plan.layer_bytes)
+    with pytest.raises(kvt_amd.KvtError) as e:
+        plan.pack(cache, 0, 2, packed, 1 << 44)                         # layer 1 would land 16 TiB further
+    assert e.value.code == 1 and "packed buffer" in str(e.value)
+    with pytest.raises(kvt_amd.KvtError):
+        plan.unpack(cache, 0, 1, np.zeros(32 << 20, dtype=np.uint8), plan.layer_bytes)
+    torch.cuda.synchronize()
 
 
 def test_empty_plan_is_a_no_op():
