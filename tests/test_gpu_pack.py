@@ -755,3 +755,50 @@ def test_transposing_pack_random_geometry_sweep():
                     [[int(x) for x in dst_ids[2 * i:2 * i + 2]]]] for i in range(2)]
         w.xform = (heads, ntpb, row)
         _transposing(w, seed=seed + 40)
+
+
+def test_many_threads_build_launch_and_drop_plans_at_once():
+    """The reference runs one sender thread per destination (kvtransfer/src/client.cpp:94-104).
+    Here every thread parses its own batches, builds plans (the table pool and its upload
+    stream are shared), packs from ONE registered cache on a stream of its own and drops the
+    plan right after the launch. ctypes releases the GIL inside the library."""
+    import threading
+    n_threads, rounds = 6, 8
+    base = workloads.llama8b_batch(n_layers=4, src_pool=1024, dst_pool=4096, n_req=4,
+                                   min_tok=200, max_tok=1500)
+    src_layers = _make_caches(base, "src", 81)
+    sc = kvt_amd.Cache(0, src_layers, base.capacities("src"))
+    src_h = [_host(src_layers[l][0]) for l in range(base.n_layers)]
+    errors, checked = [], [0] * n_threads
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream()
+            for r in range(rounds):
+                w = workloads.llama8b_batch(n_layers=4, src_pool=1024, dst_pool=4096, n_req=4,
+                                            min_tok=200, max_tok=1500, seed=1000 + 17 * i + r)
+                plan, lists = pipeline.build_plan(w, 0)
+                stride = plan.layer_bytes
+                packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+                done = torch.cuda.Event()
+                done.record()                       # the zero fill ran on the default stream
+                stream.wait_event(done)
+                plan.pack(sc, 0, w.n_layers, packed, stride, stream.cuda_stream)
+                runs = lists.tensor(0)
+                plan.close()                        # dropped while its launch may still be queued
+                stream.synchronize()
+                got = packed.cpu().numpy()
+                for l in range(w.n_layers):
+                    blob = checkers.oracle_pack(src_h[l], runs)
+                    assert np.array_equal(got[l * stride:l * stride + len(blob)], blob), (i, r, l)
+                checked[i] += 1
+        except Exception as e:                      # an exception in a thread is otherwise lost
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(n_threads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert checked == [rounds] * n_threads
