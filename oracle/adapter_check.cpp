@@ -8,6 +8,7 @@
 // exception they throw must be identical. Compiled by oracle/Makefile (target
 // `adapter`) with the reference sources where they lie; output in oracle/_ref/.
 #include <bitset>
+#include <cstring>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -16,6 +17,7 @@
 #include "ref_convert.h"
 
 #include "kvt_blade_adapter.hpp"
+#include "kvt_loopback_channel.hpp"
 
 using namespace blade_llm;
 using namespace kvt_ref;
@@ -81,6 +83,69 @@ int kvtadp_compare(int parser_id, const kvt_worker_info* src, const kvt_worker_i
         return 3;
   }
   return 0;
+}
+
+// Drives kvt_adapter::LoopbackChannel through the IChannel protocol the way
+// KvSendStub::TaskContext does (kvtransfer/src/tx_stub.cpp:227-300): connect once, then per
+// batch register_data -> send_data(layer) for every layer -> flush. `lists[t]` / `n[t]` are
+// tensor t's ranges (written back after register_data, which may merge them in place:
+// n[t] receives the new count). kind: 0 PEQD, 1 PLTD, 2 PGTD. alloc / release supply the
+// transfer buffer. Returns 0, or 1 out_of_range, 2 overflow_error, 3 other exception;
+// metrics (capacity metrics_cap) receives flush()'s string or the exception text.
+int kvtadp_loopback_send(int device, void* const* src_layers, const uint64_t* src_capacity,
+                         void* const* dst_layers, const uint64_t* dst_capacity,
+                         uint32_t n_layers, uint32_t n_tensors, kvt_ipc_block* const* lists,
+                         uint64_t* n, int kind, uint32_t batches, void* compute_stream,
+                         void* (*alloc)(size_t), void (*release)(void*), char* metrics,
+                         size_t metrics_cap) {
+  auto say = [&](const std::string& text) {
+    if (metrics && metrics_cap) {
+      std::strncpy(metrics, text.c_str(), metrics_cap - 1);
+      metrics[metrics_cap - 1] = 0;
+    }
+  };
+  try {
+    const size_t cells = static_cast<size_t>(n_layers) * n_tensors;
+    std::unique_ptr<IChannel> ch(new kvt_adapter::LoopbackChannel(
+        device, std::vector<void*>(src_layers, src_layers + cells),
+        std::vector<uint64_t>(src_capacity, src_capacity + n_tensors),
+        std::vector<void*>(dst_layers, dst_layers + cells),
+        std::vector<uint64_t>(dst_capacity, dst_capacity + n_tensors), n_layers, compute_stream,
+        alloc, release));
+    ch->connect(WorkerInfo("decode-0", 0));
+    std::string out;
+    for (uint32_t b = 0; b < batches; ++b) {
+      std::vector<std::vector<IpcBlock>> data(n_tensors);
+      for (uint32_t t = 0; t < n_tensors; ++t)
+        for (uint64_t i = 0; i < n[t]; ++i)
+          data[t].emplace_back(lists[t][i].src_offset, lists[t][i].dst_offset, lists[t][i].length);
+      ch->register_data(data, static_cast<TPKind>(kind));
+      for (uint32_t l = 0; l < n_layers; ++l) ch->send_data(l);
+      ch->flush(out);
+      if (b + 1 == batches)
+        for (uint32_t t = 0; t < n_tensors; ++t) {
+          n[t] = data[t].size();
+          for (size_t i = 0; i < data[t].size(); ++i) {
+            lists[t][i].src_offset = data[t][i].src_offset;
+            lists[t][i].dst_offset = data[t][i].dst_offset;
+            lists[t][i].length = data[t][i].length;
+          }
+        }
+    }
+    const bool was_active = ch->is_active();
+    ch->close();
+    say(out + (was_active && !ch->is_active() ? "closed=1," : "closed=0,"));
+    return 0;
+  } catch (const std::out_of_range& e) {
+    say(e.what());
+    return 1;
+  } catch (const std::overflow_error& e) {
+    say(e.what());
+    return 2;
+  } catch (const std::exception& e) {
+    say(e.what());
+    return 3;
+  }
 }
 
 }  // extern "C"
