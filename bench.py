@@ -381,6 +381,71 @@ def leg_launchers(c, out):
     # pinned-host staging of packed layers, double buffered against the pack kernel
 
 
+def leg_fp8_plan(c, out):
+    """Config 6 only (TP2 -> TP1): the same batch with an fp8 receiver. The sender's plan
+    converts bf16 to fp8 while it gathers (per-token arithmetic still in the kernel); checked
+    against the oracle on the first layer."""
+    torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
+    if args.config != 6 or args.plan != "runs":
+        return
+    import dataclasses
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import checkers
+    w, side = c.wls[0], c.sides[0]
+    d_info = dict(w.dst_info)
+    d_info["token_sizes"] = [t // 2 for t in d_info["token_sizes"]]
+    d_info["block_sizes"] = [b // 2 for b in d_info["block_sizes"]]
+    w8 = dataclasses.replace(w, dst_info=d_info, notes=dict(w.notes, fp8=True),
+                             name=w.name + ", fp8 receiver")
+    t0 = time.perf_counter()
+    plan, runs = pipeline.build_plan_runs(w8, 0, args.chunk_bytes)
+    host_ms = (time.perf_counter() - t0) * 1e3
+    dst_cache = kvt.Cache(0, side.dst, w8.capacities("dst"))      # the fp8 pool: half the bytes
+    stride = plan.layer_bytes
+    P8 = plan.tensor_bytes(0) * w8.n_layers                        # fp8 bytes on the wire
+    packed = c.packed[0]
+    assert packed.numel() >= stride * w8.n_layers
+    a, b, d = c.new_event(), c.new_event(), c.new_event()
+    pk, un = [], []
+    for rep in range(4):
+        lib.kvt_event_record(a, c.sh)
+        plan.pack(side.src_cache, 0, w8.n_layers, packed, stride, c.sh)
+        lib.kvt_event_record(b, c.sh)
+        plan.unpack(dst_cache, 0, w8.n_layers, packed, stride, c.sh)
+        lib.kvt_event_record(d, c.sh)
+        lib.kvt_event_synchronize(d)
+        if rep:
+            pk.append(ev_ms(lib, a, b))
+            un.append(ev_ms(lib, b, d))
+    s_info, dd_info = w8.worker_infos()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w8.cache_shape, s_info, dd_info)
+    rc2, outs = checkers.oracle_parse(pid, s_info, dd_info, valid, tps, tpr, w8.task_bufs(), fp8=True)
+    assert rc == 0 and rc2 == 0
+    ranges = np.ascontiguousarray(outs[0], dtype=np.uint64)
+    layer0 = side.src[0][0].cpu().numpy()
+    blob = np.zeros(int(ranges[:, 2].sum()), dtype=np.uint8)
+    checkers.oracle().kvto_pack_bf16_to_fp8(layer0.ctypes.data, ranges.ctypes.data, len(ranges),
+                                            blob.ctypes.data)
+    parity = bool(np.array_equal(packed[:len(blob)].cpu().numpy(), blob))
+    exp = np.zeros(w8.capacities("dst")[0], dtype=np.uint8)
+    got = side.dst[0][0][:len(exp)].cpu().numpy()
+    exp[:] = got
+    checkers.oracle_unpack(exp, ranges, blob)      # idempotent on what the GPU already scattered
+    parity &= bool(np.array_equal(got, exp))
+    out["converting_plan"] = {
+        "workload": w8.name, "fp8_payload_bytes": P8, "table_entries_per_layer": plan.num_chunks,
+        "ranges_per_layer": int(len(ranges)), "host_parse_plan_ms": round(host_ms, 3),
+        "pack_ms": round(statistics.mean(pk), 4), "unpack_ms": round(statistics.mean(un), 4),
+        "pack_gbps": round(3.0 * P8 / (statistics.mean(pk) * 1e-3) / 1e9, 1),
+        "unpack_gbps": round(2.0 * P8 / (statistics.mean(un) * 1e-3) / 1e9, 1),
+        "parity_vs_oracle": parity,
+        "note": "pack reads 2 bytes and writes 1 per element (bf16 -> fp8 E4M3), unpack moves "
+                "the fp8 bytes; GB/s = bytes read + bytes written"}
+    plan.close()
+    runs.close()
+    dst_cache.close()
+
+
 def leg_frames(c, out):
     """Layer messages (TCP frame format) built around the GPU's output and consumed again:
     header + range metadata written by the host, blobs packed in HBM and placed by DMA;
@@ -803,8 +868,8 @@ def main():
     if not args.skip_cpu:
         leg_cpu(c, out)
     if not args.skip_extras:
-        for leg in (leg_latency, leg_session, leg_launchers, leg_frames, leg_store_objects,
-                    leg_staging):
+        for leg in (leg_latency, leg_session, leg_launchers, leg_fp8_plan, leg_frames,
+                    leg_store_objects, leg_staging):
             leg(c, out)
 
     print(json.dumps(out), flush=True)

@@ -205,6 +205,19 @@ void kvt_plan_destroy(kvt_plan* p);
  * less is refused with KVT_ERR_INVALID. */
 int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
                          const uint64_t* dst_capacity, uint32_t chunk_bytes, kvt_plan** out);
+/* The same for a sender whose cache holds bf16 while the transfer buffer and the receiver
+ * hold fp8 (BLLM_KVTRANS_BF162FP8_CONV: the P > D parsers then emit fp8 lengths, and
+ * copy_d2h_bf16_to_fp8 converts while it gathers, kvtransfer/src/copy_kernels.cpp:733-959,
+ * parse_block_common.cpp:81-129). The lists are what kvt_parse_block_runs produces with
+ * kvt_parse_opts.bf16_to_fp8 set: every length counts fp8 bytes, i.e. elements; source offsets
+ * and strides count bytes of the bf16 cache (they must be even), where 2 * length bytes are
+ * read. kvt_pack converts (round to nearest even, saturating, like the launcher
+ * kvt_launch_copy_d2h_bf16_to_fp8) with the per-token arithmetic still done by the kernel;
+ * kvt_unpack scatters the fp8 bytes unchanged. A plain list goes through
+ * kvt_run_lists_compress first. */
+int kvt_plan_create_runs_bf16_to_fp8(int device, const kvt_run_lists* lists,
+                                     const uint64_t* src_capacity, const uint64_t* dst_capacity,
+                                     uint32_t chunk_bytes, kvt_plan** out);
 /* Table entries that stayed strided (0 for a plan made from plain lists). */
 uint64_t kvt_plan_num_strided_chunks(const kvt_plan* p);
 /* Inspection without a GPU: a plan created with device = KVT_DEVICE_NONE keeps

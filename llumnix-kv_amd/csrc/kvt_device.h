@@ -53,6 +53,13 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
                                  const StrideTable& shapes, bool words, hipStream_t stream);
+// Converting gather (bf16 -> fp8 E4M3) of a chunk table, plain and strided chunks alike; lengths
+// and packed positions count fp8 bytes, cache offsets and strides bytes of the bf16 cache.
+hipError_t launch_convert_chunks(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                 uint8_t* const* layer_ptrs, uint32_t n_tensors,
+                                 uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
+                                 uint64_t layer_stride, const BlobOffsets& blobs,
+                                 const StrideTable& shapes, hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

@@ -268,6 +268,61 @@ __global__ __launch_bounds__(kThreads) void convert_ranges_kernel(
   }
 }
 
+// Converting gather of a resident chunk table (the pack direction of a plan whose source
+// cache holds bf16 and whose transfer buffer and destination hold fp8): chunk lengths,
+// packed positions and record lengths count fp8 bytes, i.e. elements; cache offsets and
+// strides count bytes of the bf16 cache, so element e of a contiguous piece is read at byte
+// 2e. One workgroup converts 4096 elements (8 KiB in, 4 KiB out), 16 per lane. Strided
+// chunks (shape != 0) are 16-byte aligned on both sides by construction.
+__global__ __launch_bounds__(kThreads) void convert_chunks_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs, StrideTable shapes) {
+  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
+  if (b >= n_slices) return;
+  const Chunk c = chunks[b >> sub_shift];
+  const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
+  if (off >= c.len) return;
+  const uint32_t len = min(kSlice, c.len - off);
+  const uint32_t layer = blockIdx.y;
+  const uint8_t* cache =
+      layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
+  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
+  const u32x4* sv;
+  if (c.shape == 0) {
+    const uint8_t* s8 = cache + 2ull * off;
+    if (((reinterpret_cast<uintptr_t>(s8) | reinterpret_cast<uintptr_t>(pk)) & 15u) != 0) {
+      const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s8);
+      for (uint32_t j = threadIdx.x; j < len; j += kThreads)
+        pk[j] = static_cast<uint8_t>(bf16_to_e4m3(s16[j]));
+      return;
+    }
+    const uint32_t done = (len >> 4) << 4;
+    if (threadIdx.x < len - done)
+      pk[done + threadIdx.x] = static_cast<uint8_t>(
+          bf16_to_e4m3(reinterpret_cast<const uint16_t*>(s8)[done + threadIdx.x]));
+    if (threadIdx.x >= (len >> 4)) return;
+    sv = reinterpret_cast<const u32x4*>(s8) + 2 * threadIdx.x;
+  } else {
+    if (threadIdx.x >= (len >> 4)) return;
+    const StrideShape& s = shapes.shape[c.shape - 1u];
+    const uint32_t v = (off >> 4) + threadIdx.x;  // output vector index inside the chunk
+    const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
+    const uint32_t col = v - rec * s.vlen;
+    const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
+    const uint32_t i = rec - o * s.n_inner;
+    sv = reinterpret_cast<const u32x4*>(cache + o * s.outer[0] + i * s.inner[0] + (col << 5));
+  }
+  const u32x4 lo = __builtin_nontemporal_load(sv);
+  const u32x4 hi = __builtin_nontemporal_load(sv + 1);
+  u32x4 r;
+  r.x = cvt4(lo.x, lo.y);
+  r.y = cvt4(lo.z, lo.w);
+  r.z = cvt4(hi.x, hi.y);
+  r.w = cvt4(hi.z, hi.w);
+  __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(pk) + threadIdx.x);
+}
+
 // Plain linear copy with the gather kernel's slice shape (calibration / ceiling).
 __global__ __launch_bounds__(kThreads) void copy_linear_kernel(uint8_t* __restrict__ dst,
                                                                const uint8_t* __restrict__ src,
@@ -318,6 +373,19 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
   else if (!words) KVT_LAUNCH_STRIDED(false, false);
   else KVT_LAUNCH_STRIDED(false, true);
 #undef KVT_LAUNCH_STRIDED
+  return hipGetLastError();
+}
+
+hipError_t launch_convert_chunks(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                 uint8_t* const* layer_ptrs, uint32_t n_tensors,
+                                 uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
+                                 uint64_t layer_stride, const BlobOffsets& blobs,
+                                 const StrideTable& shapes, hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  const uint32_t n_slices = n_chunks << sub_shift;
+  hipLaunchKernelGGL(convert_chunks_kernel, dim3(round8(n_slices), n_layers), dim3(kThreads), 0,
+                     stream, chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer,
+                     packed, layer_stride, blobs, shapes);
   return hipGetLastError();
 }
 

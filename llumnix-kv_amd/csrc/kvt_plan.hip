@@ -256,9 +256,12 @@ int kvt_plan_create_objects(int device, const kvt_block_lists* lists, const uint
   });
 }
 
-int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
-                         const uint64_t* dst_capacity, uint32_t chunk_bytes, kvt_plan** out) {
-  return guarded([&]() -> int {
+// Plan from strided runs. convert: the pack direction converts bf16 to fp8, every length
+// counts fp8 bytes (elements) and the source side reads twice as many bytes.
+static int create_runs_plan(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
+                            const uint64_t* dst_capacity, uint32_t chunk_bytes, bool convert,
+                            kvt_plan** out) {
+  {
     if (!lists || !src_capacity || !dst_capacity || !out)
       return fail(KVT_ERR_INVALID, "kvt_plan_create_runs: null argument");
     if (lists->tensors.empty() || lists->tensors.size() > KVT_MAX_TENSORS)
@@ -275,6 +278,8 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
     p->n_tensors = static_cast<uint32_t>(lists->tensors.size());
     p->src_cap.assign(src_capacity, src_capacity + p->n_tensors);
     p->dst_cap.assign(dst_capacity, dst_capacity + p->n_tensors);
+    p->convert = convert;
+    const uint64_t src_scale = convert ? 2 : 1;  // source bytes per packed byte
 
     // A span is contiguous on the packed side: either one plain range, or the
     // records of one outermost iteration of a run that stays strided.
@@ -306,14 +311,19 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
                 __builtin_add_overflow(d_max, dd, &d_max) ||
                 __builtin_mul_overflow(count, static_cast<uint64_t>(r.n[k]), &count);
         }
-        uint64_t total = 0;
+        uint64_t total = 0, src_len = 0;
         bad = bad || __builtin_mul_overflow(count, r.length, &total) ||
-              s_max > p->src_cap[t] || r.length > p->src_cap[t] - s_max ||
+              __builtin_mul_overflow(r.length, src_scale, &src_len) ||
+              s_max > p->src_cap[t] || src_len > p->src_cap[t] - s_max ||
               d_max > p->dst_cap[t] || r.length > p->dst_cap[t] - d_max;
         if (bad)
           return fail(KVT_ERR_OUT_OF_RANGE, "kvt_plan_create_runs: run " + std::to_string(ri) +
                                                 " of tensor " + std::to_string(t) +
                                                 " exceeds the stated capacity");
+        if (convert && ((r.src_offset | r.src_stride[0] | r.src_stride[1] | r.src_stride[2]) & 1u))
+          return fail(KVT_ERR_INVALID, "kvt_plan_create_runs_bf16_to_fp8: run " + std::to_string(ri) +
+                                           " of tensor " + std::to_string(t) +
+                                           " does not start on a bf16 element");
         // effective levels (n > 1), outermost first
         int lv[3], n_lv = 0;
         for (int k = 0; k < 3; ++k)
@@ -401,7 +411,7 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
     for (const Span& sp : spans) {
       if (sp.group == 0) {
         for (uint64_t o = 0; o < sp.bytes; o += chunk_bytes)
-          pieces.push_back(Piece{sp.src + o, sp.dst + o, sp.packed + o,
+          pieces.push_back(Piece{sp.src + src_scale * o, sp.dst + o, sp.packed + o,
                                  static_cast<uint32_t>(std::min<uint64_t>(chunk_bytes, sp.bytes - o)),
                                  sp.tensor, 0, 0});
       } else {
@@ -419,6 +429,21 @@ int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t*
     if (int rc = finish_plan(p.get(), pieces)) return rc;
     *out = p.release();
     return KVT_OK;
+  }
+}
+
+int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
+                         const uint64_t* dst_capacity, uint32_t chunk_bytes, kvt_plan** out) {
+  return guarded([&]() -> int {
+    return create_runs_plan(device, lists, src_capacity, dst_capacity, chunk_bytes, false, out);
+  });
+}
+
+int kvt_plan_create_runs_bf16_to_fp8(int device, const kvt_run_lists* lists,
+                                     const uint64_t* src_capacity, const uint64_t* dst_capacity,
+                                     uint32_t chunk_bytes, kvt_plan** out) {
+  return guarded([&]() -> int {
+    return create_runs_plan(device, lists, src_capacity, dst_capacity, chunk_bytes, true, out);
   });
 }
 
@@ -532,7 +557,15 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
                   "blob offsets (16-byte aligned ones take the fast path)");
     words = (mis & 15u) != 0;
   }
+  if (p->convert && pack && p->strided && words)
+    return fail(KVT_ERR_INVALID,
+                "a converting strided plan needs 16-byte aligned layer tensors, packed buffer, "
+                "stride and blob offsets");
   const hipError_t e =
+      p->convert && pack ? launch_convert_chunks(table, n, p->sub_shift, cache->dev_ptrs,
+                                                 p->n_tensors, first_layer, n_layers,
+                                                 static_cast<uint8_t*>(packed), layer_stride,
+                                                 blobs, p->shapes, s) :
       p->strided ? launch_strided_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                          p->n_tensors, first_layer, n_layers,
                                          static_cast<uint8_t*>(packed), layer_stride, blobs,

@@ -219,6 +219,7 @@ struct kvt_plan {
   bool strided = false;            // some chunks carry a record shape (kvt_plan_create_runs)
   kvt::StrideTable shapes{};
   uint64_t n_strided = 0;
+  bool convert = false;            // pack converts bf16 -> fp8: lengths count fp8 bytes (elements)
   std::vector<kvt::Chunk> host_table;   // device == KVT_DEVICE_NONE only: the tables, kept on the host
   uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
   kvt::Chunk* dev_chunks = nullptr;     // [0, n_chunks): pack order; [n_chunks, 2 n_chunks): unpack order

@@ -72,6 +72,7 @@ SIGNATURES = {
     "kvt_run_lists_expand": (_int, [_vp, _vp]),
     "kvt_run_lists_compress": (_int, [_vp, _vp]),
     "kvt_plan_create_runs": (_int, [_int, _vp, _P(_u64), _P(_u64), _u32, _P(_vp)]),
+    "kvt_plan_create_runs_bf16_to_fp8": (_int, [_int, _vp, _P(_u64), _P(_u64), _u32, _P(_vp)]),
     "kvt_plan_num_strided_chunks": (_u64, [_vp]),
     "kvt_plan_create_objects": (_int, [_int, _vp, _P(_u64), _P(_u64), _u64, _u64, _u32, _P(_vp)]),
     "kvt_plan_host_tables": (_int, [_vp, _P(_vp), _P(_u64), _P(_u32), _P(_vp)]),
@@ -410,8 +411,9 @@ class Cache:
 
 class Plan:
     def __init__(self, device, lists, src_capacity, dst_capacity, xform=None, chunk_bytes=0,
-                 objects=None):
-        """objects = (object_bytes, object_stride): per-block objects spanning all layers."""
+                 objects=None, bf16_to_fp8=False):
+        """objects = (object_bytes, object_stride): per-block objects spanning all layers.
+        bf16_to_fp8 (RunLists parsed in that mode only): pack converts while it gathers."""
         n = lists.num_tensors()
         sc = (_u64 * max(1, n))(*src_capacity)
         dc = (_u64 * max(1, n))(*dst_capacity)
@@ -426,9 +428,12 @@ class Plan:
         if isinstance(lists, RunLists):
             if xform is not None:
                 raise ValueError("no layout transform for a plan made from runs")
-            check(lib().kvt_plan_create_runs(device, lists.h, sc, dc, chunk_bytes,
-                                             C.byref(self.h)))
+            create = (lib().kvt_plan_create_runs_bf16_to_fp8 if bf16_to_fp8
+                      else lib().kvt_plan_create_runs)
+            check(create(device, lists.h, sc, dc, chunk_bytes, C.byref(self.h)))
             return
+        if bf16_to_fp8:
+            raise ValueError("a converting plan is made from RunLists (RunLists.compress for plain lists)")
         check(lib().kvt_plan_create(device, lists.h, sc, dc, xf, chunk_bytes, C.byref(self.h)))
 
     @property

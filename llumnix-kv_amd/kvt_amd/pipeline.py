@@ -43,9 +43,11 @@ def parse_batch_runs(cache_shape, src, dst, task_bufs, fp8=False, pad=True):
 
 
 def build_plan_runs(workload, device=0, chunk_bytes=0):
-    """Workload -> (Plan whose per-token arithmetic runs on the device, RunLists)."""
+    """Workload -> (Plan whose per-token arithmetic runs on the device, RunLists). A workload
+    whose receiver holds fp8 (notes["fp8"]) is parsed in that mode and packs converting."""
     src, dst = workload.worker_infos()
-    runs, _ = parse_batch_runs(workload.cache_shape, src, dst, workload.task_bufs())
+    fp8 = bool(workload.notes.get("fp8"))
+    runs, _ = parse_batch_runs(workload.cache_shape, src, dst, workload.task_bufs(), fp8=fp8)
     plan = binding.Plan(device, runs, workload.capacities("src"), workload.capacities("dst"),
-                        chunk_bytes=chunk_bytes)
+                        chunk_bytes=chunk_bytes, bf16_to_fp8=fp8)
     return plan, runs

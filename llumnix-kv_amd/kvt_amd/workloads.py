@@ -188,15 +188,17 @@ def qwen3next_uniform_pages(n_layers=12, pool=1024, n_req=128, tokens=4096, n_gd
 
 def tp_split(layout="flash", p_tp=2, d_tp=1, rank=0, n_layers=32, src_pool=16384,
              dst_pool=24576, n_req=64, min_tok=1024, max_tok=8192, total_heads=8, head_dim=128,
-             ntpb=16, seed=20257):
+             ntpb=16, seed=20257, fp8_dst=False):
     """A TP-remapping batch (prefill TP != decode TP): every token's K and V rows are split
     between / gathered from several ranks, i.e. one short range per token (and per head for
     the HND page layout). layout = "flash" ([2, nblk, bs, h, d]), "hnd" ([nblk, 2, h, bs, d])
-    or "ragged" ([nblk, bs, 2, h, d], the only one with a P<D parser); bf16. `rank` is the sending rank when p_tp > d_tp, the receiving rank otherwise."""
+    or "ragged" ([nblk, bs, 2, h, d], the only one with a P<D parser); bf16. `rank` is the sending rank when p_tp > d_tp, the receiving rank otherwise.
+    fp8_dst: the receiver's cache holds fp8 (half the token size); parse with fp8=True, the
+    sender converts while it gathers."""
     rng = np.random.default_rng(seed)
     row = head_dim * 2
     pT = 2 * (total_heads // p_tp) * row
-    dT = 2 * (total_heads // d_tp) * row
+    dT = 2 * (total_heads // d_tp) * row // (2 if fp8_dst else 1)
     lens = rng.integers(min_tok, max_tok + 1, size=n_req)
     src, dst = _tables(rng, n_req, lens, ntpb, src_pool, dst_pool)
     gn = max(p_tp, d_tp) // min(p_tp, d_tp)
@@ -213,7 +215,7 @@ def tp_split(layout="flash", p_tp=2, d_tp=1, rank=0, n_layers=32, src_pool=16384
         raise ValueError("the reference has a P<D parser only for the ragged layout")
     return Workload("%s TP%d->TP%d %dreq x %d-%d tok" % (layout, p_tp, d_tp, n_req, min_tok, max_tok),
                     shape, "%s_%s" % (fam, kind), n_layers, s_info, d_info, tasks, seed=seed,
-                    notes=dict(tokens=int(lens.sum())))
+                    notes=dict(tokens=int(lens.sum()), fp8=bool(fp8_dst)))
 
 
 def parser_id(w):

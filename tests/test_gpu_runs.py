@@ -175,3 +175,90 @@ def test_random_synthetic_runs_on_the_gpu(seed):
     exp = np.full(cap, 0xA5, dtype=np.uint8)
     checkers.oracle_unpack(exp, expect, blob)
     assert np.array_equal(_host(dst), exp)
+
+
+# ------------------------------------------- bf16 -> fp8 while gathering (resident plan)
+
+def _oracle_pack_fp8(layer_h, ranges):
+    """ranges: (src byte offset in the bf16 cache, dst, length in fp8 bytes = elements)"""
+    r = np.ascontiguousarray(ranges, dtype=np.uint64)
+    out = np.zeros(int(r[:, 2].sum()), dtype=np.uint8)
+    checkers.oracle().kvto_pack_bf16_to_fp8(layer_h.ctypes.data, r.ctypes.data, len(r),
+                                            out.ctypes.data)
+    return out
+
+
+# (ragged with p_tp = 2 d_tp is left out: an fp8 receiver then has the sender's token size, which
+# the reference's dispatch takes for a replicated cache, tx_stub.cpp:451-590)
+@pytest.mark.parametrize("layout,p_tp,d_tp,rank", [("flash", 2, 1, 1), ("flash", 4, 2, 3),
+                                                   ("ragged", 8, 2, 5), ("ragged", 4, 1, 2)])
+@pytest.mark.parametrize("chunk", [0, 4096, 65536])
+@pytest.mark.parametrize("content", ["bf16", "raw"])
+def test_converting_run_plan_bf16_sender_fp8_receiver(layout, p_tp, d_tp, rank, chunk, content):
+    """The reference's BLLM_KVTRANS_BF162FP8_CONV mode: the P > D parsers emit fp8 lengths and
+    the sender converts while it gathers. `raw` content makes every bf16 bit pattern
+    (NaNs, infinities, denormals) likely."""
+    w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=2, src_pool=300, dst_pool=400,
+                           n_req=4, min_tok=60, max_tok=900, fp8_dst=True)
+    plan, runs = pipeline.build_plan_runs(w, 0, chunk)
+    assert plan.num_strided_chunks > 0
+    src_i, dst_i = w.worker_infos()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, src_i, dst_i)
+    assert rc == 0 and kind != 0
+    rc, outs = checkers.oracle_parse(pid, src_i, dst_i, valid, tps, tpr, w.task_bufs(), fp8=True)
+    assert rc == 0
+    ranges = outs[0]
+    assert np.array_equal(runs.expand().tensor(0), ranges)
+    src_layers = _make_caches(w, "src", 91, dtype=content)
+    dst_layers = _make_caches(w, "dst", 92, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    stride = plan.layer_bytes
+    assert plan.tensor_bytes(0) == int(ranges[:, 2].sum())        # fp8 bytes on the wire
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, w.n_layers, packed, stride)
+    plan.unpack(dc, 0, w.n_layers, packed, stride)
+    torch.cuda.synchronize()
+    packed_h = _host(packed)
+    for l in range(w.n_layers):
+        blob = _oracle_pack_fp8(_host(src_layers[l][0]), ranges)
+        assert np.array_equal(packed_h[l * stride:l * stride + len(blob)], blob), ("pack", l)
+        exp = np.full(w.capacities("dst")[0], 0xA5, dtype=np.uint8)
+        checkers.oracle_unpack(exp, ranges, blob)
+        assert np.array_equal(_host(dst_layers[l][0]), exp), ("unpack", l)
+
+
+def test_converting_plan_of_plain_unaligned_ranges_takes_the_element_path():
+    rng = np.random.default_rng(5)
+    cap_s, cap_d = 1 << 20, 1 << 19
+    n = 24
+    lens = rng.integers(1, 9000, size=n)                       # elements, any remainder mod 16
+    s_off = np.sort(rng.choice(cap_s // 32768, size=n, replace=False)) * 32768 + 2 * rng.integers(0, 8, size=n)
+    d_off = np.sort(rng.choice(cap_d // 16384, size=n, replace=False)) * 16384 + rng.integers(0, 16, size=n)
+    ranges = np.stack([s_off, d_off, lens], axis=1).astype(np.uint64)
+    lists = kvt_amd.BlockLists()
+    lists.append(0, ranges)
+    runs = kvt_amd.RunLists.compress(lists)
+    plan = kvt_amd.Plan(0, runs, [cap_s], [cap_d], bf16_to_fp8=True)
+    src = _dev_bytes(cap_s, 7, "raw")
+    dst = torch.full((cap_d,), 0xA5, dtype=torch.uint8, device="cuda")
+    packed = torch.zeros(max(plan.layer_bytes, 16), dtype=torch.uint8, device="cuda")
+    plan.pack(kvt_amd.Cache(0, [[src]], [cap_s]), 0, 1, packed, plan.layer_bytes)
+    plan.unpack(kvt_amd.Cache(0, [[dst]], [cap_d]), 0, 1, packed, plan.layer_bytes)
+    torch.cuda.synchronize()
+    blob = _oracle_pack_fp8(_host(src), ranges)
+    assert np.array_equal(_host(packed)[:len(blob)], blob)
+    exp = np.full(cap_d, 0xA5, dtype=np.uint8)
+    checkers.oracle_unpack(exp, ranges, blob)
+    assert np.array_equal(_host(dst), exp)
+    # an odd source offset is not a bf16 element boundary
+    bad = kvt_amd.BlockLists()
+    bad.append(0, [(3, 0, 64)])
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.Plan(0, kvt_amd.RunLists.compress(bad), [cap_s], [cap_d], bf16_to_fp8=True)
+    # the source side is checked at twice the length
+    edge = kvt_amd.BlockLists()
+    edge.append(0, [(cap_s - 64, 0, 64)])
+    kvt_amd.Plan(0, kvt_amd.RunLists.compress(edge), [cap_s], [cap_d]).close()
+    with pytest.raises(kvt_amd.KvtError):
+        kvt_amd.Plan(0, kvt_amd.RunLists.compress(edge), [cap_s], [cap_d], bf16_to_fp8=True)
