@@ -13,8 +13,24 @@ import kvt_amd
 from kvt_amd import pipeline, workloads
 
 
-def emulate(table, chunk_bytes, shapes, caches, tensor_offset, packed, pack):
+_FP8_LUT = None
+
+
+def _fp8_lut():
+    global _FP8_LUT
+    if _FP8_LUT is None:
+        o = checkers.oracle()
+        _FP8_LUT = np.array([o.kvto_bf16_to_fp8(b) for b in range(65536)], dtype=np.uint8)
+    return _FP8_LUT
+
+
+def emulate(table, chunk_bytes, shapes, caches, tensor_offset, packed, pack, convert=False):
+    """convert (pack only): lengths count fp8 bytes = elements, the cache side holds bf16:
+    a contiguous piece reads element e at byte 2e, a strided record 32 source bytes per
+    16-byte output vector (convert_chunks_kernel)."""
     side = 0 if pack else 1
+    scale = 2 if convert else 1
+    assert pack or not convert
     touched = [np.zeros(len(c), dtype=bool) for c in caches]
     for c in table:
         n = int(c["len"])
@@ -23,7 +39,8 @@ def emulate(table, chunk_bytes, shapes, caches, tensor_offset, packed, pack):
         pk0 = tensor_offset[t] + int(c["packed"])
         assert pk0 + n <= len(packed)
         if c["shape"] == 0:
-            idx = int(c["cache"]) + np.arange(n, dtype=np.int64)
+            idx = int(c["cache"]) + np.arange(scale * n, dtype=np.int64)
+            assert not convert or int(c["cache"]) % 2 == 0
         else:
             s = shapes[int(c["shape"]) - 1]
             vlen, inv, n_inner = int(s["vlen"]), int(s["inv_vlen"]), int(s["n_inner"])
@@ -38,11 +55,14 @@ def emulate(table, chunk_bytes, shapes, caches, tensor_offset, packed, pack):
             col = v - rec * np.uint64(vlen)
             o, i = rec // np.uint64(n_inner), rec % np.uint64(n_inner)
             at = (o * np.uint64(int(s["outer"][side])) + i * np.uint64(int(s["inner"][side]))
-                  + col * np.uint64(16)).astype(np.int64) + int(c["cache"])
+                  + col * np.uint64(16 * scale)).astype(np.int64) + int(c["cache"])
             assert (at % 16 == 0).all()
-            idx = (at[:, None] + np.arange(16, dtype=np.int64)[None, :]).reshape(-1)
+            idx = (at[:, None] + np.arange(16 * scale, dtype=np.int64)[None, :]).reshape(-1)
         assert idx.min() >= 0 and idx.max() < len(caches[t]), "access outside the cache tensor"
-        if pack:
+        if convert:
+            pairs = caches[t][idx].reshape(-1, 2).astype(np.uint32)
+            packed[pk0:pk0 + n] = _fp8_lut()[pairs[:, 0] | (pairs[:, 1] << 8)]
+        elif pack:
             packed[pk0:pk0 + n] = caches[t][idx]
         else:
             assert not touched[t][idx].any(), "two table entries write the same bytes"
@@ -208,3 +228,58 @@ def test_run_lists_append_refuses_empty_runs():
     bad["length"], bad["n"] = 16, [[1, 0, 1]]
     with pytest.raises(kvt_amd.KvtError):
         kvt_amd.RunLists().append(0, bad)
+
+
+@pytest.mark.parametrize("chunk", [0, 4096, 65536])
+@pytest.mark.parametrize("layout,p_tp,d_tp,rank", [("flash", 2, 1, 1), ("flash", 4, 1, 2),
+                                                   ("ragged", 4, 1, 3)])
+def test_converting_plan_tables_bf16_sender_fp8_receiver(layout, p_tp, d_tp, rank, chunk):
+    w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=1, src_pool=40, dst_pool=60,
+                           n_req=4, min_tok=5, max_tok=150, total_heads=4, head_dim=32,
+                           fp8_dst=True)
+    src, dst = w.worker_infos()
+    runs, _ = pipeline.parse_batch_runs(w.cache_shape, src, dst, w.task_bufs(), fp8=True)
+    s_cap, d_cap = w.capacities("src"), w.capacities("dst")
+    plan = kvt_amd.Plan(-1, runs, s_cap, d_cap, chunk_bytes=chunk, bf16_to_fp8=True)
+    assert plan.num_strided_chunks > 0
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, src, dst)
+    rc, outs = checkers.oracle_parse(pid, src, dst, valid, tps, tpr, w.task_bufs(), fp8=True)
+    assert rc == 0 and np.array_equal(runs.expand().tensor(0), outs[0])
+    ranges = np.ascontiguousarray(outs[0], dtype=np.uint64)
+    pack_t, unpack_t, cb, shapes = plan.host_tables()
+    rng = np.random.default_rng(11)
+    cache = rng.integers(0, 256, s_cap[0], dtype=np.uint8)
+    packed = np.zeros(plan.layer_bytes, dtype=np.uint8)
+    emulate(pack_t, cb, shapes, [cache], [plan.tensor_offset(0)], packed, True, convert=True)
+    blob = np.zeros(int(ranges[:, 2].sum()), dtype=np.uint8)
+    checkers.oracle().kvto_pack_bf16_to_fp8(cache.ctypes.data, ranges.ctypes.data, len(ranges),
+                                            blob.ctypes.data)
+    assert plan.tensor_bytes(0) == len(blob) and np.array_equal(packed[:len(blob)], blob)
+    dst_c = [np.full(d_cap[0], 0xA5, dtype=np.uint8)]
+    emulate(unpack_t, cb, shapes, dst_c, [plan.tensor_offset(0)], packed, False)
+    exp = np.full(d_cap[0], 0xA5, dtype=np.uint8)
+    checkers.oracle_unpack(exp, ranges, blob)
+    assert np.array_equal(dst_c[0], exp)
+
+
+def test_converting_plan_checks_the_source_at_twice_the_length_and_on_element_bounds():
+    cap_s, cap_d = 1 << 20, 1 << 19
+    edge = kvt_amd.BlockLists()
+    edge.append(0, [(cap_s - 64, 0, 64)])
+    kvt_amd.Plan(-1, kvt_amd.RunLists.compress(edge), [cap_s], [cap_d]).close()
+    with pytest.raises(kvt_amd.KvtError) as e:
+        kvt_amd.Plan(-1, kvt_amd.RunLists.compress(edge), [cap_s], [cap_d], bf16_to_fp8=True)
+    assert e.value.code == 1
+    odd = kvt_amd.BlockLists()
+    odd.append(0, [(3, 0, 64)])
+    with pytest.raises(kvt_amd.KvtError) as e:
+        kvt_amd.Plan(-1, kvt_amd.RunLists.compress(odd), [cap_s], [cap_d], bf16_to_fp8=True)
+    assert e.value.code == 3
+    # plain pieces: the k-th chunk of a long range starts 2 * k * chunk_bytes into the source
+    long = kvt_amd.BlockLists()
+    long.append(0, [(4096, 128, 100000)])
+    plan = kvt_amd.Plan(-1, kvt_amd.RunLists.compress(long), [cap_s], [cap_d], chunk_bytes=32768,
+                        bf16_to_fp8=True)
+    pack_t, unpack_t, cb, _ = plan.host_tables()
+    assert pack_t["cache"].tolist() == [4096 + 2 * 32768 * k for k in range(4)]
+    assert unpack_t["cache"].tolist() == [128 + 32768 * k for k in range(4)]
