@@ -67,6 +67,12 @@ def build_workload(cfg, scale):
         return [W.qwen3next_uniform_pages(n_layers=max(2, int(12 * scale)),
                                           pool=max(16, int(1024 * scale)),
                                           n_req=max(2, int(128 * scale)))]
+    if cfg == 10:
+        # config 9's model between a TP2 prefill and a TP1 decode instance: attention rows
+        # split per token, GDN conv rows per channel group, SSM states, tail fill
+        return [W.qwen3next_tp_split(2, 1, 0, n_layers=max(2, int(12 * scale)),
+                                     pool=max(16, int(1024 * scale)),
+                                     n_req=max(2, int(128 * scale)))]
     if cfg in (6, 7, 8):
         # TP-remapping batches (not among the baseline configurations): config 2's batch with
         # the sender on TP2 and the receiver on TP1 (6), TP1 -> TP2 on the ragged layout (7),
@@ -652,7 +658,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, help="1-5: BASELINE.json configs[] index + 1; 6-8: TP-remapping batches; "
-                         "9: config 5 with the reference's uniform 2 MiB pages")
+                         "9: config 5 with the reference's uniform 2 MiB pages; 10: the same "
+                         "model TP2 -> TP1")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")
     ap.add_argument("--chunk-bytes", type=int, default=0)
     ap.add_argument("--plan", choices=["ranges", "runs"], default="ranges",

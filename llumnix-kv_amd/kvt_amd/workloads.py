@@ -186,6 +186,61 @@ def qwen3next_uniform_pages(n_layers=12, pool=1024, n_req=128, tokens=4096, n_gd
                     seed=seed)
 
 
+def qwen3next_tp_split(p_tp=2, d_tp=1, rank=0, n_layers=12, pool=1024, n_req=128, tokens=4096,
+                       n_gdn=3, kv_heads=2, head_dim=256, key_heads=16, value_heads=32,
+                       state_dim=128, conv_rows=3, kernel_block=16, seed=20259):
+    """The hybrid model of config 5 between a TP`p_tp` prefill and a TP`d_tp` decode instance
+    (p_tp > d_tp), in the reference's arrangement (one tensor per full-attention layer, uniform
+    pages shared with `n_gdn` GDN layers). Every rank holds kv_heads / tp attention heads
+    (bf16), conv state rows of 2 * key_dim + value_dim bf16 channels and an fp32 SSM state of
+    value_heads / tp x state_dim x state_dim, so a sending rank's pieces interleave into the
+    receiver's wider rows: per token and K / V for attention (inside kernel blocks of
+    `kernel_block` tokens), per conv row and channel group (q, k, v) plus one SSM range for a
+    GDN state (parse_block_qwen3_next.cpp:108-413, 532-711). `rank` is the sending rank."""
+    if p_tp <= d_tp or p_tp % d_tp or kv_heads % p_tp or key_heads % p_tp or value_heads % p_tp:
+        raise ValueError("need p_tp a multiple of d_tp and heads divisible by p_tp")
+    rng = np.random.default_rng(seed)
+    gn = p_tp // d_tp
+
+    def side(tp):
+        tok = 2 * (kv_heads // tp) * head_dim * 2
+        key_dim, value_dim = key_heads // tp * state_dim, value_heads // tp * state_dim
+        chans = [key_dim, key_dim, value_dim]
+        conv = conv_rows * sum(chans) * 2
+        ssm = (value_heads // tp) * state_dim * state_dim * 4
+        return tok, chans, conv + ssm
+
+    pT, p_ch, p_state = side(p_tp)
+    dT, d_ch, d_state = side(d_tp)
+    ntpb = -(-d_state // dT)                       # tokens per page: the page holds a D state
+    ntpb = -(-ntpb // kernel_block) * kernel_block
+    assert pT * ntpb >= p_state
+    n_attn = (tokens + ntpb - 1) // ntpb
+    per_req = n_gdn + n_attn
+    if per_req * n_req > pool:
+        raise ValueError("pool too small for disjoint tables: %d > %d" % (per_req * n_req, pool))
+    sperm, dperm = rng.permutation(pool), rng.permutation(pool)
+    tasks = []
+    for r in range(n_req):
+        s = [int(x) for x in sperm[r * per_req:(r + 1) * per_req]]
+        d = [int(x) for x in dperm[r * per_req:(r + 1) * per_req]]
+        tasks.append([0, tokens, True, [[s[g]] for g in range(n_gdn)] + [s[n_gdn:]],
+                      [[d[g]] for g in range(n_gdn)] + [d[n_gdn:]]])
+
+    def info(tp, rk, tok, chans):
+        return dict(block_sizes=[tok * ntpb], token_sizes=[tok], layer_num_blocks=pool, tp=tp,
+                    rank=rk, num_kv_heads=kv_heads, num_layers=n_layers, num_gdn_layers=n_gdn,
+                    attn_kernel_blk_ntpb=kernel_block,
+                    conv_state_shape=[pool, conv_rows, sum(chans)],
+                    ssm_state_shape=[pool, value_heads // tp, state_dim, state_dim],
+                    gdn_conv_channel_dims=chans, gdn_conv_elem_size=2, gdn_ssm_elem_size=4)
+
+    return Workload("qwen3-next hybrid TP%d->TP%d, uniform pages %dreq x %d tok" %
+                    (p_tp, d_tp, n_req, tokens), SHAPE_QWEN3_NEXT_FLASH, "HYBRID_PGTD", n_layers,
+                    info(p_tp, rank, pT, p_ch), info(d_tp, rank // gn, dT, d_ch), tasks, seed=seed,
+                    notes=dict(tokens=tokens * n_req, page_tokens=ntpb))
+
+
 def tp_split(layout="flash", p_tp=2, d_tp=1, rank=0, n_layers=32, src_pool=16384,
              dst_pool=24576, n_req=64, min_tok=1024, max_tok=8192, total_heads=8, head_dim=128,
              ntpb=16, seed=20257, fp8_dst=False):

@@ -69,6 +69,20 @@ def test_tp_split_batches_through_a_run_plan(layout, p_tp, d_tp, rank, strided, 
     _check(w, plan, o_lists, 51, strided)
 
 
+@pytest.mark.parametrize("p_tp,d_tp,rank", [(2, 1, 0), (2, 1, 1)])
+def test_hybrid_model_between_tp2_prefill_and_tp1_decode(p_tp, d_tp, rank):
+    """Attention pages split per token inside kernel blocks, GDN conv rows split per channel
+    group, one SSM range, and the zero fill of the receiver's last page, all in one batch;
+    destination tables are disjoint, so the scatter is checked as well."""
+    w = workloads.qwen3next_tp_split(p_tp, d_tp, rank, n_layers=2, pool=64, n_req=6, tokens=1500)
+    plan, runs = pipeline.build_plan_runs(w, 0)
+    o_lists = _oracle_ranges(w)
+    assert np.array_equal(runs.expand().tensor(0), o_lists[0])
+    lens = o_lists[0][:, 2]
+    assert lens.min() <= 512 and lens.max() >= 1 << 20          # token rows up to SSM states
+    _check(w, plan, o_lists, 71, True)
+
+
 def test_receiver_compresses_plain_ranges_then_unpacks_strided():
     w = workloads.tp_split("flash", 2, 1, 0, n_layers=2, src_pool=200, dst_pool=300, n_req=4,
                            min_tok=100, max_tok=700)
