@@ -121,7 +121,8 @@ int kvt_run_lists_totals(const kvt_run_lists* l, uint32_t tensor, uint64_t* n_ra
  * run form: expanding what this appends equals what kvt_parse_block appends. */
 int kvt_parse_block_runs(const kvt_parser* p, const kvt_task* task, kvt_run_lists* lists);
 /* Appends the expansion of every run to `out` (e.g. the range metadata of a
- * layer message for a peer that expects plain ranges). */
+ * layer message for a peer that expects plain ranges). More than 2^31 ranges in
+ * one tensor are refused (KVT_ERR_INVALID). */
 int kvt_run_lists_expand(const kvt_run_lists* l, kvt_block_lists* out);
 /* The inverse, for a receiver that got plain ranges: finds the arithmetic
  * progressions (innermost first, three levels) and appends runs whose expansion

@@ -315,7 +315,8 @@ static int create_runs_plan(int device, const kvt_run_lists* lists, const uint64
         bad = bad || __builtin_mul_overflow(count, r.length, &total) ||
               __builtin_mul_overflow(r.length, src_scale, &src_len) ||
               s_max > p->src_cap[t] || src_len > p->src_cap[t] - s_max ||
-              d_max > p->dst_cap[t] || r.length > p->dst_cap[t] - d_max;
+              d_max > p->dst_cap[t] || r.length > p->dst_cap[t] - d_max ||
+              total > p->dst_cap[t];  // disjoint destination ranges cannot add up to more
         if (bad)
           return fail(KVT_ERR_OUT_OF_RANGE, "kvt_plan_create_runs: run " + std::to_string(ri) +
                                                 " of tensor " + std::to_string(t) +

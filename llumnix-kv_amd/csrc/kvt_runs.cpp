@@ -145,6 +145,17 @@ int kvt_run_lists_totals(const kvt_run_lists* l, uint32_t tensor, uint64_t* n_ra
 int kvt_run_lists_expand(const kvt_run_lists* l, kvt_block_lists* out) {
   return guarded([&]() -> int {
     if (!l || !out) return fail(KVT_ERR_INVALID, "kvt_run_lists_expand: null argument");
+    // a run is 88 bytes however many ranges it stands for: refuse to be made to allocate
+    // without bound by a few of them
+    for (const std::vector<kvt_run>& runs : l->tensors) {
+      uint64_t ranges = 0;
+      for (const kvt_run& r : runs) {
+        uint64_t c = 0;
+        if (__builtin_mul_overflow(static_cast<uint64_t>(r.n[0]) * r.n[1], static_cast<uint64_t>(r.n[2]), &c) ||
+            __builtin_add_overflow(ranges, c, &ranges) || ranges > (1ull << 31))
+          return fail(KVT_ERR_INVALID, "kvt_run_lists_expand: more than 2^31 ranges in one tensor");
+      }
+    }
     if (out->tensors.size() < l->tensors.size()) out->tensors.resize(l->tensors.size());
     for (size_t t = 0; t < l->tensors.size(); ++t) {
       RunList& dst = out->tensors[t];

@@ -312,12 +312,58 @@ static void fuzz_range_plans(int iters) {
   std::printf("range plans: %ld accepted, %ld as store objects\n", accepted, objects);
 }
 
+// Runs whose counts and strides are garbage (a run is 88 bytes however many ranges it stands
+// for): every entry point must answer within the watchdog's limit and without exhausting memory.
+static void fuzz_hostile_runs(int iters) {
+  long accepted = 0;
+  for (int it = 0; it < iters; ++it) {
+    std::snprintf(g_case, sizeof(g_case), "hostile run it=%d", it);
+    alarm(30);
+    kvt_run r{};
+    r.length = rnd(3) ? 1 + rnd(1 << 16) : 1 + rnd(1ull << 40);
+    r.src_offset = rnd(1 << 20);
+    r.dst_offset = rnd(1 << 20);
+    for (int k = 0; k < 3; ++k) {
+      static const uint32_t counts[] = {1, 2, 1000, 1u << 20, 0x7FFFFFFFu, 0xFFFFFFFFu};
+      r.n[k] = counts[rnd(6)];
+      r.src_stride[k] = rnd(3) ? rnd(1 << 16) : 0;
+      r.dst_stride[k] = rnd(3) ? rnd(1 << 16) : 0;
+    }
+    kvt_run_lists* lists = nullptr;
+    CHECK(kvt_run_lists_create(&lists) == KVT_OK);
+    CHECK(kvt_run_lists_append(lists, 0, &r, 1) == KVT_OK);
+    const uint64_t s_cap = rnd(2) ? ~0ull >> rnd(40) : rnd(1ull << 34);
+    const uint64_t d_cap = rnd(1ull << 26);     // what an accepted plan may have to enumerate
+    kvt_plan* plan = nullptr;
+    const int rc = rnd(2) ? kvt_plan_create_runs(KVT_DEVICE_NONE, lists, &s_cap, &d_cap, 0, &plan)
+                          : kvt_plan_create_runs_bf16_to_fp8(KVT_DEVICE_NONE, lists, &s_cap, &d_cap,
+                                                             0, &plan);
+    CHECK((rc == KVT_OK) == (plan != nullptr));
+    if (plan) {
+      ++accepted;
+      CHECK(kvt_plan_tensor_bytes(plan, 0) <= d_cap);
+      kvt_plan_destroy(plan);
+    }
+    kvt_block_lists* plain = nullptr;
+    CHECK(kvt_block_lists_create(&plain) == KVT_OK);
+    uint64_t ranges = 0;
+    CHECK(kvt_run_lists_totals(lists, 0, &ranges, nullptr) == KVT_OK);
+    const int rc2 = ranges <= (1u << 22) ? kvt_run_lists_expand(lists, plain) : KVT_ERR_INVALID;
+    CHECK(rc2 == KVT_OK || rc2 == KVT_ERR_INVALID);
+    kvt_block_lists_destroy(plain);
+    kvt_run_lists_destroy(lists);
+  }
+  alarm(0);
+  std::printf("hostile runs: %ld of %d accepted\n", accepted, iters);
+}
+
 int main(int argc, char** argv) {
   std::signal(SIGALRM, on_alarm);
   const int scale = argc > 1 ? std::atoi(argv[1]) : 1;
   if (argc > 2) rng.seed(std::strtoull(argv[2], nullptr, 10));
   fuzz_run_plans(400 * scale);
   fuzz_range_plans(200 * scale);
+  fuzz_hostile_runs(300 * scale);
   std::printf("plan fuzz ok\n");
   return 0;
 }
