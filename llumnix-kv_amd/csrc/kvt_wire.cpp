@@ -27,9 +27,12 @@ uint64_t get64(const uint8_t* p) {
   return v;
 }
 
+// Sum of the range lengths; saturates, so that lengths chosen to wrap around to a plausible
+// total cannot pass for it.
 uint64_t blob_bytes_of(const RunList& runs) {
   uint64_t total = 0;
-  for (const kvt_ipc_block& r : runs) total += r.length;
+  for (const kvt_ipc_block& r : runs)
+    if (__builtin_add_overflow(total, r.length, &total)) return ~0ull;
   return total;
 }
 
@@ -46,7 +49,8 @@ int layout_of(int format, const kvt_block_lists& lists, kvt_wire_layout* out) {
       cur += 8 + lists.tensors[t].size() * sizeof(kvt_ipc_block) + 8;
       out->blob_offset[t] = cur;
       out->blob_bytes[t] = blob_bytes_of(lists.tensors[t]);
-      cur += out->blob_bytes[t];
+      if (__builtin_add_overflow(cur, out->blob_bytes[t], &cur))
+        return fail(KVT_ERR_OVERFLOW, "wire: frame size does not fit 64 bits");
     }
   } else if (format == KVT_WIRE_RDMA_STAGED) {
     if (nt != 1) return fail(KVT_ERR_INVALID, "wire: the staged RDMA frame carries one tensor per layer");
@@ -55,7 +59,8 @@ int layout_of(int format, const kvt_block_lists& lists, kvt_wire_layout* out) {
     cur += 8 + lists.tensors[0].size() * sizeof(kvt_ipc_block);
     out->blob_offset[0] = cur;
     out->blob_bytes[0] = blob_bytes_of(lists.tensors[0]);
-    cur += out->blob_bytes[0];
+    if (__builtin_add_overflow(cur, out->blob_bytes[0], &cur))
+      return fail(KVT_ERR_OVERFLOW, "wire: frame size does not fit 64 bits");
   } else {
     return fail(KVT_ERR_INVALID, "wire: unknown frame format");
   }
