@@ -730,15 +730,18 @@ def main():
     infos = [w.worker_infos() for w in wls]
     tasks = [w.task_bufs() for w in wls]
 
+    # per destination, once: parser selection and compilation (refresh_dst_info in the reference)
+    senders = [pipeline.Sender(w.cache_shape, infos[i][0], infos[i][1]) for i, w in enumerate(wls)]
+    caps = [(w.capacities("src"), w.capacities("dst")) for w in wls]
+
     def prepare(i):
         """host part of a step for workload i: ParseBlock + merge + plan upload"""
         w = wls[i]
         if args.plan == "runs":
-            runs, _ = pipeline.parse_batch_runs(w.cache_shape, infos[i][0], infos[i][1], tasks[i])
-            return kvt.Plan(0, runs, w.capacities("src"), w.capacities("dst"),
-                            chunk_bytes=args.chunk_bytes), runs
-        lists, _ = pipeline.parse_batch(w.cache_shape, infos[i][0], infos[i][1], tasks[i])
-        plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
+            runs = senders[i].parse_runs(tasks[i])
+            return kvt.Plan(0, runs, caps[i][0], caps[i][1], chunk_bytes=args.chunk_bytes), runs
+        lists = senders[i].parse(tasks[i])
+        plan = kvt.Plan(0, lists, caps[i][0], caps[i][1], xform=w.xform,
                         chunk_bytes=args.chunk_bytes)
         return plan, lists
 

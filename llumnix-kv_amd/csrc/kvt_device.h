@@ -60,6 +60,18 @@ hipError_t launch_convert_chunks(const Chunk* chunks, uint32_t n_chunks, uint32_
                                  uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                  uint64_t layer_stride, const BlobOffsets& blobs,
                                  const StrideTable& shapes, hipStream_t stream);
+// A table of at most kSmallTable entries travels in the kernel arguments (2 KiB): a short
+// request then needs no table upload, no upload event and no cross-stream wait before its
+// first launch.
+constexpr uint32_t kSmallTable = 64;
+struct SmallTable {
+  Chunk c[kSmallTable];
+};
+hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t n_chunks,
+                                    uint32_t sub_shift, uint8_t* const* layer_ptrs,
+                                    uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
+                                    uint8_t* packed, uint64_t layer_stride,
+                                    const BlobOffsets& blobs, hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

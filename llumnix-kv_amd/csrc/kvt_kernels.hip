@@ -82,6 +82,29 @@ __global__ __launch_bounds__(kThreads) void copy_chunks_kernel(
     copy_slice(cache, pk, len, threadIdx.x);
 }
 
+// The same for a table short enough to be a kernel argument (read through the scalar cache
+// like any other argument; the index is uniform across the workgroup).
+template <bool PACK>
+__global__ __launch_bounds__(kThreads) void copy_chunks_small_kernel(
+    const SmallTable table, uint32_t n_slices, uint32_t sub_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
+  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
+  if (b >= n_slices) return;
+  const Chunk& c = table.c[b >> sub_shift];
+  const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
+  if (off >= c.len) return;
+  const uint32_t len = min(kSlice, c.len - off);
+  const uint32_t layer = blockIdx.y;
+  uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] +
+                   c.cache + off;
+  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
+  if (PACK)
+    copy_slice(pk, cache, len, threadIdx.x);
+  else
+    copy_slice(cache, pk, len, threadIdx.x);
+}
+
 // Gather / scatter of a table whose chunks may be strided on the cache side:
 // the token -> offset arithmetic of the TP-remapping layouts (one short range
 // per token, per head, K and V) is evaluated here, per 16-byte vector, instead
@@ -351,6 +374,25 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                        layer_stride, blobs);
   else
     hipLaunchKernelGGL((copy_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
+                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
+                       layer_stride, blobs);
+  return hipGetLastError();
+}
+
+hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t n_chunks,
+                                    uint32_t sub_shift, uint8_t* const* layer_ptrs,
+                                    uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
+                                    uint8_t* packed, uint64_t layer_stride,
+                                    const BlobOffsets& blobs, hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  const uint32_t n_slices = n_chunks << sub_shift;
+  const dim3 grid(round8(n_slices), n_layers);
+  if (pack)
+    hipLaunchKernelGGL((copy_chunks_small_kernel<true>), grid, dim3(kThreads), 0, stream, table,
+                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
+                       layer_stride, blobs);
+  else
+    hipLaunchKernelGGL((copy_chunks_small_kernel<false>), grid, dim3(kThreads), 0, stream, table,
                        n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
                        layer_stride, blobs);
   return hipGetLastError();

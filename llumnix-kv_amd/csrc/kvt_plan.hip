@@ -79,6 +79,15 @@ static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
     build(p->host_table.data());
     return KVT_OK;
   }
+  if (n != 0 && n <= kSmallTable && !p->xform && !p->strided && !p->convert) {
+    // short enough to travel in the kernel arguments
+    Chunk both[2 * kSmallTable];
+    build(both);
+    std::memcpy(p->small_pack.c, both, n * sizeof(Chunk));
+    std::memcpy(p->small_unpack.c, both + n, n * sizeof(Chunk));
+    p->small = true;
+    return KVT_OK;
+  }
   DeviceGuard g;
   if (int rc = g.enter(p->device)) return rc;
   if (n != 0) {
@@ -545,6 +554,14 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
     if (int rc = check_device_span(packed, extent, pack ? "kvt_pack: the packed buffer"
                                                         : "kvt_unpack: the packed buffer"))
       return rc;
+  }
+  if (p->small) {
+    const hipError_t e = launch_copy_chunks_small(
+        pack, pack ? p->small_pack : p->small_unpack, static_cast<uint32_t>(p->n_chunks),
+        p->sub_shift, cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
+        static_cast<uint8_t*>(packed), layer_stride, blobs, s);
+    if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
+    return KVT_OK;
   }
   const Chunk* table = p->dev_chunks + (pack ? 0 : p->n_chunks);
   const uint32_t n = static_cast<uint32_t>(p->n_chunks);

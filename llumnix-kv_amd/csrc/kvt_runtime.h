@@ -222,6 +222,10 @@ struct kvt_plan {
   bool convert = false;            // pack converts bf16 -> fp8: lengths count fp8 bytes (elements)
   std::vector<kvt::Chunk> host_table;   // device == KVT_DEVICE_NONE only: the tables, kept on the host
   uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
+  // plain plans of at most kSmallTable entries: both tables kept here and passed to the
+  // kernel by value; no device table, no upload
+  bool small = false;
+  kvt::SmallTable small_pack{}, small_unpack{};
   kvt::Chunk* dev_chunks = nullptr;     // [0, n_chunks): pack order; [n_chunks, 2 n_chunks): unpack order
   kvt::TableBuf* buf = nullptr;         // storage of dev_chunks (recycled through the table pool)
   hipEvent_t uploaded = nullptr;   // completes when the table has reached the device

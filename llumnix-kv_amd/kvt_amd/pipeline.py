@@ -8,17 +8,43 @@ from . import binding
 from .ctypes_defs import TP_PEQD
 
 
+class Sender:
+    """What TaskContext keeps per destination (refresh_dst_info, kvtransfer/src/tx_stub.cpp:
+    417-591): the valid ranks, this rank's place among them, the TP relation and the parser,
+    chosen and compiled ONCE; every batch for that destination then only parses."""
+
+    def __init__(self, cache_shape, src, dst, fp8=False, pad=True):
+        valid, tp_size, tp_rank, parser_id, self.tp_kind = binding.select_parser(cache_shape, src, dst)
+        self.parser = binding.Parser(parser_id, src, dst, valid, tp_size, tp_rank, fp8=fp8, pad=pad)
+
+    def parse(self, task_bufs):
+        """-> BlockLists of the batch, merged when the TP relation is P==D. Raises KvtError on
+        the first failing request."""
+        lists = binding.BlockLists()
+        for t in task_bufs:
+            binding.check(self.parser.parse(t.struct, lists))
+        if self.tp_kind == TP_PEQD:
+            lists.merge()
+        return lists
+
+    def parse_runs(self, task_bufs):
+        """-> RunLists: the same ranges in closed form (one run per block segment), never merged."""
+        runs = binding.RunLists()
+        for t in task_bufs:
+            binding.check(self.parser.parse_runs(t.struct, runs))
+        return runs
+
+    def close(self):
+        self.parser.close()
+
+
 def parse_batch(cache_shape, src, dst, task_bufs, fp8=False, pad=True):
     """-> (BlockLists, tp_kind). Raises KvtError on the first failing request."""
-    valid, tp_size, tp_rank, parser_id, tp_kind = binding.select_parser(cache_shape, src, dst)
-    parser = binding.Parser(parser_id, src, dst, valid, tp_size, tp_rank, fp8=fp8, pad=pad)
-    lists = binding.BlockLists()
-    for t in task_bufs:
-        binding.check(parser.parse(t.struct, lists))
-    parser.close()
-    if tp_kind == TP_PEQD:
-        lists.merge()
-    return lists, tp_kind
+    sender = Sender(cache_shape, src, dst, fp8=fp8, pad=pad)
+    try:
+        return sender.parse(task_bufs), sender.tp_kind
+    finally:
+        sender.close()
 
 
 def build_plan(workload, device=0, chunk_bytes=0):
@@ -33,13 +59,11 @@ def build_plan(workload, device=0, chunk_bytes=0):
 def parse_batch_runs(cache_shape, src, dst, task_bufs, fp8=False, pad=True):
     """-> (RunLists, tp_kind): the same ranges in closed form (one run per block segment).
     Runs are never merged; for P==D use parse_batch()."""
-    valid, tp_size, tp_rank, parser_id, tp_kind = binding.select_parser(cache_shape, src, dst)
-    parser = binding.Parser(parser_id, src, dst, valid, tp_size, tp_rank, fp8=fp8, pad=pad)
-    runs = binding.RunLists()
-    for t in task_bufs:
-        binding.check(parser.parse_runs(t.struct, runs))
-    parser.close()
-    return runs, tp_kind
+    sender = Sender(cache_shape, src, dst, fp8=fp8, pad=pad)
+    try:
+        return sender.parse_runs(task_bufs), sender.tp_kind
+    finally:
+        sender.close()
 
 
 def build_plan_runs(workload, device=0, chunk_bytes=0):

@@ -290,6 +290,50 @@ def test_cache_registration_checks_what_the_runtime_knows_about_the_memory():
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("n_ranges", [1, 63, 64, 65])
+def test_short_plans_travel_in_the_kernel_arguments(n_ranges):
+    """Up to 64 table entries are passed to the kernel by value, 65 take the resident table:
+    the same bytes either way, also inside a stream capture taken right after creation (there
+    is no table upload to wait for) and on two layers at once."""
+    rng = np.random.default_rng(n_ranges)
+    cap = 4 << 20
+    slots = np.sort(rng.choice(cap // 32768, size=n_ranges, replace=False))
+    lens = rng.integers(1, 32768, size=n_ranges)
+    d_slots = rng.permutation(cap // 32768)[:n_ranges]
+    ranges = np.stack([slots * 32768 + rng.integers(0, 3, size=n_ranges) * 16, d_slots * 32768,
+                       lens], axis=1).astype(np.uint64)
+    ranges[:, 2] = np.minimum(ranges[:, 2], 32768 - 48)
+    lists = kvt_amd.BlockLists()
+    lists.append(0, ranges)
+    plan = kvt_amd.Plan(0, lists, [cap], [cap], chunk_bytes=32768)
+    assert plan.num_chunks == n_ranges
+    src = [[_dev_bytes(cap, 40 + l, "raw")] for l in range(2)]
+    dst = [[torch.full((cap,), 0xA5, dtype=torch.uint8, device="cuda")] for l in range(2)]
+    sc, dc = kvt_amd.Cache(0, src, [cap]), kvt_amd.Cache(0, dst, [cap])
+    stride = plan.layer_bytes
+    packed = torch.zeros(2 * stride, dtype=torch.uint8, device="cuda")
+    s = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    if n_ranges <= 64:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(s):
+            with torch.cuda.graph(graph, stream=s):
+                plan.pack(sc, 0, 2, packed, stride, s.cuda_stream)
+                plan.unpack(dc, 0, 2, packed, stride, s.cuda_stream)
+        graph.replay()
+    else:
+        plan.pack(sc, 0, 2, packed, stride, s.cuda_stream)
+        plan.unpack(dc, 0, 2, packed, stride, s.cuda_stream)
+    torch.cuda.synchronize()
+    packed_h = _host(packed)
+    for l in range(2):
+        blob = checkers.oracle_pack(_host(src[l][0]), ranges)
+        assert np.array_equal(packed_h[l * stride:l * stride + len(blob)], blob), l
+        exp = np.full(cap, 0xA5, dtype=np.uint8)
+        checkers.oracle_unpack(exp, ranges, blob)
+        assert np.array_equal(_host(dst[l][0]), exp), l
+
+
 def test_empty_plan_is_a_no_op():
     lists = kvt_amd.BlockLists()
     lists.append(0, np.zeros((0, 3), dtype=np.uint64))
