@@ -362,6 +362,11 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
                                     int threads_per_wg, void* stream);
 
 enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
+/* stands in for initialize_copy_method_profile() kvtransfer/include/copy_kernels.h:15-22
+ * (called once per copy thread, kvtransfer/src/copy_utils.cpp:52). There is
+ * nothing to measure at start-up here; the call checks that `device` is a usable
+ * gfx950 part and returns. */
+int kvt_initialize_copy_method_profile(int device);
 /* replaces copy_handle_data_with_kernel()       kvtransfer/include/copy_kernels.h:87-97,
  *                                               kvtransfer/src/copy_kernels.cpp:733-827
  * Same calling convention: blocks[i].dst_offset is the GPU-side offset for BOTH
@@ -370,7 +375,12 @@ enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
  * caller's metadata buffers (>= 3 * 8 * max_block_num bytes each, host_meta
  * pinned); more than max_block_num ranges are processed in batches with a
  * stream synchronisation after each, like the reference. max_block_num <= 0
- * means 8192 (BLLM_KVTRANS_KERNEL_COPY_MAX_BLOCK_NUM's default). */
+ * means 8192 (BLLM_KVTRANS_KERNEL_COPY_MAX_BLOCK_NUM's default).
+ * Like the reference's, this entry point may decide against its kernel: at most
+ * 16 ranges of at least 8 MiB each are handed to the DMA engines, one
+ * hipMemcpyAsync per range on `stream` (the reference picks between a memcpy
+ * loop and the kernel from a start-up profile, copy_kernels.cpp:495-619; here
+ * the rule is fixed from measurements on MI355X). */
 int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
                                      const kvt_ipc_block* blocks, uint64_t n,
                                      uint64_t tensor_data_size, int direction, int device,

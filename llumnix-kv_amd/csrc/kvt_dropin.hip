@@ -41,6 +41,8 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
   return KVT_OK;
 }
 
+constexpr uint64_t kDmaMaxRanges = 16, kDmaMinBytes = 8ull << 20;
+
 // Workgroups per range when the lengths are known on the host: the mean number of slices
 // per range (bounded). Equal lengths then get exactly one slice per workgroup, the fastest
 // shape; in a mixed list the few long ranges are strided over by their `rows` workgroups
@@ -62,11 +64,12 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     return fail(KVT_ERR_INVALID, "copy_handle_data: bad direction");
   if (int rc = check_device(device)) return rc;
   if (max_block_num <= 0) max_block_num = 8192;
-  uint64_t total = 0, layer_extent = 0;
+  uint64_t total = 0, layer_extent = 0, shortest = ~0ull;
   for (uint64_t i = 0; i < n; ++i) {
     if (blocks[i].length == 0) return fail(KVT_ERR_INVALID, "copy_handle_data: zero-length range");
     if (halve && (blocks[i].length & 1)) return fail(KVT_ERR_INVALID, "odd bf16 byte length");
     total += blocks[i].length;
+    shortest = std::min(shortest, blocks[i].length);
     layer_extent = std::max(layer_extent, blocks[i].dst_offset + blocks[i].length);
   }
   if (total != tensor_data_size)
@@ -79,6 +82,24 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
   if (int rc = check_device_span(layer_gpu_ptr, layer_extent, "copy_handle_data: the layer tensor"))
     return rc;
   const hipStream_t s = static_cast<hipStream_t>(stream);
+  // A few very large ranges go to the DMA engines, one copy each. The reference makes this
+  // choice (memcpy loop or kernel) from a profile it takes at start-up
+  // (copy_kernels.cpp:495-619); here it is fixed from measurements on MI355X: against pinned
+  // host memory a copy of 128 MiB runs at 57 GB/s where the kernel's stores across PCIe reach
+  // 54, the kernel wins below about 8 MiB per copy (2 MiB: 53 against 33 GB/s).
+  if (!halve && n <= kDmaMaxRanges && shortest >= kDmaMinBytes) {
+    uint64_t cursor = 0;
+    for (uint64_t i = 0; i < n; ++i) {
+      uint8_t* host = static_cast<uint8_t*>(tensor_buf) + cursor;
+      uint8_t* dev = static_cast<uint8_t*>(layer_gpu_ptr) + blocks[i].dst_offset;
+      if (direction == KVT_COPY_D2H)
+        KVT_HIP(hipMemcpyAsync(host, dev, blocks[i].length, hipMemcpyDefault, s));
+      else
+        KVT_HIP(hipMemcpyAsync(dev, host, blocks[i].length, hipMemcpyDefault, s));
+      cursor += blocks[i].length;
+    }
+    return KVT_OK;
+  }
   uint64_t host_cursor = 0;
   for (uint64_t first = 0; first < n; first += static_cast<uint64_t>(max_block_num)) {
     const uint64_t m = std::min<uint64_t>(static_cast<uint64_t>(max_block_num), n - first);
@@ -201,6 +222,10 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
     return launch_ranges(true, gpu_src_base, dst, src_offsets, dst_offsets, lengths, n, num_wg,
                          threads_per_wg, stream);
   });
+}
+
+int kvt_initialize_copy_method_profile(int device) {
+  return guarded([&]() { return check_device(device); });
 }
 
 int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,

@@ -88,6 +88,7 @@ SIGNATURES = {
     "kvt_launch_copy_d2h_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
+    "kvt_initialize_copy_method_profile": (_int, [_int]),
     "kvt_copy_handle_data_with_kernel": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp, _vp,
                                                _vp, _i64]),
     "kvt_copy_handle_data_kernel_direct": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp, _vp,

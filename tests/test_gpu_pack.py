@@ -382,6 +382,40 @@ def test_launch_copy_direct_gather_and_scatter(n, maxlen):
     assert np.array_equal(_host(dst), exp)
 
 
+def test_copy_handle_data_hands_a_few_very_large_ranges_to_the_dma_engines():
+    lib = kvt_amd.lib()
+    assert lib.kvt_initialize_copy_method_profile(0) == 0
+    assert lib.kvt_initialize_copy_method_profile(99) != 0
+    cap = 64 << 20
+    lens = [(9 << 20) + 48, 8 << 20, (12 << 20) + 7]             # all >= 8 MiB, any remainder
+    offs = [1 << 20, (12 << 20) + 16, (30 << 20) + 3]
+    runs = np.array([[0, o, n] for o, n in zip(offs, lens)], dtype=np.uint64)
+    total = int(sum(lens))
+    layer = _dev_bytes(cap, 31, "raw")
+    pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
+    dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
+    host_meta = torch.zeros(3 * 8192, dtype=torch.int64).pin_memory()
+    s = torch.cuda.Stream()
+    rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(), runs.ctypes.data,
+                                              len(runs), total, 1, 0, s.cuda_stream,
+                                              dev_meta.data_ptr(), host_meta.data_ptr(), 0)
+    assert rc == 0, lib.kvt_last_error()
+    s.synchronize()
+    gather = np.stack([runs[:, 1], runs[:, 1], runs[:, 2]], axis=1)
+    blob = checkers.oracle_pack(_host(layer), gather)
+    assert np.array_equal(pinned.numpy(), blob)
+    dst = torch.full((cap,), 0x3C, dtype=torch.uint8, device="cuda")
+    rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), dst.data_ptr(), runs.ctypes.data,
+                                              len(runs), total, 0, 0, s.cuda_stream,
+                                              dev_meta.data_ptr(), host_meta.data_ptr(), 0)
+    assert rc == 0, lib.kvt_last_error()
+    s.synchronize()
+    exp = np.full(cap, 0x3C, dtype=np.uint8)
+    checkers.oracle_unpack(exp, gather, blob)
+    assert np.array_equal(_host(dst), exp)
+    assert (host_meta == 0).all()           # the kernel's metadata buffers were not needed
+
+
 @pytest.mark.parametrize("max_block_num", [0, 7])
 def test_copy_handle_data_with_kernel_pinned_host_buffer(max_block_num):
     w = workloads.llama8b_single(n_layers=1, pool=64, tokens=300)
