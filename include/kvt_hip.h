@@ -367,6 +367,19 @@ enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
  * nothing to measure at start-up here; the call checks that `device` is a usable
  * gfx950 part and returns. */
 int kvt_initialize_copy_method_profile(int device);
+/* replaces get_kernel_copy_buffer()             kvtransfer/include/copy_utils.h:127,
+ *                                               kvtransfer/src/copy_utils.cpp:9-57,137-146
+ * The calling THREAD's metadata buffers for kvt_copy_handle_data_with_kernel: device and
+ * pinned host memory of 3 * 8 * max_block_num bytes each (max_block_num <= 0: 8192), created on
+ * first use, re-created when the thread asks for another device or more ranges, released
+ * when the thread ends. */
+int kvt_get_kernel_copy_buffer(int device, int64_t max_block_num, int64_t** dev_meta,
+                               int64_t** host_meta);
+/* replaces get_thread_local_h2d_stream() / get_thread_local_d2h_stream()
+ *                                               kvtransfer/src/copy_utils.cpp:59-95,148-154
+ * direction = KVT_COPY_H2D / KVT_COPY_D2H: the calling thread's non-blocking stream for that
+ * direction on `device` (the reference's live on the device of the thread's buffers). */
+int kvt_get_thread_local_stream(int device, int direction, void** stream);
 /* replaces copy_handle_data_with_kernel()       kvtransfer/include/copy_kernels.h:87-97,
  *                                               kvtransfer/src/copy_kernels.cpp:733-827
  * Same calling convention: blocks[i].dst_offset is the GPU-side offset for BOTH

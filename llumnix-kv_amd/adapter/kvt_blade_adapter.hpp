@@ -26,6 +26,7 @@
 #include <stdexcept>
 #include <string>
 #include <tuple>
+#include <utility>
 #include <vector>
 
 #include "channel.h"
@@ -231,6 +232,27 @@ inline void validate_ipc_block_bounds(const std::vector<blade_llm::IpcBlock>& bl
                                       blocks.size(), capacity,
                                       kind == blade_llm::IpcBlockOffset::DESTINATION ? 1 : 0,
                                       length_scale, &bad));
+}
+
+// get_kernel_copy_buffer (kvtransfer/include/copy_utils.h:127): the calling thread's
+// {device, pinned host} metadata buffers; {nullptr, nullptr} on failure like the reference.
+inline std::pair<char*, char*> get_kernel_copy_buffer(int device_id, int64_t max_block_num = 0) {
+  int64_t *dev = nullptr, *host = nullptr;
+  if (kvt_get_kernel_copy_buffer(device_id, max_block_num, &dev, &host) != KVT_OK)
+    return {nullptr, nullptr};
+  return {reinterpret_cast<char*>(dev), reinterpret_cast<char*>(host)};
+}
+
+// get_thread_local_h2d_stream / _d2h_stream (copy_utils.h:128-129) as void* stream handles.
+inline void* get_thread_local_h2d_stream(int device_id) {
+  void* s = nullptr;
+  raise(kvt_get_thread_local_stream(device_id, KVT_COPY_H2D, &s));
+  return s;
+}
+inline void* get_thread_local_d2h_stream(int device_id) {
+  void* s = nullptr;
+  raise(kvt_get_thread_local_stream(device_id, KVT_COPY_D2H, &s));
+  return s;
 }
 
 }  // namespace kvt_adapter

@@ -224,6 +224,83 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
   });
 }
 
+// Per-thread metadata buffers and streams of the copy threads (CopyKernelCtx,
+// kvtransfer/src/copy_utils.cpp:9-154): created on first use, re-created when the thread
+// moves to another device or asks for more ranges, released when the thread ends.
+namespace {
+struct CopyThreadCtx {
+  int device = -1;
+  int64_t capacity = 0;  // ranges
+  int64_t* dev = nullptr;
+  int64_t* host = nullptr;
+  hipStream_t streams[2] = {nullptr, nullptr};  // KVT_COPY_H2D, KVT_COPY_D2H
+
+  void release() {
+    if (device >= 0) (void)hipSetDevice(device);
+    for (hipStream_t& st : streams)
+      if (st) {
+        (void)hipStreamSynchronize(st);  // the streams may still reference the buffers
+        (void)hipStreamDestroy(st);
+        st = nullptr;
+      }
+    if (dev) (void)hipFree(dev);
+    if (host) (void)hipHostFree(host);
+    dev = host = nullptr;
+    capacity = 0;
+  }
+  ~CopyThreadCtx() { release(); }
+};
+thread_local CopyThreadCtx g_copy_ctx;
+}  // namespace
+
+int kvt_get_kernel_copy_buffer(int device, int64_t max_block_num, int64_t** dev_meta,
+                               int64_t** host_meta) {
+  return guarded([&]() -> int {
+    if (!dev_meta || !host_meta)
+      return fail(KVT_ERR_INVALID, "kvt_get_kernel_copy_buffer: null argument");
+    if (int rc = check_device(device)) return rc;
+    if (max_block_num <= 0) max_block_num = 8192;
+    CopyThreadCtx& c = g_copy_ctx;
+    if (c.device != device || c.capacity < max_block_num) {
+      DeviceGuard g;
+      if (int rc = g.enter(device)) return rc;
+      c.release();
+      c.device = device;
+      const size_t bytes = 3 * sizeof(int64_t) * static_cast<size_t>(max_block_num);
+      KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c.dev), bytes));
+      const hipError_t e = hipHostMalloc(reinterpret_cast<void**>(&c.host), bytes, hipHostMallocDefault);
+      if (e != hipSuccess) {
+        c.release();
+        return hip_fail(e, "kvt_get_kernel_copy_buffer: pinned metadata buffer");
+      }
+      c.capacity = max_block_num;
+    }
+    *dev_meta = c.dev;
+    *host_meta = c.host;
+    return KVT_OK;
+  });
+}
+
+int kvt_get_thread_local_stream(int device, int direction, void** stream) {
+  return guarded([&]() -> int {
+    if (!stream || (direction != KVT_COPY_H2D && direction != KVT_COPY_D2H))
+      return fail(KVT_ERR_INVALID, "kvt_get_thread_local_stream: bad argument");
+    if (int rc = check_device(device)) return rc;
+    CopyThreadCtx& c = g_copy_ctx;
+    if (c.device != device) {
+      c.release();
+      c.device = device;
+    }
+    if (!c.streams[direction]) {
+      DeviceGuard g;
+      if (int rc = g.enter(device)) return rc;
+      KVT_HIP(hipStreamCreateWithFlags(&c.streams[direction], hipStreamNonBlocking));
+    }
+    *stream = c.streams[direction];
+    return KVT_OK;
+  });
+}
+
 int kvt_initialize_copy_method_profile(int device) {
   return guarded([&]() { return check_device(device); });
 }

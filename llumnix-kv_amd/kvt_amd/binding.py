@@ -89,6 +89,8 @@ SIGNATURES = {
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_initialize_copy_method_profile": (_int, [_int]),
+    "kvt_get_kernel_copy_buffer": (_int, [_int, _i64, _P(_vp), _P(_vp)]),
+    "kvt_get_thread_local_stream": (_int, [_int, _int, _P(_vp)]),
     "kvt_copy_handle_data_with_kernel": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp, _vp,
                                                _vp, _i64]),
     "kvt_copy_handle_data_kernel_direct": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp, _vp,

@@ -416,6 +416,52 @@ def test_copy_handle_data_hands_a_few_very_large_ranges_to_the_dma_engines():
     assert (host_meta == 0).all()           # the kernel's metadata buffers were not needed
 
 
+def test_copy_threads_get_their_own_metadata_buffers_and_streams():
+    """get_kernel_copy_buffer / get_thread_local_{h2d,d2h}_stream of the reference's copy
+    threads (copy_utils.cpp:9-154): per thread, created on first use, used for a real copy."""
+    import threading
+    lib = kvt_amd.lib()
+    w = workloads.llama8b_single(n_layers=1, pool=64, tokens=300)
+    runs = _oracle_lists(w)[0]
+    cap = w.capacities("src")[0]
+    layer = _dev_bytes(cap, 9)
+    layer_h = _host(layer)
+    total = int(runs[:, 2].sum())
+    kb = np.stack([np.zeros(len(runs), dtype=np.uint64), runs[:, 0], runs[:, 2]], axis=1).copy()
+    seen, errors = {}, []
+
+    def work(i):
+        try:
+            dev, host, st, st2 = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+            assert lib.kvt_get_kernel_copy_buffer(0, 0, C.byref(dev), C.byref(host)) == 0
+            d2, h2 = C.c_void_p(), C.c_void_p()
+            assert lib.kvt_get_kernel_copy_buffer(0, 100, C.byref(d2), C.byref(h2)) == 0
+            assert (d2.value, h2.value) == (dev.value, host.value)       # large enough already
+            assert lib.kvt_get_thread_local_stream(0, 1, C.byref(st)) == 0
+            assert lib.kvt_get_thread_local_stream(0, 1, C.byref(st2)) == 0 and st.value == st2.value
+            assert lib.kvt_get_thread_local_stream(0, 0, C.byref(st2)) == 0 and st.value != st2.value
+            pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
+            rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(),
+                                                      kb.ctypes.data, len(kb), total, 1, 0, st,
+                                                      dev, host, 0)
+            assert rc == 0, lib.kvt_last_error()
+            assert lib.kvt_stream_synchronize(st) == 0
+            assert np.array_equal(pinned.numpy(), checkers.oracle_pack(layer_h, runs))
+            seen[i] = (dev.value, host.value, st.value)
+        except Exception as e:
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(3)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert len(seen) == 3
+    bad = C.c_void_p()
+    assert lib.kvt_get_thread_local_stream(0, 7, C.byref(bad)) != 0
+
+
 @pytest.mark.parametrize("max_block_num", [0, 7])
 def test_copy_handle_data_with_kernel_pinned_host_buffer(max_block_num):
     w = workloads.llama8b_single(n_layers=1, pool=64, tokens=300)
