@@ -668,8 +668,8 @@ def main():
     ap.add_argument("--sequential", action="store_true",
                     help="config 5 only: pack everything, then unpack everything, instead of the "
                          "mixed mode (half of the requests packing while the other half unpacks)")
-    ap.add_argument("--cpu-layers", type=int, default=12,
-                    help="layers in the CPU baseline sample (12 layers x 5 passes of config 2 are "
+    ap.add_argument("--cpu-layers", type=int, default=16,
+                    help="layers in the CPU baseline sample (16 layers x 5 passes of config 2 are "
                          "about 10 s of single-thread CPU work)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
