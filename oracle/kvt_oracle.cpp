@@ -17,7 +17,10 @@
 //     config-shaped inputs (tests/test_oracle_vs_ref.py), against the golden
 //     vectors committed under tests/golden/ (written by the compiled reference),
 //     and against the known-answer numbers of the reference's own tests
-//     (tests/test_oracle_known_answers.py).
+//     (tests/test_oracle_known_answers.py). For the RAGGED, FLASH and DPSK cache
+//     shapes the reference's second, descriptor-driven generator
+//     (kvtransfer/src/cache_transfer_spec.cpp) states the same byte mapping
+//     independently (tests/test_descriptor_path.py, through the product parser).
 //   * valid-rank selection / dispatch: known answers of the reference tests.
 //   * merge: known answers of the reference tests (incl. overlapping prefix).
 //   * pack / unpack: brute-force byte model in numpy + round-trip invariants.
