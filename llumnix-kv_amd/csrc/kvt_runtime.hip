@@ -48,17 +48,23 @@ int check_device(int device) {
 // lie inside. A framework's caching allocator hands out pieces of larger allocations, so this
 // catches an extent that overshoots the underlying allocation, not one that overshoots the
 // tensor. Spans that passed are remembered per thread (a serving loop reuses its buffers),
-// so the steady state costs a few comparisons and no runtime call.
+// so the steady state costs a few comparisons and no runtime call; an entry is trusted for
+// 256 uses and then asked for again, since the memory behind an address can change hands.
 int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) {
   if (bytes == 0) return KVT_OK;
   struct Span {
     uintptr_t lo = 0, hi = 0;
+    unsigned uses = 0;
   };
   static thread_local Span seen[8];
   static thread_local unsigned next = 0;
   const uintptr_t p = reinterpret_cast<uintptr_t>(ptr);
-  for (const Span& s : seen)
-    if (p >= s.lo && p < s.hi && bytes <= s.hi - p) return KVT_OK;
+  for (Span& s : seen)
+    if (p >= s.lo && p < s.hi && bytes <= s.hi - p) {
+      if (++s.uses < 256) return KVT_OK;
+      s = Span{};  // ask the runtime again below
+      break;
+    }
   hipPointerAttribute_t attr{};
   if (hipPointerGetAttributes(&attr, ptr) != hipSuccess) {
     (void)hipGetLastError();
@@ -78,7 +84,7 @@ int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) 
                 what + ": " + std::to_string(bytes) +
                     " bytes reach beyond the allocation that holds the pointer (" +
                     std::to_string(p < lo || p - lo > size ? 0 : size - (p - lo)) + " bytes left)");
-  seen[next++ % 8] = Span{lo, lo + size};
+  seen[next++ % 8] = Span{lo, lo + size, 0};
   return KVT_OK;
 }
 
