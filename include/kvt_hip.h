@@ -189,7 +189,10 @@ typedef struct kvt_xform {
  * against; pack refuses a cache smaller than src_capacity, unpack one smaller
  * than dst_capacity. chunk_bytes bounds one table entry: a power of two in
  * [4096, 524288], or 0 to derive it from the median range length (at most
- * 32 KiB). Every entry is moved by ceil(len / 4096) workgroups. */
+ * 32 KiB). Every entry is moved by ceil(len / 4096) workgroups. The tables of a
+ * plan of at most 64 entries (one short request) are passed to the kernel by
+ * value: such a plan needs no upload and can be launched, or captured into a
+ * graph, the moment it is created. */
 typedef struct kvt_plan kvt_plan;
 int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
                     const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
@@ -203,7 +206,9 @@ void kvt_plan_destroy(kvt_plan* p);
  * With 16-byte aligned layer base pointers, packed buffer, layer stride and blob
  * positions a strided entry moves one 16-byte vector per lane; 4-byte alignment
  * (a blob inside a layer message) is served by a slower word-wise path; anything
- * less is refused with KVT_ERR_INVALID. */
+ * less is refused with KVT_ERR_INVALID. Every range of a run must fit the stated
+ * capacities, and a run may not describe more bytes than the destination tensor
+ * holds (its ranges are meant to be disjoint there): KVT_ERR_OUT_OF_RANGE. */
 int kvt_plan_create_runs(int device, const kvt_run_lists* lists, const uint64_t* src_capacity,
                          const uint64_t* dst_capacity, uint32_t chunk_bytes, kvt_plan** out);
 /* The same for a sender whose cache holds bf16 while the transfer buffer and the receiver
