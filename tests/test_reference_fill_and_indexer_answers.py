@@ -257,3 +257,13 @@ def test_ple_state_p_lt_d_fans_out_complete(d_rank):
     o = _pltd("HYBRID_PLTD", src, dst, TaskBuf(0, 1, True, *PLE_GROUPS), 4)
     want = (150 * int(src.block_sizes[0]), 220 * int(dst.block_sizes[0]), 3 * 4 * 2)
     assert o.count(want) == 1
+
+
+# send_stub_test.cpp:23-41 (Qwen4PleParseBlockTest.PEqDCopiesFullPaddedBlock calls the PLE helper
+# directly: 64-byte pages, PLE block group 2, block 2 -> 5): the same record through the
+# top-level P == D parser with empty GDN and attention groups
+def test_ple_state_p_eq_d_copies_the_full_padded_page():
+    kw = dict(num_gdn_layers=1, num_kv_heads=1, **PLE)
+    w = make_worker_info([64], [64], 16, tp=1, rank=0, **kw)
+    o = _both("HYBRID_PEQD", w, w, TaskBuf(0, 0, True, [[], [], [2]], [[], [], [5]]), 1)
+    assert o == [(2 * 64, 5 * 64, 64)]
