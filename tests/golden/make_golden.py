@@ -51,7 +51,32 @@ def config_shaped():
                     tasks=[[0, 40, False, [[6], [7], [8], [3, 4, 5]], [[10], [11], [12], [7, 8, 9]]],
                            [5, 50, True, [[16], [17], [18], [13, 14, 15, 19]],
                             [[20], [21], [22], [23, 24, 25, 26]]]]))
+    # the reference's own hybrid arrangement (uniform pages shared by attention and GDN states),
+    # at P == D and between a TP2 prefill and a TP1 decode instance; a FLASH TP2 -> TP1 batch
+    from kvt_amd import workloads
+    for tag, w in (("cfg/qwen3_next_uniform_pages", workloads.qwen3next_uniform_pages(
+                        n_layers=1, pool=40, n_req=3, tokens=2500)),
+                   ("cfg/qwen3_next_tp2_to_tp1_rank0", workloads.qwen3next_tp_split(
+                        2, 1, 0, n_layers=1, pool=16, n_req=1, tokens=200, head_dim=64, state_dim=32)),
+                   ("cfg/qwen3_next_tp2_to_tp1_rank1", workloads.qwen3next_tp_split(
+                        2, 1, 1, n_layers=1, pool=16, n_req=1, tokens=200, head_dim=64, state_dim=32)),
+                   ("cfg/flash_tp2_to_tp1", workloads.tp_split(
+                        "flash", 2, 1, 1, n_layers=1, src_pool=32, dst_pool=48, n_req=2,
+                        min_tok=20, max_tok=100))):
+        out.append(workload_case(tag, w))
     return out
+
+
+def workload_case(name, w, fp8=False):
+    """A kvt_amd.workloads.Workload as a golden case (dispatch values from the oracle's
+    restatement of refresh_dst_info, which the valid-rank known answers pin)."""
+    src, dst = w.worker_infos()
+    rc, valid, tps, tpr, pid, kind = checkers.oracle_select(w.cache_shape, src, dst)
+    assert rc == 0
+    from kvt_amd.ctypes_defs import PARSER
+    parser = [k for k, v in PARSER.items() if v == pid][0]
+    return dict(name=name, parser=parser, src=w.src_info, dst=w.dst_info, valid=int(valid),
+                tp_size=int(tps), tp_rank=int(tpr), fp8=fp8, tasks=w.tasks)
 
 
 def run_cases(case_list):
@@ -77,6 +102,10 @@ def main():
                 c["name"] += "/fp8"
                 # the converting path reads 2x the length at the source: give the source pool room
                 lst.append(c)
+        from kvt_amd import workloads
+        lst.append(workload_case("cfg/flash_tp2_to_tp1/fp8", workloads.tp_split(
+            "flash", 2, 1, 1, n_layers=1, src_pool=32, dst_pool=48, n_req=2, min_tok=20,
+            max_tok=100, fp8_dst=True), fp8=True))
         json.dump(run_cases(lst), sys.stdout)
         return
     assert checkers.ref() is not None, "build oracle/_ref first (make -C oracle ref)"
