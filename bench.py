@@ -657,7 +657,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", type=int, default=2, help="1-5: BASELINE.json configs[] index + 1; 6-8: TP-remapping batches; "
+    ap.add_argument("--config", type=int, default=2, help="1-5: the five benchmark configurations (1 = the CPU-runnable case, 2 = the headline); 6-8: TP-remapping batches; "
                          "9: config 5 with the reference's uniform 2 MiB pages; 10: the same "
                          "model TP2 -> TP1")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")

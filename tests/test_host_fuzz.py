@@ -4,7 +4,8 @@ ABI must survive malformed frames, garbage geometries and bad block tables
 without a memory error, and its invariants must hold. tests/plan_fuzz.cpp does
 the same for the copy-plan builder, which lives in HIP translation units: hipcc
 builds them with the sanitizers on the host side only, and host-only plans
-(device = -1) need no GPU. CPU only."""
+(device = -1) need no GPU. tests/thread_check.cpp runs the host entry points
+from eight threads that share parsers, under ThreadSanitizer. CPU only."""
 import os
 import shutil
 import subprocess
@@ -30,6 +31,19 @@ def test_host_entry_points_under_sanitizers(tmp_path):
         res = subprocess.run([exe, "2", seed], capture_output=True, text=True, env=env, timeout=600)
         assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-6000:]
         assert "host fuzz ok" in res.stdout
+
+
+def test_shared_parsers_under_thread_sanitizer(tmp_path):
+    exe = str(tmp_path / "thread_check")
+    cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=thread",
+           "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+           os.path.join(ROOT, "tests", "thread_check.cpp")]
+    cmd += [os.path.join(CSRC, s) for s in HOST_SOURCES] + ["-o", exe, "-lpthread"]
+    subprocess.check_call(cmd)
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1:abort_on_error=1")
+    res = subprocess.run([exe, "40", "31337"], capture_output=True, text=True, env=env, timeout=600)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-6000:]
+    assert "thread check ok" in res.stdout
 
 
 HIPCC = shutil.which("hipcc") or ("/opt/rocm/bin/hipcc" if os.path.exists("/opt/rocm/bin/hipcc") else None)
