@@ -891,14 +891,25 @@ def main():
                               wls=wls, sides=sides, full_wls=full_wls, full_sides=full_sides,
                               mixed=mixed, infos=infos, tasks=tasks, first=first, strides=strides,
                               packed=packed, stream=stream, sh=sh, new_event=new_event, keep=keep)
-    if not args.skip_cpu:
-        leg_cpu(c, out)
+    # The timed region is over: a failure in a side leg must not take the measured line with
+    # it. It is reported in "errors" (and on stderr, with the traceback) and fails the run.
+    legs = [] if args.skip_cpu else [leg_cpu]
     if not args.skip_extras:
-        for leg in (leg_latency, leg_session, leg_launchers, leg_fp8_plan, leg_frames,
-                    leg_store_objects, leg_staging):
+        legs += [leg_latency, leg_session, leg_launchers, leg_fp8_plan, leg_frames,
+                 leg_store_objects, leg_staging]
+    errors = {}
+    for leg in legs:
+        try:
             leg(c, out)
-
+        except Exception as e:          # noqa: BLE001 - reported, not swallowed
+            import traceback
+            traceback.print_exc(file=sys.stderr)
+            errors[leg.__name__] = "%s: %s" % (type(e).__name__, e)
+    if errors:
+        out["errors"] = errors
     print(json.dumps(out), flush=True)
+    if errors:
+        raise SystemExit(1)
 
 
 if __name__ == "__main__":
