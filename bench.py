@@ -333,6 +333,33 @@ def leg_session(c, out):
     sess.close()
 
 
+def leg_cu_usage(c, out):
+    """Pack and unpack of the same batch with the copy launches limited to a share of the CUs
+    (the reference's BLLM_KVTRANS_KERNEL_COPY_SM_USAGE): what a transfer that overlaps a
+    forward pass gives up for leaving the rest of the device alone."""
+    kvt, lib, sh, new_event = c.kvt, c.lib, c.sh, c.new_event
+    w, side, plan0 = c.wls[0], c.sides[0], c.first[0][0]
+    pay0 = sum(plan0.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
+    rows = []
+    try:
+        for usage in (1.0, 0.5, 0.25, 0.125, 0.0625):
+            kvt.set_copy_cu_usage(0, usage)
+            e = [new_event() for _ in range(3)]
+            for rep in range(2):   # second run is the measurement
+                lib.kvt_event_record(e[0], sh)
+                plan0.pack(side.src_cache, 0, w.n_layers, c.packed[0], c.strides[0], sh)
+                lib.kvt_event_record(e[1], sh)
+                plan0.unpack(side.dst_cache, 0, w.n_layers, c.packed[0], c.strides[0], sh)
+                lib.kvt_event_record(e[2], sh)
+            lib.kvt_event_synchronize(e[2])
+            rows.append({"usage": usage, "workgroups": kvt.get_copy_cu_usage(0)[1] or "one per slice",
+                         "pack_gbps": round(2.0 * pay0 / (ev_ms(lib, e[0], e[1]) * 1e-3) / 1e9, 1),
+                         "unpack_gbps": round(2.0 * pay0 / (ev_ms(lib, e[1], e[2]) * 1e-3) / 1e9, 1)})
+    finally:
+        kvt.set_copy_cu_usage(0, 1.0)
+    out["cu_usage"] = rows
+
+
 def leg_launchers(c, out):
     """The reference-shaped entry points on the same ranges."""
     torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
@@ -895,7 +922,7 @@ def main():
     # it. It is reported in "errors" (and on stderr, with the traceback) and fails the run.
     legs = [] if args.skip_cpu else [leg_cpu]
     if not args.skip_extras:
-        legs += [leg_latency, leg_session, leg_launchers, leg_fp8_plan, leg_frames,
+        legs += [leg_latency, leg_session, leg_cu_usage, leg_launchers, leg_fp8_plan, leg_frames,
                  leg_store_objects, leg_staging]
     errors = {}
     for leg in legs:

@@ -366,6 +366,22 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
                                     const int64_t* lengths, int64_t n, int num_wg,
                                     int threads_per_wg, void* stream);
 
+/* replaces env_kernel_copy_sm_usage(), BLLM_KVTRANS_KERNEL_COPY_SM_USAGE
+ *                                               kvtransfer/src/envcfg.cpp:311-326,
+ * as CopyKernelConfig::initialize applies it    kvtransfer/src/copy_kernels.cpp:327-335
+ * (blocks of a copy launch = resident blocks per SM x SMs x usage): the share of the
+ * device's CUs a copy launch may occupy, for an engine that overlaps transfers with its
+ * forward pass. usage in (0, 1]; 1 (the default) keeps one workgroup per 4 KiB slice, the
+ * fastest shape. Below 1 every copy launch of this library on `device` (plans, sessions,
+ * stagers, the launchers below) runs as at most usage x CUs x 8 persistent 256-lane
+ * workgroups, rounded down to a multiple of 8 and at least 8, that stride over the same
+ * work; results are identical. Takes effect for launches issued after the call (a launch
+ * captured into a graph keeps the shape it was captured with). Passing num_wg > 0 to a
+ * launcher still bounds that launch further. */
+int kvt_set_copy_cu_usage(int device, double usage);
+/* The current setting and the workgroup limit it stands for (0 = none); either may be NULL. */
+int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
+
 enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
 /* stands in for initialize_copy_method_profile() kvtransfer/include/copy_kernels.h:15-22
  * (called once per copy thread, kvtransfer/src/copy_utils.cpp:52). There is

@@ -255,6 +255,13 @@ inline void* get_thread_local_d2h_stream(int device_id) {
   return s;
 }
 
+// What CopyKernelConfig::initialize does with BLLM_KVTRANS_KERNEL_COPY_SM_USAGE
+// (kvtransfer/src/copy_kernels.cpp:327-335): hand the configured share to the library, once,
+// where the reference initialises its copy threads.
+inline void apply_kernel_copy_sm_usage(int device_id) {
+  raise(kvt_set_copy_cu_usage(device_id, blade_llm::env_kernel_copy_sm_usage()));
+}
+
 }  // namespace kvt_adapter
 
 #endif  // KVT_BLADE_ADAPTER_HPP_

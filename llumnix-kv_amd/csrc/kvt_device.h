@@ -48,18 +48,22 @@ struct StrideTable {
   StrideShape shape[kMaxShapes];
 };
 
+// Chunk launchers. max_wgs = 0: one workgroup per (4 KiB slice, layer), the fastest shape.
+// max_wgs > 0: at most that many workgroups (a multiple of 8), striding over the same items,
+// for a caller that wants the copy to leave part of the device to other kernels.
 hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, bool words, hipStream_t stream);
+                                 const StrideTable& shapes, bool words, uint32_t max_wgs,
+                                 hipStream_t stream);
 // Converting gather (bf16 -> fp8 E4M3) of a chunk table, plain and strided chunks alike; lengths
 // and packed positions count fp8 bytes, cache offsets and strides bytes of the bf16 cache.
 hipError_t launch_convert_chunks(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                  uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                  uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                  uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, hipStream_t stream);
+                                 const StrideTable& shapes, uint32_t max_wgs, hipStream_t stream);
 // A table of at most kSmallTable entries travels in the kernel arguments (2 KiB): a short
 // request then needs no table upload, no upload event and no cross-stream wait before its
 // first launch.
@@ -71,23 +75,25 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
-                                    const BlobOffsets& blobs, hipStream_t stream);
+                                    const BlobOffsets& blobs, uint32_t max_wgs,
+                                    hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, const BlobOffsets& blobs, hipStream_t stream);
+                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs,
+                              hipStream_t stream);
 hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               hipStream_t stream);
+                               uint32_t max_wgs, hipStream_t stream);
 // rows = workgroups striding over the 4 KiB slices of each range
 hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                               const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,
-                              int rows, hipStream_t stream);
+                              int rows, uint32_t max_wgs, hipStream_t stream);
 hipError_t launch_convert_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                                  const int64_t* dst_off, const int64_t* lens, int64_t n,
-                                 int num_wg, int rows, hipStream_t stream);
+                                 int num_wg, int rows, uint32_t max_wgs, hipStream_t stream);
 hipError_t launch_copy_linear(void* dst, const void* src, uint64_t bytes, hipStream_t stream);
 
 }  // namespace kvt

@@ -35,8 +35,11 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
   // short one more (enough to fill the device when its ranges are long).
   const int rows = static_cast<int>(std::max<int64_t>(2, std::min<int64_t>(64, (8192 + n - 1) / n)));
   const hipStream_t s = static_cast<hipStream_t>(stream);
-  const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, s)
-                               : launch_copy_ranges(src, dst, so, dof, len, n, wgs, rows, s);
+  int device = 0;   // these entry points name no device: the caller's current one
+  KVT_HIP(hipGetDevice(&device));
+  const uint32_t cap = copy_wg_cap(device);
+  const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s)
+                               : launch_copy_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s);
   if (e != hipSuccess) return hip_fail(e, "range copy launch");
   return KVT_OK;
 }
@@ -122,16 +125,17 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     const int64_t* d_lens = dev_meta + 2 * m;
     const int wgs = static_cast<int>(m);
     const int rows = rows_for(slices, m);
+    const uint32_t cap = copy_wg_cap(device);
     hipError_t e;
     if (halve)
       e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
-                                static_cast<int64_t>(m), wgs, rows, s);
+                                static_cast<int64_t>(m), wgs, rows, cap, s);
     else if (direction == KVT_COPY_D2H)
       e = launch_copy_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
-                             static_cast<int64_t>(m), wgs, rows, s);
+                             static_cast<int64_t>(m), wgs, rows, cap, s);
     else
       e = launch_copy_ranges(tensor_buf, layer_gpu_ptr, d_contig, d_gpu, d_lens,
-                             static_cast<int64_t>(m), wgs, rows, s);
+                             static_cast<int64_t>(m), wgs, rows, cap, s);
     if (e != hipSuccess) return hip_fail(e, "copy_handle_data launch");
     // the metadata buffers are reused by the next batch
     if (first + m < n) KVT_HIP(hipStreamSynchronize(s));
@@ -185,9 +189,9 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
   const hipError_t e =
       direction == KVT_COPY_D2H
           ? launch_copy_ranges(layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
-                               static_cast<int64_t>(n), static_cast<int>(n), rows, s)
+                               static_cast<int64_t>(n), static_cast<int>(n), rows, copy_wg_cap(device), s)
           : launch_copy_ranges(tensor_buf, layer_gpu_ptr, src_dev, dst_dev, len_dev,
-                               static_cast<int64_t>(n), static_cast<int>(n), rows, s);
+                               static_cast<int64_t>(n), static_cast<int>(n), rows, copy_wg_cap(device), s);
   if (e != hipSuccess) return hip_fail(e, "copy_handle_data_kernel_direct launch");
   return KVT_OK;
 }

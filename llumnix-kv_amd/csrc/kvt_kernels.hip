@@ -32,6 +32,28 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t b, uint32_t n) {
   return (b & 7u) * per + (b >> 3);
 }
 
+// Which (slice, layer) items a workgroup handles. The normal launch has one workgroup per
+// item: grid (slices rounded up to 8, layers). A launch capped to a share of the device
+// (CAPPED) has a one-dimensional grid of that many workgroups, a multiple of 8, which stride
+// over the same items layer by layer; since the stride and the rounded slice count are both
+// multiples of 8, a workgroup keeps meeting slices of the eighth that belongs to its XCD.
+template <bool CAPPED, class Body>
+__device__ __forceinline__ void for_items(uint32_t n_slices, uint32_t n_layers, Body body) {
+  if (!CAPPED) {
+    body(xcd_remap(blockIdx.x, n_slices), static_cast<uint32_t>(blockIdx.y));
+    return;
+  }
+  const uint32_t per_layer = (n_slices + 7u) & ~7u;
+  uint32_t layer = 0;
+  for (uint32_t s = blockIdx.x;; s += gridDim.x) {
+    while (s >= per_layer) {
+      s -= per_layer;
+      if (++layer >= n_layers) return;
+    }
+    body(xcd_remap(s, n_slices), layer);
+  }
+}
+
 // Copies len (<= 4096) bytes with the whole workgroup. Fast path: 16-byte
 // aligned on both sides; one vector per lane, stragglers byte-wise.
 __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst,
@@ -61,48 +83,48 @@ __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst,
 // Gather (PACK) / scatter of a resident chunk table. Workgroup b handles slice
 // (b & mask) of chunk (b >> sub_shift); chunks are at most 4096 << sub_shift
 // bytes, so a chunk shorter than that simply leaves its last workgroups idle.
-template <bool PACK>
+template <bool PACK, bool CAPPED>
 __global__ __launch_bounds__(kThreads) void copy_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
-  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
-  if (b >= n_slices) return;
-  const Chunk c = chunks[b >> sub_shift];
-  const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-  if (off >= c.len) return;
-  const uint32_t len = min(kSlice, c.len - off);
-  const uint32_t layer = blockIdx.y;
-  uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] +
-                   c.cache + off;
-  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-  if (PACK)
-    copy_slice(pk, cache, len, threadIdx.x);
-  else
-    copy_slice(cache, pk, len, threadIdx.x);
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
+  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
+    if (b >= n_slices) return;
+    const Chunk c = chunks[b >> sub_shift];
+    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
+    if (off >= c.len) return;
+    const uint32_t len = min(kSlice, c.len - off);
+    uint8_t* cache =
+        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache + off;
+    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
+    if (PACK)
+      copy_slice(pk, cache, len, threadIdx.x);
+    else
+      copy_slice(cache, pk, len, threadIdx.x);
+  });
 }
 
 // The same for a table short enough to be a kernel argument (read through the scalar cache
 // like any other argument; the index is uniform across the workgroup).
-template <bool PACK>
+template <bool PACK, bool CAPPED>
 __global__ __launch_bounds__(kThreads) void copy_chunks_small_kernel(
     const SmallTable table, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
-  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
-  if (b >= n_slices) return;
-  const Chunk& c = table.c[b >> sub_shift];
-  const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-  if (off >= c.len) return;
-  const uint32_t len = min(kSlice, c.len - off);
-  const uint32_t layer = blockIdx.y;
-  uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] +
-                   c.cache + off;
-  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-  if (PACK)
-    copy_slice(pk, cache, len, threadIdx.x);
-  else
-    copy_slice(cache, pk, len, threadIdx.x);
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
+  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
+    if (b >= n_slices) return;
+    const Chunk& c = table.c[b >> sub_shift];
+    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
+    if (off >= c.len) return;
+    const uint32_t len = min(kSlice, c.len - off);
+    uint8_t* cache =
+        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache + off;
+    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
+    if (PACK)
+      copy_slice(pk, cache, len, threadIdx.x);
+    else
+      copy_slice(cache, pk, len, threadIdx.x);
+  });
 }
 
 // Gather / scatter of a table whose chunks may be strided on the cache side:
@@ -114,90 +136,92 @@ __global__ __launch_bounds__(kThreads) void copy_chunks_small_kernel(
 // needs 16-byte aligned base pointers and blob positions (one vector per lane),
 // WORDS = true moves 4-byte words instead (a blob inside a received layer
 // message sits at 4 or 12 modulo 16; that path is PCIe-bound anyway).
-template <bool PACK, bool WORDS>
+template <bool PACK, bool WORDS, bool CAPPED>
 __global__ __launch_bounds__(kThreads) void strided_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs, StrideTable shapes) {
-  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
-  if (b >= n_slices) return;
-  const Chunk c = chunks[b >> sub_shift];
-  const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-  if (off >= c.len) return;
-  const uint32_t len = min(kSlice, c.len - off);
-  const uint32_t layer = blockIdx.y;
-  uint8_t* cache =
-      layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
-  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-  if (c.shape == 0) {
-    if (PACK)
-      copy_slice(pk, cache + off, len, threadIdx.x);
-    else
-      copy_slice(cache + off, pk, len, threadIdx.x);
-    return;
-  }
-  const StrideShape& s = shapes.shape[c.shape - 1u];
-  const uint64_t outer = s.outer[PACK ? 0 : 1], inner = s.inner[PACK ? 0 : 1];
-  if (!WORDS) {
-    if (threadIdx.x >= (len >> 4)) return;
-    const uint32_t v = (off >> 4) + threadIdx.x;  // vector index inside the chunk, < 2^15
-    const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
-    const uint32_t col = v - rec * s.vlen;
-    const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
-    const uint32_t i = rec - o * s.n_inner;
-    u32x4* cv = reinterpret_cast<u32x4*>(cache + o * outer + i * inner + (col << 4));
-    u32x4* pv = reinterpret_cast<u32x4*>(pk) + threadIdx.x;
-    if (PACK)
-      __builtin_nontemporal_store(__builtin_nontemporal_load(cv), pv);
-    else
-      __builtin_nontemporal_store(__builtin_nontemporal_load(pv), cv);
-  } else {
-    const uint32_t wlen = s.vlen << 2;  // record length in words, < 1024
-    for (uint32_t t = threadIdx.x; t < (len >> 2); t += kThreads) {
-      const uint32_t w = (off >> 2) + t;          // word index inside the chunk, < 2^17
-      const uint32_t rec = __umulhi(w, s.inv_wlen);
-      const uint32_t col = w - rec * wlen;
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes) {
+  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
+    if (b >= n_slices) return;
+    const Chunk c = chunks[b >> sub_shift];
+    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
+    if (off >= c.len) return;
+    const uint32_t len = min(kSlice, c.len - off);
+    uint8_t* cache =
+        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
+    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
+    if (c.shape == 0) {
+      if (PACK)
+        copy_slice(pk, cache + off, len, threadIdx.x);
+      else
+        copy_slice(cache + off, pk, len, threadIdx.x);
+      return;
+    }
+    const StrideShape& s = shapes.shape[c.shape - 1u];
+    const uint64_t outer = s.outer[PACK ? 0 : 1], inner = s.inner[PACK ? 0 : 1];
+    if (!WORDS) {
+      if (threadIdx.x >= (len >> 4)) return;
+      const uint32_t v = (off >> 4) + threadIdx.x;  // vector index inside the chunk, < 2^15
+      const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
+      const uint32_t col = v - rec * s.vlen;
       const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
       const uint32_t i = rec - o * s.n_inner;
-      uint32_t* cw = reinterpret_cast<uint32_t*>(cache + o * outer + i * inner + (col << 2));
-      uint32_t* pw = reinterpret_cast<uint32_t*>(pk) + t;
+      u32x4* cv = reinterpret_cast<u32x4*>(cache + o * outer + i * inner + (col << 4));
+      u32x4* pv = reinterpret_cast<u32x4*>(pk) + threadIdx.x;
       if (PACK)
-        *pw = *cw;
+        __builtin_nontemporal_store(__builtin_nontemporal_load(cv), pv);
       else
-        *cw = *pw;
+        __builtin_nontemporal_store(__builtin_nontemporal_load(pv), cv);
+    } else {
+      const uint32_t wlen = s.vlen << 2;  // record length in words, < 1024
+      for (uint32_t t = threadIdx.x; t < (len >> 2); t += kThreads) {
+        const uint32_t w = (off >> 2) + t;          // word index inside the chunk, < 2^17
+        const uint32_t rec = __umulhi(w, s.inv_wlen);
+        const uint32_t col = w - rec * wlen;
+        const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
+        const uint32_t i = rec - o * s.n_inner;
+        uint32_t* cw = reinterpret_cast<uint32_t*>(cache + o * outer + i * inner + (col << 2));
+        uint32_t* pw = reinterpret_cast<uint32_t*>(pk) + t;
+        if (PACK)
+          *pw = *cw;
+        else
+          *cw = *pw;
+      }
     }
-  }
+  });
 }
 
 // HND <-> NHD page transform. A chunk covers tokens [t0, t0 + len/(heads*row))
 // of one K or V half page whose base is c.cache. Packed side: [token][head][row]
 // contiguous from c.packed; cache side: [head][ntpb][row]. Lane v of the chunk
 // moves the v-th 16-byte vector of the packed side; a row is vrow vectors.
-template <bool PACK>
+template <bool PACK, bool CAPPED>
 __global__ __launch_bounds__(kThreads) void xform_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs, XformDev x) {
-  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
-  if (b >= n_slices) return;
-  const Chunk c = chunks[b >> sub_shift];
-  const uint32_t v = ((b & ((1u << sub_shift) - 1u)) << 8) + threadIdx.x;  // 256 vectors per slice
-  if (v >= (c.len >> 4)) return;
-  const uint32_t layer = blockIdx.y;
-  u32x4* cv = reinterpret_cast<u32x4*>(
-      layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache);
-  u32x4* pv =
-      reinterpret_cast<u32x4*>(packed + layer * layer_stride + blobs.off[c.tensor] + c.packed);
-  // exact quotients by multiply-high (operands < 2^16); a divisor of 1 has no such constant
-  const uint32_t r = x.vrow == 1 ? v : __umulhi(v, x.inv_vrow);  // packed-side row: t_local*heads + h
-  const uint32_t col = v - r * x.vrow;
-  const uint32_t t_local = x.heads == 1 ? r : __umulhi(r, x.inv_heads);
-  const uint32_t h = r - t_local * x.heads;
-  const uint32_t cidx = (h * x.ntpb + c.t0 + t_local) * x.vrow + col;
-  if (PACK)
-    __builtin_nontemporal_store(__builtin_nontemporal_load(cv + cidx), pv + v);
-  else
-    __builtin_nontemporal_store(__builtin_nontemporal_load(pv + v), cv + cidx);
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    XformDev x) {
+  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
+    if (b >= n_slices) return;
+    const Chunk c = chunks[b >> sub_shift];
+    const uint32_t v = ((b & ((1u << sub_shift) - 1u)) << 8) + threadIdx.x;  // 256 vectors per slice
+    if (v >= (c.len >> 4)) return;
+    u32x4* cv = reinterpret_cast<u32x4*>(
+        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache);
+    u32x4* pv =
+        reinterpret_cast<u32x4*>(packed + layer * layer_stride + blobs.off[c.tensor] + c.packed);
+    // exact quotients by multiply-high (operands < 2^16); a divisor of 1 has no such constant
+    const uint32_t r = x.vrow == 1 ? v : __umulhi(v, x.inv_vrow);  // packed-side row: t_local*heads + h
+    const uint32_t col = v - r * x.vrow;
+    const uint32_t t_local = x.heads == 1 ? r : __umulhi(r, x.inv_heads);
+    const uint32_t h = r - t_local * x.heads;
+    const uint32_t cidx = (h * x.ntpb + c.t0 + t_local) * x.vrow + col;
+    if (PACK)
+      __builtin_nontemporal_store(__builtin_nontemporal_load(cv + cidx), pv + v);
+    else
+      __builtin_nontemporal_store(__builtin_nontemporal_load(pv + v), cv + cidx);
+  });
 }
 
 // Range-granular copy driven by three int64 device arrays (the reference's
@@ -297,53 +321,55 @@ __global__ __launch_bounds__(kThreads) void convert_ranges_kernel(
 // strides count bytes of the bf16 cache, so element e of a contiguous piece is read at byte
 // 2e. One workgroup converts 4096 elements (8 KiB in, 4 KiB out), 16 per lane. Strided
 // chunks (shape != 0) are 16-byte aligned on both sides by construction.
+template <bool CAPPED>
 __global__ __launch_bounds__(kThreads) void convert_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs, StrideTable shapes) {
-  const uint32_t b = xcd_remap(blockIdx.x, n_slices);
-  if (b >= n_slices) return;
-  const Chunk c = chunks[b >> sub_shift];
-  const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-  if (off >= c.len) return;
-  const uint32_t len = min(kSlice, c.len - off);
-  const uint32_t layer = blockIdx.y;
-  const uint8_t* cache =
-      layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
-  uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-  const u32x4* sv;
-  if (c.shape == 0) {
-    const uint8_t* s8 = cache + 2ull * off;
-    if (((reinterpret_cast<uintptr_t>(s8) | reinterpret_cast<uintptr_t>(pk)) & 15u) != 0) {
-      const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s8);
-      for (uint32_t j = threadIdx.x; j < len; j += kThreads)
-        pk[j] = static_cast<uint8_t>(bf16_to_e4m3(s16[j]));
-      return;
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes) {
+  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
+    if (b >= n_slices) return;
+    const Chunk c = chunks[b >> sub_shift];
+    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
+    if (off >= c.len) return;
+    const uint32_t len = min(kSlice, c.len - off);
+    const uint8_t* cache =
+        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
+    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
+    const u32x4* sv;
+    if (c.shape == 0) {
+      const uint8_t* s8 = cache + 2ull * off;
+      if (((reinterpret_cast<uintptr_t>(s8) | reinterpret_cast<uintptr_t>(pk)) & 15u) != 0) {
+        const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s8);
+        for (uint32_t j = threadIdx.x; j < len; j += kThreads)
+          pk[j] = static_cast<uint8_t>(bf16_to_e4m3(s16[j]));
+        return;
+      }
+      const uint32_t done = (len >> 4) << 4;
+      if (threadIdx.x < len - done)
+        pk[done + threadIdx.x] = static_cast<uint8_t>(
+            bf16_to_e4m3(reinterpret_cast<const uint16_t*>(s8)[done + threadIdx.x]));
+      if (threadIdx.x >= (len >> 4)) return;
+      sv = reinterpret_cast<const u32x4*>(s8) + 2 * threadIdx.x;
+    } else {
+      if (threadIdx.x >= (len >> 4)) return;
+      const StrideShape& s = shapes.shape[c.shape - 1u];
+      const uint32_t v = (off >> 4) + threadIdx.x;  // output vector index inside the chunk
+      const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
+      const uint32_t col = v - rec * s.vlen;
+      const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
+      const uint32_t i = rec - o * s.n_inner;
+      sv = reinterpret_cast<const u32x4*>(cache + o * s.outer[0] + i * s.inner[0] + (col << 5));
     }
-    const uint32_t done = (len >> 4) << 4;
-    if (threadIdx.x < len - done)
-      pk[done + threadIdx.x] = static_cast<uint8_t>(
-          bf16_to_e4m3(reinterpret_cast<const uint16_t*>(s8)[done + threadIdx.x]));
-    if (threadIdx.x >= (len >> 4)) return;
-    sv = reinterpret_cast<const u32x4*>(s8) + 2 * threadIdx.x;
-  } else {
-    if (threadIdx.x >= (len >> 4)) return;
-    const StrideShape& s = shapes.shape[c.shape - 1u];
-    const uint32_t v = (off >> 4) + threadIdx.x;  // output vector index inside the chunk
-    const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
-    const uint32_t col = v - rec * s.vlen;
-    const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
-    const uint32_t i = rec - o * s.n_inner;
-    sv = reinterpret_cast<const u32x4*>(cache + o * s.outer[0] + i * s.inner[0] + (col << 5));
-  }
-  const u32x4 lo = __builtin_nontemporal_load(sv);
-  const u32x4 hi = __builtin_nontemporal_load(sv + 1);
-  u32x4 r;
-  r.x = cvt4(lo.x, lo.y);
-  r.y = cvt4(lo.z, lo.w);
-  r.z = cvt4(hi.x, hi.y);
-  r.w = cvt4(hi.z, hi.w);
-  __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(pk) + threadIdx.x);
+    const u32x4 lo = __builtin_nontemporal_load(sv);
+    const u32x4 hi = __builtin_nontemporal_load(sv + 1);
+    u32x4 r;
+    r.x = cvt4(lo.x, lo.y);
+    r.y = cvt4(lo.z, lo.w);
+    r.z = cvt4(hi.x, hi.y);
+    r.w = cvt4(hi.z, hi.w);
+    __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(pk) + threadIdx.x);
+  });
 }
 
 // Plain linear copy with the gather kernel's slice shape (calibration / ceiling).
@@ -361,21 +387,38 @@ __global__ __launch_bounds__(kThreads) void copy_linear_kernel(uint8_t* __restri
 
 static uint32_t round8(uint32_t n) { return (n + 7u) & ~7u; }
 
+// Grid of a chunk launch: one workgroup per (slice, layer); or, when the caller limits the
+// launch to max_wgs workgroups and there are more items than that, max_wgs workgroups
+// (rounded down to a multiple of 8, at least 8) that stride over the items.
+struct ChunkGrid {
+  dim3 grid;
+  bool capped;
+};
+static ChunkGrid chunk_grid(uint32_t n_slices, uint32_t n_layers, uint32_t max_wgs) {
+  const uint32_t per_layer = round8(n_slices);
+  const uint32_t cap = max_wgs < 8u ? 8u : (max_wgs & ~7u);
+  if (max_wgs == 0 || static_cast<uint64_t>(per_layer) * n_layers <= cap)
+    return ChunkGrid{dim3(per_layer, n_layers), false};
+  return ChunkGrid{dim3(cap), true};
+}
+
+#define KVT_LAUNCH_CHUNKS(KERNEL, ...)                                                          \
+  hipLaunchKernelGGL(KERNEL, g.grid, dim3(kThreads), 0, stream, __VA_ARGS__)
+
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, const BlobOffsets& blobs, hipStream_t stream) {
+                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs,
+                              hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
-  const dim3 grid(round8(n_slices), n_layers);
-  if (pack)
-    hipLaunchKernelGGL((copy_chunks_kernel<true>), grid, dim3(kThreads), 0, stream, chunks,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs);
-  else
-    hipLaunchKernelGGL((copy_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs);
+  const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+  if (pack && !g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, false>), KVT_ARGS);
+  else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, true>), KVT_ARGS);
+  else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, false>), KVT_ARGS);
+  else KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, true>), KVT_ARGS);
+#undef KVT_ARGS
   return hipGetLastError();
 }
 
@@ -383,18 +426,17 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
-                                    const BlobOffsets& blobs, hipStream_t stream) {
+                                    const BlobOffsets& blobs, uint32_t max_wgs,
+                                    hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
-  const dim3 grid(round8(n_slices), n_layers);
-  if (pack)
-    hipLaunchKernelGGL((copy_chunks_small_kernel<true>), grid, dim3(kThreads), 0, stream, table,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs);
-  else
-    hipLaunchKernelGGL((copy_chunks_small_kernel<false>), grid, dim3(kThreads), 0, stream, table,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs);
+  const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+#define KVT_ARGS table, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+  if (pack && !g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, false>), KVT_ARGS);
+  else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, true>), KVT_ARGS);
+  else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, false>), KVT_ARGS);
+  else KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, true>), KVT_ARGS);
+#undef KVT_ARGS
   return hipGetLastError();
 }
 
@@ -402,19 +444,23 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, bool words, hipStream_t stream) {
+                                 const StrideTable& shapes, bool words, uint32_t max_wgs,
+                                 hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
-  const dim3 grid(round8(n_slices), n_layers);
-#define KVT_LAUNCH_STRIDED(P, W)                                                                \
-  hipLaunchKernelGGL((strided_chunks_kernel<P, W>), grid, dim3(kThreads), 0, stream, chunks,   \
-                     n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,           \
-                     layer_stride, blobs, shapes)
-  if (pack && !words) KVT_LAUNCH_STRIDED(true, false);
-  else if (pack) KVT_LAUNCH_STRIDED(true, true);
-  else if (!words) KVT_LAUNCH_STRIDED(false, false);
-  else KVT_LAUNCH_STRIDED(false, true);
-#undef KVT_LAUNCH_STRIDED
+  const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+#define KVT_STRIDED(P, W)                                                                       \
+  do {                                                                                          \
+    if (g.capped) KVT_LAUNCH_CHUNKS((strided_chunks_kernel<P, W, true>), KVT_ARGS);             \
+    else KVT_LAUNCH_CHUNKS((strided_chunks_kernel<P, W, false>), KVT_ARGS);                     \
+  } while (0)
+  if (pack && !words) KVT_STRIDED(true, false);
+  else if (pack) KVT_STRIDED(true, true);
+  else if (!words) KVT_STRIDED(false, false);
+  else KVT_STRIDED(false, true);
+#undef KVT_STRIDED
+#undef KVT_ARGS
   return hipGetLastError();
 }
 
@@ -422,12 +468,15 @@ hipError_t launch_convert_chunks(const Chunk* chunks, uint32_t n_chunks, uint32_
                                  uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                  uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                  uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, hipStream_t stream) {
+                                 const StrideTable& shapes, uint32_t max_wgs,
+                                 hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
-  hipLaunchKernelGGL(convert_chunks_kernel, dim3(round8(n_slices), n_layers), dim3(kThreads), 0,
-                     stream, chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer,
-                     packed, layer_stride, blobs, shapes);
+  const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+  if (g.capped) KVT_LAUNCH_CHUNKS((convert_chunks_kernel<true>), KVT_ARGS);
+  else KVT_LAUNCH_CHUNKS((convert_chunks_kernel<false>), KVT_ARGS);
+#undef KVT_ARGS
   return hipGetLastError();
 }
 
@@ -435,41 +484,49 @@ hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               hipStream_t stream) {
+                               uint32_t max_wgs, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
-  const dim3 grid(round8(n_slices), n_layers);
-  if (pack)
-    hipLaunchKernelGGL((xform_chunks_kernel<true>), grid, dim3(kThreads), 0, stream, chunks,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs, x);
-  else
-    hipLaunchKernelGGL((xform_chunks_kernel<false>), grid, dim3(kThreads), 0, stream, chunks,
-                       n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, packed,
-                       layer_stride, blobs, x);
+  const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x
+  if (pack && !g.capped) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, false>), KVT_ARGS);
+  else if (pack) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, true>), KVT_ARGS);
+  else if (!g.capped) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<false, false>), KVT_ARGS);
+  else KVT_LAUNCH_CHUNKS((xform_chunks_kernel<false, true>), KVT_ARGS);
+#undef KVT_ARGS
   return hipGetLastError();
 }
+#undef KVT_LAUNCH_CHUNKS
 
-// grid.y is limited to 65535; the kernels stride over the ranges anyway
-static uint32_t range_wgs(int num_wg) { return num_wg < 65535 ? (num_wg < 1 ? 1 : num_wg) : 65535; }
+// grid.y is limited to 65535; the kernels stride over the ranges anyway. max_wgs > 0 limits
+// the whole grid (rows x ranges) to that many workgroups.
+static dim3 range_grid(int num_wg, int rows, uint32_t max_wgs) {
+  uint32_t gx = rows < 1 ? 1u : static_cast<uint32_t>(rows);
+  uint32_t gy = num_wg < 65535 ? (num_wg < 1 ? 1u : static_cast<uint32_t>(num_wg)) : 65535u;
+  if (max_wgs) {
+    if (gx > max_wgs) gx = max_wgs;
+    if (gy > max_wgs / gx) gy = max_wgs / gx;
+  }
+  return dim3(gx, gy);
+}
 
 hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                               const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,
-                              int rows, hipStream_t stream) {
+                              int rows, uint32_t max_wgs, hipStream_t stream) {
   if (n <= 0) return hipSuccess;
-  hipLaunchKernelGGL(copy_ranges_kernel, dim3(rows, range_wgs(num_wg)), dim3(kThreads), 0, stream,
-                     static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base),
-                     src_off, dst_off, lens, n);
+  hipLaunchKernelGGL(copy_ranges_kernel, range_grid(num_wg, rows, max_wgs), dim3(kThreads), 0,
+                     stream, static_cast<const uint8_t*>(src_base),
+                     static_cast<uint8_t*>(dst_base), src_off, dst_off, lens, n);
   return hipGetLastError();
 }
 
 hipError_t launch_convert_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                                  const int64_t* dst_off, const int64_t* lens, int64_t n,
-                                 int num_wg, int rows, hipStream_t stream) {
+                                 int num_wg, int rows, uint32_t max_wgs, hipStream_t stream) {
   if (n <= 0) return hipSuccess;
-  hipLaunchKernelGGL(convert_ranges_kernel, dim3(rows, range_wgs(num_wg)), dim3(kThreads), 0, stream,
-                     static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base),
-                     src_off, dst_off, lens, n);
+  hipLaunchKernelGGL(convert_ranges_kernel, range_grid(num_wg, rows, max_wgs), dim3(kThreads), 0,
+                     stream, static_cast<const uint8_t*>(src_base),
+                     static_cast<uint8_t*>(dst_base), src_off, dst_off, lens, n);
   return hipGetLastError();
 }
 

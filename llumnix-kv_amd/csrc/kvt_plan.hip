@@ -555,11 +555,12 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
                                                         : "kvt_unpack: the packed buffer"))
       return rc;
   }
+  const uint32_t max_wgs = copy_wg_cap(cache->device);
   if (p->small) {
     const hipError_t e = launch_copy_chunks_small(
         pack, pack ? p->small_pack : p->small_unpack, static_cast<uint32_t>(p->n_chunks),
         p->sub_shift, cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
-        static_cast<uint8_t*>(packed), layer_stride, blobs, s);
+        static_cast<uint8_t*>(packed), layer_stride, blobs, max_wgs, s);
     if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
     return KVT_OK;
   }
@@ -583,17 +584,17 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       p->convert && pack ? launch_convert_chunks(table, n, p->sub_shift, cache->dev_ptrs,
                                                  p->n_tensors, first_layer, n_layers,
                                                  static_cast<uint8_t*>(packed), layer_stride,
-                                                 blobs, p->shapes, s) :
+                                                 blobs, p->shapes, max_wgs, s) :
       p->strided ? launch_strided_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                          p->n_tensors, first_layer, n_layers,
                                          static_cast<uint8_t*>(packed), layer_stride, blobs,
-                                         p->shapes, words, s) :
+                                         p->shapes, words, max_wgs, s) :
       p->xform ? launch_xform_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                      first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                     layer_stride, blobs, p->xdev, s)
+                                     layer_stride, blobs, p->xdev, max_wgs, s)
                : launch_copy_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                     first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                    layer_stride, blobs, s);
+                                    layer_stride, blobs, max_wgs, s);
   if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
   if (p->buf) {
     // remember when the table is last read, so that its storage is not recycled too early

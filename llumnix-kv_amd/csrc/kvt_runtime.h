@@ -30,6 +30,10 @@ int usable_devices();
 // KVT_OK, or KVT_ERR_NO_DEVICE / KVT_ERR_INVALID with the message set.
 int check_device(int device);
 
+// The most workgroups one copy launch may use on `device`, or 0 for no limit
+// (kvt_set_copy_cu_usage).
+uint32_t copy_wg_cap(int device);
+
 // KVT_OK when [ptr, ptr + bytes) is, as far as the runtime can tell, memory the device may
 // touch; KVT_ERR_INVALID / KVT_ERR_OUT_OF_RANGE (message set, starting with `what`) otherwise.
 int check_device_span(const void* ptr, uint64_t bytes, const std::string& what);

@@ -1,6 +1,7 @@
 // Device selection, the chunk-table pool, cache registration and the small
 // event / stream utilities of the C ABI.
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <memory>
 
@@ -39,6 +40,19 @@ int check_device(int device) {
   if (n <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
   if (device < 0 || device >= n) return fail(KVT_ERR_INVALID, "device index out of range");
   return KVT_OK;
+}
+
+// Share of the device a copy launch may occupy. A 256-lane workgroup is four wavefronts and
+// a CU holds 32, so usage x CUs x 8 workgroups are resident at once on that share; a launch
+// capped to that many (persistent, striding over the work) leaves the rest of the CUs to
+// whatever else runs. Stored as the cap itself; 0 = one workgroup per slice, no limit.
+constexpr int kMaxDevices = 64;
+constexpr uint32_t kWgsPerCu = 8;
+static std::atomic<uint32_t> g_wg_cap[kMaxDevices];
+static std::atomic<uint32_t> g_usage_millionths[kMaxDevices];
+
+uint32_t copy_wg_cap(int device) {
+  return device >= 0 && device < kMaxDevices ? g_wg_cap[device].load(std::memory_order_relaxed) : 0;
 }
 
 // A kernel that runs past a buffer takes a GPU memory fault, which can cost the whole
@@ -100,6 +114,34 @@ using namespace kvt;
 extern "C" {
 
 int kvt_device_count(void) { return std::max(0, usable_devices()); }
+
+int kvt_set_copy_cu_usage(int device, double usage) {
+  return guarded([&]() -> int {
+    if (int rc = check_device(device)) return rc;
+    if (device >= kMaxDevices) return fail(KVT_ERR_INVALID, "kvt_set_copy_cu_usage: device index too large");
+    if (!(usage > 0.0 && usage <= 1.0))
+      return fail(KVT_ERR_INVALID, "kvt_set_copy_cu_usage: usage must be in (0, 1]");
+    uint32_t cap = 0;
+    if (usage < 1.0) {
+      int cus = 0;
+      KVT_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+      const double wgs = usage * static_cast<double>(cus) * kWgsPerCu;
+      cap = std::max<uint32_t>(8u, static_cast<uint32_t>(wgs) & ~7u);
+    }
+    g_usage_millionths[device].store(static_cast<uint32_t>(usage * 1e6 + 0.5), std::memory_order_relaxed);
+    g_wg_cap[device].store(cap, std::memory_order_relaxed);
+    return KVT_OK;
+  });
+}
+
+int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups) {
+  if (int rc = check_device(device)) return rc;
+  if (device >= kMaxDevices) return fail(KVT_ERR_INVALID, "kvt_get_copy_cu_usage: device index too large");
+  const uint32_t m = g_usage_millionths[device].load(std::memory_order_relaxed);
+  if (usage) *usage = m == 0 ? 1.0 : m / 1e6;
+  if (max_workgroups) *max_workgroups = g_wg_cap[device].load(std::memory_order_relaxed);
+  return KVT_OK;
+}
 
 // ------------------------------------------------------------------- cache
 

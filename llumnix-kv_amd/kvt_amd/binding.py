@@ -89,6 +89,8 @@ SIGNATURES = {
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_initialize_copy_method_profile": (_int, [_int]),
+    "kvt_set_copy_cu_usage": (_int, [_int, C.c_double]),
+    "kvt_get_copy_cu_usage": (_int, [_int, _P(C.c_double), _P(_u32)]),
     "kvt_get_kernel_copy_buffer": (_int, [_int, _i64, _P(_vp), _P(_vp)]),
     "kvt_get_thread_local_stream": (_int, [_int, _int, _P(_vp)]),
     "kvt_copy_handle_data_with_kernel": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp, _vp,
@@ -185,6 +187,19 @@ def check(rc):
 
 def device_count():
     return lib().kvt_device_count()
+
+
+def set_copy_cu_usage(device, usage):
+    """Share of the device's CUs that copy launches may occupy (the reference's
+    BLLM_KVTRANS_KERNEL_COPY_SM_USAGE, kvtransfer/src/envcfg.cpp:311-326); 1.0 = no limit."""
+    check(lib().kvt_set_copy_cu_usage(device, float(usage)))
+
+
+def get_copy_cu_usage(device):
+    """-> (usage, workgroup limit; 0 = none)"""
+    u, m = C.c_double(), _u32()
+    check(lib().kvt_get_copy_cu_usage(device, C.byref(u), C.byref(m)))
+    return u.value, m.value
 
 
 def compute_valid_ranks_pd(p_tp, d_tp, heads):

@@ -1,0 +1,94 @@
+"""The CU-share limit of copy launches (kvt_set_copy_cu_usage, the reference's
+BLLM_KVTRANS_KERNEL_COPY_SM_USAGE, kvtransfer/src/envcfg.cpp:311-326 and
+copy_kernels.cpp:327-335): with a share below 1 every kernel runs as a bounded
+number of persistent workgroups striding over the same work, so every result
+must be bit for bit what the unlimited launch gives. The parity tests of the
+other GPU test files are run again under two limits: half the device, and the
+smallest grid the library will use (8 workgroups on a 256-CU part at 0.004).
+Needs a real MI355X."""
+import ctypes as C
+import math
+
+import pytest
+
+import kvt_amd
+import test_gpu_pack as tp
+import test_gpu_runs as tr
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(params=[0.5, 0.004], ids=["half", "eight-workgroups"])
+def limited(request):
+    kvt_amd.set_copy_cu_usage(0, request.param)
+    try:
+        yield request.param
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+
+
+def test_setting_and_reading_the_share():
+    lib = kvt_amd.lib()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    try:
+        assert kvt_amd.get_copy_cu_usage(0) == (1.0, 0)
+        kvt_amd.set_copy_cu_usage(0, 0.25)
+        usage, limit = kvt_amd.get_copy_cu_usage(0)
+        assert usage == 0.25 and limit == (int(0.25 * cus * 8) & ~7) and limit % 8 == 0
+        kvt_amd.set_copy_cu_usage(0, 1e-6)
+        assert kvt_amd.get_copy_cu_usage(0)[1] == 8
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+        assert kvt_amd.get_copy_cu_usage(0) == (1.0, 0)
+        for bad in (0.0, -0.5, 1.5, math.nan, math.inf):
+            assert lib.kvt_set_copy_cu_usage(0, bad) != 0, bad
+            assert b"usage" in lib.kvt_last_error()
+        assert lib.kvt_set_copy_cu_usage(99, 0.5) != 0
+        assert lib.kvt_get_copy_cu_usage(99, None, None) != 0
+        assert lib.kvt_get_copy_cu_usage(0, None, None) == 0
+        assert kvt_amd.get_copy_cu_usage(0) == (1.0, 0)      # refused values change nothing
+    finally:
+        assert lib.kvt_set_copy_cu_usage(0, C.c_double(1.0)) == 0
+
+
+def test_plain_plans_under_a_limit(limited):
+    tp.test_config2_shape_reduced_pool(0)
+    tp.test_config2_shape_reduced_pool(65536)
+    tp.test_config4_mla_and_indexer_two_tensors()
+    tp.test_config5_reference_layout_uniform_pages_shared_by_attention_and_gdn()
+    tp.test_chunked_prefill_steps_and_ragged_tail()
+    tp.test_arbitrary_ranges_including_misaligned()
+
+
+def test_short_plans_in_kernel_arguments_under_a_limit(limited):
+    for n in (1, 63, 64, 65):
+        tp.test_short_plans_travel_in_the_kernel_arguments(n)
+
+
+def test_transposing_plans_under_a_limit(limited):
+    tp.test_config3_transposing_pack_hnd_to_nhd()
+    tp.test_transposing_pack_other_geometries(3, 5, 48)
+
+
+def test_strided_and_converting_plans_under_a_limit(limited):
+    tr.test_tp_split_batches_through_a_run_plan("flash", 2, 1, 1, True, 0)
+    tr.test_tp_split_batches_through_a_run_plan("ragged", 1, 4, 0, True, 4096)
+    tr.test_hybrid_model_between_tp2_prefill_and_tp1_decode(2, 1, 1)
+    tr.test_strided_plan_with_word_aligned_and_misaligned_blob_positions()
+    tr.test_converting_run_plan_bf16_sender_fp8_receiver("flash", 2, 1, 1, 0, "raw")
+    tr.test_converting_plan_of_plain_unaligned_ranges_takes_the_element_path()
+
+
+def test_reference_shaped_entry_points_under_a_limit(limited):
+    tp.test_launch_copy_direct_gather_and_scatter(5, 200000)
+    tp.test_launch_copy_direct_gather_and_scatter(5000, 700)
+    tp.test_copy_handle_data_with_kernel_pinned_host_buffer(7)
+    tp.test_copy_handle_data_kernel_direct(False)
+    tp.test_bf16_to_fp8_all_bit_patterns_and_converting_gather()
+
+
+def test_sessions_and_graphs_under_a_limit(limited):
+    tp.test_per_layer_session_on_side_stream()
+    tp.test_session_inside_hip_graph_replays()
+    tp.test_stager_save_load_round_trip_overlapped_with_packing()
