@@ -382,6 +382,17 @@ int kvt_set_copy_cu_usage(int device, double usage);
 /* The current setting and the workgroup limit it stands for (0 = none); either may be NULL. */
 int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
 
+/* replaces BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES / BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS
+ *                                               kvtransfer/src/copy_kernels.cpp:157-158, 496-499,
+ * the static part of select_copy_method()       kvtransfer/src/copy_kernels.cpp:610-617:
+ * kvt_copy_handle_data_with_kernel hands a list to the DMA engines (one copy per range) when it
+ * has at most max_ranges ranges and every range is at least min_range_bytes long. Defaults:
+ * 8 MiB and 16, measured on MI355X against pinned host memory (the reference's defaults,
+ * 256 KiB and 16, suit a part whose copy kernel is slower across PCIe than this one's).
+ * max_ranges = 0 switches the DMA route off. Process-wide. */
+int kvt_set_copy_memcpy_thresholds(uint64_t min_range_bytes, uint64_t max_ranges);
+int kvt_get_copy_memcpy_thresholds(uint64_t* min_range_bytes, uint64_t* max_ranges);
+
 enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
 /* stands in for initialize_copy_method_profile() kvtransfer/include/copy_kernels.h:15-22
  * (called once per copy thread, kvtransfer/src/copy_utils.cpp:52). There is

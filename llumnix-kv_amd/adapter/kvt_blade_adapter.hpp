@@ -22,6 +22,7 @@
 #define KVT_BLADE_ADAPTER_HPP_
 
 #include <bitset>
+#include <cstdlib>
 #include <cstring>
 #include <stdexcept>
 #include <string>
@@ -260,6 +261,25 @@ inline void* get_thread_local_d2h_stream(int device_id) {
 // where the reference initialises its copy threads.
 inline void apply_kernel_copy_sm_usage(int device_id) {
   raise(kvt_set_copy_cu_usage(device_id, blade_llm::env_kernel_copy_sm_usage()));
+}
+
+// BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES / BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS
+// (kvtransfer/src/copy_kernels.cpp:496-499), when set, replace the library's own thresholds
+// for handing a list to the DMA engines; unset or unparsable values leave them alone.
+inline void apply_copy_memcpy_env() {
+  uint64_t min_bytes = 0, max_ranges = 0;
+  raise(kvt_get_copy_memcpy_thresholds(&min_bytes, &max_ranges));
+  auto read = [](const char* name, uint64_t* out) {
+    const char* v = std::getenv(name);
+    if (v == nullptr || *v == '\0') return;
+    char* end = nullptr;
+    const unsigned long long x = std::strtoull(v, &end, 10);
+    if (end != v && *end == '\0') *out = x;
+  };
+  read("BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES", &min_bytes);
+  read("BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS", &max_ranges);
+  if (min_bytes == 0) min_bytes = 1;
+  raise(kvt_set_copy_memcpy_thresholds(min_bytes, max_ranges));
 }
 
 }  // namespace kvt_adapter

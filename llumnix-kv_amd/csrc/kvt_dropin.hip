@@ -2,6 +2,7 @@
 // three int64 device arrays, or kvt_ipc_block lists with caller-owned metadata
 // buffers.
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <vector>
 
@@ -44,7 +45,9 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
   return KVT_OK;
 }
 
+// When a list goes to the DMA engines instead of a kernel (kvt_set_copy_memcpy_thresholds).
 constexpr uint64_t kDmaMaxRanges = 16, kDmaMinBytes = 8ull << 20;
+std::atomic<uint64_t> g_dma_max_ranges{kDmaMaxRanges}, g_dma_min_bytes{kDmaMinBytes};
 
 // Workgroups per range when the lengths are known on the host: the mean number of slices
 // per range (bounded). Equal lengths then get exactly one slice per workgroup, the fastest
@@ -90,7 +93,8 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
   // (copy_kernels.cpp:495-619); here it is fixed from measurements on MI355X: against pinned
   // host memory a copy of 128 MiB runs at 57 GB/s where the kernel's stores across PCIe reach
   // 54, the kernel wins below about 8 MiB per copy (2 MiB: 53 against 33 GB/s).
-  if (!halve && n <= kDmaMaxRanges && shortest >= kDmaMinBytes) {
+  if (!halve && n <= g_dma_max_ranges.load(std::memory_order_relaxed) &&
+      shortest >= g_dma_min_bytes.load(std::memory_order_relaxed)) {
     uint64_t cursor = 0;
     for (uint64_t i = 0; i < n; ++i) {
       uint8_t* host = static_cast<uint8_t*>(tensor_buf) + cursor;
@@ -303,6 +307,20 @@ int kvt_get_thread_local_stream(int device, int direction, void** stream) {
     *stream = c.streams[direction];
     return KVT_OK;
   });
+}
+
+int kvt_set_copy_memcpy_thresholds(uint64_t min_range_bytes, uint64_t max_ranges) {
+  if (min_range_bytes == 0)
+    return fail(KVT_ERR_INVALID, "kvt_set_copy_memcpy_thresholds: min_range_bytes must be positive");
+  g_dma_min_bytes.store(min_range_bytes, std::memory_order_relaxed);
+  g_dma_max_ranges.store(max_ranges, std::memory_order_relaxed);
+  return KVT_OK;
+}
+
+int kvt_get_copy_memcpy_thresholds(uint64_t* min_range_bytes, uint64_t* max_ranges) {
+  if (min_range_bytes) *min_range_bytes = g_dma_min_bytes.load(std::memory_order_relaxed);
+  if (max_ranges) *max_ranges = g_dma_max_ranges.load(std::memory_order_relaxed);
+  return KVT_OK;
 }
 
 int kvt_initialize_copy_method_profile(int device) {

@@ -89,6 +89,8 @@ SIGNATURES = {
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_initialize_copy_method_profile": (_int, [_int]),
+    "kvt_set_copy_memcpy_thresholds": (_int, [_u64, _u64]),
+    "kvt_get_copy_memcpy_thresholds": (_int, [_P(_u64), _P(_u64)]),
     "kvt_set_copy_cu_usage": (_int, [_int, C.c_double]),
     "kvt_get_copy_cu_usage": (_int, [_int, _P(C.c_double), _P(_u32)]),
     "kvt_get_kernel_copy_buffer": (_int, [_int, _i64, _P(_vp), _P(_vp)]),

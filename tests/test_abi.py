@@ -71,3 +71,22 @@ def test_gpu_entry_points_fail_loudly_without_a_device():
         kvt_amd.Stager(0, 4096, 2)
     assert e.value.code == 6
     assert kvt_amd.lib().kvt_copy_linear(1, 1, 16, None) == 6
+    assert kvt_amd.lib().kvt_set_copy_cu_usage(0, 0.5) == 6
+
+
+def test_memcpy_route_thresholds_are_process_wide_settings():
+    import ctypes as C
+    lib = kvt_amd.lib()
+    a, b = C.c_uint64(), C.c_uint64()
+    assert lib.kvt_get_copy_memcpy_thresholds(C.byref(a), C.byref(b)) == 0
+    assert (a.value, b.value) == (8 << 20, 16)
+    try:
+        assert lib.kvt_set_copy_memcpy_thresholds(256 << 10, 4) == 0
+        assert lib.kvt_get_copy_memcpy_thresholds(C.byref(a), None) == 0 and a.value == 256 << 10
+        assert lib.kvt_get_copy_memcpy_thresholds(None, C.byref(b)) == 0 and b.value == 4
+        assert lib.kvt_set_copy_memcpy_thresholds(0, 4) != 0          # every range would qualify
+        assert lib.kvt_get_copy_memcpy_thresholds(C.byref(a), C.byref(b)) == 0
+        assert (a.value, b.value) == (256 << 10, 4)
+        assert lib.kvt_set_copy_memcpy_thresholds(1, 0) == 0          # route switched off
+    finally:
+        assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0

@@ -416,6 +416,48 @@ def test_copy_handle_data_hands_a_few_very_large_ranges_to_the_dma_engines():
     assert (host_meta == 0).all()           # the kernel's metadata buffers were not needed
 
 
+def test_memcpy_route_thresholds_decide_between_dma_and_kernel():
+    """BLLM_KVTRANS_COPY_MEMCPY_{BLOCK_THRESHOLD_BYTES,MAX_BLOCKS} of the reference
+    (copy_kernels.cpp:496-499, 610-617) as kvt_set_copy_memcpy_thresholds: the same three ranges
+    of 1 MiB go through the kernel by default, to the DMA engines once the thresholds admit them,
+    and through the kernel again when the route is switched off; the bytes never differ."""
+    lib = kvt_amd.lib()
+    cap = 16 << 20
+    runs = np.array([[0, (1 << 20) + 32, 1 << 20], [0, 5 << 20, (1 << 20) + 5],
+                     [0, (9 << 20) + 1, 1 << 20]], dtype=np.uint64)
+    total = int(runs[:, 2].sum())
+    layer = _dev_bytes(cap, 77, "raw")
+    gather = np.stack([runs[:, 1], runs[:, 1], runs[:, 2]], axis=1)
+    blob = checkers.oracle_pack(_host(layer), gather)
+    dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
+    s = torch.cuda.Stream()
+
+    def gather_once():
+        pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
+        host_meta = torch.zeros(3 * 8192, dtype=torch.int64).pin_memory()
+        rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(),
+                                                  runs.ctypes.data, len(runs), total, 1, 0,
+                                                  s.cuda_stream, dev_meta.data_ptr(),
+                                                  host_meta.data_ptr(), 0)
+        assert rc == 0, lib.kvt_last_error()
+        s.synchronize()
+        assert np.array_equal(pinned.numpy(), blob)
+        return bool((host_meta != 0).any())      # True: the kernel's metadata buffers were used
+
+    try:
+        assert gather_once() is True
+        assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 3) == 0
+        assert gather_once() is False
+        assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 2) == 0    # one range too many
+        assert gather_once() is True
+        assert lib.kvt_set_copy_memcpy_thresholds((1 << 20) + 1, 3) == 0   # two ranges too short
+        assert gather_once() is True
+        assert lib.kvt_set_copy_memcpy_thresholds(1, 0) == 0          # switched off
+        assert gather_once() is True
+    finally:
+        assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+
+
 def test_copy_threads_get_their_own_metadata_buffers_and_streams():
     """get_kernel_copy_buffer / get_thread_local_{h2d,d2h}_stream of the reference's copy
     threads (copy_utils.cpp:9-154): per thread, created on first use, used for a real copy."""
