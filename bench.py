@@ -28,8 +28,8 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 # file (each counter scaled by what it reads for the plain copy kernel of known size); see
 # profiles/copy_chunks_kernel_config2_hbm_traffic.md and
 # profiles/strided_and_xform_kernels_hbm_traffic.md. Keyed by (config, scale, chunk_bytes, plan).
-MEASURED_PACK_TRAFFIC = {(2, 1.0, 0, "ranges"): 70.966e9, (3, 1.0, 0, "ranges"): 85.892e9,
-                         (6, 1.0, 0, "runs"): 40.879e9}
+MEASURED_PACK_TRAFFIC = {(2, 1.0, 0, "ranges"): 70.956e9, (3, 1.0, 0, "ranges"): 85.878e9,
+                         (6, 1.0, 0, "runs"): 40.872e9}
 
 
 def log(*a):
