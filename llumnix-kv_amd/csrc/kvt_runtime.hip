@@ -49,7 +49,7 @@ int check_device(int device) {
 constexpr int kMaxDevices = 64;
 constexpr uint32_t kWgsPerCu = 8;
 static std::atomic<uint32_t> g_wg_cap[kMaxDevices];
-static std::atomic<uint32_t> g_usage_millionths[kMaxDevices];
+static std::atomic<uint64_t> g_usage_bits[kMaxDevices];   // the double as given; 0 = never set
 
 uint32_t copy_wg_cap(int device) {
   return device >= 0 && device < kMaxDevices ? g_wg_cap[device].load(std::memory_order_relaxed) : 0;
@@ -128,7 +128,9 @@ int kvt_set_copy_cu_usage(int device, double usage) {
       const double wgs = usage * static_cast<double>(cus) * kWgsPerCu;
       cap = std::max<uint32_t>(8u, static_cast<uint32_t>(wgs) & ~7u);
     }
-    g_usage_millionths[device].store(static_cast<uint32_t>(usage * 1e6 + 0.5), std::memory_order_relaxed);
+    uint64_t bits = 0;
+    std::memcpy(&bits, &usage, sizeof(bits));
+    g_usage_bits[device].store(bits, std::memory_order_relaxed);
     g_wg_cap[device].store(cap, std::memory_order_relaxed);
     return KVT_OK;
   });
@@ -137,8 +139,11 @@ int kvt_set_copy_cu_usage(int device, double usage) {
 int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups) {
   if (int rc = check_device(device)) return rc;
   if (device >= kMaxDevices) return fail(KVT_ERR_INVALID, "kvt_get_copy_cu_usage: device index too large");
-  const uint32_t m = g_usage_millionths[device].load(std::memory_order_relaxed);
-  if (usage) *usage = m == 0 ? 1.0 : m / 1e6;
+  const uint64_t bits = g_usage_bits[device].load(std::memory_order_relaxed);
+  if (usage) {
+    *usage = 1.0;
+    if (bits != 0) std::memcpy(usage, &bits, sizeof(bits));
+  }
   if (max_workgroups) *max_workgroups = g_wg_cap[device].load(std::memory_order_relaxed);
   return KVT_OK;
 }

@@ -37,6 +37,8 @@ def test_setting_and_reading_the_share():
         kvt_amd.set_copy_cu_usage(0, 0.25)
         usage, limit = kvt_amd.get_copy_cu_usage(0)
         assert usage == 0.25 and limit == (int(0.25 * cus * 8) & ~7) and limit % 8 == 0
+        kvt_amd.set_copy_cu_usage(0, 1 / 3)
+        assert kvt_amd.get_copy_cu_usage(0) == (1 / 3, int(cus * 8 / 3) & ~7)
         kvt_amd.set_copy_cu_usage(0, 1e-6)
         assert kvt_amd.get_copy_cu_usage(0)[1] == 8
         kvt_amd.set_copy_cu_usage(0, 1.0)
