@@ -617,6 +617,50 @@ def leg_store_objects(c, out):
     res["save_note"] = "%d transfers of %d layer(s) x %d objects" % (n_groups, group, len(ids))
     stg.close()
     plan.close()
+    # the same objects (one per block, all layers) through the pinned ring keyed by block hash:
+    # batches of 256 blocks, of which every fourth is stored already; then loaded back by hash
+    nb = min(1024, len(ids))
+    entry = ob * L
+    ring = kvt.ObjectRing(0, entry, nb, 16)
+    keys = [int(b).to_bytes(8, "little") + b"blockkey" for b in ids[:nb]]
+    pre = list(range(0, nb, 4))
+    e_pre, _ = ring.reserve([keys[i] for i in pre])
+    ring.commit(e_pre)
+    objs = torch.empty(256 * entry, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    t_a = time.perf_counter()
+    saved = 0
+    for first_blk in range(0, nb, 256):
+        batch = list(range(first_blk, min(nb, first_blk + 256)))
+        e, new = ring.reserve([keys[i] for i in batch])
+        todo = [i for i, n in zip(batch, new) if n]
+        lst, _ = kvt.block_object_lists(w.cache_shape, s_info, d_info, [ids[i] for i in todo],
+                                        [dst_ids[i] for i in todo])
+        pl = kvt.Plan(0, lst, w.capacities("src"), w.capacities("dst"), objects=(ob, entry))
+        pl.pack(side.src_cache, 0, L, objs, ob, ps.cuda_stream)
+        ring.save(e[new], objs.data_ptr(), entry, ps.cuda_stream)
+        c.keep.append(pl)
+        saved += len(todo)
+    ps.synchronize()
+    t_b = time.perf_counter()
+    e, found = ring.lookup(keys)
+    back = torch.empty(256 * entry, dtype=torch.uint8, device="cuda")
+    hits = e[found]
+    torch.cuda.synchronize()
+    t_c = time.perf_counter()
+    for first_blk in range(0, len(hits), 256):
+        part = hits[first_blk:first_blk + 256]
+        ring.load(part, back.data_ptr(), entry, ps.cuda_stream)
+    ps.synchronize()
+    t_d = time.perf_counter()
+    res["hash_ring"] = {"entries": nb, "entry_bytes": entry, "blocks_saved": saved,
+                        "blocks_skipped_as_stored": nb - saved,
+                        "save_gbps": round(saved * entry / (t_b - t_a) / 1e9, 2),
+                        "load_gbps": round(len(hits) * entry / (t_d - t_c) / 1e9, 2),
+                        "note": "batches of 256 blocks: reserve by hash, pack the missing blocks "
+                                "(all layers per object), DMA into the ring; load: DMA out of the "
+                                "entries found by hash"}
+    ring.close()
     out["kvstore_objects"] = res
 
 

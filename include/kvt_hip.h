@@ -523,6 +523,52 @@ int kvt_stager_wait(kvt_stager* s, uint32_t slot);
 int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats,
                      double* bytes_per_s);
 
+/* ---------------------------------------- store objects found by block hash */
+
+/* A ring of store objects in pinned host memory, found by key (the block hash): the staging
+ * tier between the paged cache and a KV store. Mirrors what FileBackend does with a block
+ *                                  blade_kvt/hybrid_connector/file_backend.py:215-285
+ * (a block whose hash is stored already is skipped on save, _blk_ready(); a load finds the
+ * block by its hash), with one entry per block holding that block of ALL layers, i.e. one
+ * object of kvt_plan_create_objects with object_stride = entry_bytes. Entries are handed out in
+ * ring order, so the new blocks of a batch are neighbours and cross PCIe as one or two large
+ * DMA copies; when the ring is full the oldest entries are given to new keys.
+ * device = KVT_DEVICE_NONE gives an index over plain host memory (no save / load), for a store
+ * that fills the entries itself. Keys are key_bytes (1..256) each, compared byte for byte.
+ * Calls may come from several threads. */
+typedef struct kvt_object_ring kvt_object_ring;
+int kvt_object_ring_create(int device, uint64_t entry_bytes, uint32_t n_entries,
+                           uint32_t key_bytes, kvt_object_ring** out);
+void kvt_object_ring_destroy(kvt_object_ring* r);
+/* Host address of an entry (for the store behind the ring: file or network IO). */
+void* kvt_object_ring_entry(kvt_object_ring* r, uint32_t entry);
+/* Save side. For each of the n keys: entries[i] = its entry; is_new[i] = 1 when the caller has
+ * to provide the block's bytes (a fresh entry was assigned, or an earlier reservation was never
+ * written), 0 when the block is stored already or appeared earlier in this call. No entry that
+ * this call refers to is given away by it; KVT_ERR_INVALID when the batch names more distinct
+ * blocks than the ring has entries. An entry given to a new key is waited for first if a
+ * transfer still uses it. */
+int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, uint32_t* entries,
+                            uint8_t* is_new);
+/* Device -> entries: object i (entry_bytes long) at dev + i * dev_stride goes to entries[i];
+ * neighbouring entries whose objects are neighbours too (dev_stride == entry_bytes) are one
+ * copy. Ordered behind the work queued on `stream` (the pack that produces the objects);
+ * `stream` continues once the objects have left the buffer. The entries count as written from
+ * here on (kvt_object_ring_wait before the HOST reads one). */
+int kvt_object_ring_save(kvt_object_ring* r, const uint32_t* entries, uint32_t n, const void* dev,
+                         uint64_t dev_stride, void* stream);
+/* Marks entries as written that the caller filled through kvt_object_ring_entry. */
+int kvt_object_ring_commit(kvt_object_ring* r, const uint32_t* entries, uint32_t n);
+/* Load side: found[i] = 1 and entries[i] when key i is stored (written or its write queued). */
+int kvt_object_ring_lookup(kvt_object_ring* r, const void* keys, uint32_t n, uint32_t* entries,
+                           uint8_t* found);
+/* Entries -> device, the mirror of save; work queued on `stream` afterwards (the unpack) sees
+ * the objects. */
+int kvt_object_ring_load(kvt_object_ring* r, const uint32_t* entries, uint32_t n, void* dev,
+                         uint64_t dev_stride, void* stream);
+/* Host-blocking: the last save / load that touches the entry has completed. */
+int kvt_object_ring_wait(kvt_object_ring* r, uint32_t entry);
+
 /* ------------------------------------------------------------- utilities */
 
 /* Plain device-to-device copy kernel with the same vector width and launch

@@ -1,0 +1,308 @@
+// A ring of store objects in pinned host memory, found by block hash: the
+// staging tier between the paged cache on the GPU and a KV store behind it.
+// The reference's file store keeps one object per (block hash, layer), skips a
+// block whose hash is already stored and loads by hash
+// (blade_kvt/hybrid_connector/file_backend.py:215-285); here an entry holds one
+// block of all layers (what one pack launch of an object plan produces per
+// block), entries are handed out in ring order so that the new blocks of a
+// batch sit side by side and cross PCIe as one or two large DMA copies, and the
+// oldest entries make room for new ones.
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "kvt_runtime.h"
+
+using namespace kvt;
+
+namespace {
+
+// One event per save / load call, shared by the entries it touched.
+struct Transfer {
+  hipEvent_t done = nullptr;
+  ~Transfer() {
+    if (done) (void)hipEventDestroy(done);
+  }
+};
+
+struct Entry {
+  std::string key;                     // empty: never used
+  bool saved = false;                  // its bytes have been written (or the write is queued)
+  uint64_t touched = 0;                // id of the last reserve call that referred to it
+  uint64_t flagged = 0;                // id of the last reserve call that reported it as new
+  std::shared_ptr<Transfer> pending;   // last transfer that reads or writes the entry
+};
+
+}  // namespace
+
+struct kvt_object_ring {
+  int device = KVT_DEVICE_NONE;
+  uint64_t entry_bytes = 0;
+  uint32_t n_entries = 0, key_bytes = 0;
+  uint8_t* arena = nullptr;
+  hipStream_t copy = nullptr;
+  hipEvent_t fence = nullptr;
+  std::mutex mu;
+  uint64_t handed_out = 0;   // entries assigned so far; the next one is handed_out % n_entries
+  uint64_t calls = 0;
+  std::vector<Entry> entries;
+  std::unordered_map<std::string, uint32_t> index;
+};
+
+namespace {
+
+int wait_entry(Entry& e) {
+  if (e.pending) {
+    KVT_HIP(hipEventSynchronize(e.pending->done));
+    e.pending.reset();
+  }
+  return KVT_OK;
+}
+
+// Runs of entries that are neighbours in the arena and in the device buffer: one copy each.
+template <class Fn>
+int for_runs(const kvt_object_ring* r, const uint32_t* entries, uint32_t n, uint64_t dev_stride,
+             Fn fn) {
+  for (uint32_t i = 0; i < n;) {
+    uint32_t j = i + 1;
+    if (dev_stride == r->entry_bytes)
+      while (j < n && entries[j] == entries[j - 1] + 1) ++j;
+    if (int rc = fn(i, j - i)) return rc;
+    i = j;
+  }
+  return KVT_OK;
+}
+
+int check_entries(const kvt_object_ring* r, const uint32_t* entries, uint32_t n, const char* who) {
+  for (uint32_t i = 0; i < n; ++i)
+    if (entries[i] >= r->n_entries || r->entries[entries[i]].key.empty())
+      return fail(KVT_ERR_OUT_OF_RANGE, std::string(who) + ": entry index not in use");
+  return KVT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int kvt_object_ring_create(int device, uint64_t entry_bytes, uint32_t n_entries,
+                           uint32_t key_bytes, kvt_object_ring** out) {
+  return guarded([&]() -> int {
+    if (!out || entry_bytes == 0 || n_entries == 0 || key_bytes == 0 || key_bytes > 256)
+      return fail(KVT_ERR_INVALID, "kvt_object_ring_create: bad argument");
+    uint64_t total = 0;
+    if (__builtin_mul_overflow(entry_bytes, static_cast<uint64_t>(n_entries), &total))
+      return fail(KVT_ERR_OVERFLOW, "kvt_object_ring_create: ring size overflows");
+    std::unique_ptr<kvt_object_ring, void (*)(kvt_object_ring*)> r(new kvt_object_ring(),
+                                                                   kvt_object_ring_destroy);
+    r->device = device;
+    r->entry_bytes = entry_bytes;
+    r->n_entries = n_entries;
+    r->key_bytes = key_bytes;
+    r->entries.resize(n_entries);
+    if (device == KVT_DEVICE_NONE) {
+      // index only (tests, or a store that fills the entries itself and never touches a GPU)
+      r->arena = static_cast<uint8_t*>(std::malloc(total));
+      if (!r->arena) return fail(KVT_ERR_INVALID, "kvt_object_ring_create: out of memory");
+    } else {
+      if (int rc = check_device(device)) return rc;
+      DeviceGuard g;
+      if (int rc = g.enter(device)) return rc;
+      KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&r->arena), total, hipHostMallocDefault));
+      KVT_HIP(hipStreamCreateWithFlags(&r->copy, hipStreamNonBlocking));
+      KVT_HIP(hipEventCreateWithFlags(&r->fence, hipEventDisableTiming));
+    }
+    *out = r.release();
+    return KVT_OK;
+  });
+}
+
+void kvt_object_ring_destroy(kvt_object_ring* r) {
+  if (!r) return;
+  if (r->copy) {
+    (void)hipStreamSynchronize(r->copy);
+    (void)hipStreamDestroy(r->copy);
+  }
+  r->entries.clear();   // drops the transfer events
+  if (r->fence) (void)hipEventDestroy(r->fence);
+  if (r->arena) {
+    if (r->device == KVT_DEVICE_NONE)
+      std::free(r->arena);
+    else
+      (void)hipHostFree(r->arena);
+  }
+  delete r;
+}
+
+void* kvt_object_ring_entry(kvt_object_ring* r, uint32_t entry) {
+  return (r && entry < r->n_entries) ? r->arena + static_cast<uint64_t>(entry) * r->entry_bytes
+                                     : nullptr;
+}
+
+int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, uint32_t* entries,
+                            uint8_t* is_new) {
+  return guarded([&]() -> int {
+    if (!r || (n && (!keys || !entries || !is_new)))
+      return fail(KVT_ERR_INVALID, "kvt_object_ring_reserve: null argument");
+    std::lock_guard<std::mutex> lock(r->mu);
+    const uint64_t call = ++r->calls;
+    const char* k = static_cast<const char*>(keys);
+    // first the keys that are here already: their entries must survive this call
+    uint32_t fresh = 0, kept = 0;
+    std::vector<std::string> ks(n);
+    for (uint32_t i = 0; i < n; ++i) {
+      ks[i].assign(k + static_cast<size_t>(i) * r->key_bytes, r->key_bytes);
+      auto it = r->index.find(ks[i]);
+      if (it != r->index.end()) {
+        Entry& e = r->entries[it->second];
+        if (e.touched != call) ++kept;
+        e.touched = call;
+      }
+    }
+    {
+      std::unordered_map<std::string, int> seen;
+      for (uint32_t i = 0; i < n; ++i)
+        if (!r->index.count(ks[i]) && seen.emplace(ks[i], 1).second) ++fresh;
+    }
+    if (static_cast<uint64_t>(fresh) + kept > r->n_entries)
+      return fail(KVT_ERR_INVALID, "kvt_object_ring_reserve: more distinct blocks than entries");
+    for (uint32_t i = 0; i < n; ++i) {
+      auto it = r->index.find(ks[i]);
+      if (it != r->index.end()) {
+        Entry& e = r->entries[it->second];
+        entries[i] = it->second;
+        // present and written: nothing to do. Reserved before but never written: the caller
+        // is asked again, once per call (a key may be repeated inside a batch).
+        is_new[i] = (!e.saved && e.flagged != call) ? 1 : 0;
+        if (is_new[i]) e.flagged = call;
+        continue;
+      }
+      uint32_t idx = 0;
+      for (;;) {   // the oldest entry that this call does not refer to
+        idx = static_cast<uint32_t>(r->handed_out++ % r->n_entries);
+        if (r->entries[idx].touched != call) break;
+      }
+      Entry& e = r->entries[idx];
+      if (int rc = wait_entry(e)) return rc;
+      if (!e.key.empty()) r->index.erase(e.key);
+      e.key = ks[i];
+      e.saved = false;
+      e.touched = call;
+      e.flagged = call;
+      r->index.emplace(ks[i], idx);
+      entries[i] = idx;
+      is_new[i] = 1;
+    }
+    return KVT_OK;
+  });
+}
+
+int kvt_object_ring_lookup(kvt_object_ring* r, const void* keys, uint32_t n, uint32_t* entries,
+                           uint8_t* found) {
+  return guarded([&]() -> int {
+    if (!r || (n && (!keys || !entries || !found)))
+      return fail(KVT_ERR_INVALID, "kvt_object_ring_lookup: null argument");
+    std::lock_guard<std::mutex> lock(r->mu);
+    const char* k = static_cast<const char*>(keys);
+    std::string key;
+    for (uint32_t i = 0; i < n; ++i) {
+      key.assign(k + static_cast<size_t>(i) * r->key_bytes, r->key_bytes);
+      auto it = r->index.find(key);
+      found[i] = (it != r->index.end() && r->entries[it->second].saved) ? 1 : 0;
+      entries[i] = found[i] ? it->second : 0;
+    }
+    return KVT_OK;
+  });
+}
+
+int kvt_object_ring_commit(kvt_object_ring* r, const uint32_t* entries, uint32_t n) {
+  return guarded([&]() -> int {
+    if (!r || (n && !entries)) return fail(KVT_ERR_INVALID, "kvt_object_ring_commit: null argument");
+    std::lock_guard<std::mutex> lock(r->mu);
+    if (int rc = check_entries(r, entries, n, "kvt_object_ring_commit")) return rc;
+    for (uint32_t i = 0; i < n; ++i) r->entries[entries[i]].saved = true;
+    return KVT_OK;
+  });
+}
+
+int kvt_object_ring_wait(kvt_object_ring* r, uint32_t entry) {
+  return guarded([&]() -> int {
+    if (!r || entry >= r->n_entries) return fail(KVT_ERR_INVALID, "kvt_object_ring_wait: bad argument");
+    std::shared_ptr<Transfer> t;
+    {
+      std::lock_guard<std::mutex> lock(r->mu);
+      t = r->entries[entry].pending;
+    }
+    if (t) KVT_HIP(hipEventSynchronize(t->done));
+    return KVT_OK;
+  });
+}
+
+// save = true: device -> entries (and the entries count as written); false: entries -> device.
+static int transfer(kvt_object_ring* r, const uint32_t* entries, uint32_t n, void* dev,
+                    uint64_t dev_stride, void* stream, bool save) {
+  const char* who = save ? "kvt_object_ring_save" : "kvt_object_ring_load";
+  if (!r || (n && (!entries || !dev))) return fail(KVT_ERR_INVALID, std::string(who) + ": null argument");
+  if (n == 0) return KVT_OK;
+  if (r->device == KVT_DEVICE_NONE)
+    return fail(KVT_ERR_NO_DEVICE, std::string(who) + ": this ring was created without a device");
+  if (dev_stride < r->entry_bytes)
+    return fail(KVT_ERR_INVALID, std::string(who) + ": device stride smaller than an entry");
+  std::lock_guard<std::mutex> lock(r->mu);
+  if (int rc = check_entries(r, entries, n, who)) return rc;
+  if (!save)
+    for (uint32_t i = 0; i < n; ++i)
+      if (!r->entries[entries[i]].saved)
+        return fail(KVT_ERR_INVALID, "kvt_object_ring_load: entry has not been written");
+  DeviceGuard g;
+  if (int rc = g.enter(r->device)) return rc;
+  if (int rc = check_device_span(dev, static_cast<uint64_t>(n - 1) * dev_stride + r->entry_bytes,
+                                 std::string(who) + ": the device buffer"))
+    return rc;
+  const hipStream_t user = static_cast<hipStream_t>(stream);
+  // behind whatever the caller's stream has queued (the pack that produces the objects, or the
+  // kernels still reading the buffer a load is about to overwrite)
+  KVT_HIP(hipEventRecord(r->fence, user));
+  KVT_HIP(hipStreamWaitEvent(r->copy, r->fence, 0));
+  uint8_t* d = static_cast<uint8_t*>(dev);
+  if (int rc = for_runs(r, entries, n, dev_stride, [&](uint32_t first, uint32_t count) -> int {
+        uint8_t* host = r->arena + static_cast<uint64_t>(entries[first]) * r->entry_bytes;
+        uint8_t* devp = d + static_cast<uint64_t>(first) * dev_stride;
+        const uint64_t bytes = static_cast<uint64_t>(count) * r->entry_bytes;
+        if (save)
+          KVT_HIP(hipMemcpyAsync(host, devp, bytes, hipMemcpyDeviceToHost, r->copy));
+        else
+          KVT_HIP(hipMemcpyAsync(devp, host, bytes, hipMemcpyHostToDevice, r->copy));
+        return KVT_OK;
+      }))
+    return rc;
+  auto t = std::make_shared<Transfer>();
+  KVT_HIP(hipEventCreateWithFlags(&t->done, hipEventDisableTiming));
+  KVT_HIP(hipEventRecord(t->done, r->copy));
+  for (uint32_t i = 0; i < n; ++i) {
+    Entry& e = r->entries[entries[i]];
+    e.pending = t;
+    if (save) e.saved = true;
+  }
+  // the caller's stream continues once the bytes have moved: a load is followed by the unpack
+  // that reads them, a save by whatever reuses the device buffer
+  KVT_HIP(hipStreamWaitEvent(user, t->done, 0));
+  return KVT_OK;
+}
+
+int kvt_object_ring_save(kvt_object_ring* r, const uint32_t* entries, uint32_t n, const void* dev,
+                         uint64_t dev_stride, void* stream) {
+  return guarded([&]() -> int {
+    return transfer(r, entries, n, const_cast<void*>(dev), dev_stride, stream, true);
+  });
+}
+
+int kvt_object_ring_load(kvt_object_ring* r, const uint32_t* entries, uint32_t n, void* dev,
+                         uint64_t dev_stride, void* stream) {
+  return guarded([&]() -> int { return transfer(r, entries, n, dev, dev_stride, stream, false); });
+}
+
+}  // extern "C"

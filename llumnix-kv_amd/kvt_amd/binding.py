@@ -89,6 +89,15 @@ SIGNATURES = {
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_initialize_copy_method_profile": (_int, [_int]),
+    "kvt_object_ring_create": (_int, [_int, _u64, _u32, _u32, _P(_vp)]),
+    "kvt_object_ring_destroy": (None, [_vp]),
+    "kvt_object_ring_entry": (_vp, [_vp, _u32]),
+    "kvt_object_ring_reserve": (_int, [_vp, _vp, _u32, _vp, _vp]),
+    "kvt_object_ring_save": (_int, [_vp, _vp, _u32, _vp, _u64, _vp]),
+    "kvt_object_ring_commit": (_int, [_vp, _vp, _u32]),
+    "kvt_object_ring_lookup": (_int, [_vp, _vp, _u32, _vp, _vp]),
+    "kvt_object_ring_load": (_int, [_vp, _vp, _u32, _vp, _u64, _vp]),
+    "kvt_object_ring_wait": (_int, [_vp, _u32]),
     "kvt_set_copy_memcpy_thresholds": (_int, [_u64, _u64]),
     "kvt_get_copy_memcpy_thresholds": (_int, [_P(_u64), _P(_u64)]),
     "kvt_set_copy_cu_usage": (_int, [_int, C.c_double]),
@@ -592,3 +601,69 @@ class Stager:
 
     def wait(self, slot):
         check(lib().kvt_stager_wait(self.h, slot))
+
+
+class ObjectRing:
+    """Pinned ring of per-block store objects found by block hash (kvt_object_ring_*).
+    Keys: bytes objects of `key_bytes` each."""
+
+    def __init__(self, device, entry_bytes, n_entries, key_bytes):
+        self.h = _vp()
+        self.entry_bytes, self.n_entries, self.key_bytes = entry_bytes, n_entries, key_bytes
+        check(lib().kvt_object_ring_create(device, entry_bytes, n_entries, key_bytes,
+                                           C.byref(self.h)))
+
+    def _keys(self, keys):
+        assert all(len(k) == self.key_bytes for k in keys)
+        return b"".join(keys)
+
+    def reserve(self, keys):
+        """-> (entries, is_new) as numpy arrays"""
+        n = len(keys)
+        e, f = np.zeros(n, dtype=np.uint32), np.zeros(n, dtype=np.uint8)
+        check(lib().kvt_object_ring_reserve(self.h, self._keys(keys), n, e.ctypes.data,
+                                            f.ctypes.data))
+        return e, f.astype(bool)
+
+    def lookup(self, keys):
+        """-> (entries, found)"""
+        n = len(keys)
+        e, f = np.zeros(n, dtype=np.uint32), np.zeros(n, dtype=np.uint8)
+        check(lib().kvt_object_ring_lookup(self.h, self._keys(keys), n, e.ctypes.data,
+                                           f.ctypes.data))
+        return e, f.astype(bool)
+
+    def save(self, entries, dev_ptr, dev_stride, stream=None):
+        e = np.ascontiguousarray(entries, dtype=np.uint32)
+        check(lib().kvt_object_ring_save(self.h, e.ctypes.data, len(e), dev_ptr, dev_stride,
+                                         stream))
+
+    def load(self, entries, dev_ptr, dev_stride, stream=None):
+        e = np.ascontiguousarray(entries, dtype=np.uint32)
+        check(lib().kvt_object_ring_load(self.h, e.ctypes.data, len(e), dev_ptr, dev_stride,
+                                         stream))
+
+    def commit(self, entries):
+        e = np.ascontiguousarray(entries, dtype=np.uint32)
+        check(lib().kvt_object_ring_commit(self.h, e.ctypes.data, len(e)))
+
+    def wait(self, entry):
+        check(lib().kvt_object_ring_wait(self.h, int(entry)))
+
+    def entry(self, entry):
+        """The entry's bytes as a numpy view of the ring's host memory."""
+        p = lib().kvt_object_ring_entry(self.h, int(entry))
+        if not p:
+            raise IndexError(entry)
+        return np.ctypeslib.as_array(C.cast(p, C.POINTER(C.c_uint8)), shape=(self.entry_bytes,))
+
+    def close(self):
+        if self.h:
+            lib().kvt_object_ring_destroy(self.h)
+            self.h = _vp()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
