@@ -13,6 +13,8 @@
 //     every byte a kernel would touch must lie inside the stated capacity and the packed
 //     layer, and the byte-to-byte mapping must equal the one obtained by expanding the runs
 //     to plain ranges and concatenating them (the definition of pack / unpack).
+// The index of the object ring (kvt_object_ring_*, host-only rings) gets random batches of
+// keys as well: entries carry the key they were handed out for, so that a stale mapping shows.
 #include <algorithm>
 #include <csignal>
 #include <cstdio>
@@ -357,6 +359,78 @@ static void fuzz_hostile_runs(int iters) {
   std::printf("hostile runs: %ld of %d accepted\n", accepted, iters);
 }
 
+// The object ring's index on host-only rings: every entry carries the key it was given for
+// (written through the entry pointer when the ring asks for the block), so a lookup that
+// names a stale or foreign entry is seen at once; exact-size key buffers let the sanitizer
+// see a read past the last key.
+static void fuzz_object_rings(int iters) {
+  long reserved = 0, refused = 0, hits = 0;
+  for (int it = 0; it < iters; ++it) {
+    std::snprintf(g_case, sizeof(g_case), "object ring it=%d", it);
+    const uint32_t n_entries = 1 + static_cast<uint32_t>(rnd(9));
+    const uint32_t key_bytes = 1 + static_cast<uint32_t>(rnd(3) ? rnd(16) : rnd(256));
+    const uint64_t entry_bytes = key_bytes + rnd(40);
+    kvt_object_ring* r = nullptr;
+    CHECK(kvt_object_ring_create(KVT_DEVICE_NONE, entry_bytes, n_entries, key_bytes, &r) == KVT_OK);
+    const uint32_t universe = 2 + static_cast<uint32_t>(rnd(3 * n_entries));
+    auto key_of = [&](uint32_t id, uint8_t* out) {
+      for (uint32_t b = 0; b < key_bytes; ++b) out[b] = static_cast<uint8_t>((id * 131u + b * 7u) ^ (b < 4 ? id >> (8 * b) : 0));
+    };
+    // distinct ids must give distinct keys: with one-byte keys keep the universe small
+    const uint32_t ids = key_bytes == 1 ? std::min<uint32_t>(universe, 2) : universe;
+    for (int step = 0; step < 40; ++step) {
+      const uint32_t n = static_cast<uint32_t>(rnd(2 * n_entries + 2));
+      std::vector<uint32_t> id(n);
+      std::vector<uint8_t> keys(static_cast<size_t>(n) * key_bytes);
+      for (uint32_t i = 0; i < n; ++i) {
+        id[i] = static_cast<uint32_t>(rnd(ids));
+        key_of(id[i], keys.data() + static_cast<size_t>(i) * key_bytes);
+      }
+      std::vector<uint32_t> entries(n);
+      std::vector<uint8_t> flag(n);
+      const int rc = kvt_object_ring_reserve(r, keys.data(), n, entries.data(), flag.data());
+      if (rc != KVT_OK) {
+        CHECK(rc == KVT_ERR_INVALID);
+        ++refused;
+      } else {
+        ++reserved;
+        std::vector<uint32_t> fresh;
+        for (uint32_t i = 0; i < n; ++i) {
+          CHECK(entries[i] < n_entries);
+          uint8_t* e = static_cast<uint8_t*>(kvt_object_ring_entry(r, entries[i]));
+          CHECK(e != nullptr);
+          if (flag[i]) {
+            std::memcpy(e, keys.data() + static_cast<size_t>(i) * key_bytes, key_bytes);
+            if (rnd(4)) fresh.push_back(entries[i]);
+          } else {
+            // stored already, or asked for earlier in this very call: either way the entry
+            // holds this key
+            CHECK(std::memcmp(e, keys.data() + static_cast<size_t>(i) * key_bytes, key_bytes) == 0);
+          }
+          for (uint32_t j = 0; j < i; ++j)   // same key, same entry; different keys, different entries
+            CHECK((id[i] == id[j]) == (entries[i] == entries[j]));
+        }
+        CHECK(kvt_object_ring_commit(r, fresh.data(), static_cast<uint32_t>(fresh.size())) == KVT_OK);
+      }
+      const uint32_t m = static_cast<uint32_t>(rnd(6));
+      std::vector<uint8_t> probe(static_cast<size_t>(m) * key_bytes);
+      for (uint32_t i = 0; i < m; ++i) key_of(static_cast<uint32_t>(rnd(ids)), probe.data() + static_cast<size_t>(i) * key_bytes);
+      std::vector<uint32_t> pe(m);
+      std::vector<uint8_t> found(m);
+      CHECK(kvt_object_ring_lookup(r, probe.data(), m, pe.data(), found.data()) == KVT_OK);
+      for (uint32_t i = 0; i < m; ++i)
+        if (found[i]) {
+          ++hits;
+          CHECK(pe[i] < n_entries);
+          CHECK(std::memcmp(kvt_object_ring_entry(r, pe[i]), probe.data() + static_cast<size_t>(i) * key_bytes, key_bytes) == 0);
+        }
+    }
+    kvt_object_ring_destroy(r);
+  }
+  std::printf("object rings: %ld batches reserved, %ld refused, %ld lookups hit\n", reserved, refused, hits);
+  CHECK(reserved > iters && refused > 0 && hits > iters);
+}
+
 int main(int argc, char** argv) {
   std::signal(SIGALRM, on_alarm);
   const int scale = argc > 1 ? std::atoi(argv[1]) : 1;
@@ -364,6 +438,7 @@ int main(int argc, char** argv) {
   fuzz_run_plans(400 * scale);
   fuzz_range_plans(200 * scale);
   fuzz_hostile_runs(300 * scale);
+  fuzz_object_rings(150 * scale);
   std::printf("plan fuzz ok\n");
   return 0;
 }
