@@ -31,6 +31,7 @@ class FileBlockStore:
     def __init__(self, cachedir, device=0, rank=0, ring_entries=256):
         self._dir, self._device, self._rank, self._ring_entries = cachedir, device, rank, ring_entries
         self._kv = None
+        self._step = None
 
     def register_kv_caches(self, kv_caches):
         """kv_caches: {layer name: tensor [2, num_blocks, block_size, heads, head_dim]} on the
@@ -101,6 +102,47 @@ class FileBlockStore:
                     pass
                 written += 1
         return written
+
+    def save_kv_layer(self, layer_idx, blks):
+        """The layer-wise form, called once per layer while the forward pass runs (FileBackend.
+        async_save_kv_layer / _save_layer, file_backend.py:258-300): layer `layer_idx` of the
+        not-yet-ready blocks is packed behind the work queued on torch's current stream; after
+        the last layer the objects are written out and marked ready (:282-283). One batch (at
+        most ring_entries new blocks) is in flight at a time. -> blocks written by this call."""
+        torch = self._torch
+        n_layers = len(self._kv)
+        if layer_idx == 0:
+            todo, seen = [], set()
+            for blkid, blkhash in blks:
+                if blkhash not in seen and not _blk_ready(self._path(blkhash)[0]):
+                    seen.add(blkhash)
+                    todo.append((blkid, blkhash))
+            if len(todo) > self._ring_entries:
+                raise ValueError("more new blocks in one step than the ring has entries")
+            self._step = None
+            if todo:
+                entries, _ = self._ring.reserve([self._key(h) for _, h in todo])
+                objs = torch.empty(len(todo) * self._entry, dtype=torch.uint8, device="cuda")
+                self._step = (todo, entries, objs, self._plan([b for b, _ in todo]))
+        if self._step is None:
+            return 0
+        todo, entries, objs, plan = self._step
+        self._stream.wait_stream(torch.cuda.current_stream())      # the layer has been computed
+        plan.pack(self._cache, layer_idx, 1, objs[layer_idx * self._obj:], self._obj,
+                  self._stream.cuda_stream)
+        if layer_idx != n_layers - 1:
+            return 0
+        self._ring.save(entries, objs.data_ptr(), self._entry, self._stream.cuda_stream)
+        self._stream.synchronize()
+        for (blkid, blkhash), idx in zip(todo, entries):
+            blkdir, datapath = self._path(blkhash)
+            os.makedirs(blkdir, exist_ok=True)
+            self._ring.entry(idx).tofile(datapath)
+            with open(os.path.join(blkdir, "ready"), "w"):
+                pass
+        plan.close()
+        self._step = None
+        return len(todo)
 
     def load_blocks(self, blks):
         """blks: [(blkid, blkhash)]: every block must be ready (file_backend.py:219-221); its

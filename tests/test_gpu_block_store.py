@@ -82,3 +82,28 @@ def test_save_skip_and_load_like_the_file_backend(tmp_path):
     with pytest.raises(KeyError):
         other.load_blocks([(5, "never_saved")])
     other.close()
+
+
+def test_layer_wise_save_while_the_layers_are_being_produced(tmp_path):
+    """async_save_kv_layer's shape: each layer is handed over right after the kernel that
+    writes it has been queued; a block is ready only after the last layer."""
+    kv = _caches(3, zeros=True)
+    final = _caches(3)
+    store = FileBlockStore(str(tmp_path), ring_entries=8)
+    store.register_kv_caches(kv)
+    blks = [(4, "a_1"), (21, "a_2"), (8, "a_3")]
+    names = list(kv)
+    for l, name in enumerate(names):
+        kv[name].copy_(final[name])                 # "the forward pass" fills layer l on torch's stream
+        done = store.save_kv_layer(l, blks)
+        if l < len(names) - 1:
+            assert done == 0 and not (tmp_path / "a_1" / "ready").exists()
+    assert done == 3
+    for blkid, blkhash in blks:
+        assert (tmp_path / blkhash / "ready").is_file()
+        assert np.array_equal(np.fromfile(tmp_path / blkhash / "0.data", dtype=np.uint8),
+                              _expected_file(final, blkid)), blkhash
+    # a later step with the same blocks has nothing to do
+    for l in range(len(names)):
+        assert store.save_kv_layer(l, blks) == 0
+    store.close()
