@@ -14,7 +14,7 @@
  *     is usable; there is no CPU fallback inside this library.
  *   - buffers handed to a launch whose extent the host knows (layer tensors at
  *     registration, the packed buffer of kvt_pack / kvt_unpack, both sides of
- *     the copy_handle_data calls, stager transfers) are checked against what the
+ *     the copy_handle_data calls, stager and object-ring transfers) are checked against what the
  *     runtime knows about the pointer: memory the device cannot address gives
  *     KVT_ERR_INVALID, an extent beyond the allocation holding the pointer
  *     KVT_ERR_OUT_OF_RANGE, instead of a GPU memory fault. Not checked inside a
@@ -22,7 +22,8 @@
  *   - threads: parsers, caches and plans are immutable once created and may be
  *     used from any number of threads at once (a plan may be launched on several
  *     streams); list containers (kvt_block_lists, kvt_run_lists), sessions and
- *     stagers belong to one thread at a time unless stated otherwise.
+ *     stagers belong to one thread at a time unless stated otherwise; an object
+ *     ring locks itself.
  *
  * Each declaration cites the reference interface it replaces (paths relative
  * to the reference checkout).
