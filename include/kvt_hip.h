@@ -536,7 +536,9 @@ int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats
  * DMA copies; when the ring is full the oldest entries are given to new keys.
  * device = KVT_DEVICE_NONE gives an index over plain host memory (no save / load), for a store
  * that fills the entries itself. Keys are key_bytes (1..256) each, compared byte for byte.
- * Calls may come from several threads. */
+ * Calls may come from several threads: an entry whose bytes a caller was asked for stays with
+ * its key until that caller has written it (save / commit) or given up (release), so EVERY
+ * is_new answer must be followed by one of the three; a load can name the keys it expects. */
 typedef struct kvt_object_ring kvt_object_ring;
 int kvt_object_ring_create(int device, uint64_t entry_bytes, uint32_t n_entries,
                            uint32_t key_bytes, kvt_object_ring** out);
@@ -546,9 +548,9 @@ void* kvt_object_ring_entry(kvt_object_ring* r, uint32_t entry);
 /* Save side. For each of the n keys: entries[i] = its entry; is_new[i] = 1 when the caller has
  * to provide the block's bytes (a fresh entry was assigned, or an earlier reservation was never
  * written), 0 when the block is stored already or appeared earlier in this call. No entry that
- * this call refers to is given away by it; KVT_ERR_INVALID when the batch names more distinct
- * blocks than the ring has entries. An entry given to a new key is waited for first if a
- * transfer still uses it. */
+ * this call refers to is given away by it, nor one that some caller has yet to write;
+ * KVT_ERR_INVALID (nothing reserved) when the batch has more new blocks than the entries that
+ * are left. An entry given to a new key is waited for first if a transfer still uses it. */
 int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, uint32_t* entries,
                             uint8_t* is_new);
 /* Device -> entries: object i (entry_bytes long) at dev + i * dev_stride goes to entries[i];
@@ -560,13 +562,19 @@ int kvt_object_ring_save(kvt_object_ring* r, const uint32_t* entries, uint32_t n
                          uint64_t dev_stride, void* stream);
 /* Marks entries as written that the caller filled through kvt_object_ring_entry. */
 int kvt_object_ring_commit(kvt_object_ring* r, const uint32_t* entries, uint32_t n);
+/* Gives up being asked for these entries' bytes (a failed batch). When nobody else was asked
+ * for the same block and it has not been written, its key is forgotten and the entry may be
+ * given away again. */
+int kvt_object_ring_release(kvt_object_ring* r, const uint32_t* entries, uint32_t n);
 /* Load side: found[i] = 1 and entries[i] when key i is stored (written or its write queued). */
 int kvt_object_ring_lookup(kvt_object_ring* r, const void* keys, uint32_t n, uint32_t* entries,
                            uint8_t* found);
 /* Entries -> device, the mirror of save; work queued on `stream` afterwards (the unpack) sees
- * the objects. */
-int kvt_object_ring_load(kvt_object_ring* r, const uint32_t* entries, uint32_t n, void* dev,
-                         uint64_t dev_stride, void* stream);
+ * the objects. keys (may be NULL): the n keys the lookup was made with; when another thread's
+ * reserve has given one of the entries to a different block meanwhile, nothing is copied and
+ * KVT_ERR_OUT_OF_RANGE says so (look up again). */
+int kvt_object_ring_load(kvt_object_ring* r, const uint32_t* entries, const void* keys, uint32_t n,
+                         void* dev, uint64_t dev_stride, void* stream);
 /* Host-blocking: the last save / load that touches the entry has completed. */
 int kvt_object_ring_wait(kvt_object_ring* r, uint32_t entry);
 

@@ -32,6 +32,8 @@ struct Transfer {
 struct Entry {
   std::string key;                     // empty: never used
   bool saved = false;                  // its bytes have been written (or the write is queued)
+  uint32_t claims = 0;                 // callers that were asked for the block's bytes and have
+                                       // neither written nor released yet; the entry stays put
   uint64_t touched = 0;                // id of the last reserve call that referred to it
   uint64_t flagged = 0;                // id of the last reserve call that reported it as new
   std::shared_ptr<Transfer> pending;   // last transfer that reads or writes the entry
@@ -167,8 +169,16 @@ int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, ui
       for (uint32_t i = 0; i < n; ++i)
         if (!r->index.count(ks[i]) && seen.emplace(ks[i], 1).second) ++fresh;
     }
-    if (static_cast<uint64_t>(fresh) + kept > r->n_entries)
-      return fail(KVT_ERR_INVALID, "kvt_object_ring_reserve: more distinct blocks than entries");
+    // entries that may be given away: not referred to by this call, and not claimed by a caller
+    // who has yet to write them (another thread between its reserve and its save)
+    uint32_t available = 0;
+    for (const Entry& e : r->entries)
+      if (e.touched != call && e.claims == 0) ++available;
+    (void)kept;
+    if (fresh > available)
+      return fail(KVT_ERR_INVALID,
+                  "kvt_object_ring_reserve: more new blocks than entries that may be given away "
+                  "(entries this batch refers to and reservations not yet written stay)");
     for (uint32_t i = 0; i < n; ++i) {
       auto it = r->index.find(ks[i]);
       if (it != r->index.end()) {
@@ -177,19 +187,23 @@ int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, ui
         // present and written: nothing to do. Reserved before but never written: the caller
         // is asked again, once per call (a key may be repeated inside a batch).
         is_new[i] = (!e.saved && e.flagged != call) ? 1 : 0;
-        if (is_new[i]) e.flagged = call;
+        if (is_new[i]) {
+          e.flagged = call;
+          ++e.claims;
+        }
         continue;
       }
       uint32_t idx = 0;
-      for (;;) {   // the oldest entry that this call does not refer to
+      for (;;) {   // the oldest entry that may be given away
         idx = static_cast<uint32_t>(r->handed_out++ % r->n_entries);
-        if (r->entries[idx].touched != call) break;
+        if (r->entries[idx].touched != call && r->entries[idx].claims == 0) break;
       }
       Entry& e = r->entries[idx];
       if (int rc = wait_entry(e)) return rc;
       if (!e.key.empty()) r->index.erase(e.key);
       e.key = ks[i];
       e.saved = false;
+      e.claims = 1;
       e.touched = call;
       e.flagged = call;
       r->index.emplace(ks[i], idx);
@@ -223,7 +237,30 @@ int kvt_object_ring_commit(kvt_object_ring* r, const uint32_t* entries, uint32_t
     if (!r || (n && !entries)) return fail(KVT_ERR_INVALID, "kvt_object_ring_commit: null argument");
     std::lock_guard<std::mutex> lock(r->mu);
     if (int rc = check_entries(r, entries, n, "kvt_object_ring_commit")) return rc;
-    for (uint32_t i = 0; i < n; ++i) r->entries[entries[i]].saved = true;
+    for (uint32_t i = 0; i < n; ++i) {
+      Entry& e = r->entries[entries[i]];
+      e.saved = true;
+      if (e.claims) --e.claims;
+    }
+    return KVT_OK;
+  });
+}
+
+int kvt_object_ring_release(kvt_object_ring* r, const uint32_t* entries, uint32_t n) {
+  return guarded([&]() -> int {
+    if (!r || (n && !entries)) return fail(KVT_ERR_INVALID, "kvt_object_ring_release: null argument");
+    std::lock_guard<std::mutex> lock(r->mu);
+    for (uint32_t i = 0; i < n; ++i)
+      if (entries[i] >= r->n_entries)
+        return fail(KVT_ERR_OUT_OF_RANGE, "kvt_object_ring_release: entry index out of range");
+    for (uint32_t i = 0; i < n; ++i) {
+      Entry& e = r->entries[entries[i]];
+      if (e.key.empty() || e.claims == 0) continue;   // nothing claimed here
+      if (--e.claims == 0 && !e.saved) {              // nobody is going to write it: forget the key
+        r->index.erase(e.key);
+        e.key.clear();
+      }
+    }
     return KVT_OK;
   });
 }
@@ -243,7 +280,7 @@ int kvt_object_ring_wait(kvt_object_ring* r, uint32_t entry) {
 
 // save = true: device -> entries (and the entries count as written); false: entries -> device.
 static int transfer(kvt_object_ring* r, const uint32_t* entries, uint32_t n, void* dev,
-                    uint64_t dev_stride, void* stream, bool save) {
+                    uint64_t dev_stride, void* stream, bool save, const void* keys = nullptr) {
   const char* who = save ? "kvt_object_ring_save" : "kvt_object_ring_load";
   if (!r || (n && (!entries || !dev))) return fail(KVT_ERR_INVALID, std::string(who) + ": null argument");
   if (n == 0) return KVT_OK;
@@ -254,9 +291,14 @@ static int transfer(kvt_object_ring* r, const uint32_t* entries, uint32_t n, voi
   std::lock_guard<std::mutex> lock(r->mu);
   if (int rc = check_entries(r, entries, n, who)) return rc;
   if (!save)
-    for (uint32_t i = 0; i < n; ++i)
-      if (!r->entries[entries[i]].saved)
-        return fail(KVT_ERR_INVALID, "kvt_object_ring_load: entry has not been written");
+    for (uint32_t i = 0; i < n; ++i) {
+      const Entry& e = r->entries[entries[i]];
+      if (!e.saved) return fail(KVT_ERR_INVALID, "kvt_object_ring_load: entry has not been written");
+      if (keys && std::memcmp(e.key.data(), static_cast<const char*>(keys) + static_cast<size_t>(i) * r->key_bytes,
+                              r->key_bytes) != 0)
+        return fail(KVT_ERR_OUT_OF_RANGE,
+                    "kvt_object_ring_load: an entry was given to another block since the lookup");
+    }
   DeviceGuard g;
   if (int rc = g.enter(r->device)) return rc;
   if (int rc = check_device_span(dev, static_cast<uint64_t>(n - 1) * dev_stride + r->entry_bytes,
@@ -285,7 +327,10 @@ static int transfer(kvt_object_ring* r, const uint32_t* entries, uint32_t n, voi
   for (uint32_t i = 0; i < n; ++i) {
     Entry& e = r->entries[entries[i]];
     e.pending = t;
-    if (save) e.saved = true;
+    if (save) {
+      e.saved = true;
+      if (e.claims) --e.claims;
+    }
   }
   // the caller's stream continues once the bytes have moved: a load is followed by the unpack
   // that reads them, a save by whatever reuses the device buffer
@@ -300,9 +345,11 @@ int kvt_object_ring_save(kvt_object_ring* r, const uint32_t* entries, uint32_t n
   });
 }
 
-int kvt_object_ring_load(kvt_object_ring* r, const uint32_t* entries, uint32_t n, void* dev,
-                         uint64_t dev_stride, void* stream) {
-  return guarded([&]() -> int { return transfer(r, entries, n, dev, dev_stride, stream, false); });
+int kvt_object_ring_load(kvt_object_ring* r, const uint32_t* entries, const void* keys, uint32_t n,
+                         void* dev, uint64_t dev_stride, void* stream) {
+  return guarded([&]() -> int {
+    return transfer(r, entries, n, dev, dev_stride, stream, false, keys);
+  });
 }
 
 }  // extern "C"

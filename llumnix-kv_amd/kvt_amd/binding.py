@@ -96,7 +96,8 @@ SIGNATURES = {
     "kvt_object_ring_save": (_int, [_vp, _vp, _u32, _vp, _u64, _vp]),
     "kvt_object_ring_commit": (_int, [_vp, _vp, _u32]),
     "kvt_object_ring_lookup": (_int, [_vp, _vp, _u32, _vp, _vp]),
-    "kvt_object_ring_load": (_int, [_vp, _vp, _u32, _vp, _u64, _vp]),
+    "kvt_object_ring_load": (_int, [_vp, _vp, _vp, _u32, _vp, _u64, _vp]),
+    "kvt_object_ring_release": (_int, [_vp, _vp, _u32]),
     "kvt_object_ring_wait": (_int, [_vp, _u32]),
     "kvt_set_copy_memcpy_thresholds": (_int, [_u64, _u64]),
     "kvt_get_copy_memcpy_thresholds": (_int, [_P(_u64), _P(_u64)]),
@@ -638,10 +639,17 @@ class ObjectRing:
         check(lib().kvt_object_ring_save(self.h, e.ctypes.data, len(e), dev_ptr, dev_stride,
                                          stream))
 
-    def load(self, entries, dev_ptr, dev_stride, stream=None):
+    def load(self, entries, dev_ptr, dev_stride, stream=None, keys=None):
+        """keys: the keys the entries were looked up with (checked against the entries)."""
         e = np.ascontiguousarray(entries, dtype=np.uint32)
-        check(lib().kvt_object_ring_load(self.h, e.ctypes.data, len(e), dev_ptr, dev_stride,
+        k = self._keys(keys) if keys is not None else None
+        assert keys is None or len(keys) == len(e)
+        check(lib().kvt_object_ring_load(self.h, e.ctypes.data, k, len(e), dev_ptr, dev_stride,
                                          stream))
+
+    def release(self, entries):
+        e = np.ascontiguousarray(entries, dtype=np.uint32)
+        check(lib().kvt_object_ring_release(self.h, e.ctypes.data, len(e)))
 
     def commit(self, entries):
         e = np.ascontiguousarray(entries, dtype=np.uint32)

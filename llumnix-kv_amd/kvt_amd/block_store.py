@@ -169,7 +169,8 @@ class FileBlockStore:
                 self._ring.commit(np.asarray(filled, dtype=np.uint32))
             objs = torch.empty(len(part) * self._entry, dtype=torch.uint8, device="cuda")
             self._stream.wait_stream(torch.cuda.current_stream())
-            self._ring.load(entries, objs.data_ptr(), self._entry, self._stream.cuda_stream)
+            self._ring.load(entries, objs.data_ptr(), self._entry, self._stream.cuda_stream,
+                            keys=keys)
             plan = self._plan([b for b, _ in part])
             plan.unpack(self._cache, 0, len(self._kv), objs, self._obj, self._stream.cuda_stream)
             self._stream.synchronize()

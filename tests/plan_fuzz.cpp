@@ -411,6 +411,9 @@ static void fuzz_object_rings(int iters) {
             CHECK((id[i] == id[j]) == (entries[i] == entries[j]));
         }
         CHECK(kvt_object_ring_commit(r, fresh.data(), static_cast<uint32_t>(fresh.size())) == KVT_OK);
+        // what was not written is given up half of the time (written entries are left alone),
+        // otherwise it stays reserved and narrows the ring
+        if (rnd(2)) CHECK(kvt_object_ring_release(r, entries.data(), n) == KVT_OK);
       }
       const uint32_t m = static_cast<uint32_t>(rnd(6));
       std::vector<uint8_t> probe(static_cast<size_t>(m) * key_bytes);

@@ -100,7 +100,11 @@ def test_save_by_hash_skips_stored_blocks_and_load_restores_them_elsewhere():
     torch.cuda.synchronize()
     dst_blocks = [2, 19, 8, 14]
     objs = torch.empty(len(hit) * ENTRY, dtype=torch.uint8, device="cuda")
-    ring.load(hit, objs.data_ptr(), ENTRY, s.cuda_stream)
+    hit_keys = [k for k, f in zip(want_keys, found) if f]
+    with pytest.raises(kvt_amd.KvtError) as ex:           # the entries do not hold these keys
+        ring.load(hit, objs.data_ptr(), ENTRY, s.cuda_stream, keys=hit_keys[::-1])
+    assert ex.value.code == 1 and "given to another block" in str(ex.value)
+    ring.load(hit, objs.data_ptr(), ENTRY, s.cuda_stream, keys=hit_keys)
     _plan(dst_blocks, dst_blocks).unpack(_cache_handle(new_cache), 0, N_LAYERS, objs, B,
                                          s.cuda_stream)
     s.synchronize()

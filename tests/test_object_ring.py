@@ -69,12 +69,62 @@ def test_a_batch_larger_than_the_ring_is_refused_but_repeats_do_not_count():
     r = ring(4)
     with pytest.raises(kvt_amd.KvtError) as ex:
         r.reserve([key(i) for i in range(5)])
-    assert ex.value.code == 3 and "more distinct blocks" in str(ex.value)
+    assert ex.value.code == 3 and "more new blocks" in str(ex.value)
     e, new = r.reserve([key(i % 4) for i in range(12)])
     assert e.tolist() == [0, 1, 2, 3] * 3 and new.tolist() == [True] * 4 + [False] * 8
     r.commit(e[:1])
     with pytest.raises(kvt_amd.KvtError):       # one stored block referred to + four new ones
         r.reserve([key(0), key(30), key(31), key(32), key(33)])
+
+
+def test_a_reservation_stays_until_it_is_written_or_released():
+    """Between one thread's reserve and its save another thread's batch must not be given the
+    same entries: what somebody has yet to write is not given away."""
+    r = ring(4)
+    mine, _ = r.reserve([key(1), key(2)])               # not written yet
+    theirs, new = r.reserve([key(3), key(4)])
+    assert sorted(mine.tolist() + theirs.tolist()) == [0, 1, 2, 3] and new.all()
+    with pytest.raises(kvt_amd.KvtError):                # all four entries are spoken for
+        r.reserve([key(5)])
+    r.commit(theirs)
+    e, _ = r.reserve([key(5)])                           # a written entry may go
+    assert e.tolist() == [int(theirs[0])]
+    r.release(mine[:1])                                  # key 1 will not be written after all
+    _, found = r.lookup([key(1)])
+    assert not found.any()
+    e, new = r.reserve([key(1)])                         # forgotten: a fresh reservation,
+    assert new.all() and e.tolist() == [int(theirs[1])]   # in the next entry in ring order
+    r.commit(e)
+    r.release(e)                                         # written and nobody waiting: left alone
+    _, found = r.lookup([key(1)])
+    assert found.all()
+    with pytest.raises(kvt_amd.KvtError):
+        r.release(np.array([4], dtype=np.uint32))
+
+
+def test_two_callers_asked_for_the_same_block():
+    r = ring(2)
+    a, new_a = r.reserve([key(7)])
+    b, new_b = r.reserve([key(7)])                       # the first has not written it yet
+    assert a.tolist() == b.tolist() == [0] and new_a.all() and new_b.all()
+    r.release(a)                                         # the first gives up: the second still holds it
+    e, new = r.reserve([key(8), key(9)][:1])
+    assert e.tolist() == [1] and new.all()
+    with pytest.raises(kvt_amd.KvtError):                # entry 0 is still somebody's
+        r.reserve([key(9)])
+    r.commit(b)
+    _, found = r.lookup([key(7)])
+    assert found.all()
+    # and the other way round: written by one while the other is still at it -> stays put
+    r2 = ring(1)
+    a, _ = r2.reserve([key(1)])
+    b, _ = r2.reserve([key(1)])
+    r2.commit(a)
+    with pytest.raises(kvt_amd.KvtError):
+        r2.reserve([key(2)])
+    r2.commit(b)
+    e, new = r2.reserve([key(2)])
+    assert e.tolist() == [0] and new.all()
 
 
 def test_entries_are_separate_pieces_of_host_memory():
@@ -123,33 +173,51 @@ class Model:
 
     def __init__(self, n):
         self.n, self.handed_out = n, 0
-        self.key, self.saved, self.index = [None] * n, [False] * n, {}
+        self.key, self.saved, self.claims, self.index = [None] * n, [False] * n, [0] * n, {}
+
+    def _may_go(self, idx, touched):
+        return idx not in touched and self.claims[idx] == 0
 
     def reserve(self, keys):
         touched = {self.index[k] for k in keys if k in self.index}
         fresh = {k for k in keys if k not in self.index}
-        if len(touched) + len(fresh) > self.n:
+        if len(fresh) > sum(self._may_go(i, touched) for i in range(self.n)):
             return None
         flagged, out = set(), []
         for k in keys:
             if k in self.index:
                 idx = self.index[k]
                 new = (not self.saved[idx]) and idx not in flagged
+                if new:
+                    self.claims[idx] += 1
             else:
                 while True:
                     idx = self.handed_out % self.n
                     self.handed_out += 1
-                    if idx not in touched:
+                    if self._may_go(idx, touched):
                         break
                 if self.key[idx] is not None:
                     del self.index[self.key[idx]]
-                self.key[idx], self.saved[idx], self.index[k] = k, False, idx
+                self.key[idx], self.saved[idx], self.claims[idx], self.index[k] = k, False, 1, idx
                 touched.add(idx)
                 new = True
             if new:
                 flagged.add(idx)
             out.append((idx, new))
         return out
+
+    def commit(self, entries):
+        for idx in entries:
+            self.saved[idx] = True
+            self.claims[idx] = max(0, self.claims[idx] - 1)
+
+    def release(self, entries):
+        for idx in entries:
+            if self.key[idx] is not None and self.claims[idx] > 0:
+                self.claims[idx] -= 1
+                if self.claims[idx] == 0 and not self.saved[idx]:
+                    del self.index[self.key[idx]]
+                    self.key[idx] = None
 
     def lookup(self, keys):
         return [(k in self.index and self.saved[self.index[k]]) for k in keys]
@@ -173,8 +241,15 @@ def test_random_traffic_against_the_model(seed):
         if len(keys) and rng.random() < 0.8:              # write some of what was asked for
             todo = sorted({idx for idx, is_new in want if is_new and rng.random() < 0.7})
             r.commit(np.array(todo, dtype=np.uint32))
-            for idx in todo:
-                m.saved[idx] = True
+            m.commit(todo)
+            rest = sorted({idx for idx, is_new in want if is_new} - set(todo))
+            if rest and rng.random() < 0.6:               # give up what was not written
+                r.release(np.array(rest, dtype=np.uint32))
+                m.release(rest)
+        if rng.random() < 0.2:                            # stray releases change nothing they should not
+            drop = [int(i) for i in rng.integers(0, n, size=int(rng.integers(0, n + 1)))]
+            r.release(np.array(drop, dtype=np.uint32))
+            m.release(drop)
         probe = [universe[int(i)] for i in rng.integers(0, len(universe), size=5)]
         e, found = r.lookup(probe)
         assert found.tolist() == m.lookup(probe)

@@ -69,3 +69,51 @@ def test_error_message_is_per_thread():
     b.join()
     assert "null argument" in seen["failing"]
     assert "null argument" not in seen["clean_before"]
+
+
+def test_object_ring_reservations_of_one_thread_survive_the_others():
+    """Eight threads push batches through one small ring (host-only): between a thread's reserve
+    and its commit nobody else may be handed its entries, so the tag it wrote is still there."""
+    n_entries, batch = 12, 3
+    ring = kvt_amd.ObjectRing(-1, 32, n_entries, 16)
+    errors, done = [], [0] * 8
+
+    def work(tid):
+        try:
+            rng = np.random.default_rng(tid)
+            for step in range(300):
+                ids = rng.integers(0, 40, size=batch)
+                keys = [int(i).to_bytes(8, "little") + b"thread%02d" % 0 for i in ids]
+                try:
+                    entries, new = ring.reserve(keys)
+                except kvt_amd.KvtError:
+                    continue                  # the others hold everything right now
+                mine = sorted({int(e) for e, n in zip(entries, new) if n})
+                tag = (tid << 16) | step
+                for e in mine:
+                    ring.entry(e).view(np.uint32)[0] = tag
+                for e in mine:                # (several threads may be asked for the same
+                    got = int(ring.entry(e).view(np.uint32)[0])   # block; then the tag is one of theirs)
+                    assert (got & 0xFFFF) < 300 and (got >> 16) < 8
+                if step % 5 == 4:
+                    ring.release(np.array(mine, dtype=np.uint32))
+                else:
+                    ring.commit(np.array(mine, dtype=np.uint32))
+                _, found = ring.lookup(keys)
+                done[tid] += int(found.sum())
+        except Exception as exc:              # noqa: BLE001
+            errors.append((tid, repr(exc)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert sum(done) > 0
+    # the index is still consistent: every key found names a distinct entry
+    keys = [int(i).to_bytes(8, "little") + b"thread00" for i in range(40)]
+    e, found = ring.lookup(keys)
+    hit = e[found].tolist()
+    assert len(hit) == len(set(hit)) and len(hit) <= n_entries
+    ring.close()
