@@ -950,9 +950,12 @@ def main():
         "mode": ("mixed: (pack A || unpack B) then (pack B || unpack A) on two streams; pack_ms = "
                  "unpack_ms = mean phase time") if mixed else "sequential: pack all, then unpack all",
         "roofline": {"bound": "hbm",
-                     "kernel": "strided_chunks_kernel<pack>" if first[0][0].num_strided_chunks
-                     else ("copy_chunks_kernel<pack>" if not wls[0].xform
-                           else "xform_chunks_kernel<pack>"),
+                     # instantiation names as a profiler prints them: <pack, [words,] capped>
+                     "kernel": "kvt::strided_chunks_kernel<true, false, false> (pack)"
+                     if first[0][0].num_strided_chunks
+                     else ("kvt::copy_chunks_small_kernel<true, false> (pack)" if first[0][0].num_chunks <= 64
+                           else "kvt::copy_chunks_kernel<true, false> (pack)") if not wls[0].xform
+                     else "kvt::xform_chunks_kernel<true, false> (pack)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4),
                      "traffic": MEASURED_PACK_TRAFFIC.get((args.config, args.scale,
