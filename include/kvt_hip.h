@@ -383,6 +383,14 @@ int kvt_set_copy_cu_usage(int device, double usage);
 /* The current setting and the workgroup limit it stands for (0 = none); either may be NULL. */
 int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
 
+/* replaces launch_copy_int64_array_h2d_kernel()  kvtransfer/src/copy_kernels.cu:93-103
+ * (declared for the channels, kvtransfer/src/copy_kernels.cpp:101-108): a kernel reads
+ * num_elements int64 from pinned (device-visible) host memory and writes them to device_dst,
+ * the metadata upload without a DMA copy. num_wg / threads_per_wg are accepted and ignored. */
+int kvt_launch_copy_int64_array_h2d(const int64_t* host_src, int64_t* device_dst,
+                                    int64_t num_elements, int num_wg, int threads_per_wg,
+                                    void* stream);
+
 /* replaces BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES / BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS
  *                                               kvtransfer/src/copy_kernels.cpp:157-158, 496-499,
  * the static part of select_copy_method()       kvtransfer/src/copy_kernels.cpp:610-617:

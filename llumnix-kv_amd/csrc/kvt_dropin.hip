@@ -232,6 +232,28 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
   });
 }
 
+int kvt_launch_copy_int64_array_h2d(const int64_t* host_src, int64_t* device_dst,
+                                    int64_t num_elements, int num_wg, int threads_per_wg,
+                                    void* stream) {
+  (void)num_wg;          // one 256-lane workgroup per 4 KiB, like every other copy here
+  (void)threads_per_wg;
+  return guarded([&]() -> int {
+    if (num_elements == 0) return KVT_OK;
+    if (num_elements < 0 || !host_src || !device_dst)
+      return fail(KVT_ERR_INVALID, "launch_copy_int64_array_h2d: bad argument");
+    if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+    if (num_elements > (1ll << 40)) return fail(KVT_ERR_INVALID, "launch_copy_int64_array_h2d: too large");
+    const uint64_t bytes = static_cast<uint64_t>(num_elements) * sizeof(int64_t);
+    // both sides must be memory a kernel can touch: the source is pinned host memory
+    if (int rc = check_device_span(host_src, bytes, "launch_copy_int64_array_h2d: the host array")) return rc;
+    if (int rc = check_device_span(device_dst, bytes, "launch_copy_int64_array_h2d: the device array"))
+      return rc;
+    const hipError_t e = launch_copy_linear(device_dst, host_src, bytes, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "int64 array copy launch");
+    return KVT_OK;
+  });
+}
+
 // Per-thread metadata buffers and streams of the copy threads (CopyKernelCtx,
 // kvtransfer/src/copy_utils.cpp:9-154): created on first use, re-created when the thread
 // moves to another device or asks for more ranges, released when the thread ends.

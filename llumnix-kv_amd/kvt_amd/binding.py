@@ -88,6 +88,7 @@ SIGNATURES = {
     "kvt_launch_copy_d2h_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_h2d_direct": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "kvt_launch_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
+    "kvt_launch_copy_int64_array_h2d": (_int, [_vp, _vp, _i64, _int, _int, _vp]),
     "kvt_initialize_copy_method_profile": (_int, [_int]),
     "kvt_object_ring_create": (_int, [_int, _u64, _u32, _u32, _P(_vp)]),
     "kvt_object_ring_destroy": (None, [_vp]),

@@ -416,6 +416,31 @@ def test_copy_handle_data_hands_a_few_very_large_ranges_to_the_dma_engines():
     assert (host_meta == 0).all()           # the kernel's metadata buffers were not needed
 
 
+@pytest.mark.parametrize("n", [1, 2, 3, 511, 8192 * 3, 100001])
+def test_launch_copy_int64_array_h2d(n):
+    """launch_copy_int64_array_h2d_kernel of the reference (copy_kernels.cu:93-103): pinned
+    int64 metadata read by a kernel, any count, also from an address that is only 8-byte
+    aligned."""
+    lib = kvt_amd.lib()
+    rng = np.random.default_rng(n)
+    host = torch.from_numpy(rng.integers(-2**62, 2**62, size=n + 1, dtype=np.int64)).pin_memory()
+    dev = torch.full((n + 3,), -7, dtype=torch.int64, device="cuda")
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    for shift in (0, 1):
+        rc = lib.kvt_launch_copy_int64_array_h2d(host.data_ptr() + 8 * shift, dev.data_ptr() + 8,
+                                                 n, 0, 0, s.cuda_stream)
+        assert rc == 0, lib.kvt_last_error()
+        s.synchronize()
+        got = dev.cpu()
+        assert got[0] == -7 and (got[n + 1:] == -7).all()
+        assert torch.equal(got[1:n + 1], host[shift:shift + n])
+    assert lib.kvt_launch_copy_int64_array_h2d(host.data_ptr(), dev.data_ptr(), 0, 0, 0, None) == 0
+    assert lib.kvt_launch_copy_int64_array_h2d(None, dev.data_ptr(), 4, 0, 0, None) != 0
+    pageable = np.zeros(8, dtype=np.int64)                 # not device-visible: refused, no fault
+    assert lib.kvt_launch_copy_int64_array_h2d(pageable.ctypes.data, dev.data_ptr(), 8, 0, 0, None) != 0
+
+
 def test_memcpy_route_thresholds_decide_between_dma_and_kernel():
     """BLLM_KVTRANS_COPY_MEMCPY_{BLOCK_THRESHOLD_BYTES,MAX_BLOCKS} of the reference
     (copy_kernels.cpp:496-499, 610-617) as kvt_set_copy_memcpy_thresholds: the same three ranges
