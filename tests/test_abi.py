@@ -90,3 +90,15 @@ def test_memcpy_route_thresholds_are_process_wide_settings():
         assert lib.kvt_set_copy_memcpy_thresholds(1, 0) == 0          # route switched off
     finally:
         assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+
+
+def test_launcher_stand_in_exports_the_reference_names():
+    """libkvt_blade_launchers.so: the extern "C" names kvtransfer/src/copy_kernels.cpp:52-85,
+    101-108 declares (no calls here: they launch kernels)."""
+    import ctypes as C
+    import os
+    kvt_amd.lib()
+    shim = C.CDLL(os.path.join(os.path.dirname(kvt_amd.LIB_PATH), "libkvt_blade_launchers.so"))
+    for name in ("launch_copy_int64_array_h2d_kernel", "launch_copy_h2d_direct_kernel",
+                 "launch_copy_d2h_direct_kernel", "launch_copy_d2h_bf16_to_fp8_kernel"):
+        assert hasattr(shim, name), name

@@ -382,6 +382,65 @@ def test_launch_copy_direct_gather_and_scatter(n, maxlen):
     assert np.array_equal(_host(dst), exp)
 
 
+def test_reference_launcher_names_link_level_stand_in():
+    """libkvt_blade_launchers.so exports the four extern "C" names that the reference's
+    copy_kernels.cpp calls (copy_kernels.cpp:52-85, 101-108), with its argument order and a
+    void return; called here the way that file calls them, persistent grid arguments included."""
+    import ctypes as C
+    import os
+    lib = kvt_amd.lib()                                    # libkvt_hip.so first
+    shim = C.CDLL(os.path.join(os.path.dirname(kvt_amd.LIB_PATH), "libkvt_blade_launchers.so"))
+    vp, i64, ci = C.c_void_p, C.c_int64, C.c_int
+    for name in ("launch_copy_d2h_direct_kernel", "launch_copy_h2d_direct_kernel",
+                 "launch_copy_d2h_bf16_to_fp8_kernel"):
+        fn = getattr(shim, name)
+        fn.restype, fn.argtypes = None, [vp, vp, vp, vp, vp, i64, ci, ci, vp]
+    shim.launch_copy_int64_array_h2d_kernel.restype = None
+    shim.launch_copy_int64_array_h2d_kernel.argtypes = [vp, vp, i64, ci, ci, vp]
+
+    n, cap = 700, 8 << 20
+    rng = np.random.default_rng(12)
+    lens = rng.integers(1, 300, size=n) * 16
+    gpu_off = np.sort(rng.choice(cap // 8192, size=n, replace=False)) * 8192
+    contig = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    total = int(lens.sum())
+    src = _dev_bytes(cap, 5, "bf16")
+    meta_h = torch.from_numpy(np.concatenate([gpu_off, contig, lens]).astype(np.int64)).pin_memory()
+    meta_d = torch.zeros(3 * n, dtype=torch.int64, device="cuda")
+    out = torch.zeros(total, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    st = s.cuda_stream
+    shim.launch_copy_int64_array_h2d_kernel(meta_h.data_ptr(), meta_d.data_ptr(), 3 * n, 2048, 512, st)
+    so, do, ln = (meta_d.data_ptr() + 8 * n * k for k in range(3))
+    shim.launch_copy_d2h_direct_kernel(src.data_ptr(), out.data_ptr(), so, do, ln, n, 2048, 512, st)
+    s.synchronize()
+    runs = np.stack([gpu_off, gpu_off, lens], axis=1).astype(np.uint64)
+    blob = checkers.oracle_pack(_host(src), runs)
+    assert np.array_equal(_host(out), blob)
+    dst = torch.full((cap,), 0x3C, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    shim.launch_copy_h2d_direct_kernel(out.data_ptr(), dst.data_ptr(), do, so, ln, n, 2048, 512, st)
+    s.synchronize()
+    exp = np.full(cap, 0x3C, dtype=np.uint8)
+    checkers.oracle_unpack(exp, runs, blob)
+    assert np.array_equal(_host(dst), exp)
+    # converting gather: lengths are element counts, destination offsets in fp8 bytes
+    meta_h[n:2 * n] = torch.from_numpy((contig // 2).astype(np.int64))
+    meta_h[2 * n:] = torch.from_numpy((lens // 2).astype(np.int64))
+    out8 = torch.zeros(total // 2, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    shim.launch_copy_int64_array_h2d_kernel(meta_h.data_ptr(), meta_d.data_ptr(), 3 * n, 2048, 512, st)
+    shim.launch_copy_d2h_bf16_to_fp8_kernel(src.data_ptr(), out8.data_ptr(), so, do, ln, n, 2048, 512, st)
+    s.synchronize()
+    want = torch.from_numpy(blob.copy()).view(torch.bfloat16).to(torch.float32).clamp(-448, 448) \
+        .to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(_host(out8), want)
+    # a refused call leaves a message, not a crash
+    shim.launch_copy_d2h_direct_kernel(None, out.data_ptr(), so, do, ln, n, 1, 1, st)
+    assert b"bad argument" in lib.kvt_last_error()
+
+
 def test_copy_handle_data_hands_a_few_very_large_ranges_to_the_dma_engines():
     lib = kvt_amd.lib()
     assert lib.kvt_initialize_copy_method_profile(0) == 0
