@@ -395,7 +395,9 @@ int kvt_launch_copy_int64_array_h2d(const int64_t* host_src, int64_t* device_dst
  *                                               kvtransfer/src/copy_kernels.cpp:157-158, 496-499,
  * the static part of select_copy_method()       kvtransfer/src/copy_kernels.cpp:610-617:
  * kvt_copy_handle_data_with_kernel hands a list to the DMA engines (one copy per range) when it
- * has at most max_ranges ranges and every range is at least min_range_bytes long. Defaults:
+ * has at most max_ranges ranges and every range is at least min_range_bytes long; in a longer or
+ * mixed list whose lengths differ, the ranges of at least min_range_bytes still go there one by
+ * one and the kernel moves the rest (enqueue_hybrid_copy, copy_kernels.cpp:675-722). Defaults:
  * 8 MiB and 16, measured on MI355X against pinned host memory (the reference's defaults,
  * 256 KiB and 16, suit a part whose copy kernel is slower across PCIe than this one's).
  * max_ranges = 0 switches the DMA route off. Process-wide. */

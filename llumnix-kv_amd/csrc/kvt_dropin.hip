@@ -70,12 +70,13 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     return fail(KVT_ERR_INVALID, "copy_handle_data: bad direction");
   if (int rc = check_device(device)) return rc;
   if (max_block_num <= 0) max_block_num = 8192;
-  uint64_t total = 0, layer_extent = 0, shortest = ~0ull;
+  uint64_t total = 0, layer_extent = 0, shortest = ~0ull, longest = 0;
   for (uint64_t i = 0; i < n; ++i) {
     if (blocks[i].length == 0) return fail(KVT_ERR_INVALID, "copy_handle_data: zero-length range");
     if (halve && (blocks[i].length & 1)) return fail(KVT_ERR_INVALID, "odd bf16 byte length");
     total += blocks[i].length;
     shortest = std::min(shortest, blocks[i].length);
+    longest = std::max(longest, blocks[i].length);
     layer_extent = std::max(layer_extent, blocks[i].dst_offset + blocks[i].length);
   }
   if (total != tensor_data_size)
@@ -107,20 +108,45 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     }
     return KVT_OK;
   }
-  uint64_t host_cursor = 0;
-  for (uint64_t first = 0; first < n; first += static_cast<uint64_t>(max_block_num)) {
-    const uint64_t m = std::min<uint64_t>(static_cast<uint64_t>(max_block_num), n - first);
+  // What the kernel has to move: {position in the contiguous buffer, cache offset, length}.
+  // In a list of mixed lengths the ranges long enough for a DMA copy go there one by one and
+  // only the rest to the kernel (the reference's enqueue_hybrid_copy, copy_kernels.cpp:675-722,
+  // with its per-range rule select_single_block_method, :621-631).
+  static thread_local std::vector<kvt_ipc_block> work;
+  work.clear();
+  const uint64_t dma_min = g_dma_min_bytes.load(std::memory_order_relaxed);
+  const bool split = !halve && shortest != longest && longest >= dma_min &&
+                     g_dma_max_ranges.load(std::memory_order_relaxed) != 0;
+  {
+    uint64_t cursor = 0;
+    for (uint64_t i = 0; i < n; ++i) {
+      const kvt_ipc_block& b = blocks[i];
+      if (split && b.length >= dma_min) {
+        uint8_t* host = static_cast<uint8_t*>(tensor_buf) + cursor;
+        uint8_t* dev = static_cast<uint8_t*>(layer_gpu_ptr) + b.dst_offset;
+        if (direction == KVT_COPY_D2H)
+          KVT_HIP(hipMemcpyAsync(host, dev, b.length, hipMemcpyDefault, s));
+        else
+          KVT_HIP(hipMemcpyAsync(dev, host, b.length, hipMemcpyDefault, s));
+      } else {
+        work.push_back(kvt_ipc_block{cursor, b.dst_offset, b.length});
+      }
+      cursor += halve ? b.length / 2 : b.length;
+    }
+  }
+  const uint64_t n_work = work.size();
+  for (uint64_t first = 0; first < n_work; first += static_cast<uint64_t>(max_block_num)) {
+    const uint64_t m = std::min<uint64_t>(static_cast<uint64_t>(max_block_num), n_work - first);
     int64_t* contig = host_meta;
     int64_t* gpu = host_meta + m;
     int64_t* lens = host_meta + 2 * m;
     const uint64_t unit = halve ? 8192 : 4096;  // source bytes of one workgroup's slice
     uint64_t slices = 0;
     for (uint64_t i = 0; i < m; ++i) {
-      const kvt_ipc_block& b = blocks[first + i];
-      contig[i] = static_cast<int64_t>(host_cursor);
+      const kvt_ipc_block& b = work[first + i];
+      contig[i] = static_cast<int64_t>(b.src_offset);
       gpu[i] = static_cast<int64_t>(b.dst_offset);
       lens[i] = static_cast<int64_t>(halve ? b.length / 2 : b.length);
-      host_cursor += halve ? b.length / 2 : b.length;
       slices += (b.length + unit - 1) / unit;
     }
     KVT_HIP(hipMemcpyAsync(dev_meta, host_meta, 3 * m * sizeof(int64_t), hipMemcpyHostToDevice, s));
@@ -142,7 +168,7 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
                              static_cast<int64_t>(m), wgs, rows, cap, s);
     if (e != hipSuccess) return hip_fail(e, "copy_handle_data launch");
     // the metadata buffers are reused by the next batch
-    if (first + m < n) KVT_HIP(hipStreamSynchronize(s));
+    if (first + m < n_work) KVT_HIP(hipStreamSynchronize(s));
   }
   return KVT_OK;
 }

@@ -532,12 +532,66 @@ def test_memcpy_route_thresholds_decide_between_dma_and_kernel():
         assert gather_once() is True
         assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 3) == 0
         assert gather_once() is False
-        assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 2) == 0    # one range too many
-        assert gather_once() is True
+        # one range too many for the whole-list rule; the lengths differ, so the per-range rule
+        # of mixed lists still sends each of them to the DMA engines
+        assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 2) == 0
+        assert gather_once() is False
         assert lib.kvt_set_copy_memcpy_thresholds((1 << 20) + 1, 3) == 0   # two ranges too short
         assert gather_once() is True
         assert lib.kvt_set_copy_memcpy_thresholds(1, 0) == 0          # switched off
         assert gather_once() is True
+    finally:
+        assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+
+
+@pytest.mark.parametrize("max_block_num", [0, 2])
+def test_mixed_lists_send_their_long_ranges_to_the_dma_engines(max_block_num):
+    """enqueue_hybrid_copy of the reference (copy_kernels.cpp:675-722): in a list of mixed
+    lengths the ranges at or above the threshold are copied one by one, the kernel gets the
+    rest with their true positions in the contiguous buffer."""
+    lib = kvt_amd.lib()
+    cap = 16 << 20
+    lens = [(1 << 20) + 32, 4096, 2 << 20, 65536 + 5, 4096, 1 << 20]
+    offs = [0, 3 << 20, 4 << 20, 7 << 20, (8 << 20) + 3, 9 << 20]
+    runs = np.array([[0, o, n] for o, n in zip(offs, lens)], dtype=np.uint64)
+    total = int(sum(lens))
+    layer = _dev_bytes(cap, 78, "raw")
+    gather = np.stack([runs[:, 1], runs[:, 1], runs[:, 2]], axis=1)
+    blob = checkers.oracle_pack(_host(layer), gather)
+    dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
+    host_meta = torch.zeros(3 * 8192, dtype=torch.int64).pin_memory()
+    pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
+    s = torch.cuda.Stream()
+    try:
+        assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 16) == 0
+        rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(),
+                                                  runs.ctypes.data, len(runs), total, 1, 0,
+                                                  s.cuda_stream, dev_meta.data_ptr(),
+                                                  host_meta.data_ptr(), max_block_num)
+        assert rc == 0, lib.kvt_last_error()
+        s.synchronize()
+        assert np.array_equal(pinned.numpy(), blob)
+        # the kernel was given the three short ranges only (the last batch is still in the buffer)
+        small = [(sum(lens[:i]), offs[i], lens[i]) for i in (1, 3, 4)]
+        last = small if max_block_num == 0 else small[2:]
+        m = len(last)
+        got = host_meta[:3 * m].numpy().reshape(3, m).T.tolist()
+        assert got == [list(t) for t in last]
+        if max_block_num == 0:
+            assert not host_meta[3 * m:64].any()
+        else:                                     # the batch before it had two ranges
+            assert not host_meta[6:64].any()
+        dst = torch.full((cap,), 0x3C, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), dst.data_ptr(),
+                                                  runs.ctypes.data, len(runs), total, 0, 0,
+                                                  s.cuda_stream, dev_meta.data_ptr(),
+                                                  host_meta.data_ptr(), max_block_num)
+        assert rc == 0, lib.kvt_last_error()
+        s.synchronize()
+        exp = np.full(cap, 0x3C, dtype=np.uint8)
+        checkers.oracle_unpack(exp, gather, blob)
+        assert np.array_equal(_host(dst), exp)
     finally:
         assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
 
