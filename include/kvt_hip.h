@@ -548,7 +548,8 @@ int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats
  * that fills the entries itself. Keys are key_bytes (1..256) each, compared byte for byte.
  * Calls may come from several threads: an entry whose bytes a caller was asked for stays with
  * its key until that caller has written it (save / commit) or given up (release), so EVERY
- * is_new answer must be followed by one of the three; a load can name the keys it expects. */
+ * is_new answer must be followed by exactly one of the three (an answer that is never settled
+ * keeps its entry out of circulation); a load can name the keys it expects. */
 typedef struct kvt_object_ring kvt_object_ring;
 int kvt_object_ring_create(int device, uint64_t entry_bytes, uint32_t n_entries,
                            uint32_t key_bytes, kvt_object_ring** out);

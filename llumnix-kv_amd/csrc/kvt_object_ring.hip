@@ -153,15 +153,13 @@ int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, ui
     const uint64_t call = ++r->calls;
     const char* k = static_cast<const char*>(keys);
     // first the keys that are here already: their entries must survive this call
-    uint32_t fresh = 0, kept = 0;
+    uint32_t fresh = 0;
     std::vector<std::string> ks(n);
     for (uint32_t i = 0; i < n; ++i) {
       ks[i].assign(k + static_cast<size_t>(i) * r->key_bytes, r->key_bytes);
       auto it = r->index.find(ks[i]);
       if (it != r->index.end()) {
-        Entry& e = r->entries[it->second];
-        if (e.touched != call) ++kept;
-        e.touched = call;
+        r->entries[it->second].touched = call;
       }
     }
     {
@@ -174,7 +172,6 @@ int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, ui
     uint32_t available = 0;
     for (const Entry& e : r->entries)
       if (e.touched != call && e.claims == 0) ++available;
-    (void)kept;
     if (fresh > available)
       return fail(KVT_ERR_INVALID,
                   "kvt_object_ring_reserve: more new blocks than entries that may be given away "

@@ -86,11 +86,16 @@ class FileBlockStore:
             entries, new = self._ring.reserve([self._key(h) for _, h in part])
             fresh = [b for (b, _), n in zip(part, new) if n]
             if fresh:
-                objs = torch.empty(len(fresh) * self._entry, dtype=torch.uint8, device="cuda")
-                self._stream.wait_stream(torch.cuda.current_stream())
-                plan = self._plan(fresh)
-                plan.pack(self._cache, 0, len(self._kv), objs, self._obj, self._stream.cuda_stream)
-                self._ring.save(entries[new], objs.data_ptr(), self._entry, self._stream.cuda_stream)
+                try:
+                    objs = torch.empty(len(fresh) * self._entry, dtype=torch.uint8, device="cuda")
+                    self._stream.wait_stream(torch.cuda.current_stream())
+                    plan = self._plan(fresh)
+                    plan.pack(self._cache, 0, len(self._kv), objs, self._obj, self._stream.cuda_stream)
+                    self._ring.save(entries[new], objs.data_ptr(), self._entry,
+                                    self._stream.cuda_stream)
+                except Exception:
+                    self._ring.release(entries[new])    # every "new" answer is settled exactly once
+                    raise
                 self._stream.synchronize()
                 plan.close()
             for (blkid, blkhash), idx in zip(part, entries):
@@ -160,12 +165,16 @@ class FileBlockStore:
                 # every entry this batch refers to is kept by the reservation
                 entries, new = self._ring.reserve(keys)
                 filled = []
-                for i, (idx, n) in enumerate(zip(entries, new)):
-                    if n:
-                        data = np.fromfile(self._path(part[i][1])[1], dtype=np.uint8)
-                        assert data.size == self._entry
-                        self._ring.entry(idx)[:] = data
-                        filled.append(idx)
+                try:
+                    for i, (idx, n) in enumerate(zip(entries, new)):
+                        if n:
+                            data = np.fromfile(self._path(part[i][1])[1], dtype=np.uint8)
+                            assert data.size == self._entry
+                            self._ring.entry(idx)[:] = data
+                            filled.append(idx)
+                except Exception:
+                    self._ring.release(entries[new])
+                    raise
                 self._ring.commit(np.asarray(filled, dtype=np.uint32))
             objs = torch.empty(len(part) * self._entry, dtype=torch.uint8, device="cuda")
             self._stream.wait_stream(torch.cuda.current_stream())
