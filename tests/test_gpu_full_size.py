@@ -156,3 +156,52 @@ def test_config3_full_size_transposing_pack():
             del want, exp, picked
         del src, dst, sc, dc, packed
         torch.cuda.empty_cache()
+
+
+def _run_runs(w, seed):
+    """The same check for a TP-remapping batch through a run plan (the per-token arithmetic
+    evaluated in the kernel): the oracle's per-token lists, unmerged, drive torch's gather and
+    scatter."""
+    plan, runs = pipeline.build_plan_runs(w, 0)
+    o_lists = _oracle_lists(w)
+    assert plan.num_strided_chunks > 0
+    src, dst = _caches(w, seed)
+    sc = kvt_amd.Cache(0, src, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst, w.capacities("dst"))
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, w.n_layers, packed, stride)
+    plan.unpack(dc, 0, w.n_layers, packed, stride)
+    torch.cuda.synchronize()
+    for t in range(w.n_tensors):
+        ranges = o_lists[t]
+        s_idx = torch.from_numpy(_unit_index(ranges[:, 0], ranges[:, 2])).cuda()
+        d_idx = torch.from_numpy(_unit_index(ranges[:, 1], ranges[:, 2])).cuda()
+        assert len(torch.unique(d_idx)) == len(d_idx)
+        nb = int(ranges[:, 2].sum())
+        assert plan.tensor_bytes(t) == nb
+        off = plan.tensor_offset(t)
+        for l in range(w.n_layers):
+            blob = packed[l * stride + off: l * stride + off + nb].view(-1, 16)
+            assert _gathered_equals(src[l][t].view(-1, 16), s_idx, blob), ("pack", l, t)
+            exp = torch.full_like(dst[l][t], 0xA5).view(-1, 16)
+            _scatter(exp, d_idx, blob)
+            assert torch.equal(dst[l][t].view(-1, 16), exp), ("unpack", l, t)
+            del exp
+    return plan, o_lists
+
+
+def test_tp2_to_tp1_batch_full_size_through_a_run_plan():
+    """Config 2's batch sent from TP2 to TP1: 623 786 per-token ranges of 1 KiB per layer,
+    32 layers, 19 GiB payload."""
+    w = workloads.tp_split("flash", 2, 1, 0, n_layers=32, src_pool=16384, dst_pool=24576,
+                           n_req=64, min_tok=1024, max_tok=8192)
+    plan, o_lists = _run_runs(w, 7)
+    assert len(o_lists[0]) > 600000 and plan.num_chunks < 50000
+
+
+def test_hybrid_tp2_to_tp1_full_size_through_a_run_plan():
+    """The hybrid model between a TP2 prefill and a TP1 decode instance at the size of the
+    benchmark (128 requests x 4096 tokens, 12 attention layers with their GDN states)."""
+    w = workloads.qwen3next_tp_split(2, 1, 0, n_layers=12, pool=1024, n_req=128)
+    _run_runs(w, 8)
