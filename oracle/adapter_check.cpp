@@ -148,4 +148,15 @@ int kvtadp_loopback_send(int device, void* const* src_layers, const uint64_t* sr
   }
 }
 
+// The adapter's helper that hands BLLM_KVTRANS_COPY_MEMCPY_* to the library (read from the
+// environment at the time of the call). Returns 0, or 1 when it threw.
+int kvtadp_apply_copy_memcpy_env(void) {
+  try {
+    kvt_adapter::apply_copy_memcpy_env();
+    return 0;
+  } catch (const std::exception&) {
+    return 1;
+  }
+}
+
 }  // extern "C"

@@ -65,3 +65,28 @@ def test_adapter_on_the_golden_cases():
         rc, ref_rc, n = _compare(lib, case)
         assert rc == 0, case["name"]
         assert (ref_rc != 0) == (case["rc"] != 0)
+
+
+def test_adapter_hands_the_memcpy_variables_to_the_library(monkeypatch):
+    """BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES / _MAX_BLOCKS (copy_kernels.cpp:496-499):
+    set values replace the library's thresholds, unset or unparsable ones leave them alone."""
+    lib, k = _lib(), kvt_amd.lib()
+    a, b = C.c_uint64(), C.c_uint64()
+
+    def current():
+        assert k.kvt_get_copy_memcpy_thresholds(C.byref(a), C.byref(b)) == 0
+        return a.value, b.value
+
+    try:
+        monkeypatch.delenv("BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES", raising=False)
+        monkeypatch.delenv("BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS", raising=False)
+        assert lib.kvtadp_apply_copy_memcpy_env() == 0 and current() == (8 << 20, 16)
+        monkeypatch.setenv("BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES", "262144")
+        assert lib.kvtadp_apply_copy_memcpy_env() == 0 and current() == (262144, 16)
+        monkeypatch.setenv("BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS", "4")
+        monkeypatch.setenv("BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES", "12k")   # not a number
+        assert lib.kvtadp_apply_copy_memcpy_env() == 0 and current() == (262144, 4)
+        monkeypatch.setenv("BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS", "0")               # route off
+        assert lib.kvtadp_apply_copy_memcpy_env() == 0 and current() == (262144, 0)
+    finally:
+        assert k.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
