@@ -588,6 +588,16 @@ int kvt_object_ring_load(kvt_object_ring* r, const uint32_t* entries, const void
                          void* dev, uint64_t dev_stride, void* stream);
 /* Host-blocking: the last save / load that touches the entry has completed. */
 int kvt_object_ring_wait(kvt_object_ring* r, uint32_t entry);
+/* Counters since creation (what a store reports as its hit rate and traffic). */
+typedef struct kvt_object_ring_counters {
+  uint64_t blocks_asked_for;      /* is_new answers of reserve                                   */
+  uint64_t blocks_already_here;   /* the other answers: stored, or repeated inside a batch       */
+  uint64_t entries_given_away;    /* stored or reserved keys dropped to make room                */
+  uint64_t lookups_found, lookups_missed;
+  uint64_t bytes_saved, bytes_loaded;   /* through kvt_object_ring_save / _load                  */
+  uint64_t entries_in_use;        /* keys in the index now                                       */
+} kvt_object_ring_counters;
+int kvt_object_ring_stats(kvt_object_ring* r, kvt_object_ring_counters* out);
 
 /* ------------------------------------------------------------- utilities */
 

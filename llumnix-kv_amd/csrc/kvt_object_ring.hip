@@ -53,6 +53,7 @@ struct kvt_object_ring {
   uint64_t calls = 0;
   std::vector<Entry> entries;
   std::unordered_map<std::string, uint32_t> index;
+  kvt_object_ring_counters stats{};   // under mu
 };
 
 namespace {
@@ -187,6 +188,9 @@ int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, ui
         if (is_new[i]) {
           e.flagged = call;
           ++e.claims;
+          ++r->stats.blocks_asked_for;
+        } else {
+          ++r->stats.blocks_already_here;
         }
         continue;
       }
@@ -197,7 +201,11 @@ int kvt_object_ring_reserve(kvt_object_ring* r, const void* keys, uint32_t n, ui
       }
       Entry& e = r->entries[idx];
       if (int rc = wait_entry(e)) return rc;
-      if (!e.key.empty()) r->index.erase(e.key);
+      if (!e.key.empty()) {
+        r->index.erase(e.key);
+        ++r->stats.entries_given_away;
+      }
+      ++r->stats.blocks_asked_for;
       e.key = ks[i];
       e.saved = false;
       e.claims = 1;
@@ -224,6 +232,7 @@ int kvt_object_ring_lookup(kvt_object_ring* r, const void* keys, uint32_t n, uin
       auto it = r->index.find(key);
       found[i] = (it != r->index.end() && r->entries[it->second].saved) ? 1 : 0;
       entries[i] = found[i] ? it->second : 0;
+      ++(found[i] ? r->stats.lookups_found : r->stats.lookups_missed);
     }
     return KVT_OK;
   });
@@ -260,6 +269,14 @@ int kvt_object_ring_release(kvt_object_ring* r, const uint32_t* entries, uint32_
     }
     return KVT_OK;
   });
+}
+
+int kvt_object_ring_stats(kvt_object_ring* r, kvt_object_ring_counters* out) {
+  if (!r || !out) return fail(KVT_ERR_INVALID, "kvt_object_ring_stats: null argument");
+  std::lock_guard<std::mutex> lock(r->mu);
+  *out = r->stats;
+  out->entries_in_use = r->index.size();
+  return KVT_OK;
 }
 
 int kvt_object_ring_wait(kvt_object_ring* r, uint32_t entry) {
@@ -318,6 +335,7 @@ static int transfer(kvt_object_ring* r, const uint32_t* entries, uint32_t n, voi
         return KVT_OK;
       }))
     return rc;
+  (save ? r->stats.bytes_saved : r->stats.bytes_loaded) += static_cast<uint64_t>(n) * r->entry_bytes;
   auto t = std::make_shared<Transfer>();
   KVT_HIP(hipEventCreateWithFlags(&t->done, hipEventDisableTiming));
   KVT_HIP(hipEventRecord(t->done, r->copy));

@@ -100,6 +100,7 @@ SIGNATURES = {
     "kvt_object_ring_load": (_int, [_vp, _vp, _vp, _u32, _vp, _u64, _vp]),
     "kvt_object_ring_release": (_int, [_vp, _vp, _u32]),
     "kvt_object_ring_wait": (_int, [_vp, _u32]),
+    "kvt_object_ring_stats": (_int, [_vp, _vp]),
     "kvt_set_copy_memcpy_thresholds": (_int, [_u64, _u64]),
     "kvt_get_copy_memcpy_thresholds": (_int, [_P(_u64), _P(_u64)]),
     "kvt_set_copy_cu_usage": (_int, [_int, C.c_double]),
@@ -658,6 +659,15 @@ class ObjectRing:
 
     def wait(self, entry):
         check(lib().kvt_object_ring_wait(self.h, int(entry)))
+
+    STATS = ("blocks_asked_for", "blocks_already_here", "entries_given_away", "lookups_found",
+             "lookups_missed", "bytes_saved", "bytes_loaded", "entries_in_use")
+
+    def stats(self):
+        """-> dict of the ring's counters (kvt_object_ring_counters)."""
+        out = (C.c_uint64 * len(self.STATS))()
+        check(lib().kvt_object_ring_stats(self.h, out))
+        return dict(zip(self.STATS, out))
 
     def entry(self, entry):
         """The entry's bytes as a numpy view of the ring's host memory."""

@@ -113,6 +113,11 @@ def test_save_by_hash_skips_stored_blocks_and_load_restores_them_elsewhere():
         for k, d in zip((8, 3, 1, 6), dst_blocks):
             exp[:, d] = kv[l][:, src_block_of[k]]
         assert torch.equal(new_cache[l].view(torch.int16), exp.view(torch.int16)), l
+    st = ring.stats()
+    assert st["bytes_saved"] == 9 * ENTRY and st["bytes_loaded"] == 4 * ENTRY
+    assert st["blocks_asked_for"] == 9 and st["blocks_already_here"] == 2
+    assert st["entries_given_away"] == 1 and st["entries_in_use"] == 8
+    assert st["lookups_found"] == 4 and st["lookups_missed"] == 2
     ring.close()
 
 

@@ -254,3 +254,16 @@ def test_random_traffic_against_the_model(seed):
         e, found = r.lookup(probe)
         assert found.tolist() == m.lookup(probe)
         assert all(m.index[k] == int(idx) for k, idx, f in zip(probe, e, found) if f)
+
+
+def test_counters():
+    r = ring(4)
+    e, _ = r.reserve([key(1), key(2), key(1)])
+    r.commit(e[:2])
+    r.reserve([key(1), key(3)])
+    r.lookup([key(1), key(2), key(3), key(9)])
+    e, _ = r.reserve([key(4), key(5)])          # entry 3, then key 1's entry makes room
+    st = r.stats()
+    assert st == {"blocks_asked_for": 5, "blocks_already_here": 2, "entries_given_away": 1,
+                  "lookups_found": 2, "lookups_missed": 2, "bytes_saved": 0, "bytes_loaded": 0,
+                  "entries_in_use": 4}
