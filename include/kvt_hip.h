@@ -605,6 +605,9 @@ int kvt_object_ring_stats(kvt_object_ring* r, kvt_object_ring_counters* out);
  * shape as the gather kernel; used to calibrate profiler counters and as the
  * "no scatter" bandwidth reference. */
 int kvt_copy_linear(void* dst, const void* src, uint64_t bytes, void* stream);
+/* The HIP runtime's own device-to-device copy (hipMemcpyAsync) of the same bytes: a copy rate
+ * of the part that owes nothing to this library's kernels, timed beside them. */
+int kvt_copy_runtime_d2d(void* dst, const void* src, uint64_t bytes, void* stream);
 /* Average duration in milliseconds of the GPU work queued on `stream` between
  * two internally created events around `fn`-less region helpers: */
 int kvt_event_create(void** ev);

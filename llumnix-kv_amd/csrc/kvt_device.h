@@ -82,6 +82,14 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                               uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs,
                               hipStream_t stream);
+// The capped launch of a plain table with 16-byte aligned entries of at most 16 KiB
+// (sub_shift 2) or 32 KiB (sub_shift 3): `wgs` persistent workgroups (a multiple of 8), one
+// table entry per trip, software-pipelined. Every address and length involved must be a
+// multiple of 16.
+hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                               uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                               uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                               const BlobOffsets& blobs, uint32_t wgs, hipStream_t stream);
 hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

@@ -15,6 +15,7 @@
 // rows that are contiguous on both sides, so it is a pure index permutation.
 #include <hip/hip_runtime.h>
 
+#include <cstddef>
 #include <cstdint>
 
 #include "kvt_device.h"
@@ -32,25 +33,34 @@ __device__ __forceinline__ uint32_t xcd_remap(uint32_t b, uint32_t n) {
   return (b & 7u) * per + (b >> 3);
 }
 
-// Which (slice, layer) items a workgroup handles. The normal launch has one workgroup per
-// item: grid (slices rounded up to 8, layers). A launch capped to a share of the device
-// (CAPPED) has a one-dimensional grid of that many workgroups, a multiple of 8, which stride
-// over the same items layer by layer; since the stride and the rounded slice count are both
-// multiples of 8, a workgroup keeps meeting slices of the eighth that belongs to its XCD.
-template <bool CAPPED, class Body>
-__device__ __forceinline__ void for_items(uint32_t n_slices, uint32_t n_layers, Body body) {
-  if (!CAPPED) {
-    body(xcd_remap(blockIdx.x, n_slices), static_cast<uint32_t>(blockIdx.y));
-    return;
-  }
-  const uint32_t per_layer = (n_slices + 7u) & ~7u;
-  uint32_t layer = 0;
-  for (uint32_t s = blockIdx.x;; s += gridDim.x) {
-    while (s >= per_layer) {
-      s -= per_layer;
-      if (++layer >= n_layers) return;
-    }
-    body(xcd_remap(s, n_slices), layer);
+// Every pointer a kernel here follows is device-visible global memory, also where the
+// compiler cannot tell (layer pointers are loaded from a table): saying so gives global
+// instead of generic ("flat") memory instructions.
+typedef __attribute__((address_space(1))) u32x4 g_u32x4;
+__device__ __forceinline__ u32x4 load_vec(const uint8_t* p) {
+  return __builtin_nontemporal_load((const g_u32x4*)(p));
+}
+__device__ __forceinline__ void store_vec(uint8_t* p, u32x4 v) {
+  __builtin_nontemporal_store(v, (g_u32x4*)(p));
+}
+
+// Copies len (<= 4096) bytes with the whole workgroup when the two sides are not both
+// 16-byte aligned: 4-byte words where possible, else bytes.
+__device__ __forceinline__ void copy_slice_odd(uint8_t* __restrict__ dst,
+                                               const uint8_t* __restrict__ src, uint32_t len,
+                                               uint32_t tid) {
+  const uintptr_t mis = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
+  if ((mis & 3u) == 0) {
+    const uint32_t nw = len >> 2;
+    const uint32_t* __restrict__ s = reinterpret_cast<const uint32_t*>(src);
+    uint32_t* __restrict__ d = reinterpret_cast<uint32_t*>(dst);
+#pragma clang loop vectorize(disable) unroll(disable)
+    for (uint32_t i = tid; i < nw; i += kThreads) d[i] = s[i];
+    const uint32_t done = nw << 2;
+    if (tid < len - done) dst[done + tid] = src[done + tid];
+  } else {
+#pragma clang loop vectorize(disable) unroll(disable)
+    for (uint32_t j = tid; j < len; j += kThreads) dst[j] = src[j];
   }
 }
 
@@ -60,71 +70,266 @@ __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst,
                                            const uint8_t* __restrict__ src, uint32_t len,
                                            uint32_t tid) {
   const uintptr_t mis = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src);
-  if ((mis & 15u) == 0) {
-    const uint32_t nvec = len >> 4;
-    if (tid < nvec)
-      __builtin_nontemporal_store(
-          __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + tid),
-          reinterpret_cast<u32x4*>(dst) + tid);
-    const uint32_t done = nvec << 4;
-    if (tid < len - done) dst[done + tid] = src[done + tid];
-  } else if ((mis & 3u) == 0) {
-    const uint32_t nw = len >> 2;
-    const uint32_t* __restrict__ s = reinterpret_cast<const uint32_t*>(src);
-    uint32_t* __restrict__ d = reinterpret_cast<uint32_t*>(dst);
-    for (uint32_t i = tid; i < nw; i += kThreads) d[i] = s[i];
-    const uint32_t done = nw << 2;
-    if (tid < len - done) dst[done + tid] = src[done + tid];
-  } else {
-    for (uint32_t j = tid; j < len; j += kThreads) dst[j] = src[j];
+  if ((mis & 15u) != 0) return copy_slice_odd(dst, src, len, tid);
+  const uint32_t nvec = len >> 4;
+  if (tid < nvec) store_vec(dst + (tid << 4), load_vec(src + (tid << 4)));
+  const uint32_t done = nvec << 4;
+  if (tid < len - done) dst[done + tid] = src[done + tid];
+}
+
+// ------------------------------------------------------------ chunk kernels
+//
+// Workgroup item b of a layer handles slice (b & mask) of table entry (b >> sub_shift);
+// entries hold at most 4096 << sub_shift bytes, so a shorter one simply leaves its last
+// workgroups idle. The normal launch has one workgroup per (slice, layer) item: grid (slices
+// rounded up to 8, layers). A launch capped to a share of the device (CAPPED) has a
+// one-dimensional grid of that many workgroups, a multiple of 8, which stride over the same
+// items layer by layer; since the stride and the rounded slice count are both multiples of 8,
+// a workgroup keeps meeting slices of the eighth that belongs to its XCD.
+//
+// A capped workgroup is persistent, and with one 16-byte vector per lane in flight its rate
+// would follow the number of resident wavefronts (half the wave slots, half the rate), each
+// item paying for three dependent loads in a row (table entry, layer pointer, data). So it
+// takes kBatch items per trip in phases: the kBatch table entries (independent scalar
+// loads), then the kBatch layer pointers, then the lanes' addresses, then the kBatch vector
+// loads back to back and only then the stores: a lane has kBatch x 16 bytes in flight.
+
+constexpr int kBatch = 4;
+
+// The uniform arguments of a chunk launch.
+struct Launch {
+  uint32_t n_slices, sub_shift;
+  uint8_t* const* layer_ptrs;
+  uint32_t n_tensors, first_layer, n_layers;
+  uint8_t* packed;
+  uint64_t layer_stride;
+  const BlobOffsets* blobs;
+};
+
+// A table entry as the kernels read it: the Chunk's two 16-bit fields as one word (a 16-bit
+// field would be fetched with a vector load, everything else here with scalar loads).
+struct __attribute__((may_alias, aligned(16))) Entry {
+  uint64_t cache, packed;
+  uint32_t len, tensor_t0, shape, reserved;
+  __device__ __forceinline__ uint32_t tensor() const { return tensor_t0 & 0xFFFFu; }
+  __device__ __forceinline__ uint32_t t0() const { return tensor_t0 >> 16; }
+};
+static_assert(sizeof(Entry) == sizeof(Chunk) && offsetof(Chunk, tensor) == offsetof(Entry, tensor_t0) &&
+                  offsetof(Chunk, t0) == offsetof(Entry, tensor_t0) + 2 &&
+                  offsetof(Chunk, shape) == offsetof(Entry, shape),
+              "Entry must mirror Chunk");
+
+// One (slice, layer) item, uniform across the workgroup.
+struct Item {
+  Entry c;
+  uint8_t* cache;  // the layer tensor's base + c.cache
+  uint8_t* pk;     // where the entry's packed bytes start in this layer
+  uint32_t sub;    // slice index inside the entry
+};
+
+// One lane's vector move: uniform base addresses (they stay in scalar registers) plus the
+// lane's byte offsets. `on` = the lane has a vector to move.
+struct Move {
+  const uint8_t* src;
+  uint8_t* dst;
+  uint64_t src_off, dst_off;
+  bool on;
+};
+#define KVT_NO_MOVE (Move{nullptr, nullptr, 0, 0, false})
+
+// `fetch(entry)` reads a table entry; `place(item)` turns an item into the lane's move. Odd
+// cases (misaligned slices, stragglers behind the last whole vector) `place` may move itself.
+template <bool CAPPED, class Fetch, class Place>
+__device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place place) {
+  if (!CAPPED) {
+    // no branch before the last scalar load has been issued: a workgroup's life is three
+    // dependent round trips (arguments, table entry, layer pointer) and then its vector
+    const uint32_t b = xcd_remap(blockIdx.x, L.n_slices), layer = blockIdx.y;
+    const uint32_t bc = min(b, L.n_slices - 1u);
+    Item it;
+    it.c = fetch(bc >> L.sub_shift);
+    it.sub = bc & ((1u << L.sub_shift) - 1u);
+    it.cache = L.layer_ptrs[static_cast<uint64_t>(L.first_layer + layer) * L.n_tensors + it.c.tensor()] +
+               it.c.cache;
+    it.pk = L.packed + layer * L.layer_stride + L.blobs->off[it.c.tensor()] + it.c.packed;
+    if (b >= L.n_slices) return;
+    const Move m = place(it);
+    if (m.on) store_vec(m.dst + m.dst_off, load_vec(m.src + m.src_off));
+    return;
+  }
+  // lanes without a vector load from here: the layer pointer table, at least 16 bytes long
+  const uint8_t* const idle = reinterpret_cast<const uint8_t*>(L.layer_ptrs);
+  const uint32_t per_layer = (L.n_slices + 7u) & ~7u;
+  const uint32_t d_layer = gridDim.x / per_layer, d_slice = gridDim.x - d_layer * per_layer;
+  uint32_t layer = blockIdx.x / per_layer, s = blockIdx.x - layer * per_layer;
+  while (layer < L.n_layers) {
+    Item it[kBatch];
+    uint32_t lay[kBatch];
+    bool valid[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {  // which items, and their table entries
+      const uint32_t b = xcd_remap(s, L.n_slices);
+      valid[j] = layer < L.n_layers && b < L.n_slices;
+      lay[j] = min(layer, L.n_layers - 1u);
+      const uint32_t bc = min(b, L.n_slices - 1u);
+      it[j].c = fetch(bc >> L.sub_shift);
+      it[j].sub = bc & ((1u << L.sub_shift) - 1u);
+      s += d_slice;
+      layer += d_layer;
+      if (s >= per_layer) {
+        s -= per_layer;
+        ++layer;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {  // their layer tensors
+      it[j].cache =
+          L.layer_ptrs[static_cast<uint64_t>(L.first_layer + lay[j]) * L.n_tensors + it[j].c.tensor()] +
+          it[j].c.cache;
+      it[j].pk = L.packed + lay[j] * L.layer_stride + L.blobs->off[it[j].c.tensor()] + it[j].c.packed;
+    }
+    Move m[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      m[j] = KVT_NO_MOVE;
+      if (valid[j]) m[j] = place(it[j]);
+    }
+    u32x4 r[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) r[j] = load_vec(m[j].on ? m[j].src + m[j].src_off : idle);
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j)
+      if (m[j].on) store_vec(m[j].dst + m[j].dst_off, r[j]);
   }
 }
 
-// Gather (PACK) / scatter of a resident chunk table. Workgroup b handles slice
-// (b & mask) of chunk (b >> sub_shift); chunks are at most 4096 << sub_shift
-// bytes, so a chunk shorter than that simply leaves its last workgroups idle.
+// The lane's share of one contiguous slice: `on` when the slice is 16-byte aligned on both
+// sides and the lane has a whole vector of it; stragglers behind the last whole vector and
+// slices that are not aligned are moved here.
+__device__ __forceinline__ Move slice_move(uint8_t* d, const uint8_t* s, uint32_t len) {
+  const uint32_t tid = threadIdx.x;
+  const uintptr_t mis = reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(s);
+  if ((mis & 15u) != 0) {
+    copy_slice_odd(d, s, len, tid);
+    return KVT_NO_MOVE;
+  }
+  const uint32_t nvec = len >> 4, done = nvec << 4;
+  if (tid < len - done) d[done + tid] = s[done + tid];
+  return Move{s, d, tid << 4, tid << 4, tid < nvec};
+}
+
+template <bool PACK>
+__device__ __forceinline__ Move plain_move(const Item& it) {
+  const uint32_t off = it.sub << kSliceShift;
+  const uint32_t len = off < it.c.len ? min(kSlice, it.c.len - off) : 0u;  // 0: an idle workgroup
+  uint8_t* cache = it.cache + off;
+  uint8_t* pk = it.pk + off;
+  return slice_move(PACK ? pk : cache, PACK ? cache : pk, len);
+}
+
+#define KVT_LAUNCH_STRUCT \
+  const Launch L{n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, &blobs}
+
+// Gather (PACK) / scatter of a resident chunk table.
 template <bool PACK, bool CAPPED>
-__global__ __launch_bounds__(kThreads) void copy_chunks_kernel(
+__global__ __launch_bounds__(kThreads, 8) void copy_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
-  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
-    if (b >= n_slices) return;
-    const Chunk c = chunks[b >> sub_shift];
-    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-    if (off >= c.len) return;
-    const uint32_t len = min(kSlice, c.len - off);
-    uint8_t* cache =
-        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache + off;
-    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-    if (PACK)
-      copy_slice(pk, cache, len, threadIdx.x);
-    else
-      copy_slice(cache, pk, len, threadIdx.x);
-  });
+  KVT_LAUNCH_STRUCT;
+  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; },
+                    [&](const Item& it) { return plain_move<PACK>(it); });
 }
 
 // The same for a table short enough to be a kernel argument (read through the scalar cache
 // like any other argument; the index is uniform across the workgroup).
 template <bool PACK, bool CAPPED>
-__global__ __launch_bounds__(kThreads) void copy_chunks_small_kernel(
+__global__ __launch_bounds__(kThreads, 8) void copy_chunks_small_kernel(
     const SmallTable table, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
-  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
-    if (b >= n_slices) return;
-    const Chunk& c = table.c[b >> sub_shift];
-    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-    if (off >= c.len) return;
-    const uint32_t len = min(kSlice, c.len - off);
-    uint8_t* cache =
-        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache + off;
-    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-    if (PACK)
-      copy_slice(pk, cache, len, threadIdx.x);
-    else
-      copy_slice(cache, pk, len, threadIdx.x);
-  });
+  KVT_LAUNCH_STRUCT;
+  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(table.c)[e]; },
+                    [&](const Item& it) { return plain_move<PACK>(it); });
+}
+
+// The capped launch of a plain table whose entries are whole multiples of 16 bytes, 16-byte
+// aligned on both sides, and 16 or 32 KiB at most (V = 4 or 8 slices): persistent workgroups
+// again, but one table ENTRY per trip -- one descriptor fetch and one pair of buffer
+// descriptors for up to 32 KiB, V vectors per lane -- and software-pipelined over three
+// register sets: the loads of entry k+1 are issued before the stores of entry k, and a set is
+// loaded again only two trips after its stores were issued, so that a wave does not sit out
+// the acknowledgement of stores it has just issued (one counter covers a wave's loads and
+// stores, in issue order). Lanes beyond an entry's length are switched off by the
+// descriptor's range check (loads return zero, stores are dropped), so the loop has no
+// branch but its exit. Entries of a layer are dealt to the XCDs in eighths like the slices of
+// the other kernels, neighbouring workgroups of an XCD taking neighbouring entries.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const uint8_t* base, uint32_t bytes) {
+  // raw buffer of `bytes` bytes, no stride, no swizzle; 0x00020000: 32-bit data format
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(base), 0, bytes, 0x00020000);
+}
+constexpr int kNonTemporal = 2;  // cache-policy operand of the buffer builtins: the nt bit
+
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
+  const uint32_t per8 = (n_chunks + 7u) >> 3;
+  const uint32_t xcd = blockIdx.x & 7u;
+  const uint32_t nloc = gridDim.x >> 3;  // workgroups per XCD
+  const uint32_t step_layer = nloc / per8, step_within = nloc - step_layer * per8;
+  uint32_t layer = (blockIdx.x >> 3) / per8, within = (blockIdx.x >> 3) - layer * per8;
+  const uint32_t off = threadIdx.x << 4;
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  // this workgroup's next entry as two descriptors (empty ones past the end); false past the end
+  auto next = [&](rsrc_t& src, rsrc_t& dst) -> bool {
+    const bool live = layer < n_layers;
+    const uint32_t b = xcd * per8 + within;
+    const bool valid = live && b < n_chunks;
+    const uint32_t lay = min(layer, n_layers - 1u);
+    const Entry c = table[min(b, n_chunks - 1u)];
+    uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
+    uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed;
+    const uint32_t bytes = valid ? c.len : 0u;
+    src = make_rsrc(PACK ? cache : pk, bytes);
+    dst = make_rsrc(PACK ? pk : cache, bytes);
+    within += step_within;
+    layer += step_layer;
+    const bool wrap = within >= per8;
+    within -= wrap ? per8 : 0u;
+    layer += wrap ? 1u : 0u;
+    return live;
+  };
+  auto load = [&](rsrc_t src, u32x4* r) {
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      r[v] = __builtin_amdgcn_raw_buffer_load_b128(src, off + (v << kSliceShift), 0, kNonTemporal);
+  };
+  auto store = [&](rsrc_t dst, const u32x4* r) {
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      __builtin_amdgcn_raw_buffer_store_b128(r[v], dst, off + (v << kSliceShift), 0, kNonTemporal);
+  };
+  rsrc_t s0, d0, s1, d1, s2, d2;
+  u32x4 r0[V], r1[V], r2[V];
+  if (!next(s0, d0)) return;
+  load(s0, r0);
+  for (;;) {
+    const bool l1 = next(s1, d1);
+    load(s1, r1);
+    store(d0, r0);
+    if (!l1) break;
+    const bool l2 = next(s2, d2);
+    load(s2, r2);
+    store(d1, r1);
+    if (!l2) break;
+    const bool l0 = next(s0, d0);
+    load(s0, r0);
+    store(d2, r2);
+    if (!l0) break;
+  }
 }
 
 // Gather / scatter of a table whose chunks may be strided on the cache side:
@@ -137,58 +342,47 @@ __global__ __launch_bounds__(kThreads) void copy_chunks_small_kernel(
 // WORDS = true moves 4-byte words instead (a blob inside a received layer
 // message sits at 4 or 12 modulo 16; that path is PCIe-bound anyway).
 template <bool PACK, bool WORDS, bool CAPPED>
-__global__ __launch_bounds__(kThreads) void strided_chunks_kernel(
+__global__ __launch_bounds__(kThreads, 8) void strided_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     StrideTable shapes) {
-  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
-    if (b >= n_slices) return;
-    const Chunk c = chunks[b >> sub_shift];
-    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-    if (off >= c.len) return;
-    const uint32_t len = min(kSlice, c.len - off);
-    uint8_t* cache =
-        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
-    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-    if (c.shape == 0) {
-      if (PACK)
-        copy_slice(pk, cache + off, len, threadIdx.x);
-      else
-        copy_slice(cache + off, pk, len, threadIdx.x);
-      return;
-    }
-    const StrideShape& s = shapes.shape[c.shape - 1u];
+  KVT_LAUNCH_STRUCT;
+  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; }, [&](const Item& it) -> Move {
+    if (it.c.shape == 0) return plain_move<PACK>(it);
+    const uint32_t off = it.sub << kSliceShift;
+    if (off >= it.c.len) return KVT_NO_MOVE;
+    const uint32_t len = min(kSlice, it.c.len - off);
+    uint8_t* cache = it.cache;
+    uint8_t* pk = it.pk + off;
+    const StrideShape& s = shapes.shape[it.c.shape - 1u];
     const uint64_t outer = s.outer[PACK ? 0 : 1], inner = s.inner[PACK ? 0 : 1];
     if (!WORDS) {
-      if (threadIdx.x >= (len >> 4)) return;
       const uint32_t v = (off >> 4) + threadIdx.x;  // vector index inside the chunk, < 2^15
       const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
       const uint32_t col = v - rec * s.vlen;
       const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
       const uint32_t i = rec - o * s.n_inner;
-      u32x4* cv = reinterpret_cast<u32x4*>(cache + o * outer + i * inner + (col << 4));
-      u32x4* pv = reinterpret_cast<u32x4*>(pk) + threadIdx.x;
-      if (PACK)
-        __builtin_nontemporal_store(__builtin_nontemporal_load(cv), pv);
-      else
-        __builtin_nontemporal_store(__builtin_nontemporal_load(pv), cv);
-    } else {
-      const uint32_t wlen = s.vlen << 2;  // record length in words, < 1024
-      for (uint32_t t = threadIdx.x; t < (len >> 2); t += kThreads) {
-        const uint32_t w = (off >> 2) + t;          // word index inside the chunk, < 2^17
-        const uint32_t rec = __umulhi(w, s.inv_wlen);
-        const uint32_t col = w - rec * wlen;
-        const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
-        const uint32_t i = rec - o * s.n_inner;
-        uint32_t* cw = reinterpret_cast<uint32_t*>(cache + o * outer + i * inner + (col << 2));
-        uint32_t* pw = reinterpret_cast<uint32_t*>(pk) + t;
-        if (PACK)
-          *pw = *cw;
-        else
-          *cw = *pw;
-      }
+      const uint64_t cv = o * outer + i * inner + (col << 4), pv = threadIdx.x << 4;
+      return Move{PACK ? cache : pk, PACK ? pk : cache, PACK ? cv : pv, PACK ? pv : cv,
+                  threadIdx.x < (len >> 4)};
     }
+    const uint32_t wlen = s.vlen << 2;  // record length in words, < 1024
+#pragma clang loop vectorize(disable) unroll(disable)
+    for (uint32_t t = threadIdx.x; t < (len >> 2); t += kThreads) {
+      const uint32_t w = (off >> 2) + t;          // word index inside the chunk, < 2^17
+      const uint32_t rec = __umulhi(w, s.inv_wlen);
+      const uint32_t col = w - rec * wlen;
+      const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
+      const uint32_t i = rec - o * s.n_inner;
+      uint32_t* cw = reinterpret_cast<uint32_t*>(cache + o * outer + i * inner + (col << 2));
+      uint32_t* pw = reinterpret_cast<uint32_t*>(pk) + t;
+      if (PACK)
+        *pw = *cw;
+      else
+        *cw = *pw;
+    }
+    return KVT_NO_MOVE;
   });
 }
 
@@ -197,30 +391,23 @@ __global__ __launch_bounds__(kThreads) void strided_chunks_kernel(
 // contiguous from c.packed; cache side: [head][ntpb][row]. Lane v of the chunk
 // moves the v-th 16-byte vector of the packed side; a row is vrow vectors.
 template <bool PACK, bool CAPPED>
-__global__ __launch_bounds__(kThreads) void xform_chunks_kernel(
+__global__ __launch_bounds__(kThreads, 8) void xform_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     XformDev x) {
-  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
-    if (b >= n_slices) return;
-    const Chunk c = chunks[b >> sub_shift];
-    const uint32_t v = ((b & ((1u << sub_shift) - 1u)) << 8) + threadIdx.x;  // 256 vectors per slice
-    if (v >= (c.len >> 4)) return;
-    u32x4* cv = reinterpret_cast<u32x4*>(
-        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache);
-    u32x4* pv =
-        reinterpret_cast<u32x4*>(packed + layer * layer_stride + blobs.off[c.tensor] + c.packed);
+  KVT_LAUNCH_STRUCT;
+  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; }, [&](const Item& it) -> Move {
+    const uint32_t v = (it.sub << 8) + threadIdx.x;  // 256 vectors per slice
     // exact quotients by multiply-high (operands < 2^16); a divisor of 1 has no such constant
     const uint32_t r = x.vrow == 1 ? v : __umulhi(v, x.inv_vrow);  // packed-side row: t_local*heads + h
     const uint32_t col = v - r * x.vrow;
     const uint32_t t_local = x.heads == 1 ? r : __umulhi(r, x.inv_heads);
     const uint32_t h = r - t_local * x.heads;
-    const uint32_t cidx = (h * x.ntpb + c.t0 + t_local) * x.vrow + col;
-    if (PACK)
-      __builtin_nontemporal_store(__builtin_nontemporal_load(cv + cidx), pv + v);
-    else
-      __builtin_nontemporal_store(__builtin_nontemporal_load(pv + v), cv + cidx);
+    const uint32_t cidx = (h * x.ntpb + it.c.t0() + t_local) * x.vrow + col;
+    const uint64_t cv = static_cast<uint64_t>(cidx) << 4, pv = v << 4;
+    return Move{PACK ? it.cache : it.pk, PACK ? it.pk : it.cache, PACK ? cv : pv, PACK ? pv : cv,
+                v < (it.c.len >> 4)};
   });
 }
 
@@ -322,53 +509,53 @@ __global__ __launch_bounds__(kThreads) void convert_ranges_kernel(
 // 2e. One workgroup converts 4096 elements (8 KiB in, 4 KiB out), 16 per lane. Strided
 // chunks (shape != 0) are 16-byte aligned on both sides by construction.
 template <bool CAPPED>
-__global__ __launch_bounds__(kThreads) void convert_chunks_kernel(
+__global__ __launch_bounds__(kThreads, 8) void convert_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     StrideTable shapes) {
-  for_items<CAPPED>(n_slices, n_layers, [&](uint32_t b, uint32_t layer) {
-    if (b >= n_slices) return;
-    const Chunk c = chunks[b >> sub_shift];
-    const uint32_t off = (b & ((1u << sub_shift) - 1u)) << kSliceShift;
-    if (off >= c.len) return;
-    const uint32_t len = min(kSlice, c.len - off);
-    const uint8_t* cache =
-        layer_ptrs[static_cast<uint64_t>(first_layer + layer) * n_tensors + c.tensor] + c.cache;
-    uint8_t* pk = packed + layer * layer_stride + blobs.off[c.tensor] + c.packed + off;
-    const u32x4* sv;
-    if (c.shape == 0) {
+  KVT_LAUNCH_STRUCT;
+  // two loads and a conversion per store: `place` moves everything itself
+  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; }, [&](const Item& it) -> Move {
+    const uint32_t off = it.sub << kSliceShift;
+    if (off >= it.c.len) return KVT_NO_MOVE;
+    const uint32_t len = min(kSlice, it.c.len - off);
+    const uint8_t* cache = it.cache;
+    uint8_t* pk = it.pk + off;
+    const uint8_t* sv;
+    if (it.c.shape == 0) {
       const uint8_t* s8 = cache + 2ull * off;
       if (((reinterpret_cast<uintptr_t>(s8) | reinterpret_cast<uintptr_t>(pk)) & 15u) != 0) {
         const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s8);
         for (uint32_t j = threadIdx.x; j < len; j += kThreads)
           pk[j] = static_cast<uint8_t>(bf16_to_e4m3(s16[j]));
-        return;
+        return KVT_NO_MOVE;
       }
       const uint32_t done = (len >> 4) << 4;
       if (threadIdx.x < len - done)
         pk[done + threadIdx.x] = static_cast<uint8_t>(
             bf16_to_e4m3(reinterpret_cast<const uint16_t*>(s8)[done + threadIdx.x]));
-      if (threadIdx.x >= (len >> 4)) return;
-      sv = reinterpret_cast<const u32x4*>(s8) + 2 * threadIdx.x;
+      if (threadIdx.x >= (len >> 4)) return KVT_NO_MOVE;
+      sv = s8 + (threadIdx.x << 5);
     } else {
-      if (threadIdx.x >= (len >> 4)) return;
-      const StrideShape& s = shapes.shape[c.shape - 1u];
+      if (threadIdx.x >= (len >> 4)) return KVT_NO_MOVE;
+      const StrideShape& s = shapes.shape[it.c.shape - 1u];
       const uint32_t v = (off >> 4) + threadIdx.x;  // output vector index inside the chunk
       const uint32_t rec = s.vlen == 1 ? v : __umulhi(v, s.inv_vlen);
       const uint32_t col = v - rec * s.vlen;
       const uint32_t o = s.n_inner == 1 ? rec : (s.n_inner == 2 ? rec >> 1 : rec / s.n_inner);
       const uint32_t i = rec - o * s.n_inner;
-      sv = reinterpret_cast<const u32x4*>(cache + o * s.outer[0] + i * s.inner[0] + (col << 5));
+      sv = cache + o * s.outer[0] + i * s.inner[0] + (col << 5);
     }
-    const u32x4 lo = __builtin_nontemporal_load(sv);
-    const u32x4 hi = __builtin_nontemporal_load(sv + 1);
+    const u32x4 lo = load_vec(sv);
+    const u32x4 hi = load_vec(sv + 16);
     u32x4 r;
     r.x = cvt4(lo.x, lo.y);
     r.y = cvt4(lo.z, lo.w);
     r.z = cvt4(hi.x, hi.y);
     r.w = cvt4(hi.z, hi.w);
-    __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(pk) + threadIdx.x);
+    store_vec(pk + (threadIdx.x << 4), r);
+    return KVT_NO_MOVE;
   });
 }
 
@@ -418,6 +605,25 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
   else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, true>), KVT_ARGS);
   else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, false>), KVT_ARGS);
   else KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, true>), KVT_ARGS);
+#undef KVT_ARGS
+  return hipGetLastError();
+}
+
+hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                               uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                               uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                               const BlobOffsets& blobs, uint32_t wgs, hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  if ((sub_shift != 2 && sub_shift != 3) || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+  const dim3 grid(wgs), block(kThreads);
+#define KVT_ARGS chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+  if (sub_shift == 3) {
+    if (pack) hipLaunchKernelGGL((copy_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((copy_entries_kernel<false, 8>), grid, block, 0, stream, KVT_ARGS);
+  } else {
+    if (pack) hipLaunchKernelGGL((copy_entries_kernel<true, 4>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((copy_entries_kernel<false, 4>), grid, block, 0, stream, KVT_ARGS);
+  }
 #undef KVT_ARGS
   return hipGetLastError();
 }

@@ -33,6 +33,8 @@ int check_device(int device);
 // The most workgroups one copy launch may use on `device`, or 0 for no limit
 // (kvt_set_copy_cu_usage).
 uint32_t copy_wg_cap(int device);
+// Compute units of `device` (0 when unknown).
+uint32_t device_cu_count(int device);
 
 // KVT_OK when [ptr, ptr + bytes) is, as far as the runtime can tell, memory the device may
 // touch; KVT_ERR_INVALID / KVT_ERR_OUT_OF_RANGE (message set, starting with `what`) otherwise.
@@ -224,6 +226,7 @@ struct kvt_plan {
   kvt::StrideTable shapes{};
   uint64_t n_strided = 0;
   bool convert = false;            // pack converts bf16 -> fp8: lengths count fp8 bytes (elements)
+  bool all16 = false;              // every entry's offsets and length are multiples of 16 bytes
   std::vector<kvt::Chunk> host_table;   // device == KVT_DEVICE_NONE only: the tables, kept on the host
   uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
   // plain plans of at most kSmallTable entries: both tables kept here and passed to the

@@ -55,6 +55,22 @@ uint32_t copy_wg_cap(int device) {
   return device >= 0 && device < kMaxDevices ? g_wg_cap[device].load(std::memory_order_relaxed) : 0;
 }
 
+uint32_t device_cu_count(int device) {
+  static std::atomic<uint32_t> cached[kMaxDevices];
+  if (device < 0 || device >= kMaxDevices) return 0;
+  uint32_t n = cached[device].load(std::memory_order_relaxed);
+  if (n == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) {
+      (void)hipGetLastError();
+      return 0;
+    }
+    n = cus > 0 ? static_cast<uint32_t>(cus) : 0u;
+    cached[device].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
 // A kernel that runs past a buffer takes a GPU memory fault, which can cost the whole
 // process (and more) instead of an error code. What the runtime knows about a pointer is
 // therefore checked on the host before a launch uses it: it must be memory the device can
@@ -178,7 +194,8 @@ int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, u
                                          " tensor " + std::to_string(i % n_tensors)))
         return rc;
     }
-    KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c->dev_ptrs), n * sizeof(void*)));
+    // at least one 16-byte vector long: idle lanes of a capped launch load from its start
+    KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c->dev_ptrs), std::max<uint64_t>(16, n * sizeof(void*))));
     const hipError_t e =
         hipMemcpy(c->dev_ptrs, c->host_ptrs.data(), n * sizeof(void*), hipMemcpyHostToDevice);
     if (e != hipSuccess) {
@@ -204,6 +221,16 @@ int kvt_copy_linear(void* dst, const void* src, uint64_t bytes, void* stream) {
     if (bytes > (0x7FFFFFF0ull << 12)) return fail(KVT_ERR_INVALID, "kvt_copy_linear: too large");
     const hipError_t e = launch_copy_linear(dst, src, bytes, static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(e, "linear copy launch");
+    return KVT_OK;
+  });
+}
+
+int kvt_copy_runtime_d2d(void* dst, const void* src, uint64_t bytes, void* stream) {
+  return guarded([&]() -> int {
+    if ((!dst || !src) && bytes) return fail(KVT_ERR_INVALID, "kvt_copy_runtime_d2d: null argument");
+    if (usable_devices() <= 0) return fail(KVT_ERR_NO_DEVICE, "no usable gfx950 (MI355X) device");
+    if (bytes == 0) return KVT_OK;
+    KVT_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
     return KVT_OK;
   });
 }

@@ -130,6 +130,7 @@ SIGNATURES = {
     "kvt_stager_wait": (_int, [_vp, _u32]),
     "kvt_measure_pcie": (_int, [_int, _int, _u64, _u32, _P(C.c_double)]),
     "kvt_copy_linear": (_int, [_vp, _vp, _u64, _vp]),
+    "kvt_copy_runtime_d2d": (_int, [_vp, _vp, _u64, _vp]),
     "kvt_event_create": (_int, [_P(_vp)]),
     "kvt_event_destroy": (_int, [_vp]),
     "kvt_event_record": (_int, [_vp, _vp]),
