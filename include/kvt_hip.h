@@ -406,9 +406,10 @@ int kvt_get_copy_memcpy_thresholds(uint64_t* min_range_bytes, uint64_t* max_rang
 
 enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
 /* stands in for initialize_copy_method_profile() kvtransfer/include/copy_kernels.h:15-22
- * (called once per copy thread, kvtransfer/src/copy_utils.cpp:52). There is
- * nothing to measure at start-up here; the call checks that `device` is a usable
- * gfx950 part and returns. */
+ * (called once per copy thread, kvtransfer/src/copy_utils.cpp:52). Checks that `device` is a
+ * usable gfx950 part and looks up the address of that device's static metadata array (see
+ * kvt_copy_handle_data_kernel_direct_static; otherwise done by that entry point's first call
+ * on the device). */
 int kvt_initialize_copy_method_profile(int device);
 /* replaces get_kernel_copy_buffer()             kvtransfer/include/copy_utils.h:127,
  *                                               kvtransfer/src/copy_utils.cpp:9-57,137-146
@@ -456,6 +457,23 @@ int kvt_copy_handle_data_kernel_direct(void* tensor_buf, void* layer_gpu_ptr,
                                        void* stream, int64_t* src_offsets_dev,
                                        int64_t* dst_offsets_dev, int64_t* lengths_dev,
                                        int64_t* host_meta, int use_explicit_host_offsets);
+/* No counterpart in the reference. kvt_copy_handle_data_kernel_direct for callers that cannot
+ * allocate device memory or hand over a device workspace (code under hipGraph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the three device-side metadata arrays live
+ * in a 192 KiB array that is part of the library's code object (one copy per GPU, held until
+ * the process ends), so the caller passes inputs, outputs and the pinned host_meta staging
+ * area (3 n int64) only. The call allocates and frees nothing, on the host side of the
+ * runtime or the device: the metadata is brought over by a copy kernel reading host_meta.
+ * At most 8192 ranges per call: more are refused with KVT_ERR_INVALID. All calls on one GPU
+ * share that GPU's array, which keeps the last call's metadata until the next one overwrites
+ * it: calls whose execution may overlap on one GPU (different streams, or the same graph
+ * launched twice at once) race; calls on one stream do not. host_meta must stay untouched
+ * until the stream has run the copy. Errors as kvt_copy_handle_data_kernel_direct. */
+int kvt_copy_handle_data_kernel_direct_static(void* tensor_buf, void* layer_gpu_ptr,
+                                              const kvt_ipc_block* blocks, uint64_t n,
+                                              uint64_t tensor_data_size, int direction, int device,
+                                              void* stream, int64_t* host_meta,
+                                              int use_explicit_host_offsets);
 /* replaces copy_d2h_bf16_to_fp8()               kvtransfer/include/copy_kernels.h:112-121,
  *                                               kvtransfer/src/copy_kernels.cpp:833-959
  * blocks[i].length = bf16 bytes at the source; the contiguous side receives

@@ -4,6 +4,8 @@
 #include <algorithm>
 #include <atomic>
 #include <cstring>
+#include <mutex>
+#include <string>
 #include <vector>
 
 #include "kvt_runtime.h"
@@ -174,10 +176,13 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
 }
 
 // Single batch with separate device arrays (copy_handle_data_kernel_direct).
+// meta_by_kernel: the three device arrays are one piece of 3 n int64 starting at src_dev, and
+// the metadata reaches it through a copy kernel reading host_meta (device-visible pinned
+// memory) instead of three runtime copies.
 int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks,
                        uint64_t n, uint64_t tensor_data_size, int direction, int device,
                        void* stream, int64_t* src_dev, int64_t* dst_dev, int64_t* len_dev,
-                       int64_t* host_meta, bool explicit_host_offsets) {
+                       int64_t* host_meta, bool explicit_host_offsets, bool meta_by_kernel = false) {
   if (n == 0) return KVT_OK;
   if (!tensor_buf || !layer_gpu_ptr || !blocks || !src_dev || !dst_dev || !len_dev || !host_meta)
     return fail(KVT_ERR_INVALID, "copy_handle_data_kernel_direct: null argument");
@@ -212,9 +217,17 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
     return rc;
   const hipStream_t s = static_cast<hipStream_t>(stream);
   const size_t bytes = n * sizeof(int64_t);
-  KVT_HIP(hipMemcpyAsync(src_dev, host_meta, bytes, hipMemcpyHostToDevice, s));
-  KVT_HIP(hipMemcpyAsync(dst_dev, host_meta + n, bytes, hipMemcpyHostToDevice, s));
-  KVT_HIP(hipMemcpyAsync(len_dev, host_meta + 2 * n, bytes, hipMemcpyHostToDevice, s));
+  if (meta_by_kernel) {
+    if (int rc = check_device_span(host_meta, 3 * bytes,
+                                   "copy_handle_data_kernel_direct: the metadata staging buffer"))
+      return rc;
+    const hipError_t me = launch_copy_linear(src_dev, host_meta, 3 * bytes, s);
+    if (me != hipSuccess) return hip_fail(me, "metadata copy launch");
+  } else {
+    KVT_HIP(hipMemcpyAsync(src_dev, host_meta, bytes, hipMemcpyHostToDevice, s));
+    KVT_HIP(hipMemcpyAsync(dst_dev, host_meta + n, bytes, hipMemcpyHostToDevice, s));
+    KVT_HIP(hipMemcpyAsync(len_dev, host_meta + 2 * n, bytes, hipMemcpyHostToDevice, s));
+  }
   const int rows = rows_for(slices, n);
   const hipError_t e =
       direction == KVT_COPY_D2H
@@ -371,10 +384,6 @@ int kvt_get_copy_memcpy_thresholds(uint64_t* min_range_bytes, uint64_t* max_rang
   return KVT_OK;
 }
 
-int kvt_initialize_copy_method_profile(int device) {
-  return guarded([&]() { return check_device(device); });
-}
-
 int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
                                      const kvt_ipc_block* blocks, uint64_t n,
                                      uint64_t tensor_data_size, int direction, int device,
@@ -396,6 +405,70 @@ int kvt_copy_handle_data_kernel_direct(void* tensor_buf, void* layer_gpu_ptr,
     return handle_data_direct(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction,
                               device, stream, src_offsets_dev, dst_offsets_dev, lengths_dev,
                               host_meta, use_explicit_host_offsets != 0);
+  });
+}
+
+// ------------------------------------------------ the entry point that allocates nothing
+
+}  // extern "C"
+
+// Device-side range metadata of kvt_copy_handle_data_kernel_direct_static: three int64 arrays
+// of up to kStaticMaxRanges entries, 192 KiB, held by every GPU the library runs on until the
+// process ends. In host code the name is only a handle for hipGetSymbolAddress; each device
+// has its own copy at its own address, looked up once per device (g_scratch_ptr).
+constexpr uint64_t kStaticMaxRanges = 8192;
+static __device__ __align__(256) int64_t scratch[3 * kStaticMaxRanges];
+
+namespace {
+constexpr int kMaxStaticDevices = 64;
+std::mutex g_scratch_mu;
+int64_t* g_scratch_ptr[kMaxStaticDevices] = {};
+
+// The address of `device`'s copy of the array (looked up with that device current).
+int static_scratch(int device, int64_t** out) {
+  if (device < 0 || device >= kMaxStaticDevices)
+    return fail(KVT_ERR_INVALID, "device index too large for the static metadata array");
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[device]) {
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    void* p = nullptr;
+    KVT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(KVT_ERR_HIP, "hipGetSymbolAddress gave no address for the static metadata array");
+    g_scratch_ptr[device] = static_cast<int64_t*>(p);
+  }
+  *out = g_scratch_ptr[device];
+  return KVT_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int kvt_initialize_copy_method_profile(int device) {
+  return guarded([&]() -> int {
+    if (int rc = check_device(device)) return rc;
+    int64_t* unused = nullptr;
+    return static_scratch(device, &unused);
+  });
+}
+
+int kvt_copy_handle_data_kernel_direct_static(void* tensor_buf, void* layer_gpu_ptr,
+                                              const kvt_ipc_block* blocks, uint64_t n,
+                                              uint64_t tensor_data_size, int direction, int device,
+                                              void* stream, int64_t* host_meta,
+                                              int use_explicit_host_offsets) {
+  return guarded([&]() -> int {
+    if (n > kStaticMaxRanges)
+      return fail(KVT_ERR_INVALID,
+                  "kvt_copy_handle_data_kernel_direct_static: at most 8192 ranges per call (" +
+                      std::to_string(n) + " given)");
+    if (n == 0) return KVT_OK;
+    if (int rc = check_device(device)) return rc;
+    int64_t* meta = nullptr;
+    if (int rc = static_scratch(device, &meta)) return rc;
+    return handle_data_direct(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction,
+                              device, stream, meta, meta + n, meta + 2 * n, host_meta,
+                              use_explicit_host_offsets != 0, true);
   });
 }
 

@@ -111,6 +111,8 @@ SIGNATURES = {
                                                _vp, _i64]),
     "kvt_copy_handle_data_kernel_direct": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp, _vp,
                                                   _vp, _vp, _vp, _int]),
+    "kvt_copy_handle_data_kernel_direct_static": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _int, _vp,
+                                                         _vp, _int]),
     "kvt_copy_d2h_bf16_to_fp8": (_int, [_vp, _vp, _vp, _u64, _u64, _int, _vp, _vp, _vp, _i64]),
     "kvt_session_create": (_int, [_vp, _vp, _vp, _u64, _P(_vp)]),
     "kvt_session_destroy": (None, [_vp]),
