@@ -325,10 +325,24 @@ def leg_session(c, out):
         torch.cuda.synchronize()
         t_a = time.perf_counter()
         for _ in range(5):
+            sess.begin_step()
             graph.replay()
         torch.cuda.synchronize()
         g_ms = (time.perf_counter() - t_a) / 5 * 1e3
     out["per_layer_session"]["graph_replay_ms_all_layers"] = round(g_ms, 4)
+    # the transport's view of one replay: host time from the launch until wait_layer(l) returns,
+    # for the first and the last layer (no stream or device synchronisation involved)
+    torch.cuda.synchronize()
+    step = sess.begin_step()
+    t_a = time.perf_counter()
+    graph.replay()
+    sess.wait_layer(0, step)
+    t_first = time.perf_counter()
+    sess.wait_layer(w.n_layers - 1, step)
+    t_last = time.perf_counter()
+    out["per_layer_session"]["graph_replay_first_layer_signal_ms"] = round((t_first - t_a) * 1e3, 4)
+    out["per_layer_session"]["graph_replay_last_layer_signal_ms"] = round((t_last - t_a) * 1e3, 4)
+    torch.cuda.synchronize()
     del graph
     sess.close()
 

@@ -490,14 +490,33 @@ int kvt_copy_d2h_bf16_to_fp8(void* tensor_buf, const void* layer_gpu_ptr,
  * and the host-side wait in do_send()           kvtransfer/src/tx_stub.cpp:395-415:
  * the reference parks a host thread in cudaEventSynchronize per layer; here the
  * dependency stays on the device (event record on the compute stream, stream
- * wait on a side stream, pack launch, done event), so the sequence can be
- * captured into a hipGraph together with the forward pass. */
+ * wait on a side stream, pack launch), so the sequence can be captured into a
+ * hipGraph together with the forward pass. Completion of a layer's pack is published by the
+ * device itself (a one-lane kernel behind the pack bumps a per-layer counter mirrored in
+ * pinned host memory); the transport thread's wait polls that word. The signal is therefore
+ * the same for eagerly issued and for replayed (graph) sequences, and a wait touches neither
+ * an event nor a stream.
+ *
+ * Steps. A session serves any number of forward passes ("steps", Step objects in the
+ * reference). kvt_session_begin_step starts one; a session that only ever serves one step
+ * needs no call (the first save_layer begins step 1). The last 8 steps are tracked, i.e. the
+ * transport may lag up to 7 steps behind the forward pass. */
 typedef struct kvt_session kvt_session;
 int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packed,
                        uint64_t layer_stride, kvt_session** out);
+/* Wakes threads parked in a wait (they return KVT_ERR_INVALID), waits for them to leave and
+ * for the side stream to drain. */
 void kvt_session_destroy(kvt_session* s);
+/* Host only, never captured: starts step *step (1, 2, ...). Eager use: call before the step's
+ * first save_layer. Graph use: call before EACH launch of a graph that holds captured
+ * save_layer calls -- the layers recorded in it count as submitted from here on, so launch
+ * the graph next. `step` may be NULL. */
+int kvt_session_begin_step(kvt_session* s, uint64_t* step);
 /* save_kv_layer hook: layer `layer` of the cache is complete once the work
- * already queued on compute_stream has run. Never blocks the host. */
+ * already queued on compute_stream has run. Never blocks the host. Capturable: inside a
+ * stream capture nothing runs, the layer's pack and its completion signal become part of
+ * the graph. A failure (refused launch, HIP error) is latched in the current step: threads
+ * waiting for that step return it instead of waiting on. */
 int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream);
 /* The same for a caller that owns the per-layer events, as the reference's Python side does:
  * it creates one event per layer, hands their handles to the library at init and records
@@ -506,16 +525,22 @@ int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream)
  * `ready_event` is that hipEvent_t (torch.cuda.Event.cuda_event), already recorded on the
  * compute stream; the side stream waits for it, the host never does. */
 int kvt_session_save_layer_event(kvt_session* s, uint32_t layer, void* ready_event);
-/* Host-blocking wait until layer's packed bytes are complete (what the
+/* Host-blocking wait until the packed bytes of `layer` in step `step` are complete (what the
  * transport thread calls before send_data(layer), Step::wait_layer_ready in the
- * reference, kvtransfer/src/step.cpp:49-69). May be called from another thread
- * before save_layer(layer): it then waits for that call first. Not capturable. */
+ * reference, kvtransfer/src/step.cpp:49-69). May be called from any thread and before the
+ * step has begun or the layer has been submitted: it then waits for that first. Issues no
+ * HIP call and synchronises nothing but the calling thread. step = 0: the newest step.
+ * Errors: the latched failure of the step; KVT_ERR_INVALID when the step is no longer tracked
+ * or the session is being destroyed. A layer that the step never submits is waited for
+ * until the session is destroyed, like the reference's. */
+int kvt_session_wait_layer_step(kvt_session* s, uint64_t step, uint32_t layer);
+/* kvt_session_wait_layer_step(s, 0, layer). */
 int kvt_session_wait_layer(kvt_session* s, uint32_t layer);
 /* Makes `stream` wait for every pack issued so far (joins the side stream
  * back; required before ending a capture that included save_layer calls). */
 int kvt_session_join(kvt_session* s, void* stream);
-/* hipStream_t of the side stream (for tests / profiling). Threads: save_layer /
- * join from the thread that drives the forward pass, wait_layer from any thread. */
+/* hipStream_t of the side stream (for tests / profiling). Threads: begin_step / save_layer /
+ * join from the thread that drives the forward pass, the waits from any thread. */
 void* kvt_session_side_stream(kvt_session* s);
 
 /* ------------------------------------ pinned-host staging (KVStore path) */

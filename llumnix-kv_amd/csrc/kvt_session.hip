@@ -1,13 +1,22 @@
 // Per-layer gating sessions (event -> side stream -> pack -> done event) and
 // pinned-host staging of packed layers.
+#include <chrono>
 #include <condition_variable>
 #include <cstring>
 #include <memory>
+#include <string>
+#include <thread>
 
 #include "kvt_runtime.h"
 
 using namespace kvt;
 
+// Completion of a layer's pack is published by the device itself: a one-lane kernel behind
+// the pack on the side stream bumps the layer's counter in device memory and mirrors it into
+// pinned host memory. A host thread that waits for "the k-th pack of layer l" polls that
+// word -- no event, no stream, no device-wide synchronisation -- so the signal is the same
+// whether the sequence was issued eagerly or is replayed from a hipGraph, where a host-side
+// event wait has nothing to hold on to.
 struct kvt_session {
   const kvt_plan* plan = nullptr;
   const kvt_cache* cache = nullptr;
@@ -16,11 +25,29 @@ struct kvt_session {
   hipStream_t side = nullptr;
   std::vector<hipEvent_t> ready, done;
   hipEvent_t last_done = nullptr;
-  // which layers' packs have been issued (wait_layer may be called, from another thread,
-  // before the forward pass reaches the layer)
+  uint32_t* count_dev = nullptr;   // per layer: packs completed so far (device memory)
+  uint32_t* count_host = nullptr;  // the same, mirrored by the device into pinned host memory
+
+  // Host bookkeeping of steps (one forward pass each). target[l] of a step = which completion
+  // of layer l belongs to it (0 = not submitted yet); the last kSteps steps are kept so that a
+  // transport thread may lag behind the forward pass.
+  static constexpr uint32_t kSteps = 8;
+  struct Step {
+    uint64_t id = 0;
+    std::vector<uint32_t> target;
+    int error = KVT_OK;
+    std::string message;
+  };
   std::mutex mu;
-  std::condition_variable issued_cv;
-  std::vector<uint8_t> issued;
+  std::condition_variable cv;
+  Step steps[kSteps];
+  uint64_t cur_step = 0;                 // id of the newest step, 0 = none yet
+  std::vector<uint32_t> submitted;       // packs of layer l handed to the GPU so far
+  std::vector<uint8_t> in_graph;         // layer l's pack was recorded into a stream capture
+  bool closing = false;
+  uint32_t waiters = 0;
+
+  Step& step_slot(uint64_t id) { return steps[id % kSteps]; }
 };
 
 struct kvt_stager {
@@ -36,6 +63,61 @@ struct kvt_stager {
 extern "C" {
 
 // ----------------------------------------------------------------- session
+
+}  // extern "C"
+
+namespace {
+
+// One lane: this layer's completion count, bumped in device memory and mirrored to the host.
+// The pack kernel in front of it on the stream has ended, so its stores have left the caches.
+__global__ void publish_layer_kernel(uint32_t* count_dev, uint32_t* count_host) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const uint32_t c = *count_dev + 1u;
+  *count_dev = c;
+  __hip_atomic_store(count_host, c, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Starts a new step under s->mu. Layers whose pack lives in a captured graph are counted as
+// submitted now: the caller launches that graph next.
+uint64_t begin_step_locked(kvt_session* s) {
+  const uint64_t id = ++s->cur_step;
+  kvt_session::Step& st = s->step_slot(id);
+  st.id = id;
+  st.error = KVT_OK;
+  st.message.clear();
+  st.target.assign(s->cache->n_layers, 0);
+  for (uint32_t l = 0; l < s->cache->n_layers; ++l)
+    if (s->in_graph[l]) st.target[l] = ++s->submitted[l];
+  return id;
+}
+
+// Blocks until completion `target` of `layer` has been published, the session is being
+// destroyed, or (eager steps) the step fails.
+int poll_layer(kvt_session* s, uint32_t layer, uint32_t target) {
+  const uint32_t* word = s->count_host + layer;
+  for (uint32_t spins = 0;; ++spins) {
+    // counts only grow; the comparison survives wrap-around of the 32-bit counter
+    if (static_cast<int32_t>(__atomic_load_n(word, __ATOMIC_ACQUIRE) - target) >= 0) return KVT_OK;
+    if (spins < 2000) {
+#if defined(__x86_64__)
+      __builtin_ia32_pause();
+#endif
+      continue;
+    }
+    if ((spins & 63u) == 0) {
+      std::lock_guard<std::mutex> lock(s->mu);
+      if (s->closing) return fail(KVT_ERR_INVALID, "kvt_session_wait_layer: the session is being destroyed");
+    }
+    if (spins < 20000)
+      std::this_thread::yield();
+    else
+      std::this_thread::sleep_for(std::chrono::microseconds(50));
+  }
+}
+
+}  // namespace
+
+extern "C" {
 
 int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packed,
                        uint64_t layer_stride, kvt_session** out) {
@@ -54,14 +136,21 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
     s->cache = cache;
     s->packed = packed;
     s->layer_stride = layer_stride;
+    const uint32_t n = cache->n_layers;
     KVT_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));
-    s->ready.resize(cache->n_layers);
-    s->done.resize(cache->n_layers);
-    s->issued.assign(cache->n_layers, 0);
-    for (uint32_t l = 0; l < cache->n_layers; ++l) {
+    s->ready.resize(n);
+    s->done.resize(n);
+    s->submitted.assign(n, 0);
+    s->in_graph.assign(n, 0);
+    for (uint32_t l = 0; l < n; ++l) {
       KVT_HIP(hipEventCreateWithFlags(&s->ready[l], hipEventDisableTiming));
       KVT_HIP(hipEventCreateWithFlags(&s->done[l], hipEventDisableTiming));
     }
+    KVT_HIP(hipMalloc(reinterpret_cast<void**>(&s->count_dev), n * sizeof(uint32_t)));
+    KVT_HIP(hipMemset(s->count_dev, 0, n * sizeof(uint32_t)));
+    KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&s->count_host), n * sizeof(uint32_t),
+                          hipHostMallocCoherent));
+    std::memset(s->count_host, 0, n * sizeof(uint32_t));
     *out = s.release();
     return KVT_OK;
   });
@@ -69,6 +158,12 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
 
 void kvt_session_destroy(kvt_session* s) {
   if (!s) return;
+  {  // threads parked in wait_layer return with an error first
+    std::unique_lock<std::mutex> lock(s->mu);
+    s->closing = true;
+    s->cv.notify_all();
+    s->cv.wait(lock, [&] { return s->waiters == 0; });
+  }
   if (s->side) {
     (void)hipStreamSynchronize(s->side);
     (void)hipStreamDestroy(s->side);
@@ -77,22 +172,58 @@ void kvt_session_destroy(kvt_session* s) {
     if (e) (void)hipEventDestroy(e);
   for (hipEvent_t e : s->done)
     if (e) (void)hipEventDestroy(e);
+  if (s->count_dev) (void)hipFree(s->count_dev);
+  if (s->count_host) (void)hipHostFree(s->count_host);
   delete s;
 }
 
-// The pack of `layer` on the side stream, gated by `ready` (already recorded).
-static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
-  KVT_HIP(hipStreamWaitEvent(s->side, ready, 0));
-  uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
-  if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
-  KVT_HIP(hipEventRecord(s->done[layer], s->side));
-  {
+int kvt_session_begin_step(kvt_session* s, uint64_t* step) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_begin_step: null session");
     std::lock_guard<std::mutex> lock(s->mu);
-    s->last_done = s->done[layer];
-    s->issued[layer] = 1;
+    const uint64_t id = begin_step_locked(s);
+    if (step) *step = id;
+    s->cv.notify_all();
+    return KVT_OK;
+  });
+}
+
+// The pack of `layer` on the side stream, gated by `ready` (already recorded), and the
+// publication of its completion.
+static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
+  auto launch = [&](bool* capturing) -> int {
+    KVT_HIP(hipStreamWaitEvent(s->side, ready, 0));
+    // a side stream that waits for an event recorded inside a capture has joined that capture
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s->side, &cap) != hipSuccess) (void)hipGetLastError();
+    *capturing = cap != hipStreamCaptureStatusNone;
+    uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
+    if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
+    hipLaunchKernelGGL(publish_layer_kernel, dim3(1), dim3(64), 0, s->side, s->count_dev + layer,
+                       s->count_host + layer);
+    KVT_HIP(hipGetLastError());
+    KVT_HIP(hipEventRecord(s->done[layer], s->side));
+    return KVT_OK;
+  };
+  bool capturing = false;
+  const int rc = launch(&capturing);
+  std::lock_guard<std::mutex> lock(s->mu);
+  if (capturing) {
+    // nothing runs now: the pack belongs to every later launch of the graph being recorded
+    if (rc == KVT_OK) s->in_graph[layer] = 1;
+  } else {
+    if (s->cur_step == 0) begin_step_locked(s);  // a session used for one step needs no begin_step
+    kvt_session::Step& st = s->step_slot(s->cur_step);
+    if (rc == KVT_OK) {
+      st.target[layer] = ++s->submitted[layer];
+    } else if (st.error == KVT_OK) {   // latched: threads waiting for this step return it
+      st.error = rc;
+      st.message = kvt_last_error();
+    }
   }
-  s->issued_cv.notify_all();
-  return KVT_OK;
+  if (rc == KVT_OK) s->last_done = s->done[layer];
+  s->cv.notify_all();
+  return rc;
 }
 
 int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream) {
@@ -117,17 +248,56 @@ int kvt_session_save_layer_event(kvt_session* s, uint32_t layer, void* ready_eve
   });
 }
 
-int kvt_session_wait_layer(kvt_session* s, uint32_t layer) {
+int kvt_session_wait_layer_step(kvt_session* s, uint64_t step, uint32_t layer) {
   return guarded([&]() -> int {
     if (!s) return fail(KVT_ERR_INVALID, "kvt_session_wait_layer: null session");
     if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    // kvt_session_destroy waits until every thread has left this function
+    struct Visit {
+      kvt_session* s;
+      explicit Visit(kvt_session* session) : s(session) {
+        std::lock_guard<std::mutex> lock(s->mu);
+        ++s->waiters;
+      }
+      ~Visit() {
+        std::lock_guard<std::mutex> lock(s->mu);
+        --s->waiters;
+        s->cv.notify_all();
+      }
+    } visit(s);
+    uint32_t target = 0;
     {
       std::unique_lock<std::mutex> lock(s->mu);
-      s->issued_cv.wait(lock, [&] { return s->issued[layer] != 0; });
+      if (step == 0) step = s->cur_step ? s->cur_step : 1;  // "the current step"
+      int rc = KVT_OK;
+      s->cv.wait(lock, [&] {
+        if (s->closing) {
+          rc = fail(KVT_ERR_INVALID, "kvt_session_wait_layer: the session is being destroyed");
+          return true;
+        }
+        if (s->cur_step < step) return false;                 // the step has not begun yet
+        if (s->cur_step >= step + kvt_session::kSteps) {
+          rc = fail(KVT_ERR_INVALID, "kvt_session_wait_layer: step " + std::to_string(step) +
+                                         " is no longer tracked (the forward pass is " +
+                                         std::to_string(s->cur_step - step) + " steps ahead)");
+          return true;
+        }
+        const kvt_session::Step& st = s->step_slot(step);
+        if (st.error != KVT_OK) {
+          rc = fail(st.error, "kvt_session_wait_layer: the step failed: " + st.message);
+          return true;
+        }
+        target = st.target[layer];
+        return target != 0;
+      });
+      if (rc != KVT_OK) return rc;
     }
-    KVT_HIP(hipEventSynchronize(s->done[layer]));
-    return KVT_OK;
+    return poll_layer(s, layer, target);
   });
+}
+
+int kvt_session_wait_layer(kvt_session* s, uint32_t layer) {
+  return kvt_session_wait_layer_step(s, 0, layer);
 }
 
 int kvt_session_join(kvt_session* s, void* stream) {

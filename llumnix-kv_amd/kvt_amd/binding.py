@@ -119,6 +119,8 @@ SIGNATURES = {
     "kvt_session_save_layer": (_int, [_vp, _u32, _vp]),
     "kvt_session_save_layer_event": (_int, [_vp, _u32, _vp]),
     "kvt_session_wait_layer": (_int, [_vp, _u32]),
+    "kvt_session_wait_layer_step": (_int, [_vp, _u64, _u32]),
+    "kvt_session_begin_step": (_int, [_vp, _P(_u64)]),
     "kvt_session_join": (_int, [_vp, _vp]),
     "kvt_session_side_stream": (_vp, [_vp]),
     "kvt_stager_create": (_int, [_int, _u64, _u32, _P(_vp)]),
@@ -556,8 +558,16 @@ class Session:
         handle = getattr(ready_event, "cuda_event", ready_event)
         check(lib().kvt_session_save_layer_event(self.h, layer, handle))
 
-    def wait_layer(self, layer):
-        check(lib().kvt_session_wait_layer(self.h, layer))
+    def begin_step(self):
+        """Starts the next step (host only; before each eager step, or before each launch of a
+        graph that holds captured save_layer calls) -> its number."""
+        step = _u64()
+        check(lib().kvt_session_begin_step(self.h, C.byref(step)))
+        return step.value
+
+    def wait_layer(self, layer, step=0):
+        """Blocks until `layer` of `step` (0 = the newest step) is packed."""
+        check(lib().kvt_session_wait_layer_step(self.h, step, layer))
 
     def join(self, stream=None):
         check(lib().kvt_session_join(self.h, _ptr(stream)))
