@@ -63,6 +63,10 @@ int kvt_select_parser(int cache_shape, const kvt_worker_info* src, const kvt_wor
 /* A compiled parser: the per-destination part of ParseBlock (all divisions,
  * strides and rank gating) resolved once, the way refresh_dst_info() picks a
  * ParseBlockFunc once per destination. */
+/* Geometries the library declines: KVT_ERR_INVALID for more than 65536 tokens per block,
+ * zero sizes and the like; KVT_ERR_OVERFLOW for a hybrid layout whose indexer block (tokens
+ * per indexer block x indexer token size) reaches 4 GiB -- the reference forms that product in
+ * 32 bits (kvtransfer/src/parse_block_qwen3_next.cpp:376-413) and emits wrapped ranges there. */
 typedef struct kvt_parser kvt_parser;
 int kvt_parser_create(int parser_id, const kvt_worker_info* src, const kvt_worker_info* dst,
                       uint32_t valid_mask, uint32_t kvt_tp_size, uint32_t kvt_tp_rank,

@@ -9,9 +9,11 @@
 // task. The emitted (src_offset, dst_offset, length) sequence is identical,
 // record for record, to what the corresponding reference function appends.
 //
-// Two arithmetic notes: the reference forms a few products in 32 bits
-// (indexer token term, kernel-block index times pack size); this file uses
-// 64-bit products throughout, which differs only for pages >= 4 GiB.
+// An arithmetic note: the reference forms a few products in 32 bits. The kernel-block index
+// times the pack size never exceeds the tokens per block, a 32-bit number, so 64-bit
+// arithmetic gives the same value; the indexer's token term and length (tokens x indexer token
+// size) wrap in the reference for indexer blocks of 4 GiB or more, and kvt_parser_create
+// refuses such a geometry with KVT_ERR_OVERFLOW rather than following or "correcting" it.
 #include <algorithm>
 #include <cstring>
 #include <limits>

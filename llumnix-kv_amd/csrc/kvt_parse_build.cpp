@@ -178,6 +178,13 @@ struct Builder {
 
   void walk_indexer(u32 group, u64 sB, u64 dB, u32 sn, u32 dn, u32 tok) {
     need(sn > 0 && dn > 0, "indexer tokens per block must be positive");
+    // The reference forms the indexer's token term and length as uint32 * uint32
+    // (parse_block_qwen3_next.cpp:376-413): for an indexer block of 4 GiB or more they wrap and
+    // its ranges point anywhere. Such a geometry is refused here instead of being followed
+    // (or silently "corrected" with 64-bit products, which would differ from the reference).
+    if (static_cast<u64>(std::max(sn, dn)) * tok > 0xFFFFFFFFull)
+      throw OverflowError("KVT parse block: indexer block of 4 GiB or more (tokens per block x "
+                          "indexer token size exceeds 32 bits)");
     WalkOp& w = push(OP_WALK).walk;
     w.s.group = w.d.group = group;
     w.s.blk_tok = w.s.seg_tok = sn;

@@ -21,7 +21,15 @@
 //     shapes the reference's second, descriptor-driven generator
 //     (kvtransfer/src/cache_transfer_spec.cpp) states the same byte mapping
 //     independently (tests/test_descriptor_path.py, through the product parser).
-//   * valid-rank selection / dispatch: known answers of the reference tests.
+//   * valid-rank selection: the known answers of the reference's ComputeValidRanksTest.
+//   * dispatch (kvto_select): a literal (cache shape, TP relation, equal token sizes) ->
+//     (parser, TPKind) table transcribed from tx_stub.cpp:451-590, and the reference's tests
+//     that run through KvSendStub (send_stub_test.cpp:286-496, 499-705, 707-1130), whose
+//     literal ranges must come out of (cache shape, two workers) alone
+//     (tests/test_dispatch_pins.py); every known-answer case of the parser tests also checks
+//     that the dispatch leads to the parser and rank values it names. TPKind itself has no
+//     known answer in the reference's tests (their FakeChannel merges for every kind): it
+//     rests on the transcription alone.
 //   * merge: known answers of the reference tests (incl. overlapping prefix).
 //   * pack / unpack: brute-force byte model in numpy + round-trip invariants.
 //   * HND->NHD transposing pack: no reference function exists; pinned by the

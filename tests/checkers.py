@@ -151,3 +151,45 @@ def oracle_unpack(layer, runs, blob):
     lib = oracle()
     runs = np.ascontiguousarray(runs, dtype=np.uint64)
     lib.kvto_unpack(layer.ctypes.data, runs.ctypes.data, len(runs), blob.ctypes.data)
+
+
+# ---------------------------------------------------------------- dispatch
+
+# (prefix of the parser name, cache shape): which cache shape a parser id belongs to in the
+# reference's per-destination dispatch (refresh_dst_info, kvtransfer/src/tx_stub.cpp:451-590)
+_PARSER_SHAPES = (("RAGGED_", 1), ("FLASHINFER_", 5), ("FLASH_", 2), ("HYBRID_FI_", 7),
+                  ("HYBRID_", 3), ("DPSK_", 4), ("KIMI_K3_", 8), ("TURBOQUANT_", 6))
+_KIND_OF_SUFFIX = {"PEQD": 0, "PLTD": 1, "PGTD": 2}
+
+
+def dispatch_of(parser_name):
+    """-> (cache shape, TPKind) the reference's dispatch pairs with this parser, or None for
+    the parsers it never selects directly (the KDA state parsers are called by the Kimi-K3
+    ones). TPKind follows the name except where tx_stub.cpp says otherwise: every DPSK parser
+    and parse_block_send_p_gt_d_dpsk are registered as PEQD (tx_stub.cpp:469-470, 521-535)."""
+    for prefix, shape in _PARSER_SHAPES:
+        if parser_name.startswith(prefix):
+            if shape == 4 or parser_name == "RAGGED_PGTD_DPSK":
+                return shape, 0
+            return shape, _KIND_OF_SUFFIX[parser_name.rsplit("_", 1)[1]]
+    return None
+
+
+def assert_dispatch(parser_name, src, dst, valid=None, tp_size=None, tp_rank=None):
+    """A known-answer case names its parser and its (valid ranks, kvt_tp_size, kvt_tp_rank):
+    from (cache shape, src, dst) alone, the oracle's and the product's dispatch must arrive at
+    exactly those. valid = None: the case hands the parser rank values it did not derive from
+    the two workers (some reference tests do); then only parser and TPKind are compared."""
+    from kvt_amd.ctypes_defs import PARSER
+    import kvt_amd
+    want = dispatch_of(parser_name)
+    if want is None:     # never selected by the dispatch itself: nothing to check
+        return
+    shape, kind = want
+    exp = (valid, tp_size, tp_rank, PARSER[parser_name], kind)
+    got_o = oracle_select(shape, src, dst)
+    got_p = kvt_amd.select_parser(shape, src, dst)
+    if valid is None:
+        exp, got_o, got_p = exp[3:], (got_o[0],) + got_o[4:], got_p[3:]
+    assert got_o == (0,) + exp, ("oracle dispatch", parser_name, got_o, exp)
+    assert got_p == exp, ("product dispatch", parser_name, got_p, exp)

@@ -13,10 +13,12 @@ from kvt_amd.ctypes_defs import PARSER, TaskBuf, make_worker_info
 KB = 1024
 
 
-def _parse(parser, src, dst, tasks, valid=None, tp_size=None, tp_rank=None, **kw):
+def _parse(parser, src, dst, tasks, valid=None, tp_size=None, tp_rank=None, dispatch=True, **kw):
     valid = (1 << src.engine_tp_size) - 1 if valid is None else valid
     tp_size = bin(valid).count("1") if tp_size is None else tp_size
     tp_rank = bin(valid & ((1 << src.worker_tp_rank) - 1)).count("1") if tp_rank is None else tp_rank
+    if dispatch:   # the case reaches this parser, with these ranks, through the dispatch too
+        checkers.assert_dispatch(parser, src, dst, valid, tp_size, tp_rank)
     rc, outs = checkers.oracle_parse(PARSER[parser], src, dst, valid, tp_size, tp_rank, tasks, **kw)
     assert rc == 0
     return [[tuple(int(x) for x in r) for r in o] for o in outs]

@@ -127,7 +127,7 @@ def test_capacity_overflow_and_missing_tensor():
     assert rc_o == 1
 
 
-@pytest.mark.parametrize("shape", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("shape", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_select_parser_matches_oracle(shape):
     rng = np.random.default_rng(shape)
     for _ in range(200):

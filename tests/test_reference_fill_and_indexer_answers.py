@@ -15,6 +15,7 @@ def _both(parser, src, dst, task, heads):
     valid = checkers.oracle().kvto_valid_ranks(src.engine_tp_size, dst.engine_tp_size, heads)
     tp_size = bin(valid).count("1")
     tp_rank = bin(valid & ((1 << src.worker_tp_rank) - 1)).count("1")
+    checkers.assert_dispatch(parser, src, dst, valid, tp_size, tp_rank)
     rc, outs = checkers.oracle_parse(PARSER[parser], src, dst, valid, tp_size, tp_rank, [task])
     assert rc == 0 and len(outs) == 1
     oracle = [tuple(int(x) for x in r) for r in outs[0]]
@@ -153,6 +154,7 @@ def _pltd(parser, src, dst, task, heads):
     """The reference's P<D tests call the parser with kvt_tp_size 2, kvt_tp_rank 0."""
     valid = checkers.oracle().kvto_valid_ranks(2, 8, heads)
     assert bin(valid).count("1") == 2
+    checkers.assert_dispatch(parser, src, dst, valid, 2, 0)
     rc, outs = checkers.oracle_parse(PARSER[parser], src, dst, valid, 2, 0, [task])
     assert rc == 0 and len(outs) == 1
     oracle = [tuple(int(x) for x in r) for r in outs[0]]

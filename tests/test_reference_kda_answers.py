@@ -30,6 +30,9 @@ def _fixture(p_tp, p_rank, d_tp, d_rank, pB, dB, layout=None, kimi=None):
 
 
 def _run(parser, src, dst, task, valid, tp_size, tp_rank):
+    # the Kimi-K3 cases name the parser the dispatch must pick for these two workers (the rank
+    # values are literals of the reference tests, not derived from the workers)
+    checkers.assert_dispatch(parser, src, dst)
     rc, outs = checkers.oracle_parse(PARSER[parser], src, dst, valid, tp_size, tp_rank, [task])
     assert rc == 0 and len(outs) == 1
     oracle = [tuple(int(x) for x in r) for r in outs[0]]
