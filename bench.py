@@ -24,14 +24,6 @@ sys.path[:0] = [os.path.join(ROOT, "llumnix-kv_amd"), os.path.join(ROOT, "tests"
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 
-# HBM bytes moved by ONE pack launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (each counter scaled by what it reads for the plain copy kernel of known size); see
-# profiles/copy_chunks_kernel_config2_hbm_traffic.md and
-# profiles/strided_and_xform_kernels_hbm_traffic.md. Keyed by (config, scale, chunk_bytes, plan).
-MEASURED_PACK_TRAFFIC = {(2, 1.0, 0, "ranges"): 70.956e9, (3, 1.0, 0, "ranges"): 85.878e9,
-                         (6, 1.0, 0, "runs"): 40.872e9}
-
-
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -267,27 +259,66 @@ def leg_cpu(c, out):
 
 
 def leg_latency(c, out):
-    """GPU time of one pack launch per request (all layers of the request)."""
+    """Per-request KV pack latency. Three figures, each the median over the batch's requests:
+    * latency_p50_us: GPU time from the first pack launch of layer 0 to the completion of the
+      last layer on the side stream, the request packed layer by layer through a session (HIP
+      events on the streams involved);
+    * latency_wall_p50_us: host wall clock around the whole request -- ParseBlock, plan (cold:
+      built for this request), one gated launch per layer, until the transport's wait for the
+      last layer returns;
+    * latency_single_launch_p50_us: GPU time of ONE launch covering all layers of the request
+      (second, warm launch)."""
     torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
     wls, sides, infos, tasks, first = c.wls, c.sides, c.infos, c.tasks, c.first
     strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
     w, side = wls[0], sides[0]
-    lat = []
+    sender = c.senders[0]
+    single, gated, wall = [], [], []
     reqs = list(range(len(w.tasks)))
+    sess = None
+    a, b = new_event(), new_event()
     for r in reqs:
-        lists, _ = pipeline.parse_batch(w.cache_shape, infos[0][0], infos[0][1], [tasks[0][r]])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        lists = sender.parse([tasks[0][r]])
         plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
                         chunk_bytes=args.chunk_bytes)
-        c.keep.append(plan)
-        a, b = new_event(), new_event()
+        if sess is None:
+            sess = kvt.Session(plan, side.src_cache, packed[0], plan.layer_bytes)
+        else:
+            sess.set_plan(plan, packed[0], plan.layer_bytes)
+        step = sess.begin_step()
+        lib.kvt_event_record(a, sh)
+        for l in range(w.n_layers):
+            sess.save_layer(l, sh)
+        lib.kvt_event_record(b, sess.side_stream)
+        sess.wait_layer(w.n_layers - 1, step)
+        wall.append((time.perf_counter() - t0) * 1e6)
+        lib.kvt_event_synchronize(b)
+        gated.append(ev_ms(lib, a, b) * 1e3)
         for rep in range(2):   # second run is the measurement
             lib.kvt_event_record(a, sh)
             plan.pack(side.src_cache, 0, w.n_layers, packed[0], plan.layer_bytes, sh)
             lib.kvt_event_record(b, sh)
         lib.kvt_event_synchronize(b)
-        lat.append(ev_ms(lib, a, b) * 1e3)
-    out["latency_p50_us"] = round(statistics.median(lat), 2)
-    out["latency_note"] = "per request: one pack launch covering all %d layers, GPU time" % w.n_layers
+        single.append(ev_ms(lib, a, b) * 1e3)
+        if r + 1 < len(reqs):      # everything of this request has run: its table may be reused
+            plan.close()
+            lists.close()
+        else:
+            c.keep_objs.append((plan, lists))   # the session still names the last plan
+    torch.cuda.synchronize()
+    if sess is not None:
+        sess.close()
+    out["latency_p50_us"] = round(statistics.median(gated), 2)
+    out["latency_wall_p50_us"] = round(statistics.median(wall), 2)
+    out["latency_single_launch_p50_us"] = round(statistics.median(single), 2)
+    out["latency_note"] = ("per request (%d requests): latency_p50_us = GPU time from the first "
+                           "pack launch of layer 0 to the completion of layer %d on the side "
+                           "stream, one event-gated launch per layer; latency_wall_p50_us = host "
+                           "clock from before ParseBlock (plan built cold) until the wait for the "
+                           "last layer returns; latency_single_launch_p50_us = one warm launch "
+                           "covering all layers" % (len(reqs), w.n_layers - 1))
 
 
 def leg_session(c, out):
@@ -372,6 +403,37 @@ def leg_cu_usage(c, out):
     finally:
         kvt.set_copy_cu_usage(0, 1.0)
     out["cu_usage"] = rows
+
+
+def leg_copy_ceilings(c, out):
+    """Plain copies of the sizes the launches here have, by this library's linear copy kernel
+    and by the runtime's own device-to-device hipMemcpyAsync: what the part gives a copy that
+    gathers and scatters nothing. Each buffer pair is used once per measurement round, larger
+    than the 256 MiB memory-side cache in total, so repeated rounds do not read from it."""
+    torch, lib, sh, new_event = c.torch, c.lib, c.sh, c.new_event
+    res = {}
+    for name, n, pairs, rounds in (("64MiB", 64 << 20, 8, 6), ("4GiB", 4 << 30, 1, 4)):
+        src = [torch.full((n,), 3, dtype=torch.uint8, device="cuda") for _ in range(pairs)]
+        dst = [torch.empty(n, dtype=torch.uint8, device="cuda") for _ in range(pairs)]
+        for fn_name in ("kvt_copy_linear", "kvt_copy_runtime_d2d"):
+            fn = getattr(lib, fn_name)
+            a, b = new_event(), new_event()
+            times = []
+            for rnd in range(rounds):
+                lib.kvt_event_record(a, sh)
+                for i in range(pairs):
+                    assert fn(dst[i].data_ptr(), src[i].data_ptr(), n, sh) == 0, lib.kvt_last_error()
+                lib.kvt_event_record(b, sh)
+                lib.kvt_event_synchronize(b)
+                times.append(ev_ms(lib, a, b) / pairs)
+            t = statistics.median(times[1:])
+            res["%s_%s" % (fn_name, name)] = {"us": round(t * 1e3, 2),
+                                              "gbps": round(2.0 * n / (t * 1e-3) / 1e9, 1)}
+        assert torch.equal(src[0], dst[0])
+        del src, dst
+    res["note"] = ("GB/s = bytes read + bytes written; back-to-back launches on one stream, "
+                   "median of the rounds after the first")
+    out["copy_ceilings"] = res
 
 
 def leg_launchers(c, out):
@@ -653,7 +715,7 @@ def leg_store_objects(c, out):
         pl = kvt.Plan(0, lst, w.capacities("src"), w.capacities("dst"), objects=(ob, entry))
         pl.pack(side.src_cache, 0, L, objs, ob, ps.cuda_stream)
         ring.save(e[new], objs.data_ptr(), entry, ps.cuda_stream)
-        c.keep.append(pl)
+        c.keep_objs.append((pl, lst))
         saved += len(todo)
     ps.synchronize()
     t_b = time.perf_counter()
@@ -737,34 +799,34 @@ def leg_staging(c, out):
         stg.close()
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", type=int, default=2, help="1-5: the five benchmark configurations (1 = the CPU-runnable case, 2 = the headline); 6-8: TP-remapping batches; "
-                         "9: config 5 with the reference's uniform 2 MiB pages; 10: the same "
-                         "model TP2 -> TP1")
-    ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")
-    ap.add_argument("--chunk-bytes", type=int, default=0)
-    ap.add_argument("--plan", choices=["ranges", "runs"], default="ranges",
-                    help="runs: ParseBlock in closed form (strided runs), the per-token offset "
-                         "arithmetic done by the copy kernel")
-    ap.add_argument("--sequential", action="store_true",
-                    help="config 5 only: pack everything, then unpack everything, instead of the "
-                         "mixed mode (half of the requests packing while the other half unpacks)")
-    ap.add_argument("--cpu-layers", type=int, default=16,
-                    help="layers in the CPU baseline sample (16 layers x 5 passes of config 2 are "
-                         "about 10 s of single-thread CPU work)")
-    ap.add_argument("--skip-cpu", action="store_true")
-    ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
-    ap.add_argument("--calibrate-copy-gib", type=float, default=0.0,
-                    help="only run the plain linear copy kernel on this many GiB (profiler "
-                         "counter calibration: its HBM traffic is known, 1 read + 1 write)")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        raise SystemExit("bench.py: this build measures ONE MI355X; the path has no inter-GPU "
-                         "part, so --gpus N with N > 1 is not supported.")
+# HBM bytes moved by ONE launch over all layers, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# of this file (each counter scaled by what it reads for the plain copy kernel of known size):
+# profiles/*_hbm_traffic.md. Keyed by (config, plan); valid for scale 1 and the automatic
+# chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
+# compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
+# changed since, so a stale table cannot pass unnoticed.
+KERNELS_SHA256 = "a23c23a8eebb91c2b05f50b7b3883ac763015b442d2f98ca4cf1bc15a6f843c1"
+MEASURED_TRAFFIC = {
+    (1, "ranges"): {"pack": 134276965, "unpack": 134276496},
+    (2, "ranges"): {"pack": 71013090059, "unpack": 73358409599},
+    (3, "ranges"): {"pack": 85983221225, "unpack": 85983589735},
+    (4, "ranges"): {"pack": 22690378135, "unpack": 22690435564},
+    (5, "ranges"): {"pack": 45141182693, "unpack": 45141395897},
+}
+
+
+def measured_traffic(args, direction):
+    if args.scale != 1.0 or args.chunk_bytes != 0:
+        return None
+    row = MEASURED_TRAFFIC.get((args.config, args.plan))
+    return row[direction] if row else None
+
+
+def run_config(args, headline):
+    """One configuration: caches resident in HBM, the timed steps, the side legs. Returns the
+    dictionary that becomes the JSON line (headline) or a row of its "configs" list, and frees
+    everything it allocated."""
+    import gc
 
     import numpy as np
     import torch
@@ -773,29 +835,11 @@ def main():
     from kvt_amd import pipeline
 
     lib = kvt.lib()
-    if kvt.device_count() < 1:
-        raise SystemExit("bench.py: no usable MI355X (gfx950) device; there is no CPU fallback")
-
-    if args.calibrate_copy_gib > 0:
-        n = int(args.calibrate_copy_gib * 2**30)
-        a = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
-        b = torch.empty(n, dtype=torch.uint8, device="cuda")
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            assert lib.kvt_copy_linear(b.data_ptr(), a.data_ptr(), n, None) == 0
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / args.steps
-        assert torch.equal(a, b)
-        print(json.dumps({"calibration": "kvt_copy_linear", "bytes": n, "launches": args.steps,
-                          "gbps_read_plus_write": round(2 * n / dt / 1e9, 1)}))
-        return
-
     full_wls = build_workload(args.config, args.scale)
     t_init = time.time()
     full_sides = [DeviceSide(torch, kvt, w, 7 + i) for i, w in enumerate(full_wls)]
     torch.cuda.synchronize()
-    log("caches resident in %.1fs" % (time.time() - t_init))
+    log("config %d: caches resident in %.1fs" % (args.config, time.time() - t_init))
     mixed = args.config == 5 and not args.sequential
     if mixed:
         # halves A and B of every workload's requests, on the same caches; a step is
@@ -842,10 +886,12 @@ def main():
 
     stream = torch.cuda.Stream()
     sh = stream.cuda_stream
+    made_events = []
 
     def new_event():
         e = C.c_void_p()
         assert lib.kvt_event_create(C.byref(e)) == 0, lib.kvt_last_error()
+        made_events.append(e)
         return e
 
     s2 = torch.cuda.Stream()
@@ -937,6 +983,15 @@ def main():
     log("pack %.3f ms  unpack %.3f ms  host %.3f ms/step  wall %.3f ms/step" %
         (pack_avg, unpack_avg, statistics.mean(host_ms), ms_per_step))
 
+    # instantiation names as a profiler prints them: <pack, [words,] capped>
+    if first[0][0].num_strided_chunks:
+        kernel = "kvt::strided_chunks_kernel<true, false, false> (pack)"
+    elif wls[0].xform:
+        kernel = "kvt::xform_chunks_kernel<true, false> (pack)"
+    elif first[0][0].num_chunks <= 64:
+        kernel = "kvt::copy_chunks_small_kernel<true, false> (pack)"
+    else:
+        kernel = "kvt::copy_chunks_kernel<true, false> (pack)"
     out = {
         "metric": "pack+unpack GB/s (bytes read + bytes written per second, whole job)",
         "value": round(value, 1),
@@ -963,28 +1018,27 @@ def main():
         "host_parse_plan_ms": round(statistics.mean(host_ms), 4),
         "mode": ("mixed: (pack A || unpack B) then (pack B || unpack A) on two streams; pack_ms = "
                  "unpack_ms = mean phase time") if mixed else "sequential: pack all, then unpack all",
-        "roofline": {"bound": "hbm",
-                     # instantiation names as a profiler prints them: <pack, [words,] capped>
-                     "kernel": "kvt::strided_chunks_kernel<true, false, false> (pack)"
-                     if first[0][0].num_strided_chunks
-                     else ("kvt::copy_chunks_small_kernel<true, false> (pack)" if first[0][0].num_chunks <= 64
-                           else "kvt::copy_chunks_kernel<true, false> (pack)") if not wls[0].xform
-                     else "kvt::xform_chunks_kernel<true, false> (pack)",
+        "roofline": {"bound": "hbm", "kernel": kernel,
                      "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK, 4),
-                     "traffic": MEASURED_PACK_TRAFFIC.get((args.config, args.scale,
-                                                           args.chunk_bytes, args.plan))},
+                     "algorithmic_bytes_per_launch": 2 * P,
+                     "traffic": measured_traffic(args, "pack"),
+                     "traffic_unpack": measured_traffic(args, "unpack")},
     }
+    keep_objs = []
     c = types.SimpleNamespace(torch=torch, np=np, kvt=kvt, lib=lib, args=args, pipeline=pipeline,
                               wls=wls, sides=sides, full_wls=full_wls, full_sides=full_sides,
                               mixed=mixed, infos=infos, tasks=tasks, first=first, strides=strides,
-                              packed=packed, stream=stream, sh=sh, new_event=new_event, keep=keep)
+                              packed=packed, stream=stream, sh=sh, new_event=new_event, keep=keep,
+                              senders=senders, keep_objs=keep_objs)
     # The timed region is over: a failure in a side leg must not take the measured line with
     # it. It is reported in "errors" (and on stderr, with the traceback) and fails the run.
     legs = [] if args.skip_cpu else [leg_cpu]
     if not args.skip_extras:
-        legs += [leg_latency, leg_session, leg_cu_usage, leg_launchers, leg_fp8_plan, leg_frames,
-                 leg_store_objects, leg_staging]
+        legs += [leg_latency, leg_staging]
+        if headline:
+            legs += [leg_session, leg_cu_usage, leg_copy_ceilings, leg_launchers, leg_fp8_plan,
+                     leg_frames, leg_store_objects]
     errors = {}
     for leg in legs:
         try:
@@ -995,8 +1049,118 @@ def main():
             errors[leg.__name__] = "%s: %s" % (type(e).__name__, e)
     if errors:
         out["errors"] = errors
+    # give everything back before the next configuration builds its caches
+    torch.cuda.synchronize()
+    for batch in keep:
+        for pl, ls in batch:
+            pl.close()
+            ls.close()
+    for pl, ls in keep_objs:
+        pl.close()
+        ls.close()
+    for sd in full_sides:
+        sd.src_cache.close()
+        sd.dst_cache.close()
+    for sender in senders:
+        sender.close()
+    for e in made_events:
+        lib.kvt_event_destroy(e)
+    del c, keep, keep_objs, first, plans, packed, sides, full_sides, wls, full_wls, events
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=0,
+                    help="0 (default): the headline configuration 2 as the JSON line, followed by "
+                         "the other four baseline configurations as rows of its \"configs\" list; "
+                         "1-5: that baseline configuration alone (1 = the CPU-runnable case, 2 = "
+                         "the headline); 6-8: TP-remapping batches; 9: config 5 with the "
+                         "reference's uniform 2 MiB pages; 10: the same model TP2 -> TP1")
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")
+    ap.add_argument("--chunk-bytes", type=int, default=0)
+    ap.add_argument("--plan", choices=["ranges", "runs"], default="ranges",
+                    help="runs: ParseBlock in closed form (strided runs), the per-token offset "
+                         "arithmetic done by the copy kernel")
+    ap.add_argument("--sequential", action="store_true",
+                    help="config 5 only: pack everything, then unpack everything, instead of the "
+                         "mixed mode (half of the requests packing while the other half unpacks)")
+    ap.add_argument("--cpu-layers", type=int, default=16,
+                    help="layers in the CPU baseline sample (16 layers x 5 passes of config 2 are "
+                         "about 10 s of single-thread CPU work)")
+    ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
+    ap.add_argument("--calibrate-copy-gib", type=float, default=0.0,
+                    help="only run the plain linear copy kernel on this many GiB (profiler "
+                         "counter calibration: its HBM traffic is known, 1 read + 1 write)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py: this build measures ONE MI355X; the path has no inter-GPU "
+                         "part, so --gpus N with N > 1 is not supported.")
+
+    import torch
+
+    import kvt_amd as kvt
+
+    lib = kvt.lib()
+    if kvt.device_count() < 1:
+        raise SystemExit("bench.py: no usable MI355X (gfx950) device; there is no CPU fallback")
+
+    if args.calibrate_copy_gib > 0:
+        n = int(args.calibrate_copy_gib * 2**30)
+        a = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
+        b = torch.empty(n, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            assert lib.kvt_copy_linear(b.data_ptr(), a.data_ptr(), n, None) == 0
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        assert torch.equal(a, b)
+        print(json.dumps({"calibration": "kvt_copy_linear", "bytes": n, "launches": args.steps,
+                          "gbps_read_plus_write": round(2 * n / dt / 1e9, 1)}))
+        return
+
+    all_configs = args.config == 0
+    if all_configs:
+        args.config = 2
+    out = run_config(args, headline=True)
+    if all_configs:
+        # the other baseline configurations, full size, one after the other on the same GPU:
+        # the timed steps, parity against the oracle on a sample of layers, the request
+        # latencies and the staging path
+        rows = []
+        for cfg in (1, 3, 4, 5):
+            sub = argparse.Namespace(**vars(args))
+            sub.config, sub.plan, sub.chunk_bytes = cfg, "ranges", 0
+            sub.cpu_layers = min(args.cpu_layers, 4)
+            try:
+                r = run_config(sub, headline=False)
+            except Exception as e:      # noqa: BLE001 - reported, not swallowed
+                import traceback
+                traceback.print_exc(file=sys.stderr)
+                out.setdefault("errors", {})["config %d" % cfg] = "%s: %s" % (type(e).__name__, e)
+                continue
+            row = {"config": cfg, "workload": r["config"]["workload"],
+                   "payload_bytes_per_step": r["config"]["payload_bytes_per_step"]}
+            for key in ("value", "ms_per_step", "pack_gbps", "unpack_gbps", "pack_ms", "unpack_ms",
+                        "frac_hbm_peak", "host_parse_plan_ms", "mode", "parity_vs_oracle",
+                        "latency_p50_us", "latency_wall_p50_us", "latency_single_launch_p50_us",
+                        "staging", "roofline", "cpu_baseline", "errors"):
+                if key in r:
+                    row[key] = r[key]
+            row["frac"] = r["roofline"]["frac"]
+            rows.append(row)
+            if "errors" in r:
+                out.setdefault("errors", {})["config %d" % cfg] = r["errors"]
+        out["configs"] = rows
     print(json.dumps(out), flush=True)
-    if errors:
+    if out.get("errors"):
         raise SystemExit(1)
 
 

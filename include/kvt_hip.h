@@ -511,6 +511,13 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
 /* Wakes threads parked in a wait (they return KVT_ERR_INVALID), waits for them to leave and
  * for the side stream to drain. */
 void kvt_session_destroy(kvt_session* s);
+/* The next batch on the same session: packs issued from here on use `plan` and write to
+ * `packed` (stream, events and counters of a session are not cheap to create; a sender keeps
+ * one session per destination and gives it each batch's plan). Layers already issued keep
+ * what they were issued with. Refused once save_layer calls of this session have been captured
+ * into a graph (the graph would go on launching the old plan). Call it from the thread that
+ * drives the forward pass, between steps. */
+int kvt_session_set_plan(kvt_session* s, const kvt_plan* plan, void* packed, uint64_t layer_stride);
 /* Host only, never captured: starts step *step (1, 2, ...). Eager use: call before the step's
  * first save_layer. Graph use: call before EACH launch of a graph that holds captured
  * save_layer calls -- the layers recorded in it count as submitted from here on, so launch

@@ -163,15 +163,22 @@ class TablePool {
       delete b;
       return;
     }
-    std::lock_guard<std::mutex> lock(mu_);
-    if (idle_.size() >= 64) {
-      TableBuf* victim = idle_.front();
-      idle_.erase(idle_.begin());
+    std::vector<TableBuf*> victims;
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      // A full pool gives up its older half at once: freeing device memory waits for the whole
+      // device, so it must not happen on every release of a pool that stays full.
+      if (idle_.size() >= kMaxIdle) {
+        victims.assign(idle_.begin(), idle_.begin() + kMaxIdle / 2);
+        idle_.erase(idle_.begin(), idle_.begin() + kMaxIdle / 2);
+      }
+      idle_.push_back(b);
+    }
+    for (TableBuf* victim : victims) {
       victim->wait_idle();
       destroy(victim);
       delete victim;
     }
-    idle_.push_back(b);
   }
 
   // One upload stream per device, created on first use.
@@ -184,6 +191,7 @@ class TablePool {
   }
 
  private:
+  static constexpr size_t kMaxIdle = 256;
   static void destroy(TableBuf* b) {
     if (b->dev) (void)hipFree(b->dev);
     if (b->host) (void)hipHostFree(b->host);

@@ -23,8 +23,9 @@ struct kvt_session {
   void* packed = nullptr;
   uint64_t layer_stride = 0;
   hipStream_t side = nullptr;
-  std::vector<hipEvent_t> ready, done;
-  hipEvent_t last_done = nullptr;
+  std::vector<hipEvent_t> ready;
+  hipEvent_t joined = nullptr;     // recorded on the side stream by kvt_session_join
+  bool issued_any = false;
   uint32_t* count_dev = nullptr;   // per layer: packs completed so far (device memory)
   uint32_t* count_host = nullptr;  // the same, mirrored by the device into pinned host memory
 
@@ -139,13 +140,12 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
     const uint32_t n = cache->n_layers;
     KVT_HIP(hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking));
     s->ready.resize(n);
-    s->done.resize(n);
     s->submitted.assign(n, 0);
     s->in_graph.assign(n, 0);
     for (uint32_t l = 0; l < n; ++l) {
       KVT_HIP(hipEventCreateWithFlags(&s->ready[l], hipEventDisableTiming));
-      KVT_HIP(hipEventCreateWithFlags(&s->done[l], hipEventDisableTiming));
     }
+    KVT_HIP(hipEventCreateWithFlags(&s->joined, hipEventDisableTiming));
     KVT_HIP(hipMalloc(reinterpret_cast<void**>(&s->count_dev), n * sizeof(uint32_t)));
     KVT_HIP(hipMemset(s->count_dev, 0, n * sizeof(uint32_t)));
     KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&s->count_host), n * sizeof(uint32_t),
@@ -170,11 +170,29 @@ void kvt_session_destroy(kvt_session* s) {
   }
   for (hipEvent_t e : s->ready)
     if (e) (void)hipEventDestroy(e);
-  for (hipEvent_t e : s->done)
-    if (e) (void)hipEventDestroy(e);
+  if (s->joined) (void)hipEventDestroy(s->joined);
   if (s->count_dev) (void)hipFree(s->count_dev);
   if (s->count_host) (void)hipHostFree(s->count_host);
   delete s;
+}
+
+int kvt_session_set_plan(kvt_session* s, const kvt_plan* plan, void* packed, uint64_t layer_stride) {
+  return guarded([&]() -> int {
+    if (!s || !plan || !packed) return fail(KVT_ERR_INVALID, "kvt_session_set_plan: null argument");
+    if (plan->device != s->cache->device || plan->n_tensors != s->cache->n_tensors)
+      return fail(KVT_ERR_INVALID, "kvt_session_set_plan: the plan does not fit the session's cache");
+    if (layer_stride < plan->min_layer_stride)
+      return fail(KVT_ERR_INVALID, "kvt_session_set_plan: layer_stride smaller than one packed layer");
+    std::lock_guard<std::mutex> lock(s->mu);
+    for (uint8_t g : s->in_graph)
+      if (g)
+        return fail(KVT_ERR_INVALID,
+                    "kvt_session_set_plan: a captured graph still launches the session's old plan");
+    s->plan = plan;
+    s->packed = packed;
+    s->layer_stride = layer_stride;
+    return KVT_OK;
+  });
 }
 
 int kvt_session_begin_step(kvt_session* s, uint64_t* step) {
@@ -202,7 +220,6 @@ static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
     hipLaunchKernelGGL(publish_layer_kernel, dim3(1), dim3(64), 0, s->side, s->count_dev + layer,
                        s->count_host + layer);
     KVT_HIP(hipGetLastError());
-    KVT_HIP(hipEventRecord(s->done[layer], s->side));
     return KVT_OK;
   };
   bool capturing = false;
@@ -221,7 +238,7 @@ static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
       st.message = kvt_last_error();
     }
   }
-  if (rc == KVT_OK) s->last_done = s->done[layer];
+  if (rc == KVT_OK) s->issued_any = true;
   s->cv.notify_all();
   return rc;
 }
@@ -303,12 +320,14 @@ int kvt_session_wait_layer(kvt_session* s, uint32_t layer) {
 int kvt_session_join(kvt_session* s, void* stream) {
   return guarded([&]() -> int {
     if (!s) return fail(KVT_ERR_INVALID, "kvt_session_join: null session");
-    hipEvent_t last = nullptr;
     {
       std::lock_guard<std::mutex> lock(s->mu);
-      last = s->last_done;
+      if (!s->issued_any) return KVT_OK;
     }
-    if (last) KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), last, 0));
+    DeviceGuard g;
+    if (int rc = g.enter(s->plan->device)) return rc;
+    KVT_HIP(hipEventRecord(s->joined, s->side));
+    KVT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), s->joined, 0));
     return KVT_OK;
   });
 }

@@ -121,6 +121,7 @@ SIGNATURES = {
     "kvt_session_wait_layer": (_int, [_vp, _u32]),
     "kvt_session_wait_layer_step": (_int, [_vp, _u64, _u32]),
     "kvt_session_begin_step": (_int, [_vp, _P(_u64)]),
+    "kvt_session_set_plan": (_int, [_vp, _vp, _vp, _u64]),
     "kvt_session_join": (_int, [_vp, _vp]),
     "kvt_session_side_stream": (_vp, [_vp]),
     "kvt_stager_create": (_int, [_int, _u64, _u32, _P(_vp)]),
@@ -557,6 +558,11 @@ class Session:
         torch.cuda.Event.cuda_event), or the torch event itself."""
         handle = getattr(ready_event, "cuda_event", ready_event)
         check(lib().kvt_session_save_layer_event(self.h, layer, handle))
+
+    def set_plan(self, plan, packed, layer_stride):
+        """The next batch on the same session (its stream, events and counters are kept)."""
+        check(lib().kvt_session_set_plan(self.h, plan.h, _ptr(packed), layer_stride))
+        self._keep = (plan, self._keep[1], packed)
 
     def begin_step(self):
         """Starts the next step (host only; before each eager step, or before each launch of a

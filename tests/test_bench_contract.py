@@ -49,3 +49,25 @@ def test_the_json_line_names_every_agreed_key():
     assert '"workload"' in src and '"model"' not in src
     # nothing under _work/ and no reference checkout at run time
     assert "_work/" not in src and "/root/reference" not in src
+
+
+def test_the_measured_hbm_traffic_belongs_to_the_kernels_as_they_are_now():
+    """roofline.traffic comes from profiler counter runs and is kept in bench.py next to the
+    SHA-256 of the kernel source it was measured with. A kernel change without a new counter
+    run must not go unnoticed: the figures would be quoted for code they were not taken from."""
+    import hashlib
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", BENCH)
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    kernels = os.path.join(ROOT, "llumnix-kv_amd", "csrc", "kvt_kernels.hip")
+    sha = hashlib.sha256(open(kernels, "rb").read()).hexdigest()
+    if not bench.MEASURED_TRAFFIC:
+        assert bench.KERNELS_SHA256 == "unmeasured"
+        return
+    assert bench.KERNELS_SHA256 == sha, (
+        "llumnix-kv_amd/csrc/kvt_kernels.hip has changed since the FETCH_SIZE / WRITE_SIZE runs "
+        "behind bench.MEASURED_TRAFFIC: take the counter runs again (profiles/*_hbm_traffic.md "
+        "give the commands), or empty the table")
+    for (cfg, plan), row in bench.MEASURED_TRAFFIC.items():
+        assert set(row) == {"pack", "unpack"} and all(v > 0 for v in row.values()), (cfg, plan)

@@ -77,7 +77,7 @@ def test_graph_replays_signal_every_layer_to_a_waiting_thread():
             for l in range(w.n_layers):
                 layers[l][0].copy_(staging[l])          # the "forward pass" writes layer l
                 sess.save_layer(l, s.cuda_stream)
-                torch.cuda._sleep(4_000_000)            # a few milliseconds of other work
+                torch.cuda._sleep(10_000_000)           # some milliseconds of other work
             sess.join(s.cuda_stream)
     n_replays = 4
     transport = _Transport(sess, packed, stride, blob_len, w.n_layers, range(1, n_replays + 1))
@@ -94,15 +94,15 @@ def test_graph_replays_signal_every_layer_to_a_waiting_thread():
         with torch.cuda.stream(s):
             graph.replay()
             finished.record(s)
+        deadline = time.time() + 60
+        while (step, 0) not in transport.returned_at and transport.error is None:
+            assert time.time() < deadline
+            time.sleep(0.0001)
+        still_running.append(not finished.query())
         for l in range(w.n_layers):
             expected[(step, l)] = checkers.oracle_pack(contents[l].cpu().numpy(), lists.tensor(0))
         # the next replay overwrites the packed buffer: let the transport take this step first
         # (what a real sender does by owning one buffer per step in flight)
-        deadline = time.time() + 60
-        while (step, 0) not in transport.returned_at and transport.error is None:
-            assert time.time() < deadline
-            time.sleep(0.0002)
-        still_running.append(not finished.query())
         while (step, w.n_layers - 1) not in transport.got and transport.error is None:
             assert time.time() < deadline
             time.sleep(0.001)
