@@ -402,31 +402,58 @@ int kvt_launch_copy_int64_array_h2d(const int64_t* host_src, int64_t* device_dst
  * has at most max_ranges ranges and every range is at least min_range_bytes long; in a longer or
  * mixed list whose lengths differ, the ranges of at least min_range_bytes still go there one by
  * one and the kernel moves the rest (enqueue_hybrid_copy, copy_kernels.cpp:675-722). Defaults:
- * 8 MiB and 16, measured on MI355X against pinned host memory (the reference's defaults,
- * 256 KiB and 16, suit a part whose copy kernel is slower across PCIe than this one's).
+ * 8 MiB and 16, measured on one MI355X box against pinned host memory (the reference's
+ * defaults, 256 KiB and 16, suit a part whose copy kernel is slower across PCIe than this
+ * one's). They are the rule until kvt_initialize_copy_method_profile has measured the box at
+ * hand, and for good once they have been set through this call (both directions at once).
  * max_ranges = 0 switches the DMA route off. Process-wide. */
 int kvt_set_copy_memcpy_thresholds(uint64_t min_range_bytes, uint64_t max_ranges);
 int kvt_get_copy_memcpy_thresholds(uint64_t* min_range_bytes, uint64_t* max_ranges);
+/* Undoes kvt_set_copy_memcpy_thresholds: the defaults again, and the start-up measurement in
+ * charge again where it has run. */
+int kvt_reset_copy_memcpy_thresholds(void);
 
 enum { KVT_COPY_H2D = 0, KVT_COPY_D2H = 1 };
-/* stands in for initialize_copy_method_profile() kvtransfer/include/copy_kernels.h:15-22
+/* replaces initialize_copy_method_profile()     kvtransfer/include/copy_kernels.h:15-22,
+ *                                               kvtransfer/src/copy_kernels.cpp:495-591, 724-728
  * (called once per copy thread, kvtransfer/src/copy_utils.cpp:52). Checks that `device` is a
- * usable gfx950 part and looks up the address of that device's static metadata array (see
- * kvt_copy_handle_data_kernel_direct_static; otherwise done by that entry point's first call
- * on the device). */
+ * usable gfx950 part, looks up the address of that device's static metadata array (see
+ * kvt_copy_handle_data_kernel_direct_static) and, on the first call of the process, times
+ * loops of DMA copies against the copy kernel on pinned host memory in both directions (8
+ * ranges of 256 KiB and 2 of 16 MiB by either route). From then on, unless the thresholds
+ * above have been set by the caller, kvt_copy_handle_data_with_kernel routes a list of n
+ * ranges and `total` bytes by comparing n * dma_fixed + total * dma_per_byte with kernel_fixed
+ * + total * kernel_per_byte (select_copy_method, copy_kernels.cpp:593-619, which looks the
+ * list up in a table of measured buckets), and in a list of mixed lengths gives a range a DMA
+ * copy of its own when that beats the kernel's cost per byte for it (select_single_block_method,
+ * :621-631). Allocates and frees 32 MiB of pinned and of device memory and blocks for a few
+ * tens of milliseconds: call it at start-up, not in a serving loop. */
 int kvt_initialize_copy_method_profile(int device);
+/* What the start-up measurement found for `direction` (*measured = 0 and zeros before it has
+ * run): microseconds per DMA copy and per MiB moved by it, per kernel launch (metadata upload
+ * included) and per MiB moved by it; the shortest range that gets a DMA copy of its own in a
+ * mixed list under the rule in force (~0: none); the time the measurement took. Any pointer
+ * may be NULL. */
+int kvt_get_copy_method_profile(int direction, double* dma_fixed_us, double* dma_us_per_mib,
+                                double* kernel_fixed_us, double* kernel_us_per_mib,
+                                uint64_t* single_range_min_bytes, int* measured, double* elapsed_ms);
 /* replaces get_kernel_copy_buffer()             kvtransfer/include/copy_utils.h:127,
  *                                               kvtransfer/src/copy_utils.cpp:9-57,137-146
  * The calling THREAD's metadata buffers for kvt_copy_handle_data_with_kernel: device and
- * pinned host memory of 3 * 8 * max_block_num bytes each (max_block_num <= 0: 8192), created on
- * first use, re-created when the thread asks for another device or more ranges, released
- * when the thread ends. */
+ * pinned host memory of 3 * 8 * max_block_num bytes each (max_block_num <= 0: 8192), one pair
+ * per (thread, device), created on first use and released when the thread ends. Asking for
+ * MORE ranges on the same device replaces the pair, after the thread's two streams have
+ * drained: the pointers handed out before are invalid from then on (the reference sizes its
+ * buffers once from the environment and never regrows). A request for another device, or for
+ * a stream, leaves them alone. */
 int kvt_get_kernel_copy_buffer(int device, int64_t max_block_num, int64_t** dev_meta,
                                int64_t** host_meta);
 /* replaces get_thread_local_h2d_stream() / get_thread_local_d2h_stream()
  *                                               kvtransfer/src/copy_utils.cpp:59-95,148-154
  * direction = KVT_COPY_H2D / KVT_COPY_D2H: the calling thread's non-blocking stream for that
- * direction on `device` (the reference's live on the device of the thread's buffers). */
+ * direction on `device` (the reference's live on the device of the thread's buffers). The
+ * handle stays valid until the thread ends, whatever buffers or devices the thread asks for
+ * in between. */
 int kvt_get_thread_local_stream(int device, int direction, void** stream);
 /* replaces copy_handle_data_with_kernel()       kvtransfer/include/copy_kernels.h:87-97,
  *                                               kvtransfer/src/copy_kernels.cpp:733-827

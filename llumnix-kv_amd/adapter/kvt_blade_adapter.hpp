@@ -265,21 +265,34 @@ inline void apply_kernel_copy_sm_usage(int device_id) {
 
 // BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES / BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS
 // (kvtransfer/src/copy_kernels.cpp:496-499), when set, replace the library's own thresholds
-// for handing a list to the DMA engines; unset or unparsable values leave them alone.
+// for handing a list to the DMA engines; unset or unparsable values leave them alone (and
+// with neither set the library's start-up measurement stays free to choose them).
 inline void apply_copy_memcpy_env() {
   uint64_t min_bytes = 0, max_ranges = 0;
   raise(kvt_get_copy_memcpy_thresholds(&min_bytes, &max_ranges));
   auto read = [](const char* name, uint64_t* out) {
     const char* v = std::getenv(name);
-    if (v == nullptr || *v == '\0') return;
+    if (v == nullptr || *v == '\0') return false;
     char* end = nullptr;
     const unsigned long long x = std::strtoull(v, &end, 10);
-    if (end != v && *end == '\0') *out = x;
+    if (end == v || *end != '\0') return false;
+    *out = x;
+    return true;
   };
-  read("BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES", &min_bytes);
-  read("BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS", &max_ranges);
+  const bool a = read("BLLM_KVTRANS_COPY_MEMCPY_BLOCK_THRESHOLD_BYTES", &min_bytes);
+  const bool b = read("BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS", &max_ranges);
+  if (!a && !b) return;
   if (min_bytes == 0) min_bytes = 1;
   raise(kvt_set_copy_memcpy_thresholds(min_bytes, max_ranges));
+}
+
+// initialize_copy_method_profile as the reference's copy threads call it
+// (kvtransfer/src/copy_utils.cpp:52): BLLM_KVTRANS_COPY_PROFILE_ENABLE=0 skips the
+// measurement (kvtransfer/src/copy_kernels.cpp:501-508) and leaves the thresholds as they are.
+inline void initialize_copy_method_profile(int device_id) {
+  const char* v = std::getenv("BLLM_KVTRANS_COPY_PROFILE_ENABLE");
+  if (v != nullptr && std::atoi(v) == 0) return;  // env_bool, copy_kernels.cpp:168-174
+  raise(kvt_initialize_copy_method_profile(device_id));
 }
 
 }  // namespace kvt_adapter

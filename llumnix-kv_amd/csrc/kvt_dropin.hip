@@ -3,6 +3,7 @@
 // buffers.
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -48,8 +49,58 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
 }
 
 // When a list goes to the DMA engines instead of a kernel (kvt_set_copy_memcpy_thresholds).
+// Indexed by direction (KVT_COPY_H2D, KVT_COPY_D2H). The defaults were measured on one MI355X
+// box; kvt_initialize_copy_method_profile replaces them with what it measures on the box at
+// hand unless the caller has set them.
 constexpr uint64_t kDmaMaxRanges = 16, kDmaMinBytes = 8ull << 20;
-std::atomic<uint64_t> g_dma_max_ranges{kDmaMaxRanges}, g_dma_min_bytes{kDmaMinBytes};
+std::atomic<uint64_t> g_dma_max_ranges[2] = {{kDmaMaxRanges}, {kDmaMaxRanges}};
+std::atomic<uint64_t> g_dma_min_bytes[2] = {{kDmaMinBytes}, {kDmaMinBytes}};
+std::atomic<bool> g_dma_thresholds_set{false};  // by the caller: a profile leaves them alone
+
+// What the start-up measurement found, per direction: a list of n ranges and `total` bytes takes
+// about n * dma_fixed_us + total * dma_us_per_byte through a loop of DMA copies and
+// kernel_fixed_us + total * kernel_us_per_byte through the copy kernel (metadata upload and
+// launch included). While `measured` is set and the caller has not fixed the thresholds, the
+// route is chosen by comparing the two; the thresholds are the rule before that and the override.
+struct CopyCost {
+  double dma_fixed_us = 0, dma_us_per_byte = 0, kernel_fixed_us = 0, kernel_us_per_byte = 0;
+};
+struct CopyProfile {
+  bool measured = false;
+  CopyCost cost[2];
+  double elapsed_ms = 0;
+};
+std::mutex g_profile_mu;           // writers; readers go through g_profile_live
+CopyProfile g_profile;
+std::atomic<const CopyProfile*> g_profile_live{nullptr};  // set once, never freed
+
+enum Route { kRouteAuto = 0, kRouteKernel = 1, kRouteDma = 2 };
+
+const CopyCost* live_cost(int direction) {
+  if (g_dma_thresholds_set.load(std::memory_order_relaxed)) return nullptr;
+  const CopyProfile* p = g_profile_live.load(std::memory_order_acquire);
+  return p ? &p->cost[direction] : nullptr;
+}
+// The whole list through DMA copies?
+bool list_to_dma(int direction, uint64_t n, uint64_t total, uint64_t shortest) {
+  if (const CopyCost* c = live_cost(direction))
+    return static_cast<double>(n) * c->dma_fixed_us + static_cast<double>(total) * c->dma_us_per_byte <
+           c->kernel_fixed_us + static_cast<double>(total) * c->kernel_us_per_byte;
+  return n <= g_dma_max_ranges[direction].load(std::memory_order_relaxed) &&
+         shortest >= g_dma_min_bytes[direction].load(std::memory_order_relaxed);
+}
+// Shortest range worth a DMA copy of its own when a kernel launch moves the rest anyway
+// (~0: none).
+uint64_t single_dma_min(int direction) {
+  if (const CopyCost* c = live_cost(direction)) {
+    const double gain = c->kernel_us_per_byte - c->dma_us_per_byte;  // per byte moved by DMA instead
+    if (gain <= 0) return ~0ull;
+    const double bytes = c->dma_fixed_us / gain;
+    return bytes >= 1e18 ? ~0ull : static_cast<uint64_t>(bytes) + 1;
+  }
+  if (g_dma_max_ranges[direction].load(std::memory_order_relaxed) == 0) return ~0ull;
+  return g_dma_min_bytes[direction].load(std::memory_order_relaxed);
+}
 
 // Workgroups per range when the lengths are known on the host: the mean number of slices
 // per range (bounded). Equal lengths then get exactly one slice per workgroup, the fastest
@@ -64,7 +115,8 @@ int rows_for(uint64_t slices, uint64_t n_ranges) {
 // are element counts).
 int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks, uint64_t n,
                 uint64_t tensor_data_size, int direction, bool halve, int device, void* stream,
-                int64_t* dev_meta, int64_t* host_meta, int64_t max_block_num) {
+                int64_t* dev_meta, int64_t* host_meta, int64_t max_block_num,
+                Route route = kRouteAuto) {
   if (n == 0) return KVT_OK;
   if (!tensor_buf || !layer_gpu_ptr || !blocks || !dev_meta || !host_meta)
     return fail(KVT_ERR_INVALID, "copy_handle_data: null argument");
@@ -76,10 +128,14 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
   for (uint64_t i = 0; i < n; ++i) {
     if (blocks[i].length == 0) return fail(KVT_ERR_INVALID, "copy_handle_data: zero-length range");
     if (halve && (blocks[i].length & 1)) return fail(KVT_ERR_INVALID, "odd bf16 byte length");
-    total += blocks[i].length;
+    // sums that wrap would pass the span checks below with a small extent
+    uint64_t end = 0;
+    if (__builtin_add_overflow(total, blocks[i].length, &total) ||
+        __builtin_add_overflow(blocks[i].dst_offset, blocks[i].length, &end))
+      return fail(KVT_ERR_OUT_OF_RANGE, "copy_handle_data: offset + length exceeds 64 bits");
     shortest = std::min(shortest, blocks[i].length);
     longest = std::max(longest, blocks[i].length);
-    layer_extent = std::max(layer_extent, blocks[i].dst_offset + blocks[i].length);
+    layer_extent = std::max(layer_extent, end);
   }
   if (total != tensor_data_size)
     return fail(KVT_ERR_INVALID, "copy_handle_data: tensor_data_size != sum of range lengths");
@@ -93,11 +149,12 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
   const hipStream_t s = static_cast<hipStream_t>(stream);
   // A few very large ranges go to the DMA engines, one copy each. The reference makes this
   // choice (memcpy loop or kernel) from a profile it takes at start-up
-  // (copy_kernels.cpp:495-619); here it is fixed from measurements on MI355X: against pinned
-  // host memory a copy of 128 MiB runs at 57 GB/s where the kernel's stores across PCIe reach
-  // 54, the kernel wins below about 8 MiB per copy (2 MiB: 53 against 33 GB/s).
-  if (!halve && n <= g_dma_max_ranges.load(std::memory_order_relaxed) &&
-      shortest >= g_dma_min_bytes.load(std::memory_order_relaxed)) {
+  // (copy_kernels.cpp:495-619); so does kvt_initialize_copy_method_profile here, and before it
+  // has run the thresholds decide, fixed from measurements on one MI355X: against pinned host
+  // memory a copy of 128 MiB runs at 57 GB/s where the kernel's stores across PCIe reach 54,
+  // the kernel wins below about 8 MiB per copy (2 MiB: 53 against 33 GB/s).
+  if (route == kRouteDma ||
+      (route == kRouteAuto && !halve && list_to_dma(direction, n, total, shortest))) {
     uint64_t cursor = 0;
     for (uint64_t i = 0; i < n; ++i) {
       uint8_t* host = static_cast<uint8_t*>(tensor_buf) + cursor;
@@ -116,9 +173,8 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
   // with its per-range rule select_single_block_method, :621-631).
   static thread_local std::vector<kvt_ipc_block> work;
   work.clear();
-  const uint64_t dma_min = g_dma_min_bytes.load(std::memory_order_relaxed);
-  const bool split = !halve && shortest != longest && longest >= dma_min &&
-                     g_dma_max_ranges.load(std::memory_order_relaxed) != 0;
+  const uint64_t dma_min = route == kRouteAuto ? single_dma_min(direction) : ~0ull;
+  const bool split = !halve && shortest != longest && longest >= dma_min;
   {
     uint64_t cursor = 0;
     for (uint64_t i = 0; i < n; ++i) {
@@ -193,7 +249,11 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
   uint64_t cursor = 0, slices = 0, layer_extent = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const kvt_ipc_block& b = blocks[i];
-    layer_extent = std::max(layer_extent, b.dst_offset + b.length);
+    uint64_t end = 0;
+    if (__builtin_add_overflow(b.dst_offset, b.length, &end))
+      return fail(KVT_ERR_OUT_OF_RANGE,
+                  "copy_handle_data_kernel_direct: offset + length exceeds 64 bits");
+    layer_extent = std::max(layer_extent, end);
     const uint64_t host_off = explicit_host_offsets ? b.src_offset : cursor;
     if (b.length == 0 || host_off > tensor_data_size || b.length > tensor_data_size - host_off)
       return fail(KVT_ERR_OUT_OF_RANGE,
@@ -294,8 +354,11 @@ int kvt_launch_copy_int64_array_h2d(const int64_t* host_src, int64_t* device_dst
 }
 
 // Per-thread metadata buffers and streams of the copy threads (CopyKernelCtx,
-// kvtransfer/src/copy_utils.cpp:9-154): created on first use, re-created when the thread
-// moves to another device or asks for more ranges, released when the thread ends.
+// kvtransfer/src/copy_utils.cpp:9-154): one context per (thread, device), created on first
+// use and released when the thread ends. Streams and buffers have separate lifetimes: a
+// stream handed out stays valid until its thread ends, whatever is asked for afterwards; the
+// buffers are replaced only when the same thread asks for more ranges on the same device
+// (after both streams have drained), which invalidates the pointers handed out before.
 namespace {
 struct CopyThreadCtx {
   int device = -1;
@@ -304,22 +367,49 @@ struct CopyThreadCtx {
   int64_t* host = nullptr;
   hipStream_t streams[2] = {nullptr, nullptr};  // KVT_COPY_H2D, KVT_COPY_D2H
 
-  void release() {
-    if (device >= 0) (void)hipSetDevice(device);
-    for (hipStream_t& st : streams)
-      if (st) {
-        (void)hipStreamSynchronize(st);  // the streams may still reference the buffers
-        (void)hipStreamDestroy(st);
-        st = nullptr;
-      }
+  void drain() {
+    for (hipStream_t st : streams)
+      if (st) (void)hipStreamSynchronize(st);  // launches in flight may still read the buffers
+  }
+  void release_buffers() {
+    if (dev) forget_device_spans();
     if (dev) (void)hipFree(dev);
     if (host) (void)hipHostFree(host);
     dev = host = nullptr;
     capacity = 0;
   }
-  ~CopyThreadCtx() { release(); }
+  void release() {
+    if (device < 0) return;
+    int prev = -1;
+    const bool restore = hipGetDevice(&prev) == hipSuccess && prev != device;
+    (void)hipSetDevice(device);
+    drain();
+    for (hipStream_t& st : streams)
+      if (st) {
+        (void)hipStreamDestroy(st);
+        st = nullptr;
+      }
+    release_buffers();
+    if (restore) (void)hipSetDevice(prev);
+  }
 };
-thread_local CopyThreadCtx g_copy_ctx;
+struct CopyThreadCtxs {
+  std::vector<CopyThreadCtx*> by_device;
+  CopyThreadCtx& of(int device) {
+    for (CopyThreadCtx* c : by_device)
+      if (c->device == device) return *c;
+    by_device.push_back(new CopyThreadCtx());
+    by_device.back()->device = device;
+    return *by_device.back();
+  }
+  ~CopyThreadCtxs() {
+    for (CopyThreadCtx* c : by_device) {
+      c->release();
+      delete c;
+    }
+  }
+};
+thread_local CopyThreadCtxs g_copy_ctxs;
 }  // namespace
 
 int kvt_get_kernel_copy_buffer(int device, int64_t max_block_num, int64_t** dev_meta,
@@ -329,17 +419,19 @@ int kvt_get_kernel_copy_buffer(int device, int64_t max_block_num, int64_t** dev_
       return fail(KVT_ERR_INVALID, "kvt_get_kernel_copy_buffer: null argument");
     if (int rc = check_device(device)) return rc;
     if (max_block_num <= 0) max_block_num = 8192;
-    CopyThreadCtx& c = g_copy_ctx;
-    if (c.device != device || c.capacity < max_block_num) {
+    if (max_block_num > (int64_t(1) << 31))
+      return fail(KVT_ERR_INVALID, "kvt_get_kernel_copy_buffer: max_block_num too large");
+    CopyThreadCtx& c = g_copy_ctxs.of(device);
+    if (c.capacity < max_block_num) {
       DeviceGuard g;
       if (int rc = g.enter(device)) return rc;
-      c.release();
-      c.device = device;
+      c.drain();
+      c.release_buffers();
       const size_t bytes = 3 * sizeof(int64_t) * static_cast<size_t>(max_block_num);
       KVT_HIP(hipMalloc(reinterpret_cast<void**>(&c.dev), bytes));
       const hipError_t e = hipHostMalloc(reinterpret_cast<void**>(&c.host), bytes, hipHostMallocDefault);
       if (e != hipSuccess) {
-        c.release();
+        c.release_buffers();
         return hip_fail(e, "kvt_get_kernel_copy_buffer: pinned metadata buffer");
       }
       c.capacity = max_block_num;
@@ -355,11 +447,7 @@ int kvt_get_thread_local_stream(int device, int direction, void** stream) {
     if (!stream || (direction != KVT_COPY_H2D && direction != KVT_COPY_D2H))
       return fail(KVT_ERR_INVALID, "kvt_get_thread_local_stream: bad argument");
     if (int rc = check_device(device)) return rc;
-    CopyThreadCtx& c = g_copy_ctx;
-    if (c.device != device) {
-      c.release();
-      c.device = device;
-    }
+    CopyThreadCtx& c = g_copy_ctxs.of(device);
     if (!c.streams[direction]) {
       DeviceGuard g;
       if (int rc = g.enter(device)) return rc;
@@ -373,14 +461,17 @@ int kvt_get_thread_local_stream(int device, int direction, void** stream) {
 int kvt_set_copy_memcpy_thresholds(uint64_t min_range_bytes, uint64_t max_ranges) {
   if (min_range_bytes == 0)
     return fail(KVT_ERR_INVALID, "kvt_set_copy_memcpy_thresholds: min_range_bytes must be positive");
-  g_dma_min_bytes.store(min_range_bytes, std::memory_order_relaxed);
-  g_dma_max_ranges.store(max_ranges, std::memory_order_relaxed);
+  for (int d = 0; d < 2; ++d) {
+    g_dma_min_bytes[d].store(min_range_bytes, std::memory_order_relaxed);
+    g_dma_max_ranges[d].store(max_ranges, std::memory_order_relaxed);
+  }
+  g_dma_thresholds_set.store(true, std::memory_order_relaxed);
   return KVT_OK;
 }
 
 int kvt_get_copy_memcpy_thresholds(uint64_t* min_range_bytes, uint64_t* max_ranges) {
-  if (min_range_bytes) *min_range_bytes = g_dma_min_bytes.load(std::memory_order_relaxed);
-  if (max_ranges) *max_ranges = g_dma_max_ranges.load(std::memory_order_relaxed);
+  if (min_range_bytes) *min_range_bytes = g_dma_min_bytes[KVT_COPY_D2H].load(std::memory_order_relaxed);
+  if (max_ranges) *max_ranges = g_dma_max_ranges[KVT_COPY_D2H].load(std::memory_order_relaxed);
   return KVT_OK;
 }
 
@@ -444,12 +535,142 @@ int static_scratch(int device, int64_t** out) {
 
 extern "C" {
 
+}  // extern "C"
+
+// The start-up measurement (initialize_copy_method_profile_impl, kvtransfer/src/
+// copy_kernels.cpp:495-591): loops of DMA copies against the copy kernel on pinned host
+// memory, per direction. The reference fills a table over 6 counts x 7 sizes of up to 64 MiB
+// and looks lists up by bucket; here two list shapes per method (8 x 256 KiB and 2 x 16 MiB)
+// give each method's fixed cost and cost per byte, and a list is routed by comparing the two
+// predictions. 32 MiB of pinned and of device memory, a few tens of milliseconds, once per
+// process.
+namespace {
+struct ProfileBuffers {
+  uint8_t* host = nullptr;
+  uint8_t* dev = nullptr;
+  int64_t* meta_dev = nullptr;
+  int64_t* meta_host = nullptr;
+  hipStream_t stream = nullptr;
+  hipEvent_t a = nullptr, b = nullptr;
+  ~ProfileBuffers() {
+    if (stream) (void)hipStreamSynchronize(stream);
+    if (a) (void)hipEventDestroy(a);
+    if (b) (void)hipEventDestroy(b);
+    if (stream) (void)hipStreamDestroy(stream);
+    if (dev) forget_device_spans();
+    if (dev) (void)hipFree(dev);
+    if (meta_dev) (void)hipFree(meta_dev);
+    if (host) (void)hipHostFree(host);
+    if (meta_host) (void)hipHostFree(meta_host);
+  }
+};
+constexpr uint64_t kProfileBytes = 32ull << 20;
+constexpr uint64_t kProfileMaxRanges = 64;
+
+// Average microseconds of one list of `count` ranges of `size` bytes by one route.
+int time_copy_route(ProfileBuffers& pb, Route route, uint64_t count, uint64_t size, int direction,
+                    int device, double* us) {
+  std::vector<kvt_ipc_block> blocks(count);
+  for (uint64_t i = 0; i < count; ++i) blocks[i] = kvt_ipc_block{0, i * size, size};
+  auto enqueue = [&]() -> int {
+    return handle_data(pb.host, pb.dev, blocks.data(), count, count * size, direction, false, device,
+                       pb.stream, pb.meta_dev, pb.meta_host, kProfileMaxRanges, route);
+  };
+  constexpr int kIters = 3;
+  if (int rc = enqueue()) return rc;  // warm-up
+  KVT_HIP(hipStreamSynchronize(pb.stream));
+  KVT_HIP(hipEventRecord(pb.a, pb.stream));
+  for (int i = 0; i < kIters; ++i)
+    if (int rc = enqueue()) return rc;
+  KVT_HIP(hipEventRecord(pb.b, pb.stream));
+  KVT_HIP(hipEventSynchronize(pb.b));
+  float ms = 0;
+  KVT_HIP(hipEventElapsedTime(&ms, pb.a, pb.b));
+  *us = static_cast<double>(ms) * 1000.0 / kIters;
+  return KVT_OK;
+}
+
+int measure_copy_routes(int device, CopyProfile* out) {
+  DeviceGuard g;
+  if (int rc = g.enter(device)) return rc;
+  const auto t0 = std::chrono::steady_clock::now();
+  ProfileBuffers pb;
+  KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&pb.host), kProfileBytes, hipHostMallocDefault));
+  KVT_HIP(hipMalloc(reinterpret_cast<void**>(&pb.dev), kProfileBytes));
+  KVT_HIP(hipMemset(pb.dev, 0, kProfileBytes));
+  KVT_HIP(hipMalloc(reinterpret_cast<void**>(&pb.meta_dev), 3 * kProfileMaxRanges * sizeof(int64_t)));
+  KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&pb.meta_host), 3 * kProfileMaxRanges * sizeof(int64_t),
+                        hipHostMallocDefault));
+  KVT_HIP(hipStreamCreateWithFlags(&pb.stream, hipStreamNonBlocking));
+  KVT_HIP(hipEventCreate(&pb.a));
+  KVT_HIP(hipEventCreate(&pb.b));
+  constexpr uint64_t n1 = 8, s1 = 256ull << 10;  // many short ranges: the fixed costs show
+  constexpr uint64_t n2 = 2, s2 = 16ull << 20;   // few long ones: the cost per byte shows
+  for (int direction : {KVT_COPY_H2D, KVT_COPY_D2H}) {
+    double d1 = 0, d2 = 0, k1 = 0, k2 = 0;
+    if (int rc = time_copy_route(pb, kRouteDma, n1, s1, direction, device, &d1)) return rc;
+    if (int rc = time_copy_route(pb, kRouteDma, n2, s2, direction, device, &d2)) return rc;
+    if (int rc = time_copy_route(pb, kRouteKernel, n1, s1, direction, device, &k1)) return rc;
+    if (int rc = time_copy_route(pb, kRouteKernel, n2, s2, direction, device, &k2)) return rc;
+    CopyCost& c = out->cost[direction];
+    // DMA: d = n * fixed + n * s * per_byte, two equations in (fixed, per_byte)
+    const double t1 = static_cast<double>(n1 * s1), t2 = static_cast<double>(n2 * s2);
+    const double det = static_cast<double>(n1) * t2 - static_cast<double>(n2) * t1;
+    c.dma_fixed_us = std::max(0.0, (d1 * t2 - d2 * t1) / det);
+    c.dma_us_per_byte = std::max(0.0, (static_cast<double>(n1) * d2 - static_cast<double>(n2) * d1) / det);
+    // kernel: k = fixed + total * per_byte
+    c.kernel_us_per_byte = std::max(0.0, (k2 - k1) / (t2 - t1));
+    c.kernel_fixed_us = std::max(0.0, k1 - t1 * c.kernel_us_per_byte);
+  }
+  out->measured = true;
+  out->elapsed_ms =
+      std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  return KVT_OK;
+}
+}  // namespace
+
+extern "C" {
+
 int kvt_initialize_copy_method_profile(int device) {
   return guarded([&]() -> int {
     if (int rc = check_device(device)) return rc;
     int64_t* unused = nullptr;
-    return static_scratch(device, &unused);
+    if (int rc = static_scratch(device, &unused)) return rc;
+    std::lock_guard<std::mutex> lock(g_profile_mu);
+    if (g_profile.measured) return KVT_OK;  // once per process, like the reference's call_once
+    CopyProfile p;
+    if (int rc = measure_copy_routes(device, &p)) return rc;
+    g_profile = p;
+    g_profile_live.store(&g_profile, std::memory_order_release);
+    return KVT_OK;
   });
+}
+
+int kvt_get_copy_method_profile(int direction, double* dma_fixed_us, double* dma_us_per_mib,
+                                double* kernel_fixed_us, double* kernel_us_per_mib,
+                                uint64_t* single_range_min_bytes, int* measured, double* elapsed_ms) {
+  if (direction != KVT_COPY_H2D && direction != KVT_COPY_D2H)
+    return fail(KVT_ERR_INVALID, "kvt_get_copy_method_profile: bad direction");
+  std::lock_guard<std::mutex> lock(g_profile_mu);
+  const CopyCost& c = g_profile.cost[direction];
+  constexpr double kMiB = 1048576.0;
+  if (dma_fixed_us) *dma_fixed_us = c.dma_fixed_us;
+  if (dma_us_per_mib) *dma_us_per_mib = c.dma_us_per_byte * kMiB;
+  if (kernel_fixed_us) *kernel_fixed_us = c.kernel_fixed_us;
+  if (kernel_us_per_mib) *kernel_us_per_mib = c.kernel_us_per_byte * kMiB;
+  if (single_range_min_bytes) *single_range_min_bytes = single_dma_min(direction);
+  if (measured) *measured = g_profile.measured ? 1 : 0;
+  if (elapsed_ms) *elapsed_ms = g_profile.elapsed_ms;
+  return KVT_OK;
+}
+
+int kvt_reset_copy_memcpy_thresholds(void) {
+  for (int d = 0; d < 2; ++d) {
+    g_dma_min_bytes[d].store(kDmaMinBytes, std::memory_order_relaxed);
+    g_dma_max_ranges[d].store(kDmaMaxRanges, std::memory_order_relaxed);
+  }
+  g_dma_thresholds_set.store(false, std::memory_order_relaxed);
+  return KVT_OK;
 }
 
 int kvt_copy_handle_data_kernel_direct_static(void* tensor_buf, void* layer_gpu_ptr,

@@ -80,17 +80,25 @@ uint32_t device_cu_count(int device) {
 // tensor. Spans that passed are remembered per thread (a serving loop reuses its buffers),
 // so the steady state costs a few comparisons and no runtime call; an entry is trusted for
 // 256 uses and then asked for again, since the memory behind an address can change hands.
+static std::atomic<uint64_t> g_span_epoch{1};
+void forget_device_spans() { g_span_epoch.fetch_add(1, std::memory_order_relaxed); }
+
 int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) {
   if (bytes == 0) return KVT_OK;
   struct Span {
     uintptr_t lo = 0, hi = 0;
     unsigned uses = 0;
+    uint64_t epoch = 0;
   };
+  // Allocations the runtime has answered for lately, per thread: a lookup costs microseconds
+  // and the same few buffers come back launch after launch. An answer is trusted for a bounded
+  // number of uses and dropped as soon as the library itself frees device memory.
   static thread_local Span seen[8];
   static thread_local unsigned next = 0;
   const uintptr_t p = reinterpret_cast<uintptr_t>(ptr);
+  const uint64_t epoch = g_span_epoch.load(std::memory_order_relaxed);
   for (Span& s : seen)
-    if (p >= s.lo && p < s.hi && bytes <= s.hi - p) {
+    if (s.epoch == epoch && p >= s.lo && p < s.hi && bytes <= s.hi - p) {
       if (++s.uses < 256) return KVT_OK;
       s = Span{};  // ask the runtime again below
       break;
@@ -114,7 +122,7 @@ int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) 
                 what + ": " + std::to_string(bytes) +
                     " bytes reach beyond the allocation that holds the pointer (" +
                     std::to_string(p < lo || p - lo > size ? 0 : size - (p - lo)) + " bytes left)");
-  seen[next++ % 8] = Span{lo, lo + size, 0};
+  seen[next++ % 8] = Span{lo, lo + size, 0, epoch};
   return KVT_OK;
 }
 
@@ -209,6 +217,7 @@ int kvt_cache_register(int device, const void* const* ptrs, uint32_t n_layers, u
 
 void kvt_cache_destroy(kvt_cache* c) {
   if (!c) return;
+  forget_device_spans();  // the caller is about to free the tensors this cache named
   if (c->dev_ptrs) (void)hipFree(c->dev_ptrs);
   delete c;
 }

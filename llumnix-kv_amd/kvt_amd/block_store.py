@@ -117,6 +117,7 @@ class FileBlockStore:
         torch = self._torch
         n_layers = len(self._kv)
         if layer_idx == 0:
+            self._abandon_step()       # a step that never reached its last layer
             todo, seen = [], set()
             for blkid, blkhash in blks:
                 if blkhash not in seen and not _blk_ready(self._path(blkhash)[0]):
@@ -124,30 +125,60 @@ class FileBlockStore:
                     todo.append((blkid, blkhash))
             if len(todo) > self._ring_entries:
                 raise ValueError("more new blocks in one step than the ring has entries")
-            self._step = None
             if todo:
-                entries, _ = self._ring.reserve([self._key(h) for _, h in todo])
-                objs = torch.empty(len(todo) * self._entry, dtype=torch.uint8, device="cuda")
-                self._step = (todo, entries, objs, self._plan([b for b, _ in todo]))
+                entries, new = self._ring.reserve([self._key(h) for _, h in todo])
+                # only the entries this call was given (new) are written and settled by it; the
+                # others are being filled, or were filled, by whoever reserved them first
+                fresh = [b for (b, _), n in zip(todo, new) if n]
+                try:
+                    objs = torch.empty(len(fresh) * self._entry, dtype=torch.uint8, device="cuda")
+                    plan = self._plan(fresh) if fresh else None
+                except Exception:
+                    self._ring.release(entries[new])
+                    raise
+                self._step = (todo, entries, new, objs, plan)
         if self._step is None:
             return 0
-        todo, entries, objs, plan = self._step
-        self._stream.wait_stream(torch.cuda.current_stream())      # the layer has been computed
-        plan.pack(self._cache, layer_idx, 1, objs[layer_idx * self._obj:], self._obj,
-                  self._stream.cuda_stream)
-        if layer_idx != n_layers - 1:
-            return 0
-        self._ring.save(entries, objs.data_ptr(), self._entry, self._stream.cuda_stream)
-        self._stream.synchronize()
-        for (blkid, blkhash), idx in zip(todo, entries):
-            blkdir, datapath = self._path(blkhash)
-            os.makedirs(blkdir, exist_ok=True)
-            self._ring.entry(idx).tofile(datapath)
-            with open(os.path.join(blkdir, "ready"), "w"):
-                pass
-        plan.close()
+        todo, entries, new, objs, plan = self._step
+        try:
+            if plan is not None:
+                self._stream.wait_stream(torch.cuda.current_stream())  # the layer has been computed
+                plan.pack(self._cache, layer_idx, 1, objs[layer_idx * self._obj:], self._obj,
+                          self._stream.cuda_stream)
+            if layer_idx != n_layers - 1:
+                return 0
+            if plan is not None:
+                self._ring.save(entries[new], objs.data_ptr(), self._entry, self._stream.cuda_stream)
+                new = np.zeros_like(new)          # settled: nothing left to give back on failure
+                self._step = (todo, entries, new, objs, plan)
+                self._stream.synchronize()
+            for (blkid, blkhash), idx in zip(todo, entries):
+                blkdir, datapath = self._path(blkhash)
+                os.makedirs(blkdir, exist_ok=True)
+                self._ring.wait(idx)
+                self._ring.entry(idx).tofile(datapath)
+                with open(os.path.join(blkdir, "ready"), "w"):
+                    pass
+        except Exception:
+            self._abandon_step()
+            raise
+        if plan is not None:
+            plan.close()
         self._step = None
         return len(todo)
+
+    def _abandon_step(self):
+        """Gives back what an unfinished layer-wise step holds: its claims on ring entries (an
+        entry that stays claimed is never handed out again) and its plan."""
+        if self._step is None:
+            return
+        todo, entries, new, objs, plan = self._step
+        self._step = None
+        self._stream.synchronize()          # packs of the abandoned step still write to objs
+        if new.any():
+            self._ring.release(entries[new])
+        if plan is not None:
+            plan.close()
 
     def load_blocks(self, blks):
         """blks: [(blkid, blkhash)]: every block must be ready (file_backend.py:219-221); its
@@ -187,6 +218,7 @@ class FileBlockStore:
 
     def close(self):
         if self._kv is not None:
+            self._abandon_step()
             self._ring.close()
             self._cache.close()
             self._kv = None

@@ -89,7 +89,7 @@ def test_memcpy_route_thresholds_are_process_wide_settings():
         assert (a.value, b.value) == (256 << 10, 4)
         assert lib.kvt_set_copy_memcpy_thresholds(1, 0) == 0          # route switched off
     finally:
-        assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+        assert lib.kvt_reset_copy_memcpy_thresholds() == 0
 
 
 def test_launcher_stand_in_exports_the_reference_names():

@@ -89,4 +89,4 @@ def test_adapter_hands_the_memcpy_variables_to_the_library(monkeypatch):
         monkeypatch.setenv("BLLM_KVTRANS_COPY_MEMCPY_MAX_BLOCKS", "0")               # route off
         assert lib.kvtadp_apply_copy_memcpy_env() == 0 and current() == (262144, 0)
     finally:
-        assert k.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+        assert k.kvt_reset_copy_memcpy_thresholds() == 0

@@ -107,3 +107,33 @@ def test_layer_wise_save_while_the_layers_are_being_produced(tmp_path):
     for l in range(len(names)):
         assert store.save_kv_layer(l, blks) == 0
     store.close()
+
+
+def test_abandoned_layer_wise_steps_give_their_ring_entries_back(tmp_path):
+    """A step that never reaches its last layer (an aborted forward pass, a failing pack) must
+    not keep its entries claimed: after more abandoned steps than the ring has entries the
+    next complete step still finds room, and what it writes is exact."""
+    kv = _caches(5)
+    store = FileBlockStore(str(tmp_path), ring_entries=4)
+    store.register_kv_caches(kv)
+    names = list(kv)
+    for attempt in range(6):                       # 6 x 3 blocks > 4 entries
+        blks = [(b, "gone_%d_%d" % (attempt, b)) for b in (1, 2, 3)]
+        assert store.save_kv_layer(0, blks) == 0   # layer 0 only: the step is then dropped
+    # a pack that fails mid-step settles its claims too
+    blks = [(7, "fail_7"), (8, "fail_8")]
+    assert store.save_kv_layer(0, blks) == 0
+    with pytest.raises(Exception):
+        store.save_kv_layer(len(names) + 5, blks)  # no such layer: the pack is refused
+    assert store._step is None
+    stats = store._ring.stats()
+    assert stats["entries_in_use"] == 0, stats
+    blks = [(9, "kept_9"), (10, "kept_10"), (11, "kept_11"), (12, "kept_12")]
+    for l in range(len(names)):
+        done = store.save_kv_layer(l, blks)
+    assert done == 4
+    for blkid, blkhash in blks:
+        assert np.array_equal(np.fromfile(tmp_path / blkhash / "0.data", dtype=np.uint8),
+                              _expected_file(kv, blkid)), blkhash
+    assert not (tmp_path / "gone_0_1").exists() and not (tmp_path / "fail_7").exists()
+    store.close()

@@ -441,10 +441,50 @@ def test_reference_launcher_names_link_level_stand_in():
     assert b"bad argument" in lib.kvt_last_error()
 
 
+def test_start_up_profile_measures_both_copy_routes():
+    """initialize_copy_method_profile (copy_kernels.cpp:495-591): loops of DMA copies against
+    the copy kernel on pinned memory, once per process. What it finds must look like a PCIe
+    part (tens of GB/s either way, microseconds of fixed cost), it decides the route unless the
+    caller has set the thresholds, and either route gives the same bytes."""
+    lib = kvt_amd.lib()
+    assert lib.kvt_initialize_copy_method_profile(99) != 0
+    assert lib.kvt_reset_copy_memcpy_thresholds() == 0
+    assert lib.kvt_initialize_copy_method_profile(0) == 0, lib.kvt_last_error()
+    d_fix, d_mib, k_fix, k_mib, ms = (C.c_double() for _ in range(5))
+    single, measured = C.c_uint64(), C.c_int()
+    for direction in (0, 1):
+        assert lib.kvt_get_copy_method_profile(direction, C.byref(d_fix), C.byref(d_mib),
+                                               C.byref(k_fix), C.byref(k_mib), C.byref(single),
+                                               C.byref(measured), C.byref(ms)) == 0
+        assert measured.value == 1 and 0 < ms.value < 2000.0
+        print("copy routes %s: DMA %.1f us + %.2f us/MiB, kernel %.1f us + %.2f us/MiB, own DMA "
+              "copy from %d bytes (%.1f ms)" % ("H2D D2H".split()[direction], d_fix.value,
+                                                d_mib.value, k_fix.value, k_mib.value,
+                                                single.value, ms.value))
+        for per_mib in (d_mib.value, k_mib.value):          # 10 ... 100 GB/s across PCIe
+            assert 10.0 < per_mib < 105.0, per_mib
+        assert 0.0 <= d_fix.value < 500.0 and 0.0 <= k_fix.value < 500.0
+        assert single.value >= 64 << 10                      # never worth it for small ranges
+    # a second call measures nothing again; thresholds set by the caller win and can be undone
+    assert lib.kvt_initialize_copy_method_profile(0) == 0
+    assert lib.kvt_set_copy_memcpy_thresholds(3 << 20, 5) == 0
+    assert lib.kvt_get_copy_method_profile(1, None, None, None, None, C.byref(single), None, None) == 0
+    assert single.value == 3 << 20
+    assert lib.kvt_reset_copy_memcpy_thresholds() == 0
+    # the measured rule in charge: mixed lengths, bytes exact whichever way each range went
+    _few_very_large_ranges(lib, expect_dma=False)
+
+
 def test_copy_handle_data_hands_a_few_very_large_ranges_to_the_dma_engines():
     lib = kvt_amd.lib()
-    assert lib.kvt_initialize_copy_method_profile(0) == 0
-    assert lib.kvt_initialize_copy_method_profile(99) != 0
+    assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+    try:
+        _few_very_large_ranges(lib)
+    finally:
+        assert lib.kvt_reset_copy_memcpy_thresholds() == 0
+
+
+def _few_very_large_ranges(lib, expect_dma=True):
     cap = 64 << 20
     lens = [(9 << 20) + 48, 8 << 20, (12 << 20) + 7]             # all >= 8 MiB, any remainder
     offs = [1 << 20, (12 << 20) + 16, (30 << 20) + 3]
@@ -472,7 +512,8 @@ def test_copy_handle_data_hands_a_few_very_large_ranges_to_the_dma_engines():
     exp = np.full(cap, 0x3C, dtype=np.uint8)
     checkers.oracle_unpack(exp, gather, blob)
     assert np.array_equal(_host(dst), exp)
-    assert (host_meta == 0).all()           # the kernel's metadata buffers were not needed
+    if expect_dma:
+        assert (host_meta == 0).all()       # the kernel's metadata buffers were not needed
 
 
 @pytest.mark.parametrize("n", [1, 2, 3, 511, 8192 * 3, 100001])
@@ -529,6 +570,7 @@ def test_memcpy_route_thresholds_decide_between_dma_and_kernel():
         return bool((host_meta != 0).any())      # True: the kernel's metadata buffers were used
 
     try:
+        assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0   # the defaults, spelled out
         assert gather_once() is True
         assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 3) == 0
         assert gather_once() is False
@@ -541,7 +583,7 @@ def test_memcpy_route_thresholds_decide_between_dma_and_kernel():
         assert lib.kvt_set_copy_memcpy_thresholds(1, 0) == 0          # switched off
         assert gather_once() is True
     finally:
-        assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+        assert lib.kvt_reset_copy_memcpy_thresholds() == 0
 
 
 @pytest.mark.parametrize("max_block_num", [0, 2])
@@ -593,7 +635,7 @@ def test_mixed_lists_send_their_long_ranges_to_the_dma_engines(max_block_num):
         checkers.oracle_unpack(exp, gather, blob)
         assert np.array_equal(_host(dst), exp)
     finally:
-        assert lib.kvt_set_copy_memcpy_thresholds(8 << 20, 16) == 0
+        assert lib.kvt_reset_copy_memcpy_thresholds() == 0
 
 
 def test_copy_threads_get_their_own_metadata_buffers_and_streams():
@@ -640,6 +682,52 @@ def test_copy_threads_get_their_own_metadata_buffers_and_streams():
     assert len(seen) == 3
     bad = C.c_void_p()
     assert lib.kvt_get_thread_local_stream(0, 7, C.byref(bad)) != 0
+
+
+def test_thread_stream_survives_a_larger_buffer_request():
+    """A stream handed out stays valid when the same thread then asks for larger metadata
+    buffers (only the buffers are replaced), and the copy through the new buffers on the old
+    stream is exact."""
+    lib = kvt_amd.lib()
+    w = workloads.llama8b_single(n_layers=1, pool=64, tokens=300)
+    runs = _oracle_lists(w)[0]
+    cap = w.capacities("src")[0]
+    layer = _dev_bytes(cap, 21)
+    total = int(runs[:, 2].sum())
+    kb = np.stack([np.zeros(len(runs), dtype=np.uint64), runs[:, 0], runs[:, 2]], axis=1).copy()
+    st, st_after = C.c_void_p(), C.c_void_p()
+    dev, host, dev2, host2 = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert lib.kvt_get_thread_local_stream(0, 1, C.byref(st)) == 0
+    assert lib.kvt_get_kernel_copy_buffer(0, 0, C.byref(dev), C.byref(host)) == 0
+    assert lib.kvt_get_kernel_copy_buffer(0, 20000, C.byref(dev2), C.byref(host2)) == 0
+    assert lib.kvt_get_thread_local_stream(0, 1, C.byref(st_after)) == 0
+    assert st_after.value == st.value
+    pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
+    rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(), kb.ctypes.data,
+                                              len(kb), total, 1, 0, st, dev2, host2, 20000)
+    assert rc == 0, lib.kvt_last_error()
+    assert lib.kvt_stream_synchronize(st) == 0
+    assert np.array_equal(pinned.numpy(), checkers.oracle_pack(_host(layer), runs))
+
+
+def test_copy_handle_data_refuses_offsets_that_wrap():
+    """offset + length beyond 64 bits is an error, not a small extent that passes the checks."""
+    lib = kvt_amd.lib()
+    layer = _dev_bytes(1 << 20, 3)
+    pinned = torch.zeros(8192, dtype=torch.uint8).pin_memory()
+    meta_d = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
+    meta_h = torch.zeros(3 * 8192, dtype=torch.int64).pin_memory()
+    kb = np.array([[0, 0, 4096], [0, 2**64 - 2048, 4096]], dtype=np.uint64)
+    rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(), kb.ctypes.data,
+                                              2, 8192, 1, 0, None, meta_d.data_ptr(),
+                                              meta_h.data_ptr(), 0)
+    assert rc == 1, lib.kvt_last_error()
+    rc = lib.kvt_copy_handle_data_kernel_direct(pinned.data_ptr(), layer.data_ptr(), kb.ctypes.data,
+                                                2, 8192, 1, 0, None, meta_d.data_ptr(),
+                                                meta_d[8192:].data_ptr(), meta_d[16384:].data_ptr(),
+                                                meta_h.data_ptr(), 0)
+    assert rc == 1, lib.kvt_last_error()
+    torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("max_block_num", [0, 7])
