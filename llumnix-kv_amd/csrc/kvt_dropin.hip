@@ -576,17 +576,22 @@ int time_copy_route(ProfileBuffers& pb, Route route, uint64_t count, uint64_t si
     return handle_data(pb.host, pb.dev, blocks.data(), count, count * size, direction, false, device,
                        pb.stream, pb.meta_dev, pb.meta_host, kProfileMaxRanges, route);
   };
-  constexpr int kIters = 3;
+  // the fastest of a few separately timed runs: a run that shares the bus with somebody
+  // else's traffic reads long, never short
+  constexpr int kIters = 4;
   if (int rc = enqueue()) return rc;  // warm-up
   KVT_HIP(hipStreamSynchronize(pb.stream));
-  KVT_HIP(hipEventRecord(pb.a, pb.stream));
-  for (int i = 0; i < kIters; ++i)
+  double best = 0;
+  for (int i = 0; i < kIters; ++i) {
+    KVT_HIP(hipEventRecord(pb.a, pb.stream));
     if (int rc = enqueue()) return rc;
-  KVT_HIP(hipEventRecord(pb.b, pb.stream));
-  KVT_HIP(hipEventSynchronize(pb.b));
-  float ms = 0;
-  KVT_HIP(hipEventElapsedTime(&ms, pb.a, pb.b));
-  *us = static_cast<double>(ms) * 1000.0 / kIters;
+    KVT_HIP(hipEventRecord(pb.b, pb.stream));
+    KVT_HIP(hipEventSynchronize(pb.b));
+    float ms = 0;
+    KVT_HIP(hipEventElapsedTime(&ms, pb.a, pb.b));
+    if (i == 0 || ms < best) best = ms;
+  }
+  *us = best * 1000.0;
   return KVT_OK;
 }
 
@@ -621,6 +626,13 @@ int measure_copy_routes(int device, CopyProfile* out) {
     // kernel: k = fixed + total * per_byte
     c.kernel_us_per_byte = std::max(0.0, (k2 - k1) / (t2 - t1));
     c.kernel_fixed_us = std::max(0.0, k1 - t1 * c.kernel_us_per_byte);
+    // A bus between 5 and 87 GB/s (12 ... 200 us per MiB) and fixed costs below a millisecond,
+    // or the measurement was disturbed: then the thresholds stay in charge and a later call
+    // measures again.
+    constexpr double kMiB = 1048576.0;
+    for (double per_byte : {c.dma_us_per_byte, c.kernel_us_per_byte})
+      if (!(per_byte * kMiB > 12.0 && per_byte * kMiB < 200.0)) return KVT_OK;
+    if (c.dma_fixed_us > 1000.0 || c.kernel_fixed_us > 1000.0) return KVT_OK;
   }
   out->measured = true;
   out->elapsed_ms =
@@ -640,6 +652,7 @@ int kvt_initialize_copy_method_profile(int device) {
     if (g_profile.measured) return KVT_OK;  // once per process, like the reference's call_once
     CopyProfile p;
     if (int rc = measure_copy_routes(device, &p)) return rc;
+    if (!p.measured) return KVT_OK;
     g_profile = p;
     g_profile_live.store(&g_profile, std::memory_order_release);
     return KVT_OK;

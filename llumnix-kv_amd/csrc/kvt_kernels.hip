@@ -118,6 +118,22 @@ struct __attribute__((may_alias, aligned(16))) Entry {
   __device__ __forceinline__ uint32_t tensor() const { return tensor_t0 & 0xFFFFu; }
   __device__ __forceinline__ uint32_t t0() const { return tensor_t0 >> 16; }
 };
+// Read as one 32-byte scalar load (field by field the compiler fetches the half it needs
+// first and the rest a round trip later).
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ u32x8 fetch_entry(const void* table, uint32_t e) {
+  return static_cast<const u32x8*>(table)[e];
+}
+__device__ __forceinline__ Entry entry_of(u32x8 r) {
+  Entry c;
+  c.cache = r[0] | (static_cast<uint64_t>(r[1]) << 32);
+  c.packed = r[2] | (static_cast<uint64_t>(r[3]) << 32);
+  c.len = r[4];
+  c.tensor_t0 = r[5];
+  c.shape = r[6];
+  c.reserved = r[7];
+  return c;
+}
 static_assert(sizeof(Entry) == sizeof(Chunk) && offsetof(Chunk, tensor) == offsetof(Entry, tensor_t0) &&
                   offsetof(Chunk, t0) == offsetof(Entry, tensor_t0) + 2 &&
                   offsetof(Chunk, shape) == offsetof(Entry, shape),
@@ -146,17 +162,35 @@ struct Move {
 template <bool CAPPED, class Fetch, class Place>
 __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place place) {
   if (!CAPPED) {
-    // no branch before the last scalar load has been issued: a workgroup's life is three
-    // dependent round trips (arguments, table entry, layer pointer) and then its vector
+    // A workgroup's life is a chain of dependent round trips and then its one vector, and
+    // 2 048 resident workgroups have to hide all of it: the chain is kept to three links.
+    // (1) every argument; (2) the table entry as ONE 32-byte scalar load and, beside it, the
+    // layer pointer and blob position of tensor 0 (the only tensor of most plans: an entry of
+    // another tensor pays one more link); (3) the data. There is no branch before the last
+    // of these loads has been issued: a workgroup beyond the last slice (the grid is rounded
+    // up to a multiple of 8) runs the same code on the last entry with a length of zero.
+    // The empty asm statements pin where the loads complete: without them the compiler moves
+    // a load next to its first use, behind the branch on the tensor index, and the chain grows
+    // by a link.
     const uint32_t b = xcd_remap(blockIdx.x, L.n_slices), layer = blockIdx.y;
     const uint32_t bc = min(b, L.n_slices - 1u);
+    uint64_t stride = L.layer_stride, blob = L.blobs->off[0];
+    asm volatile("" : "+s"(stride), "+s"(blob));
+    uint8_t* const* row = L.layer_ptrs + static_cast<uint64_t>(L.first_layer + layer) * L.n_tensors;
+    u32x8 raw = fetch(bc >> L.sub_shift);
+    uint8_t* base = row[0];
+    asm volatile("" : "+s"(raw), "+s"(base));
     Item it;
-    it.c = fetch(bc >> L.sub_shift);
+    it.c = entry_of(raw);
     it.sub = bc & ((1u << L.sub_shift) - 1u);
-    it.cache = L.layer_ptrs[static_cast<uint64_t>(L.first_layer + layer) * L.n_tensors + it.c.tensor()] +
-               it.c.cache;
-    it.pk = L.packed + layer * L.layer_stride + L.blobs->off[it.c.tensor()] + it.c.packed;
-    if (b >= L.n_slices) return;
+    const uint32_t t = it.c.tensor();
+    if (__builtin_expect(t != 0u, 0)) {
+      base = row[t];
+      blob = L.blobs->off[t];
+    }
+    it.cache = base + it.c.cache;
+    it.pk = L.packed + layer * stride + blob + it.c.packed;
+    if (b >= L.n_slices) it.c.len = 0;
     const Move m = place(it);
     if (m.on) store_vec(m.dst + m.dst_off, load_vec(m.src + m.src_off));
     return;
@@ -176,7 +210,7 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place pl
       valid[j] = layer < L.n_layers && b < L.n_slices;
       lay[j] = min(layer, L.n_layers - 1u);
       const uint32_t bc = min(b, L.n_slices - 1u);
-      it[j].c = fetch(bc >> L.sub_shift);
+      it[j].c = entry_of(fetch(bc >> L.sub_shift));
       it[j].sub = bc & ((1u << L.sub_shift) - 1u);
       s += d_slice;
       layer += d_layer;
@@ -241,7 +275,7 @@ __global__ __launch_bounds__(kThreads, 8) void copy_chunks_kernel(
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; },
+  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); },
                     [&](const Item& it) { return plain_move<PACK>(it); });
 }
 
@@ -253,7 +287,7 @@ __global__ __launch_bounds__(kThreads, 8) void copy_chunks_small_kernel(
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(table.c)[e]; },
+  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(table.c, e); },
                     [&](const Item& it) { return plain_move<PACK>(it); });
 }
 
@@ -353,7 +387,7 @@ __global__ __launch_bounds__(kThreads, 8) void strided_chunks_kernel(
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     StrideTable shapes) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; }, [&](const Item& it) -> Move {
+  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     if (it.c.shape == 0) return plain_move<PACK>(it);
     const uint32_t off = it.sub << kSliceShift;
     if (off >= it.c.len) return KVT_NO_MOVE;
@@ -402,7 +436,7 @@ __global__ __launch_bounds__(kThreads, 8) void xform_chunks_kernel(
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     XformDev x) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; }, [&](const Item& it) -> Move {
+  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     const uint32_t v = (it.sub << 8) + threadIdx.x;  // 256 vectors per slice
     // exact quotients by multiply-high (operands < 2^16); a divisor of 1 has no such constant
     const uint32_t r = x.vrow == 1 ? v : __umulhi(v, x.inv_vrow);  // packed-side row: t_local*heads + h
@@ -521,7 +555,7 @@ __global__ __launch_bounds__(kThreads, 8) void convert_chunks_kernel(
     StrideTable shapes) {
   KVT_LAUNCH_STRUCT;
   // two loads and a conversion per store: `place` moves everything itself
-  for_items<CAPPED>(L, [&](uint32_t e) { return reinterpret_cast<const Entry*>(chunks)[e]; }, [&](const Item& it) -> Move {
+  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     const uint32_t off = it.sub << kSliceShift;
     if (off >= it.c.len) return KVT_NO_MOVE;
     const uint32_t len = min(kSlice, it.c.len - off);

@@ -449,20 +449,25 @@ def test_start_up_profile_measures_both_copy_routes():
     lib = kvt_amd.lib()
     assert lib.kvt_initialize_copy_method_profile(99) != 0
     assert lib.kvt_reset_copy_memcpy_thresholds() == 0
-    assert lib.kvt_initialize_copy_method_profile(0) == 0, lib.kvt_last_error()
     d_fix, d_mib, k_fix, k_mib, ms = (C.c_double() for _ in range(5))
     single, measured = C.c_uint64(), C.c_int()
+    for attempt in range(3):        # a disturbed measurement is discarded and may be repeated
+        assert lib.kvt_initialize_copy_method_profile(0) == 0, lib.kvt_last_error()
+        assert lib.kvt_get_copy_method_profile(0, None, None, None, None, None,
+                                               C.byref(measured), None) == 0
+        if measured.value:
+            break
     for direction in (0, 1):
         assert lib.kvt_get_copy_method_profile(direction, C.byref(d_fix), C.byref(d_mib),
                                                C.byref(k_fix), C.byref(k_mib), C.byref(single),
                                                C.byref(measured), C.byref(ms)) == 0
-        assert measured.value == 1 and 0 < ms.value < 2000.0
         print("copy routes %s: DMA %.1f us + %.2f us/MiB, kernel %.1f us + %.2f us/MiB, own DMA "
               "copy from %d bytes (%.1f ms)" % ("H2D D2H".split()[direction], d_fix.value,
                                                 d_mib.value, k_fix.value, k_mib.value,
                                                 single.value, ms.value))
-        for per_mib in (d_mib.value, k_mib.value):          # 10 ... 100 GB/s across PCIe
-            assert 10.0 < per_mib < 105.0, per_mib
+        assert measured.value == 1 and 0 < ms.value < 2000.0
+        for per_mib in (d_mib.value, k_mib.value):          # 5 ... 87 GB/s across PCIe
+            assert 12.0 < per_mib < 200.0, per_mib
         assert 0.0 <= d_fix.value < 500.0 and 0.0 <= k_fix.value < 500.0
         assert single.value >= 64 << 10                      # never worth it for small ranges
     # a second call measures nothing again; thresholds set by the caller win and can be undone
