@@ -275,18 +275,28 @@ def leg_latency(c, out):
     sender = c.senders[0]
     single, gated, wall = [], [], []
     reqs = list(range(len(w.tasks)))
-    sess = None
+    if len(reqs) < 5:                  # a single-request configuration: the same request again
+        reqs = reqs * 5
     a, b = new_event(), new_event()
+    # A sender keeps one session per destination (stream, events, counters): it exists before
+    # the first timed request, made with an untimed run of request 0.
+    lists = sender.parse([tasks[0][reqs[0]]])
+    plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
+                    chunk_bytes=args.chunk_bytes)
+    sess = kvt.Session(plan, side.src_cache, packed[0], plan.layer_bytes)
+    step = sess.begin_step()
+    for l in range(w.n_layers):
+        sess.save_layer(l, sh)
+    sess.wait_layer(w.n_layers - 1, step)
+    torch.cuda.synchronize()
+    held = (plan, lists)               # the session names this plan until the next set_plan
     for r in reqs:
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         lists = sender.parse([tasks[0][r]])
         plan = kvt.Plan(0, lists, w.capacities("src"), w.capacities("dst"), xform=w.xform,
                         chunk_bytes=args.chunk_bytes)
-        if sess is None:
-            sess = kvt.Session(plan, side.src_cache, packed[0], plan.layer_bytes)
-        else:
-            sess.set_plan(plan, packed[0], plan.layer_bytes)
+        sess.set_plan(plan, packed[0], plan.layer_bytes)
         step = sess.begin_step()
         lib.kvt_event_record(a, sh)
         for l in range(w.n_layers):
@@ -296,24 +306,22 @@ def leg_latency(c, out):
         wall.append((time.perf_counter() - t0) * 1e6)
         lib.kvt_event_synchronize(b)
         gated.append(ev_ms(lib, a, b) * 1e3)
+        held[0].close()                # everything of the previous request has run
+        held[1].close()
+        held = (plan, lists)
         for rep in range(2):   # second run is the measurement
             lib.kvt_event_record(a, sh)
             plan.pack(side.src_cache, 0, w.n_layers, packed[0], plan.layer_bytes, sh)
             lib.kvt_event_record(b, sh)
         lib.kvt_event_synchronize(b)
         single.append(ev_ms(lib, a, b) * 1e3)
-        if r + 1 < len(reqs):      # everything of this request has run: its table may be reused
-            plan.close()
-            lists.close()
-        else:
-            c.keep_objs.append((plan, lists))   # the session still names the last plan
     torch.cuda.synchronize()
-    if sess is not None:
-        sess.close()
+    sess.close()
+    c.keep_objs.append(held)
     out["latency_p50_us"] = round(statistics.median(gated), 2)
     out["latency_wall_p50_us"] = round(statistics.median(wall), 2)
     out["latency_single_launch_p50_us"] = round(statistics.median(single), 2)
-    out["latency_note"] = ("per request (%d requests): latency_p50_us = GPU time from the first "
+    out["latency_note"] = ("per request (%d timed): latency_p50_us = GPU time from the first "
                            "pack launch of layer 0 to the completion of layer %d on the side "
                            "stream, one event-gated launch per layer; latency_wall_p50_us = host "
                            "clock from before ParseBlock (plan built cold) until the wait for the "
@@ -805,13 +813,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "47d5474535edb955982c5d73535a9346f679295647efbce27b930d4861680ea5"
+KERNELS_SHA256 = "4110f1635d6b497895b2d2def98f1a60d22792cc55ee609f60666a54b3dbb780"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134276965, "unpack": 134276496},
-    (2, "ranges"): {"pack": 71013090059, "unpack": 73358409599},
-    (3, "ranges"): {"pack": 85983221225, "unpack": 85983589735},
-    (4, "ranges"): {"pack": 22690378135, "unpack": 22690435564},
-    (5, "ranges"): {"pack": 45141182693, "unpack": 45141395897},
+    (1, "ranges"): {"pack": 134274952, "unpack": 134275166},
+    (2, "ranges"): {"pack": 71013107935, "unpack": 73358400937},
+    (3, "ranges"): {"pack": 85983096503, "unpack": 85983587166},
+    (4, "ranges"): {"pack": 22690362891, "unpack": 22690436533},
+    (5, "ranges"): {"pack": 45141178816, "unpack": 45141392959},
 }
 
 
@@ -1112,18 +1120,25 @@ def main():
         raise SystemExit("bench.py: no usable MI355X (gfx950) device; there is no CPU fallback")
 
     if args.calibrate_copy_gib > 0:
+        # plain copies of one size, `steps` launches each of this library's linear copy kernel
+        # and of the runtime's own device-to-device copy: counter calibration (known traffic)
+        # and, under a kernel trace, the two copy ceilings for a launch of that size
         n = int(args.calibrate_copy_gib * 2**30)
         a = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
         b = torch.empty(n, dtype=torch.uint8, device="cuda")
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            assert lib.kvt_copy_linear(b.data_ptr(), a.data_ptr(), n, None) == 0
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / args.steps
-        assert torch.equal(a, b)
-        print(json.dumps({"calibration": "kvt_copy_linear", "bytes": n, "launches": args.steps,
-                          "gbps_read_plus_write": round(2 * n / dt / 1e9, 1)}))
+        res = {"calibration": "plain copies", "bytes": n, "launches": args.steps}
+        for fn_name in ("kvt_copy_linear", "kvt_copy_runtime_d2d"):
+            fn = getattr(lib, fn_name)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                assert fn(b.data_ptr(), a.data_ptr(), n, None) == 0
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / args.steps
+            assert torch.equal(a, b)
+            res[fn_name + "_gbps_read_plus_write"] = round(2 * n / dt / 1e9, 1)
+            b.zero_()
+        print(json.dumps(res))
         return
 
     all_configs = args.config == 0

@@ -44,6 +44,9 @@ struct StrideShape {
   uint64_t outer[2], inner[2];  // [0] = source side (pack), [1] = destination side (unpack)
 };
 constexpr uint32_t kMaxShapes = 16;
+// Payload (bytes moved one way) up to which a launch reads with plain loads: the size of
+// MI355X's memory-side cache. Above it non-temporal loads are faster again.
+constexpr uint64_t kTemporalMaxBytes = 256ull << 20;
 struct StrideTable {
   StrideShape shape[kMaxShapes];
 };
@@ -51,11 +54,13 @@ struct StrideTable {
 // Chunk launchers. max_wgs = 0: one workgroup per (4 KiB slice, layer), the fastest shape.
 // max_wgs > 0: at most that many workgroups (a multiple of 8), striding over the same items,
 // for a caller that wants the copy to leave part of the device to other kernels.
+// temporal: plain instead of non-temporal loads, for a launch whose data may sit in the
+// memory-side cache (ignored by a capped launch).
 hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, bool words, uint32_t max_wgs,
+                                 const StrideTable& shapes, bool words, uint32_t max_wgs, bool temporal,
                                  hipStream_t stream);
 // Converting gather (bf16 -> fp8 E4M3) of a chunk table, plain and strided chunks alike; lengths
 // and packed positions count fp8 bytes, cache offsets and strides bytes of the bf16 cache.
@@ -75,12 +80,12 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
-                                    const BlobOffsets& blobs, uint32_t max_wgs,
+                                    const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
                                     hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs,
+                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
                               hipStream_t stream);
 // The capped launch of a plain table with 16-byte aligned entries of at most 16 KiB
 // (sub_shift 2) or 32 KiB (sub_shift 3): `wgs` persistent workgroups (a multiple of 8), one
@@ -94,7 +99,7 @@ hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               uint32_t max_wgs, hipStream_t stream);
+                               uint32_t max_wgs, bool temporal, hipStream_t stream);
 // rows = workgroups striding over the 4 KiB slices of each range
 hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                               const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,

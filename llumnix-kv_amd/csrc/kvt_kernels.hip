@@ -40,6 +40,13 @@ typedef __attribute__((address_space(1))) u32x4 g_u32x4;
 __device__ __forceinline__ u32x4 load_vec(const uint8_t* p) {
   return __builtin_nontemporal_load((const g_u32x4*)(p));
 }
+// The load of a launch small enough for its data to sit in the 256 MiB memory-side cache (a
+// single request, one layer of a batch): non-temporal loads of resident lines are slower than
+// plain ones. Measured on MI355X, one request of n tokens packed / unpacked over 32 layers,
+// TB/s with non-temporal against plain loads: 64 MiB 6.27 / 5.90 -> 7.01 / 6.94; 128 MiB 5.91 /
+// 5.30 -> 6.32 / 6.70; 256 MiB 6.39 / 5.80 -> 6.93 / 7.08; 512 MiB 6.57 / 5.98 -> 6.26 / 5.70;
+// 4 GiB 6.67 / 6.18 -> 6.32 / 5.90. The launcher decides by the launch's payload (kTemporalMax).
+__device__ __forceinline__ u32x4 load_vec_temporal(const uint8_t* p) { return *(const g_u32x4*)(p); }
 // Stores are non-temporal and written through at system scope (sc0 sc1 nt): nothing of a
 // streamed copy is worth keeping in a cache. There is no builtin for that combination on a
 // global store. Measured on MI355X against the compiler's non-temporal store (nt alone):
@@ -99,6 +106,7 @@ __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst,
 // loads back to back and only then the stores: a lane has kBatch x 16 bytes in flight.
 
 constexpr int kBatch = 4;
+constexpr uint32_t kTemporalFlag = 0x100u;  // in a kernel's sub_shift argument: Launch::temporal
 
 // The uniform arguments of a chunk launch.
 struct Launch {
@@ -108,6 +116,7 @@ struct Launch {
   uint8_t* packed;
   uint64_t layer_stride;
   const BlobOffsets* blobs;
+  bool temporal;  // plain instead of non-temporal loads (bit 8 of the sub_shift argument)
 };
 
 // A table entry as the kernels read it: the Chunk's two 16-bit fields as one word (a 16-bit
@@ -192,7 +201,21 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place pl
     it.pk = L.packed + layer * stride + blob + it.c.packed;
     if (b >= L.n_slices) it.c.len = 0;
     const Move m = place(it);
-    if (m.on) store_vec(m.dst + m.dst_off, load_vec(m.src + m.src_off));
+    if (m.on) {
+      const uint8_t* src = m.src + m.src_off;
+      u32x4 v;
+      if (L.temporal) {
+        v = load_vec_temporal(src);
+      } else {
+        // Written out: given the builtin, the compiler merges the two arms into ONE load and
+        // drops the non-temporal hint with it.
+        asm volatile("global_load_dwordx4 %0, %1, off nt\n\ts_waitcnt vmcnt(0)"
+                     : "=v"(v)
+                     : "v"(src)
+                     : "memory");
+      }
+      store_vec(m.dst + m.dst_off, v);
+    }
     return;
   }
   // lanes without a vector load from here: the layer pointer table, at least 16 bytes long
@@ -266,7 +289,8 @@ __device__ __forceinline__ Move plain_move(const Item& it) {
 }
 
 #define KVT_LAUNCH_STRUCT \
-  const Launch L{n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, &blobs}
+  const Launch L{n_slices, sub_shift & 0xFFu, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, &blobs, \
+                 (sub_shift & kTemporalFlag) != 0}
 
 // Gather (PACK) / scatter of a resident chunk table.
 template <bool PACK, bool CAPPED>
@@ -634,12 +658,13 @@ static ChunkGrid chunk_grid(uint32_t n_slices, uint32_t n_layers, uint32_t max_w
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs,
+                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
                               hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
-#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
   if (pack && !g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, false>), KVT_ARGS);
   else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, true>), KVT_ARGS);
   else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, false>), KVT_ARGS);
@@ -671,12 +696,13 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
-                                    const BlobOffsets& blobs, uint32_t max_wgs,
+                                    const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
                                     hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
-#define KVT_ARGS table, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+#define KVT_ARGS table, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
   if (pack && !g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, false>), KVT_ARGS);
   else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, true>), KVT_ARGS);
   else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, false>), KVT_ARGS);
@@ -689,12 +715,13 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, bool words, uint32_t max_wgs,
+                                 const StrideTable& shapes, bool words, uint32_t max_wgs, bool temporal,
                                  hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
-#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
 #define KVT_STRIDED(P, W)                                                                       \
   do {                                                                                          \
     if (g.capped) KVT_LAUNCH_CHUNKS((strided_chunks_kernel<P, W, true>), KVT_ARGS);             \
@@ -729,11 +756,12 @@ hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               uint32_t max_wgs, hipStream_t stream) {
+                               uint32_t max_wgs, bool temporal, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
-#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x
+  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x
   if (pack && !g.capped) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, false>), KVT_ARGS);
   else if (pack) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, true>), KVT_ARGS);
   else if (!g.capped) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<false, false>), KVT_ARGS);

@@ -110,6 +110,9 @@ static int finish_plan(kvt_plan* p, const std::vector<Piece>& pieces) {
     hipError_t e = hipEventCreateWithFlags(&p->uploaded, hipEventDisableTiming);
     if (e == hipSuccess) e = hipMemcpyAsync(p->buf->dev, p->buf->host, bytes, hipMemcpyHostToDevice, up);
     if (e == hipSuccess) e = hipEventRecord(p->uploaded, up);
+    // the copy reads the pinned twin and writes the table: the buffer counts as in use by the
+    // upload stream until it has run, so destroying the plan early never has to wait for it
+    if (e == hipSuccess && p->buf->mark_use(up) != KVT_OK) e = hipErrorUnknown;
     if (e != hipSuccess) {
       (void)hipStreamSynchronize(up);
       if (p->uploaded) (void)hipEventDestroy(p->uploaded);
@@ -477,10 +480,10 @@ int kvt_plan_host_tables(const kvt_plan* p, const void** chunks, uint64_t* n_chu
 
 void kvt_plan_destroy(kvt_plan* p) {
   if (!p) return;
-  if (p->uploaded) {
-    (void)hipEventSynchronize(p->uploaded);  // the upload reads the pinned twin
-    (void)hipEventDestroy(p->uploaded);
-  }
+  // No wait for the upload here (on a busy device the copy may sit behind a whole step of
+  // kernels that share its hardware queue): the buffer's own record of the upload keeps it
+  // out of circulation until the copy has run.
+  if (p->uploaded) (void)hipEventDestroy(p->uploaded);
   table_pool().release(p->buf);
   delete p;
 }
@@ -559,11 +562,15 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       return rc;
   }
   const uint32_t max_wgs = copy_wg_cap(cache->device);
+  // A launch whose payload fits the memory-side cache reads with plain loads (kvt_kernels.hip).
+  uint64_t payload = 0;
+  for (uint32_t t = 0; t < p->n_tensors; ++t) payload += p->tensor_bytes[t];
+  const bool temporal = payload * n_layers <= kTemporalMaxBytes;
   if (p->small) {
     const hipError_t e = launch_copy_chunks_small(
         pack, pack ? p->small_pack : p->small_unpack, static_cast<uint32_t>(p->n_chunks),
         p->sub_shift, cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
-        static_cast<uint8_t*>(packed), layer_stride, blobs, max_wgs, s);
+        static_cast<uint8_t*>(packed), layer_stride, blobs, max_wgs, temporal, s);
     if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
     return KVT_OK;
   }
@@ -614,13 +621,13 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       p->strided ? launch_strided_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                          p->n_tensors, first_layer, n_layers,
                                          static_cast<uint8_t*>(packed), layer_stride, blobs,
-                                         p->shapes, words, max_wgs, s) :
+                                         p->shapes, words, max_wgs, temporal, s) :
       p->xform ? launch_xform_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                      first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                     layer_stride, blobs, p->xdev, max_wgs, s)
+                                     layer_stride, blobs, p->xdev, max_wgs, temporal, s)
                : launch_copy_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                     first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                    layer_stride, blobs, max_wgs, s);
+                                    layer_stride, blobs, max_wgs, temporal, s);
   if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
   if (p->buf) {
     // remember when the table is last read, so that its storage is not recycled too early

@@ -139,6 +139,7 @@ class TablePool {
       }
       if (best != idle_.size()) {
         *out = idle_[best];
+        idle_bytes_ -= idle_[best]->cap;
         idle_.erase(idle_.begin() + best);
         (*out)->forget_uses();
         return KVT_OK;
@@ -168,13 +169,22 @@ class TablePool {
     std::vector<TableBuf*> victims;
     {
       std::lock_guard<std::mutex> lock(mu_);
-      // A full pool gives up its older half at once: freeing device memory waits for the whole
-      // device, so it must not happen on every release of a pool that stays full.
-      if (idle_.size() >= kMaxIdle) {
-        victims.assign(idle_.begin(), idle_.begin() + kMaxIdle / 2);
-        idle_.erase(idle_.begin(), idle_.begin() + kMaxIdle / 2);
-      }
       idle_.push_back(b);
+      idle_bytes_ += b->cap;
+      // Freeing device memory waits for the whole device, so a serving loop must not get
+      // here: the pool is bounded by the memory it holds (tables are 64 KiB to a few MiB; the
+      // bound is hundreds of batches), not by a count that a burst of small plans reaches.
+      // Over the bound it shrinks to three quarters at once, oldest first.
+      if (idle_bytes_ > kMaxIdleBytes || idle_.size() > kMaxIdle) {
+        size_t n = 0;
+        while (n + 1 < idle_.size() &&
+               (idle_bytes_ > kMaxIdleBytes / 4 * 3 || idle_.size() - n > kMaxIdle / 4 * 3)) {
+          idle_bytes_ -= idle_[n]->cap;
+          ++n;
+        }
+        victims.assign(idle_.begin(), idle_.begin() + n);
+        idle_.erase(idle_.begin(), idle_.begin() + n);
+      }
     }
     for (TableBuf* victim : victims) {
       victim->wait_idle();
@@ -193,7 +203,8 @@ class TablePool {
   }
 
  private:
-  static constexpr size_t kMaxIdle = 256;
+  static constexpr size_t kMaxIdle = 4096;
+  static constexpr size_t kMaxIdleBytes = size_t(256) << 20;  // device memory, and as much pinned
   static void destroy(TableBuf* b) {
     if (b->dev) (void)hipFree(b->dev);
     if (b->host) (void)hipHostFree(b->host);
@@ -203,6 +214,7 @@ class TablePool {
   }
   std::mutex mu_;
   std::vector<TableBuf*> idle_;
+  size_t idle_bytes_ = 0;
   std::vector<hipStream_t> streams_;
 };
 
