@@ -832,13 +832,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "4110f1635d6b497895b2d2def98f1a60d22792cc55ee609f60666a54b3dbb780"
+KERNELS_SHA256 = "080ddefed4a033ceecc445124b98a0fd1e48134bf5bb88f6fb2125e97a89e479"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134274952, "unpack": 134275166},
-    (2, "ranges"): {"pack": 71013107935, "unpack": 73358400937},
-    (3, "ranges"): {"pack": 85983096503, "unpack": 85983587166},
-    (4, "ranges"): {"pack": 22690362891, "unpack": 22690436533},
-    (5, "ranges"): {"pack": 45141178816, "unpack": 45141392959},
+    (1, "ranges"): {"pack": 134275251, "unpack": 134274995},
+    (2, "ranges"): {"pack": 71013059978, "unpack": 73358401491},
+    (3, "ranges"): {"pack": 85983095265, "unpack": 85983587976},
+    (4, "ranges"): {"pack": 22690363317, "unpack": 22690411274},
+    (5, "ranges"): {"pack": 45141180992, "unpack": 45141391124},
 }
 
 

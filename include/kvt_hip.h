@@ -387,6 +387,20 @@ int kvt_set_copy_cu_usage(int device, double usage);
 /* The current setting and the workgroup limit it stands for (0 = none); either may be NULL. */
 int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
 
+/* No counterpart in the reference (its copy kernel uses one load flavour). A pack / unpack
+ * launch whose payload (bytes moved one way, all layers of the launch) is at most
+ * payload_bytes reads with plain loads, a larger one with non-temporal loads. Plain loads are
+ * faster when the data sits in the 256 MiB memory-side cache -- a layer packed right behind
+ * the kernel that wrote it (sessions, layer-wise saves), a request packed again -- and slower
+ * when it has to come from HBM anyway: measured on MI355X, one request per launch, 64 / 128 /
+ * 256 MiB of payload: +12 / +7 / +8 % (pack) and +18 / +26 / +22 % (unpack) on cached data,
+ * -5 / -7 / -7 % (pack) and +-1 % (unpack) on data cycled through 2-4 GiB. Default: 256 MiB.
+ * 0 = non-temporal loads always. Process-wide; takes effect for launches issued after the
+ * call (a launch captured into a graph keeps what it was captured with). Results are identical
+ * either way. */
+int kvt_set_copy_cached_load_max(uint64_t payload_bytes);
+uint64_t kvt_get_copy_cached_load_max(void);
+
 /* replaces launch_copy_int64_array_h2d_kernel()  kvtransfer/src/copy_kernels.cu:93-103
  * (declared for the channels, kvtransfer/src/copy_kernels.cpp:101-108): a kernel reads
  * num_elements int64 from pinned (device-visible) host memory and writes them to device_dst,

@@ -44,8 +44,9 @@ struct StrideShape {
   uint64_t outer[2], inner[2];  // [0] = source side (pack), [1] = destination side (unpack)
 };
 constexpr uint32_t kMaxShapes = 16;
-// Payload (bytes moved one way) up to which a launch reads with plain loads: the size of
-// MI355X's memory-side cache. Above it non-temporal loads are faster again.
+// Default payload (bytes moved one way) up to which a launch reads with plain loads: the
+// size of MI355X's memory-side cache. Above it non-temporal loads are faster whether or not
+// the data was cached (kvt_set_copy_cached_load_max moves the limit).
 constexpr uint64_t kTemporalMaxBytes = 256ull << 20;
 struct StrideTable {
   StrideShape shape[kMaxShapes];

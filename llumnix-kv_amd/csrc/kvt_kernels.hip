@@ -41,11 +41,16 @@ __device__ __forceinline__ u32x4 load_vec(const uint8_t* p) {
   return __builtin_nontemporal_load((const g_u32x4*)(p));
 }
 // The load of a launch small enough for its data to sit in the 256 MiB memory-side cache (a
-// single request, one layer of a batch): non-temporal loads of resident lines are slower than
-// plain ones. Measured on MI355X, one request of n tokens packed / unpacked over 32 layers,
-// TB/s with non-temporal against plain loads: 64 MiB 6.27 / 5.90 -> 7.01 / 6.94; 128 MiB 5.91 /
-// 5.30 -> 6.32 / 6.70; 256 MiB 6.39 / 5.80 -> 6.93 / 7.08; 512 MiB 6.57 / 5.98 -> 6.26 / 5.70;
-// 4 GiB 6.67 / 6.18 -> 6.32 / 5.90. The launcher decides by the launch's payload (kTemporalMax).
+// layer packed right behind the kernel that wrote it, a request packed again): non-temporal
+// loads of resident lines are slower than plain ones, plain loads of lines that have to come
+// from HBM anyway are slower than non-temporal ones. Measured on MI355X, one request of n
+// tokens packed / unpacked over 32 layers, TB/s with non-temporal against plain loads, the same
+// request again and again (cached): 64 MiB 6.27 / 5.90 -> 7.01 / 6.94; 128 MiB 5.91 / 5.30 ->
+// 6.32 / 6.70; 256 MiB 6.39 / 5.80 -> 6.93 / 7.08; 512 MiB 6.57 / 5.98 -> 6.26 / 5.70; 4 GiB
+// 6.67 / 6.18 -> 6.32 / 5.90. Cycling over requests that hold 2-4 GiB together (not cached):
+// 64 MiB 5.82 / 5.36 -> 5.52 / 5.29; 128 MiB 5.82 / 5.17 -> 5.43 / 5.11; 256 MiB 6.21 / 5.38 ->
+// 5.74 / 5.30. The launcher decides by the launch's payload against a limit the caller can
+// move (kvt_set_copy_cached_load_max).
 __device__ __forceinline__ u32x4 load_vec_temporal(const uint8_t* p) { return *(const g_u32x4*)(p); }
 // Stores are non-temporal and written through at system scope (sc0 sc1 nt): nothing of a
 // streamed copy is worth keeping in a cache. There is no builtin for that combination on a

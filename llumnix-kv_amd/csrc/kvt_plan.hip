@@ -565,7 +565,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   // A launch whose payload fits the memory-side cache reads with plain loads (kvt_kernels.hip).
   uint64_t payload = 0;
   for (uint32_t t = 0; t < p->n_tensors; ++t) payload += p->tensor_bytes[t];
-  const bool temporal = payload * n_layers <= kTemporalMaxBytes;
+  const bool temporal = payload * n_layers <= copy_cached_load_max_bytes();
   if (p->small) {
     const hipError_t e = launch_copy_chunks_small(
         pack, pack ? p->small_pack : p->small_unpack, static_cast<uint32_t>(p->n_chunks),

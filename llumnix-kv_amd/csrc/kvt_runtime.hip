@@ -80,6 +80,9 @@ uint32_t device_cu_count(int device) {
 // tensor. Spans that passed are remembered per thread (a serving loop reuses its buffers),
 // so the steady state costs a few comparisons and no runtime call; an entry is trusted for
 // 256 uses and then asked for again, since the memory behind an address can change hands.
+static std::atomic<uint64_t> g_cached_load_max{kTemporalMaxBytes};
+uint64_t copy_cached_load_max_bytes() { return g_cached_load_max.load(std::memory_order_relaxed); }
+
 static std::atomic<uint64_t> g_span_epoch{1};
 void forget_device_spans() { g_span_epoch.fetch_add(1, std::memory_order_relaxed); }
 
@@ -138,6 +141,12 @@ using namespace kvt;
 extern "C" {
 
 int kvt_device_count(void) { return std::max(0, usable_devices()); }
+
+int kvt_set_copy_cached_load_max(uint64_t payload_bytes) {
+  g_cached_load_max.store(payload_bytes, std::memory_order_relaxed);
+  return KVT_OK;
+}
+uint64_t kvt_get_copy_cached_load_max(void) { return copy_cached_load_max_bytes(); }
 
 int kvt_set_copy_cu_usage(int device, double usage) {
   return guarded([&]() -> int {

@@ -102,3 +102,14 @@ def test_launcher_stand_in_exports_the_reference_names():
     for name in ("launch_copy_int64_array_h2d_kernel", "launch_copy_h2d_direct_kernel",
                  "launch_copy_d2h_direct_kernel", "launch_copy_d2h_bf16_to_fp8_kernel"):
         assert hasattr(shim, name), name
+
+
+def test_cached_load_threshold_is_a_process_wide_setting():
+    lib = kvt_amd.lib()
+    assert lib.kvt_get_copy_cached_load_max() == 256 << 20
+    try:
+        assert lib.kvt_set_copy_cached_load_max(0) == 0 and lib.kvt_get_copy_cached_load_max() == 0
+        assert lib.kvt_set_copy_cached_load_max(1 << 40) == 0
+        assert lib.kvt_get_copy_cached_load_max() == 1 << 40
+    finally:
+        assert lib.kvt_set_copy_cached_load_max(256 << 20) == 0

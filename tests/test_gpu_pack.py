@@ -1199,3 +1199,20 @@ def test_many_threads_build_launch_and_drop_plans_at_once():
         t.join()
     assert not errors, errors
     assert checked == [rounds] * n_threads
+
+
+@pytest.mark.parametrize("limit", [0, 1 << 40])
+def test_either_load_flavour_moves_the_same_bytes(limit):
+    """kvt_set_copy_cached_load_max: non-temporal loads always (0) or plain loads always (a huge
+    limit) -- a plain table from the kernel arguments, a table in device memory, a transposing
+    and a strided plan all give the oracle's bytes either way."""
+    lib = kvt_amd.lib()
+    assert lib.kvt_set_copy_cached_load_max(limit) == 0
+    try:
+        test_short_plans_travel_in_the_kernel_arguments(64)
+        test_config2_shape_reduced_pool(0)
+        test_config3_transposing_pack_hnd_to_nhd()
+        test_config4_mla_and_indexer_two_tensors()
+        test_arbitrary_ranges_including_misaligned()
+    finally:
+        assert lib.kvt_set_copy_cached_load_max(256 << 20) == 0
