@@ -832,13 +832,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "080ddefed4a033ceecc445124b98a0fd1e48134bf5bb88f6fb2125e97a89e479"
+KERNELS_SHA256 = "33947a87031d7205b5b98821106f4621a0eebd23842d40acc8943266b6283121"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134275251, "unpack": 134274995},
-    (2, "ranges"): {"pack": 71013059978, "unpack": 73358401491},
-    (3, "ranges"): {"pack": 85983095265, "unpack": 85983587976},
-    (4, "ranges"): {"pack": 22690363317, "unpack": 22690411274},
-    (5, "ranges"): {"pack": 45141180992, "unpack": 45141391124},
+    (1, "ranges"): {"pack": 134276572, "unpack": 134276572},
+    (2, "ranges"): {"pack": 71013031477, "unpack": 73358401189},
+    (3, "ranges"): {"pack": 85983097824, "unpack": 85983590876},
+    (4, "ranges"): {"pack": 22690378407, "unpack": 22690438908},
+    (5, "ranges"): {"pack": 45141180458, "unpack": 45141389609},
 }
 
 

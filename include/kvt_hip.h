@@ -389,15 +389,17 @@ int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
 
 /* No counterpart in the reference (its copy kernel uses one load flavour). A pack / unpack
  * launch whose payload (bytes moved one way, all layers of the launch) is at most
- * payload_bytes reads with plain loads, a larger one with non-temporal loads. Plain loads are
- * faster when the data sits in the 256 MiB memory-side cache -- a layer packed right behind
- * the kernel that wrote it (sessions, layer-wise saves), a request packed again -- and slower
- * when it has to come from HBM anyway: measured on MI355X, one request per launch, 64 / 128 /
- * 256 MiB of payload: +12 / +7 / +8 % (pack) and +18 / +26 / +22 % (unpack) on cached data,
- * -5 / -7 / -7 % (pack) and +-1 % (unpack) on data cycled through 2-4 GiB. Default: 256 MiB.
- * 0 = non-temporal loads always. Process-wide; takes effect for launches issued after the
- * call (a launch captured into a graph keeps what it was captured with). Results are identical
- * either way. */
+ * payload_bytes reads with plain loads, a larger one with non-temporal loads. Default: 0,
+ * non-temporal loads always -- they are the faster ones whenever a launch's data is read
+ * once, whether it comes from HBM or was left in the 256 MiB memory-side cache by the kernel
+ * that produced it (MI355X, one request per launch, 32 to 256 MiB: 1 to 6 % faster on
+ * uncached data, 2 to 22 % faster right behind a producer). Plain loads pay when the SAME data
+ * is read again while it is still cached (one layer gathered for several destinations, blocks
+ * stored and sent): the second reader then hits, 64 / 128 / 256 MiB of payload back to back:
+ * +12 / +7 / +8 % (pack), +18 / +26 / +22 % (unpack); beyond 256 MiB they lose again. A caller
+ * with such a pattern sets the limit to the largest launch it repeats. Process-wide; takes
+ * effect for launches issued after the call (a launch captured into a graph keeps what it was
+ * captured with). Results are identical either way. */
 int kvt_set_copy_cached_load_max(uint64_t payload_bytes);
 uint64_t kvt_get_copy_cached_load_max(void);
 

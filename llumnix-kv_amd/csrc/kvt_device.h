@@ -44,10 +44,9 @@ struct StrideShape {
   uint64_t outer[2], inner[2];  // [0] = source side (pack), [1] = destination side (unpack)
 };
 constexpr uint32_t kMaxShapes = 16;
-// Default payload (bytes moved one way) up to which a launch reads with plain loads: the
-// size of MI355X's memory-side cache. Above it non-temporal loads are faster whether or not
-// the data was cached (kvt_set_copy_cached_load_max moves the limit).
-constexpr uint64_t kTemporalMaxBytes = 256ull << 20;
+// Default payload (bytes moved one way) up to which a launch reads with plain loads: none.
+// Plain loads pay only when the same data is read again soon (kvt_set_copy_cached_load_max).
+constexpr uint64_t kTemporalMaxBytes = 0;
 struct StrideTable {
   StrideShape shape[kMaxShapes];
 };

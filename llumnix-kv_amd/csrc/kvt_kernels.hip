@@ -40,17 +40,20 @@ typedef __attribute__((address_space(1))) u32x4 g_u32x4;
 __device__ __forceinline__ u32x4 load_vec(const uint8_t* p) {
   return __builtin_nontemporal_load((const g_u32x4*)(p));
 }
-// The load of a launch small enough for its data to sit in the 256 MiB memory-side cache (a
-// layer packed right behind the kernel that wrote it, a request packed again): non-temporal
-// loads of resident lines are slower than plain ones, plain loads of lines that have to come
-// from HBM anyway are slower than non-temporal ones. Measured on MI355X, one request of n
-// tokens packed / unpacked over 32 layers, TB/s with non-temporal against plain loads, the same
-// request again and again (cached): 64 MiB 6.27 / 5.90 -> 7.01 / 6.94; 128 MiB 5.91 / 5.30 ->
-// 6.32 / 6.70; 256 MiB 6.39 / 5.80 -> 6.93 / 7.08; 512 MiB 6.57 / 5.98 -> 6.26 / 5.70; 4 GiB
-// 6.67 / 6.18 -> 6.32 / 5.90. Cycling over requests that hold 2-4 GiB together (not cached):
-// 64 MiB 5.82 / 5.36 -> 5.52 / 5.29; 128 MiB 5.82 / 5.17 -> 5.43 / 5.11; 256 MiB 6.21 / 5.38 ->
-// 5.74 / 5.30. The launcher decides by the launch's payload against a limit the caller can
-// move (kvt_set_copy_cached_load_max).
+// Plain instead of non-temporal loads, for a caller that reads the same data more than once
+// within the reach of the 256 MiB memory-side cache (one layer sent to several destinations,
+// stored and sent): a plain load leaves its line in the cache for the next reader, a
+// non-temporal one does not. Measured on MI355X, one request of n tokens packed over 32
+// layers, non-temporal against plain loads, microseconds per launch:
+//   data not cached (cycling over 1-4 GiB):     32 MiB 16.0 / 16.1, 64 MiB 26.2 / 27.0,
+//                                               128 MiB 50.9 / 53.4, 256 MiB 92.1 / 97.7
+//   right after a kernel wrote the blocks:      32 MiB 12.9 / 13.2, 64 MiB 21.9 / 22.5,
+//                                               128 MiB 44.0 / 46.6, 256 MiB 80.8 / 99.1
+//   the same request again (back to back):      64 MiB 21.4 / 19.1, 128 MiB 45.4 / 42.5,
+//                                               256 MiB 84.0 / 77.5, 512 MiB 163 / 171
+// Non-temporal loads are the default: they win whenever the data is read once, also when a
+// producer's stores have just left it in the cache. The launcher switches by the launch's
+// payload against a limit the caller sets (kvt_set_copy_cached_load_max, 0 by default).
 __device__ __forceinline__ u32x4 load_vec_temporal(const uint8_t* p) { return *(const g_u32x4*)(p); }
 // Stores are non-temporal and written through at system scope (sc0 sc1 nt): nothing of a
 // streamed copy is worth keeping in a cache. There is no builtin for that combination on a

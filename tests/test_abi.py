@@ -106,10 +106,10 @@ def test_launcher_stand_in_exports_the_reference_names():
 
 def test_cached_load_threshold_is_a_process_wide_setting():
     lib = kvt_amd.lib()
-    assert lib.kvt_get_copy_cached_load_max() == 256 << 20
+    assert lib.kvt_get_copy_cached_load_max() == 0
     try:
         assert lib.kvt_set_copy_cached_load_max(0) == 0 and lib.kvt_get_copy_cached_load_max() == 0
         assert lib.kvt_set_copy_cached_load_max(1 << 40) == 0
         assert lib.kvt_get_copy_cached_load_max() == 1 << 40
     finally:
-        assert lib.kvt_set_copy_cached_load_max(256 << 20) == 0
+        assert lib.kvt_set_copy_cached_load_max(0) == 0

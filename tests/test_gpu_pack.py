@@ -1215,4 +1215,4 @@ def test_either_load_flavour_moves_the_same_bytes(limit):
         test_config4_mla_and_indexer_two_tensors()
         test_arbitrary_ranges_including_misaligned()
     finally:
-        assert lib.kvt_set_copy_cached_load_max(256 << 20) == 0
+        assert lib.kvt_set_copy_cached_load_max(0) == 0
