@@ -832,13 +832,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "33947a87031d7205b5b98821106f4621a0eebd23842d40acc8943266b6283121"
+KERNELS_SHA256 = "8abacba752ead0dc5b2f1b0f13713e8636dac148a950658b018e86e6934c4415"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134276572, "unpack": 134276572},
-    (2, "ranges"): {"pack": 71013031477, "unpack": 73358401189},
-    (3, "ranges"): {"pack": 85983097824, "unpack": 85983590876},
-    (4, "ranges"): {"pack": 22690378407, "unpack": 22690438908},
-    (5, "ranges"): {"pack": 45141180458, "unpack": 45141389609},
+    (1, "ranges"): {"pack": 134276273, "unpack": 134276742},
+    (2, "ranges"): {"pack": 71012987616, "unpack": 73358401976},
+    (3, "ranges"): {"pack": 85983095476, "unpack": 85983588827},
+    (4, "ranges"): {"pack": 22690385291, "unpack": 22690437216},
+    (5, "ranges"): {"pack": 45141180660, "unpack": 45141394120},
 }
 
 
