@@ -193,8 +193,9 @@ typedef struct kvt_xform {
  * src_capacity / dst_capacity: per-tensor byte sizes the ranges were validated
  * against; pack refuses a cache smaller than src_capacity, unpack one smaller
  * than dst_capacity. chunk_bytes bounds one table entry: a power of two in
- * [4096, 524288], or 0 to derive it from the median range length (at most
- * 32 KiB). Every entry is moved by ceil(len / 4096) workgroups. The tables of a
+ * [4096, 524288], or 0 for the largest size up to 32 KiB that leaves at most
+ * 2 % of the launched workgroups without bytes to move. Every entry is served
+ * by chunk_bytes / 4096 workgroups. The tables of a
  * plan of at most 64 entries (one short request) are passed to the kernel by
  * value: such a plan needs no upload and can be launched, or captured into a
  * graph, the moment it is created. */
@@ -202,6 +203,10 @@ typedef struct kvt_plan kvt_plan;
 int kvt_plan_create(int device, const kvt_block_lists* lists, const uint64_t* src_capacity,
                     const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
                     kvt_plan** out);
+/* May be called while launches of the plan are still queued: the table's storage
+ * goes back into circulation only after the last of them has run, and the call
+ * waits for nothing. A plan whose launches were recorded into a hipGraph must
+ * outlive the last launch of that graph. */
 void kvt_plan_destroy(kvt_plan* p);
 /* A plan from runs: runs whose ranges are shorter than 4 KiB and 16-byte
  * aligned (offsets, strides, length) stay strided on the device (one table
@@ -480,11 +485,16 @@ int kvt_get_thread_local_stream(int device, int direction, void** stream);
  * pinned); more than max_block_num ranges are processed in batches with a
  * stream synchronisation after each, like the reference. max_block_num <= 0
  * means 8192 (BLLM_KVTRANS_KERNEL_COPY_MAX_BLOCK_NUM's default).
- * Like the reference's, this entry point may decide against its kernel: at most
- * 16 ranges of at least 8 MiB each are handed to the DMA engines, one
- * hipMemcpyAsync per range on `stream` (the reference picks between a memcpy
- * loop and the kernel from a start-up profile, copy_kernels.cpp:495-619; here
- * the rule is fixed from measurements on MI355X). */
+ * A single batch is only enqueued, like the reference's: host_meta (and dev_meta)
+ * must stay untouched until `stream` has run the copy, so a thread that reuses its
+ * buffers for the next call waits for the stream first.
+ * Like the reference's, this entry point may decide against its kernel and hand
+ * the list, or the longest ranges of a mixed list, to the DMA engines, one
+ * hipMemcpyAsync per range on `stream` (select_copy_method / enqueue_hybrid_copy,
+ * copy_kernels.cpp:621-722): by the cost model of kvt_initialize_copy_method_profile
+ * once that has run, before that (or when the caller has set them) by the
+ * thresholds of kvt_set_copy_memcpy_thresholds: at most 16 ranges of at least
+ * 8 MiB each. */
 int kvt_copy_handle_data_with_kernel(void* tensor_buf, void* layer_gpu_ptr,
                                      const kvt_ipc_block* blocks, uint64_t n,
                                      uint64_t tensor_data_size, int direction, int device,
@@ -588,6 +598,12 @@ int kvt_session_save_layer_event(kvt_session* s, uint32_t layer, void* ready_eve
  * or the session is being destroyed. A layer that the step never submits is waited for
  * until the session is destroyed, like the reference's. */
 int kvt_session_wait_layer_step(kvt_session* s, uint64_t step, uint32_t layer);
+/* The same with a limit (no counterpart in the reference, whose wait has none): returns
+ * KVT_ERR_TIMEOUT when the layer is not complete within timeout_us microseconds -- the step
+ * has not begun, the layer has not been submitted, or the GPU has not got to it. Nothing
+ * about the step changes; the wait can simply be repeated. For transport threads that must
+ * notice a shutdown or a stalled device between waits. */
+int kvt_session_wait_layer_for(kvt_session* s, uint64_t step, uint32_t layer, uint64_t timeout_us);
 /* kvt_session_wait_layer_step(s, 0, layer). */
 int kvt_session_wait_layer(kvt_session* s, uint32_t layer);
 /* Makes `stream` wait for every pack issued so far (joins the side stream

@@ -118,7 +118,8 @@ enum {
   KVT_ERR_INVALID = 3,       /* malformed arguments (null pointers, inconsistent metadata)  */
   KVT_ERR_UNSUPPORTED = 4,   /* std::runtime_error("unsupported cache_shape") and the like  */
   KVT_ERR_HIP = 5,           /* a HIP runtime call failed (see kvt_last_error)              */
-  KVT_ERR_NO_DEVICE = 6      /* GPU entry point called without a usable MI355X              */
+  KVT_ERR_NO_DEVICE = 6,     /* GPU entry point called without a usable MI355X              */
+  KVT_ERR_TIMEOUT = 7        /* a bounded wait ran out (kvt_session_wait_layer_for)         */
 };
 
 /* Per-worker cache geometry consumed by ParseBlock. */

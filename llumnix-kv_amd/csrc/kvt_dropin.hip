@@ -499,9 +499,9 @@ int kvt_copy_handle_data_kernel_direct(void* tensor_buf, void* layer_gpu_ptr,
   });
 }
 
-// ------------------------------------------------ the entry point that allocates nothing
-
 }  // extern "C"
+
+// ------------------------------------------------ the entry point that allocates nothing
 
 // Device-side range metadata of kvt_copy_handle_data_kernel_direct_static: three int64 arrays
 // of up to kStaticMaxRanges entries, 192 KiB, held by every GPU the library runs on until the
@@ -532,10 +532,6 @@ int static_scratch(int device, int64_t** out) {
   return KVT_OK;
 }
 }  // namespace
-
-extern "C" {
-
-}  // extern "C"
 
 // The start-up measurement (initialize_copy_method_profile_impl, kvtransfer/src/
 // copy_kernels.cpp:495-591): loops of DMA copies against the copy kernel on pinned host

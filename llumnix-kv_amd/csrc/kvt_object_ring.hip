@@ -315,9 +315,11 @@ static int transfer(kvt_object_ring* r, const uint32_t* entries, uint32_t n, voi
     }
   DeviceGuard g;
   if (int rc = g.enter(r->device)) return rc;
-  if (int rc = check_device_span(dev, static_cast<uint64_t>(n - 1) * dev_stride + r->entry_bytes,
-                                 std::string(who) + ": the device buffer"))
-    return rc;
+  uint64_t extent = 0;
+  if (__builtin_mul_overflow(static_cast<uint64_t>(n - 1), dev_stride, &extent) ||
+      __builtin_add_overflow(extent, r->entry_bytes, &extent))
+    return fail(KVT_ERR_OUT_OF_RANGE, std::string(who) + ": device stride times entries exceeds 64 bits");
+  if (int rc = check_device_span(dev, extent, std::string(who) + ": the device buffer")) return rc;
   const hipStream_t user = static_cast<hipStream_t>(stream);
   // behind whatever the caller's stream has queued (the pack that produces the objects, or the
   // kernels still reading the buffer a load is about to overwrite)

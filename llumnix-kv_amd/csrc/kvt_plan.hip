@@ -553,10 +553,16 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
     }
   }
   if (!capturing && p->n_chunks != 0 && n_layers != 0) {
-    uint64_t extent = 0;
-    for (uint32_t t = 0; t < p->n_tensors; ++t)
-      extent = std::max(extent, blobs.off[t] + p->tensor_bytes[t]);
-    extent += static_cast<uint64_t>(n_layers - 1) * layer_stride;
+    uint64_t extent = 0, layers_span = 0;
+    bool wraps = __builtin_mul_overflow(static_cast<uint64_t>(n_layers - 1), layer_stride, &layers_span);
+    for (uint32_t t = 0; t < p->n_tensors; ++t) {
+      uint64_t end = 0;
+      wraps = wraps || __builtin_add_overflow(blobs.off[t], p->tensor_bytes[t], &end);
+      extent = std::max(extent, end);
+    }
+    // a sum that wraps would pass the span check below with a small extent
+    if (wraps || __builtin_add_overflow(extent, layers_span, &extent))
+      return fail(KVT_ERR_OUT_OF_RANGE, "blob offsets and layer stride exceed 64 bits");
     if (int rc = check_device_span(packed, extent, pack ? "kvt_pack: the packed buffer"
                                                         : "kvt_unpack: the packed buffer"))
       return rc;

@@ -71,6 +71,9 @@ uint32_t device_cu_count(int device) {
   return n;
 }
 
+static std::atomic<uint64_t> g_cached_load_max{kTemporalMaxBytes};
+uint64_t copy_cached_load_max_bytes() { return g_cached_load_max.load(std::memory_order_relaxed); }
+
 // A kernel that runs past a buffer takes a GPU memory fault, which can cost the whole
 // process (and more) instead of an error code. What the runtime knows about a pointer is
 // therefore checked on the host before a launch uses it: it must be memory the device can
@@ -80,9 +83,6 @@ uint32_t device_cu_count(int device) {
 // tensor. Spans that passed are remembered per thread (a serving loop reuses its buffers),
 // so the steady state costs a few comparisons and no runtime call; an entry is trusted for
 // 256 uses and then asked for again, since the memory behind an address can change hands.
-static std::atomic<uint64_t> g_cached_load_max{kTemporalMaxBytes};
-uint64_t copy_cached_load_max_bytes() { return g_cached_load_max.load(std::memory_order_relaxed); }
-
 static std::atomic<uint64_t> g_span_epoch{1};
 void forget_device_spans() { g_span_epoch.fetch_add(1, std::memory_order_relaxed); }
 

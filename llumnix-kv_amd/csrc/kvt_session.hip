@@ -1,5 +1,6 @@
 // Per-layer gating sessions (event -> side stream -> pack -> done event) and
 // pinned-host staging of packed layers.
+#include <algorithm>
 #include <chrono>
 #include <condition_variable>
 #include <cstring>
@@ -61,11 +62,7 @@ struct kvt_stager {
   hipEvent_t fence = nullptr;
 };
 
-extern "C" {
-
 // ----------------------------------------------------------------- session
-
-}  // extern "C"
 
 namespace {
 
@@ -92,9 +89,16 @@ uint64_t begin_step_locked(kvt_session* s) {
   return id;
 }
 
+using Clock = std::chrono::steady_clock;
+
+int timed_out(uint32_t layer) {
+  return fail(KVT_ERR_TIMEOUT, "kvt_session_wait_layer_for: layer " + std::to_string(layer) +
+                                   " was not complete within the time given");
+}
+
 // Blocks until completion `target` of `layer` has been published, the session is being
-// destroyed, or (eager steps) the step fails.
-int poll_layer(kvt_session* s, uint32_t layer, uint32_t target) {
+// destroyed, or `deadline` (if any) has passed.
+int poll_layer(kvt_session* s, uint32_t layer, uint32_t target, const Clock::time_point* deadline) {
   const uint32_t* word = s->count_host + layer;
   for (uint32_t spins = 0;; ++spins) {
     // counts only grow; the comparison survives wrap-around of the 32-bit counter
@@ -109,6 +113,7 @@ int poll_layer(kvt_session* s, uint32_t layer, uint32_t target) {
       std::lock_guard<std::mutex> lock(s->mu);
       if (s->closing) return fail(KVT_ERR_INVALID, "kvt_session_wait_layer: the session is being destroyed");
     }
+    if (deadline && Clock::now() >= *deadline) return timed_out(layer);
     if (spins < 20000)
       std::this_thread::yield();
     else
@@ -265,8 +270,9 @@ int kvt_session_save_layer_event(kvt_session* s, uint32_t layer, void* ready_eve
   });
 }
 
-int kvt_session_wait_layer_step(kvt_session* s, uint64_t step, uint32_t layer) {
-  return guarded([&]() -> int {
+// deadline = nullptr: no limit.
+static int wait_layer(kvt_session* s, uint64_t step, uint32_t layer, const Clock::time_point* deadline) {
+  {
     if (!s) return fail(KVT_ERR_INVALID, "kvt_session_wait_layer: null session");
     if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
     // kvt_session_destroy waits until every thread has left this function
@@ -287,7 +293,7 @@ int kvt_session_wait_layer_step(kvt_session* s, uint64_t step, uint32_t layer) {
       std::unique_lock<std::mutex> lock(s->mu);
       if (step == 0) step = s->cur_step ? s->cur_step : 1;  // "the current step"
       int rc = KVT_OK;
-      s->cv.wait(lock, [&] {
+      auto settled = [&] {
         if (s->closing) {
           rc = fail(KVT_ERR_INVALID, "kvt_session_wait_layer: the session is being destroyed");
           return true;
@@ -306,10 +312,27 @@ int kvt_session_wait_layer_step(kvt_session* s, uint64_t step, uint32_t layer) {
         }
         target = st.target[layer];
         return target != 0;
-      });
+      };
+      if (!deadline)
+        s->cv.wait(lock, settled);
+      else if (!s->cv.wait_until(lock, *deadline, settled))
+        return timed_out(layer);
       if (rc != KVT_OK) return rc;
     }
-    return poll_layer(s, layer, target);
+    return poll_layer(s, layer, target, deadline);
+  }
+}
+
+int kvt_session_wait_layer_step(kvt_session* s, uint64_t step, uint32_t layer) {
+  return guarded([&]() -> int { return wait_layer(s, step, layer, nullptr); });
+}
+
+int kvt_session_wait_layer_for(kvt_session* s, uint64_t step, uint32_t layer, uint64_t timeout_us) {
+  return guarded([&]() -> int {
+    // far enough for any caller, near enough for the clock's range
+    const uint64_t us = std::min<uint64_t>(timeout_us, 1000ull * 1000 * 86400 * 365);
+    const Clock::time_point deadline = Clock::now() + std::chrono::microseconds(us);
+    return wait_layer(s, step, layer, &deadline);
   });
 }
 

@@ -124,6 +124,7 @@ SIGNATURES = {
     "kvt_session_save_layer_event": (_int, [_vp, _u32, _vp]),
     "kvt_session_wait_layer": (_int, [_vp, _u32]),
     "kvt_session_wait_layer_step": (_int, [_vp, _u64, _u32]),
+    "kvt_session_wait_layer_for": (_int, [_vp, _u64, _u32, _u64]),
     "kvt_session_begin_step": (_int, [_vp, _P(_u64)]),
     "kvt_session_set_plan": (_int, [_vp, _vp, _vp, _u64]),
     "kvt_session_join": (_int, [_vp, _vp]),
@@ -575,9 +576,13 @@ class Session:
         check(lib().kvt_session_begin_step(self.h, C.byref(step)))
         return step.value
 
-    def wait_layer(self, layer, step=0):
-        """Blocks until `layer` of `step` (0 = the newest step) is packed."""
-        check(lib().kvt_session_wait_layer_step(self.h, step, layer))
+    def wait_layer(self, layer, step=0, timeout_us=None):
+        """Blocks until `layer` of `step` (0 = the newest step) is packed; with timeout_us,
+        raises KvtError(ERR_TIMEOUT) when that takes longer."""
+        if timeout_us is None:
+            check(lib().kvt_session_wait_layer_step(self.h, step, layer))
+        else:
+            check(lib().kvt_session_wait_layer_for(self.h, step, layer, int(timeout_us)))
 
     def join(self, stream=None):
         check(lib().kvt_session_join(self.h, _ptr(stream)))

@@ -35,7 +35,8 @@ PARSER_NAMES = [
 ]
 PARSER = {name: i for i, name in enumerate(PARSER_NAMES)}
 
-OK, ERR_OUT_OF_RANGE, ERR_OVERFLOW, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE = range(7)
+(OK, ERR_OUT_OF_RANGE, ERR_OVERFLOW, ERR_INVALID, ERR_UNSUPPORTED, ERR_HIP, ERR_NO_DEVICE,
+ ERR_TIMEOUT) = range(8)
 
 
 class IpcBlock(C.Structure):

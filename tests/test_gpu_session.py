@@ -13,7 +13,7 @@ import pytest
 
 import checkers
 import kvt_amd
-from kvt_amd import pipeline, workloads
+from kvt_amd import ctypes_defs, pipeline, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -237,3 +237,38 @@ def test_destroying_a_session_releases_a_parked_waiter():
     t.join(30)
     assert not t.is_alive() and "returned" not in result
     assert "being destroyed" in str(result["error"])
+
+
+def test_a_bounded_wait_runs_out_and_can_be_repeated():
+    """kvt_session_wait_layer_for: a layer that is not there yet -- step not begun, layer not
+    submitted -- gives KVT_ERR_TIMEOUT after the time given instead of parking the thread, and
+    the same wait succeeds once the layer has been packed."""
+    w = workloads.llama8b_single(n_layers=2, pool=64, tokens=100)
+    plan, lists = pipeline.build_plan(w, 0)
+    cap = w.capacities("src")[0]
+    layers = [[_contents(cap, 70 + l)] for l in range(w.n_layers)]
+    cache = kvt_amd.Cache(0, layers, [cap])
+    packed = torch.zeros(w.n_layers * plan.layer_bytes, dtype=torch.uint8, device="cuda")
+    sess = kvt_amd.Session(plan, cache, packed, plan.layer_bytes)
+    compute = torch.cuda.Stream()
+    for step, layer in ((1, 0), (3, 1)):             # step 1 has not begun; step 3 is far off
+        t0 = time.perf_counter()
+        with pytest.raises(kvt_amd.KvtError) as err:
+            sess.wait_layer(layer, step, timeout_us=20_000)
+        waited = time.perf_counter() - t0
+        assert err.value.code == ctypes_defs.ERR_TIMEOUT, str(err.value)
+        assert 0.015 < waited < 5.0, waited
+    assert sess.begin_step() == 1
+    sess.save_layer(0, compute.cuda_stream)
+    with pytest.raises(kvt_amd.KvtError) as err:       # begun, but layer 1 not submitted
+        sess.wait_layer(1, 1, timeout_us=5_000)
+    assert err.value.code == ctypes_defs.ERR_TIMEOUT
+    sess.wait_layer(0, 1, timeout_us=30_000_000)
+    sess.save_layer(1, compute.cuda_stream)
+    sess.wait_layer(1, 1, timeout_us=30_000_000)
+    for l in range(w.n_layers):
+        blob = checkers.oracle_pack(layers[l][0].cpu().numpy(), lists.tensor(0))
+        got = packed[l * plan.layer_bytes:l * plan.layer_bytes + len(blob)].cpu().numpy()
+        assert np.array_equal(got, blob), l
+    compute.synchronize()
+    sess.close()

@@ -135,6 +135,20 @@ def test_pack_at_several_layers_with_a_stride_and_odd_offsets():
             assert np.array_equal(_host(dst_layers[l][t]), e), (l, t)
 
 
+def test_pack_at_refuses_blob_offsets_and_strides_that_wrap():
+    """A blob offset or layer stride near 2^64 must not wrap into an extent that fits the buffer."""
+    w = workloads.deepseek_mla(n_layers=2, pool=64, n_req=1, tokens=300)
+    plan, _ = pipeline.build_plan(w, 0)
+    sc = kvt_amd.Cache(0, _make_caches(w, "src", 43), w.capacities("src"))
+    out = torch.zeros(2 * plan.layer_bytes, dtype=torch.uint8, device="cuda")
+    for offs, stride in (([2**64 - 16, 0] + [0] * 6, plan.layer_bytes),
+                         ([0, plan.tensor_bytes(0)] + [0] * 6, 2**64 - 256)):
+        with pytest.raises(kvt_amd.KvtError) as err:
+            plan.pack_at(sc, 0, 2, out, stride, offs)
+        assert err.value.code == 1, str(err.value)
+    torch.cuda.synchronize()
+
+
 def _info(block_sizes, nblk, n_layers):
     w = kvt_amd.ctypes_defs.WorkerInfo()
     w.engine_tp_size, w.worker_tp_rank = 1, 0
