@@ -584,13 +584,38 @@ def leg_fp8_plan(c, out):
     exp[:] = got
     checkers.oracle_unpack(exp, ranges, blob)      # idempotent on what the GPU already scattered
     parity &= bool(np.array_equal(got, exp))
+    # the same two launches limited to a share of the device (pipelined persistent kernels)
+    shares = []
+    exp0 = np.zeros_like(exp)
+    checkers.oracle_unpack(exp0, ranges, blob)
+    try:
+        for usage in (0.5, 0.25, 0.125):
+            kvt.set_copy_cu_usage(0, usage)
+            packed[:len(blob)].zero_()             # layer 0 of both sides: what the check reads
+            side.dst[0][0][:len(exp)].zero_()
+            torch.cuda.synchronize()
+            for rep in range(2):   # second run is the measurement
+                lib.kvt_event_record(a, c.sh)
+                plan.pack(side.src_cache, 0, w8.n_layers, packed, stride, c.sh)
+                lib.kvt_event_record(b, c.sh)
+                plan.unpack(dst_cache, 0, w8.n_layers, packed, stride, c.sh)
+                lib.kvt_event_record(d, c.sh)
+                lib.kvt_event_synchronize(d)
+            same = bool(np.array_equal(packed[:len(blob)].cpu().numpy(), blob)) and \
+                bool(np.array_equal(side.dst[0][0][:len(exp)].cpu().numpy(), exp0))
+            shares.append({"usage": usage, "workgroups": kvt.get_copy_cu_usage(0)[1],
+                           "pack_gbps": round(3.0 * P8 / (ev_ms(lib, a, b) * 1e-3) / 1e9, 1),
+                           "unpack_gbps": round(2.0 * P8 / (ev_ms(lib, b, d) * 1e-3) / 1e9, 1),
+                           "parity_vs_oracle": same})
+    finally:
+        kvt.set_copy_cu_usage(0, 1.0)
     out["converting_plan"] = {
         "workload": w8.name, "fp8_payload_bytes": P8, "table_entries_per_layer": plan.num_chunks,
         "ranges_per_layer": int(len(ranges)), "host_parse_plan_ms": round(host_ms, 3),
         "pack_ms": round(statistics.mean(pk), 4), "unpack_ms": round(statistics.mean(un), 4),
         "pack_gbps": round(3.0 * P8 / (statistics.mean(pk) * 1e-3) / 1e9, 1),
         "unpack_gbps": round(2.0 * P8 / (statistics.mean(un) * 1e-3) / 1e9, 1),
-        "parity_vs_oracle": parity,
+        "parity_vs_oracle": parity, "cu_usage": shares,
         "note": "pack reads 2 bytes and writes 1 per element (bf16 -> fp8 E4M3), unpack moves "
                 "the fp8 bytes; GB/s = bytes read + bytes written"}
     plan.close()
@@ -832,13 +857,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "8abacba752ead0dc5b2f1b0f13713e8636dac148a950658b018e86e6934c4415"
+KERNELS_SHA256 = "e296c7bff5072869475b8982ee6877249a5849504a82c1ac888db6217ef376a5"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134276273, "unpack": 134276742},
-    (2, "ranges"): {"pack": 71012987616, "unpack": 73358401976},
-    (3, "ranges"): {"pack": 85983095476, "unpack": 85983588827},
-    (4, "ranges"): {"pack": 22690385291, "unpack": 22690437216},
-    (5, "ranges"): {"pack": 45141180660, "unpack": 45141394120},
+    (1, "ranges"): {"pack": 134263594, "unpack": 134277546},
+    (2, "ranges"): {"pack": 71013059763, "unpack": 73358396750},
+    (3, "ranges"): {"pack": 85983093249, "unpack": 85983584168},
+    (4, "ranges"): {"pack": 22690381169, "unpack": 22690437702},
+    (5, "ranges"): {"pack": 45141190235, "unpack": 45141384964},
 }
 
 

@@ -240,8 +240,9 @@ uint64_t kvt_plan_num_strided_chunks(const kvt_plan* p);
  * its two tables on the host and cannot be launched. *chunks = 2 * n_chunks
  * entries of 32 bytes {u64 cache, u64 packed, u32 len, u16 tensor, u16 t0,
  * u32 shape, u32 0}: pack order first, then unpack order; *shapes = 16 record
- * shapes of 48 bytes {u32 vlen16, u32 inv, u32 n_inner, u32 inv_words, u64 outer[2],
- * u64 inner[2]} ([0] source side, [1] destination side). Entry semantics: see
+ * shapes of 64 bytes {u32 vlen16, u32 inv, u32 n_inner, u32 inv_words, u64 outer[2],
+ * u64 inner[2], u32 inv_inner, u32 0 x 3} ([0] source side, [1] destination side).
+ * Entry semantics: see
  * csrc/kvt_device.h. Borrowed pointers, valid until the plan is destroyed. */
 #define KVT_DEVICE_NONE (-1)
 int kvt_plan_host_tables(const kvt_plan* p, const void** chunks, uint64_t* n_chunks,

@@ -37,12 +37,15 @@ struct XformDev {
 // records of vlen 16-byte vectors; record r lives in the cache at
 //   chunk.cache + (r / n_inner) * outer + (r % n_inner) * inner
 // (per token: the outer step; K and V of one token: the inner step).
-struct StrideShape {
+struct __attribute__((aligned(16))) StrideShape {
   uint32_t vlen, inv_vlen;     // inv_vlen = floor(2^32 / vlen) + 1, exact for operands < 2^32 / vlen
   uint32_t n_inner;
   uint32_t inv_wlen;           // the same reciprocal for the record length in 4-byte words (4 * vlen)
   uint64_t outer[2], inner[2];  // [0] = source side (pack), [1] = destination side (unpack)
+  uint32_t inv_inner;          // floor(2^32 / n_inner) + 1 (n_inner > 1: exact for operands < 2^16), else 0
+  uint32_t reserved[3];
 };
+static_assert(sizeof(StrideShape) == 64, "StrideShape is read as one 64-byte scalar load");
 constexpr uint32_t kMaxShapes = 16;
 // Default payload (bytes moved one way) up to which a launch reads with plain loads: none.
 // Plain loads pay only when the same data is read again soon (kvt_set_copy_cached_load_max).
@@ -95,6 +98,26 @@ hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                const BlobOffsets& blobs, uint32_t wgs, hipStream_t stream);
+// The same pipeline for strided and for transposing tables (sub_shift 2 ... 7; larger entries
+// are taken in parts of 16 or 32 KiB). Every entry must be 16-byte aligned on both sides, a multiple
+// of 16 bytes long, and span less than 2 GiB on the cache side.
+hipError_t launch_strided_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                  uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                  uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                  const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
+                                  hipStream_t stream);
+// ... and for the converting gather (entries a multiple of 16 elements long; sub_shift 1 ... 7;
+// strided entries also from sub_shift 1).
+hipError_t launch_convert_entries(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                  uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                  uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                  const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
+                                  hipStream_t stream);
+hipError_t launch_xform_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                const BlobOffsets& blobs, const XformDev& x, uint32_t wgs,
+                                hipStream_t stream);
 hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

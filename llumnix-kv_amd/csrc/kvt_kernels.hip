@@ -403,6 +403,175 @@ __global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
   }
 }
 
+// The same pipeline for tables whose cache side is not contiguous (strided records, the
+// HND <-> NHD transform): one trip moves V slices of one entry (entries of more than V slices
+// are taken in parts), the packed side through a descriptor of exactly the part's bytes, the
+// cache side through a descriptor that starts at the entry's cache position with the lane's own
+// byte offsets, computed when the part is fetched. `cache_offsets(entry, begin, bytes, off)`
+// fills the lane's V offsets for the vectors at packed offsets begin + lane * 16 + v * 4096,
+// kNoVector where that lies beyond `bytes`. Offsets are 32-bit: the launcher's caller checks
+// that no entry spans 2 GiB on the cache side.
+constexpr uint32_t kCacheWindow = 0x80000000u;  // bytes a cache-side descriptor covers
+constexpr uint32_t kNoVector = kCacheWindow;    // first offset outside it: loads give zero, stores are dropped
+
+// This workgroup's way through the (item, layer) pairs of a launch: the items of a layer are
+// dealt to the XCDs in eighths, neighbouring workgroups of an XCD take neighbouring items.
+struct EntryWalk {
+  uint32_t n_items, n_layers, per8, xcd, step_layer, step_within, layer, within;
+  __device__ __forceinline__ EntryWalk(uint32_t items, uint32_t layers) : n_items(items), n_layers(layers) {
+    per8 = (n_items + 7u) >> 3;
+    xcd = blockIdx.x & 7u;
+    const uint32_t nloc = gridDim.x >> 3;  // workgroups per XCD
+    step_layer = nloc / per8;
+    step_within = nloc - step_layer * per8;
+    layer = (blockIdx.x >> 3) / per8;
+    within = (blockIdx.x >> 3) - layer * per8;
+  }
+  // The next pair, clamped to the last one past the end (`valid` false: nothing to move there);
+  // returns false once the workgroup is past the last layer.
+  __device__ __forceinline__ bool next(uint32_t& item, uint32_t& lay, bool& valid) {
+    const bool live = layer < n_layers;
+    const uint32_t b = xcd * per8 + within;
+    valid = live && b < n_items;
+    lay = min(layer, n_layers - 1u);
+    item = min(b, n_items - 1u);
+    within += step_within;
+    layer += step_layer;
+    const bool wrap = within >= per8;
+    within -= wrap ? per8 : 0u;
+    layer += wrap ? 1u : 0u;
+    return live;
+  }
+};
+
+// Three register sets in rotation: the loads of item k+1 are issued before the stores of item k,
+// and a set is loaded again only two trips after its stores were issued.
+#define KVT_ROTATE3(NEXT, LOAD, STORE) \
+  if (!NEXT(0)) return;                \
+  LOAD(0);                             \
+  for (;;) {                           \
+    const bool l1 = NEXT(1);           \
+    LOAD(1);                           \
+    STORE(0);                          \
+    if (!l1) break;                    \
+    const bool l2 = NEXT(2);           \
+    LOAD(2);                           \
+    STORE(1);                          \
+    if (!l2) break;                    \
+    const bool l0 = NEXT(0);           \
+    LOAD(0);                           \
+    STORE(2);                          \
+    if (!l0) break;                    \
+  }
+
+template <bool PACK, int V, class CacheOffsets>
+__device__ __forceinline__ void entries_pipeline(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride,
+    const BlobOffsets& blobs, CacheOffsets cache_offsets) {
+  EntryWalk walk(n_chunks << part_shift, n_layers);
+  const uint32_t lane = threadIdx.x << 4;
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  rsrc_t cdesc[3], pdesc[3];
+  uint32_t coff[3][V];
+  u32x4 r[3][V];
+  auto next = [&](int k) -> bool {
+    uint32_t item, lay;
+    bool valid;
+    const bool live = walk.next(item, lay, valid);
+    const Entry c = table[item >> part_shift];
+    const uint32_t begin = (item & ((1u << part_shift) - 1u)) * (static_cast<uint32_t>(V) << kSliceShift);
+    uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
+    uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed + begin;
+    const uint32_t bytes =
+        valid && c.len > begin ? min(c.len - begin, static_cast<uint32_t>(V) << kSliceShift) : 0u;
+    pdesc[k] = make_rsrc(pk, bytes);
+    cdesc[k] = make_rsrc(cache, bytes ? kCacheWindow : 0u);
+    cache_offsets(c, begin, bytes, coff[k]);
+    return live;
+  };
+  auto load = [&](int k) {
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      r[k][v] = PACK ? __builtin_amdgcn_raw_buffer_load_b128(cdesc[k], coff[k][v], 0, kLoadPolicy)
+                     : __builtin_amdgcn_raw_buffer_load_b128(pdesc[k], lane + (v << kSliceShift), 0, kLoadPolicy);
+  };
+  auto store = [&](int k) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      if (PACK)
+        __builtin_amdgcn_raw_buffer_store_b128(r[k][v], pdesc[k], lane + (v << kSliceShift), 0, kStorePolicy);
+      else
+        __builtin_amdgcn_raw_buffer_store_b128(r[k][v], cdesc[k], coff[k][v], 0, kStorePolicy);
+    }
+  };
+  KVT_ROTATE3(next, load, store)
+}
+
+// Strided tables (16-byte vectors only; every entry 16-byte aligned on both sides). The
+// entry's record shape arrives as one 64-byte scalar load and the offsets are computed without
+// a branch: a contiguous entry (shape 0) is the degenerate record whose quotient is always
+// zero, so that its vectors are all "column" (both multipliers zero), and a divisor of 1,
+// which has no 32-bit reciprocal, adds the dividend itself instead.
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void strided_entries_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes) {
+  const uint32_t lane = threadIdx.x << 4;
+  entries_pipeline<PACK, V>(
+      chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride,
+      blobs, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
+        const bool plain = c.shape == 0;
+        const u32x16 raw = *reinterpret_cast<const u32x16*>(&shapes.shape[plain ? 0u : c.shape - 1u]);
+        // words of a StrideShape: 0 vlen, 1 inv_vlen, 2 n_inner, 4 + 2 side: outer, 8 + 2 side: inner,
+        // 12 inv_inner (low halves of the strides: the entry spans less than 2 GiB)
+        const uint32_t vlen = plain ? 0u : raw[0];
+        const uint32_t rec_mul = plain || raw[0] == 1u ? 0u : raw[1], rec_add = !plain && raw[0] == 1u ? 1u : 0u;
+        const uint32_t n_inner = plain ? 1u : raw[2];
+        const uint32_t o_mul = raw[12], o_add = n_inner == 1u ? 1u : 0u;
+        const uint32_t outer = raw[PACK ? 4 : 6], inner = raw[PACK ? 8 : 10];
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+          const uint32_t at = lane + (v << kSliceShift);
+          const uint32_t vi = (begin + at) >> 4;  // vector index inside the entry, < 2^15
+          const uint32_t rec = __umulhi(vi, rec_mul) + vi * rec_add;
+          const uint32_t col = vi - rec * vlen;
+          const uint32_t o = __umulhi(rec, o_mul) + rec * o_add;
+          const uint32_t i = rec - o * n_inner;
+          coff[v] = at < bytes ? o * outer + i * inner + (col << 4) : kNoVector;
+        }
+      });
+}
+
+// The HND <-> NHD transform (index arithmetic of xform_chunks_kernel).
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void xform_entries_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    XformDev x) {
+  const uint32_t lane = threadIdx.x << 4;
+  entries_pipeline<PACK, V>(
+      chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride,
+      blobs, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+          const uint32_t at = lane + (v << kSliceShift);
+          const uint32_t vi = (begin + at) >> 4;
+          const uint32_t r = x.vrow == 1 ? vi : __umulhi(vi, x.inv_vrow);
+          const uint32_t col = vi - r * x.vrow;
+          const uint32_t t_local = x.heads == 1 ? r : __umulhi(r, x.inv_heads);
+          const uint32_t h = r - t_local * x.heads;
+          const uint32_t cidx = (h * x.ntpb + c.t0() + t_local) * x.vrow + col;
+          coff[v] = at < bytes ? cidx << 4 : kNoVector;
+        }
+      });
+}
+
 // Gather / scatter of a table whose chunks may be strided on the cache side:
 // the token -> offset arithmetic of the TP-remapping layouts (one short range
 // per token, per head, K and V) is evaluated here, per 16-byte vector, instead
@@ -654,6 +823,78 @@ __global__ __launch_bounds__(kThreads, 8) void convert_chunks_kernel(
   });
 }
 
+// The pipelined capped launch of a converting table (every entry 16-byte aligned on both sides
+// and a multiple of 16 elements long): one trip converts V slices of 4096 elements of one
+// entry, lane t the groups of 8 elements t, t + 256, ... of the part, each a 16-byte load
+// through the cache-side descriptor at an offset computed when the part is fetched, and an
+// 8-byte store through the packed-side descriptor. Record arithmetic as in
+// strided_entries_kernel, in groups: a record of vlen * 16 elements is 2 * vlen groups.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <int V>
+__global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes) {
+  constexpr int G = 2 * V;  // groups per lane and trip
+  EntryWalk walk(n_chunks << part_shift, n_layers);
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  rsrc_t cdesc[3], pdesc[3];
+  u32x4 r[3][G];
+  auto next = [&](int k, uint32_t* coff) -> bool {
+    uint32_t item, lay;
+    bool valid;
+    const bool live = walk.next(item, lay, valid);
+    const Entry c = table[item >> part_shift];
+    const uint32_t begin = (item & ((1u << part_shift) - 1u)) * (static_cast<uint32_t>(V) << kSliceShift);
+    uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
+    uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed + begin;
+    const uint32_t bytes =
+        valid && c.len > begin ? min(c.len - begin, static_cast<uint32_t>(V) << kSliceShift) : 0u;
+    pdesc[k] = make_rsrc(pk, bytes);
+    cdesc[k] = make_rsrc(cache, bytes ? kCacheWindow : 0u);
+    const bool plain = c.shape == 0;
+    const u32x16 raw = *reinterpret_cast<const u32x16*>(&shapes.shape[plain ? 0u : c.shape - 1u]);
+    const uint32_t vlen = plain ? 0u : raw[0];
+    const uint32_t rec_mul = plain || raw[0] == 1u ? 0u : raw[1], rec_add = !plain && raw[0] == 1u ? 1u : 0u;
+    const uint32_t n_inner = plain ? 1u : raw[2];
+    const uint32_t o_mul = raw[12], o_add = n_inner == 1u ? 1u : 0u;
+    const uint32_t outer = raw[4], inner = raw[8];
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      const uint32_t g = threadIdx.x + (j << 8);    // group inside the part
+      const uint32_t q = (begin >> 3) + g;          // group inside the entry, < 2^16
+      const uint32_t half = q >> 1;                 // 16-element vector inside the entry
+      const uint32_t rec = __umulhi(half, rec_mul) + half * rec_add;
+      const uint32_t col = q - rec * (vlen << 1);
+      const uint32_t o = __umulhi(rec, o_mul) + rec * o_add;
+      const uint32_t i = rec - o * n_inner;
+      coff[j] = (g << 3) < bytes ? o * outer + i * inner + (col << 4) : kNoVector;
+    }
+    return live;
+  };
+  // the offsets are used up by the loads that follow at once
+  auto fetch = [&](int k) -> bool {
+    uint32_t coff[G];
+    const bool live = next(k, coff);
+#pragma unroll
+    for (int j = 0; j < G; ++j)
+      r[k][j] = __builtin_amdgcn_raw_buffer_load_b128(cdesc[k], coff[j], 0, kLoadPolicy);
+    return live;
+  };
+  auto nothing = [&](int) {};
+  auto store = [&](int k) {
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      u32x2 out;
+      out.x = cvt4(r[k][j].x, r[k][j].y);
+      out.y = cvt4(r[k][j].z, r[k][j].w);
+      __builtin_amdgcn_raw_buffer_store_b64(out, pdesc[k], (threadIdx.x + (j << 8)) << 3, 0, kStorePolicy);
+    }
+  };
+  KVT_ROTATE3(fetch, nothing, store)
+}
+
 // Plain linear copy with the gather kernel's slice shape (calibration / ceiling).
 __global__ __launch_bounds__(kThreads) void copy_linear_kernel(uint8_t* __restrict__ dst,
                                                                const uint8_t* __restrict__ src,
@@ -719,6 +960,78 @@ hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks
   } else {
     if (pack) hipLaunchKernelGGL((copy_entries_kernel<true, 4>), grid, block, 0, stream, KVT_ARGS);
     else hipLaunchKernelGGL((copy_entries_kernel<false, 4>), grid, block, 0, stream, KVT_ARGS);
+  }
+#undef KVT_ARGS
+  return hipGetLastError();
+}
+
+// V slices per trip and the parts an entry is taken in, for entries of 4096 << sub_shift bytes.
+static bool entries_shape(uint32_t sub_shift, uint32_t wgs, int max_v, int* v, uint32_t* part_shift) {
+  if (sub_shift < 1 || sub_shift > 7 || wgs < 8 || (wgs & 7u)) return false;
+  *v = sub_shift == 1 ? 2 : (sub_shift == 2 ? 4 : max_v);
+  *part_shift = sub_shift - (*v == 2 ? 1u : (*v == 4 ? 2u : 3u));
+  return true;
+}
+
+hipError_t launch_strided_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                  uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                  uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                  const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
+                                  hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  int v = 0;
+  uint32_t part_shift = 0;
+  if (!entries_shape(sub_shift, wgs, 8, &v, &part_shift)) return hipErrorInvalidValue;
+  const dim3 grid(wgs), block(kThreads);
+#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+  if (v == 8) {
+    if (pack) hipLaunchKernelGGL((strided_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((strided_entries_kernel<false, 8>), grid, block, 0, stream, KVT_ARGS);
+  } else if (v == 4) {
+    if (pack) hipLaunchKernelGGL((strided_entries_kernel<true, 4>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((strided_entries_kernel<false, 4>), grid, block, 0, stream, KVT_ARGS);
+  } else {
+    if (pack) hipLaunchKernelGGL((strided_entries_kernel<true, 2>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((strided_entries_kernel<false, 2>), grid, block, 0, stream, KVT_ARGS);
+  }
+#undef KVT_ARGS
+  return hipGetLastError();
+}
+
+hipError_t launch_convert_entries(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                  uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                  uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                  const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
+                                  hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  int v = 0;
+  uint32_t part_shift = 0;
+  if (!entries_shape(sub_shift, wgs, 4, &v, &part_shift)) return hipErrorInvalidValue;
+  const dim3 grid(wgs), block(kThreads);
+#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+  if (v == 4) hipLaunchKernelGGL((convert_entries_kernel<4>), grid, block, 0, stream, KVT_ARGS);
+  else hipLaunchKernelGGL((convert_entries_kernel<2>), grid, block, 0, stream, KVT_ARGS);
+#undef KVT_ARGS
+  return hipGetLastError();
+}
+
+hipError_t launch_xform_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                const BlobOffsets& blobs, const XformDev& x, uint32_t wgs,
+                                hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  int v = 0;
+  uint32_t part_shift = 0;
+  // the scatter keeps its offsets until the stores: 8 slices per trip would not fit the registers
+  if (sub_shift < 2 || !entries_shape(sub_shift, wgs, pack ? 8 : 4, &v, &part_shift)) return hipErrorInvalidValue;
+  const dim3 grid(wgs), block(kThreads);
+#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x
+  if (v == 8) {
+    hipLaunchKernelGGL((xform_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);
+  } else {
+    if (pack) hipLaunchKernelGGL((xform_entries_kernel<true, 4>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((xform_entries_kernel<false, 4>), grid, block, 0, stream, KVT_ARGS);
   }
 #undef KVT_ARGS
   return hipGetLastError();

@@ -158,6 +158,7 @@ static int create_plan(int device, const kvt_block_lists* lists, const uint64_t*
         return fail(KVT_ERR_INVALID, "layout transform: rows must be multiples of 16 bytes");
       tok_bytes = static_cast<uint64_t>(xform->heads) * xform->row_bytes;
       half = tok_bytes * xform->ntpb;
+      p->near = half < (1ull << 31);
       if (tok_bytes > kMaxChunk) return fail(KVT_ERR_INVALID, "layout transform: token row too large");
       p->xform = true;
       p->xdev.heads = xform->heads;
@@ -365,6 +366,7 @@ static int create_runs_plan(int device, const kvt_run_lists* lists, const uint64
           sh.inv_vlen = static_cast<uint32_t>((1ull << 32) / sh.vlen) + 1u;
           sh.n_inner = static_cast<uint32_t>(n_in);
           sh.inv_wlen = static_cast<uint32_t>((1ull << 32) / (4u * sh.vlen)) + 1u;
+          sh.inv_inner = sh.n_inner > 1 ? static_cast<uint32_t>((1ull << 32) / sh.n_inner) + 1u : 0u;
           sh.outer[0] = r.src_stride[out_k];
           sh.outer[1] = r.dst_stride[out_k];
           sh.inner[0] = in_k >= 0 ? r.src_stride[in_k] : 0;
@@ -433,6 +435,13 @@ static int create_runs_plan(int device, const kvt_run_lists* lists, const uint64
       } else {
         const uint64_t steps_per = chunk_bytes / sp.group;
         const uint64_t per = steps_per * sp.group;
+        // how far an entry reaches on the cache side, from its first byte: the pipelined capped
+        // kernels address it with 32-bit offsets
+        const StrideShape& sh = p->shapes.shape[sp.shape - 1];
+        const uint64_t reach = (steps_per - 1) * std::max(sp.s_outer, sp.d_outer) +
+                               (sh.n_inner - 1) * std::max(sh.inner[0], sh.inner[1]) +
+                               16ull * sh.vlen * src_scale;
+        if (reach >= (1ull << 31)) p->near = false;
         for (uint64_t o = 0, step = 0; o < sp.bytes; o += per, step += steps_per) {
           pieces.push_back(Piece{sp.src + step * sp.s_outer, sp.dst + step * sp.d_outer,
                                  sp.packed + o,
@@ -611,6 +620,43 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
                                                p->n_tensors, first_layer, n_layers,
                                                static_cast<uint8_t*>(packed), layer_stride, blobs,
                                                wgs, s);
+      if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
+      if (p->buf) {
+        if (capturing) p->buf->captured = true;
+        else if (int rc = p->buf->mark_use(s)) return rc;
+      }
+      return KVT_OK;
+    }
+  }
+  // The same for strided, transposing and converting tables (16-byte vectors only), whose
+  // pipeline carries 5.4-5.9 TB/s whatever the share: from half the device on the strided loop
+  // of the chunk kernels is as fast or faster (5.6 / 5.7 TB/s on the TP2 -> TP1 batch), below
+  // that its rate falls with the share (a quarter: 4.4 / 4.2, an eighth: 2.5 / 2.4). The
+  // converting gather, with two loads and a conversion per store, gains at every share (half
+  // the device: 5.1 against 4.3 TB/s of bytes read and written).
+  const bool converting = p->convert && pack;
+  const uint32_t min_shift = p->xform ? 2u : 1u;  // entries of at least 8 KiB (transposing: 16 KiB)
+  if (max_wgs != 0 && (converting || max_wgs < 4u * device_cu_count(cache->device)) && p->all16 && p->near &&
+      (p->strided || p->xform || converting) && !words && p->sub_shift >= min_shift &&
+      p->sub_shift <= 7 && cache->aligned16 && static_cast<uint64_t>(n) * n_layers > max_wgs) {
+    uint64_t mis = reinterpret_cast<uintptr_t>(packed) | (n_layers > 1 ? layer_stride : 0);
+    for (uint32_t t = 0; t < p->n_tensors; ++t) mis |= blobs.off[t];
+    const uint32_t cus = device_cu_count(cache->device) & ~7u;
+    if ((mis & 15u) == 0 && cus >= 8) {
+      // one workgroup per CU; two where a trip moves only 8 KiB
+      const uint32_t per_cu = p->sub_shift == 1 ? 2u : 1u;
+      const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, per_cu * cus));
+      uint8_t* const pk = static_cast<uint8_t*>(packed);
+      const hipError_t e =
+          converting ? launch_convert_entries(table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
+                                              first_layer, n_layers, pk, layer_stride, blobs,
+                                              p->shapes, wgs, s)
+          : p->xform ? launch_xform_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
+                                            p->n_tensors, first_layer, n_layers, pk, layer_stride,
+                                            blobs, p->xdev, wgs, s)
+                     : launch_strided_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
+                                              p->n_tensors, first_layer, n_layers, pk, layer_stride,
+                                              blobs, p->shapes, wgs, s);
       if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
       if (p->buf) {
         if (capturing) p->buf->captured = true;

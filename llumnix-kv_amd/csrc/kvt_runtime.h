@@ -251,6 +251,7 @@ struct kvt_plan {
   uint64_t n_strided = 0;
   bool convert = false;            // pack converts bf16 -> fp8: lengths count fp8 bytes (elements)
   bool all16 = false;              // every entry's offsets and length are multiples of 16 bytes
+  bool near = true;                // no entry spans 2 GiB or more on the cache side (32-bit offsets do)
   std::vector<kvt::Chunk> host_table;   // device == KVT_DEVICE_NONE only: the tables, kept on the host
   uint32_t sub_shift = 0;          // chunks hold at most 4096 << sub_shift bytes
   // plain plans of at most kSmallTable entries: both tables kept here and passed to the

@@ -391,7 +391,8 @@ class RunLists:
 CHUNK_DTYPE = np.dtype([("cache", "<u8"), ("packed", "<u8"), ("len", "<u4"), ("tensor", "<u2"),
                         ("t0", "<u2"), ("shape", "<u4"), ("reserved", "<u4")])
 SHAPE_DTYPE = np.dtype([("vlen", "<u4"), ("inv_vlen", "<u4"), ("n_inner", "<u4"),
-                        ("inv_wlen", "<u4"), ("outer", "<u8", 2), ("inner", "<u8", 2)])
+                        ("inv_wlen", "<u4"), ("outer", "<u8", 2), ("inner", "<u8", 2),
+                        ("inv_inner", "<u4"), ("reserved", "<u4", 3)])
 RUN_DTYPE = np.dtype([("src_offset", "<u8"), ("dst_offset", "<u8"), ("length", "<u8"),
                       ("n", "<u4", 3), ("reserved0", "<u4"), ("src_stride", "<u8", 3),
                       ("dst_stride", "<u8", 3)])

@@ -83,6 +83,8 @@ static void walk(const Chunk* table, uint64_t n, uint32_t chunk_bytes, const Str
       CHECK(rec == v / s.vlen);  // the reciprocal is exact over the chunk
       const uint32_t col = v - rec * s.vlen;
       const uint32_t o = rec / s.n_inner, i = rec % s.n_inner;
+      // the reciprocal the pipelined kernels divide by (a divisor of 1 has none: they add the dividend)
+      CHECK(s.n_inner == 1 ? s.inv_inner == 0 : umulhi(rec, s.inv_inner) == o);
       const uint64_t at = c.cache + o * s.outer[side] + i * s.inner[side] + col * 16 * scale;
       CHECK(at % 16 == 0 && at + 16 * scale <= cap[c.tensor]);
       for (uint32_t j = 0; j < 16; ++j) {

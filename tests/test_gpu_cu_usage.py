@@ -14,6 +14,7 @@ import pytest
 import kvt_amd
 import test_gpu_pack as tp
 import test_gpu_runs as tr
+from kvt_amd import pipeline, workloads
 
 pytestmark = pytest.mark.gpu
 
@@ -94,3 +95,30 @@ def test_sessions_and_graphs_under_a_limit(limited):
     tp.test_per_layer_session_on_side_stream()
     tp.test_session_inside_hip_graph_replays()
     tp.test_stager_save_load_round_trip_overlapped_with_packing()
+
+
+@pytest.mark.parametrize("usage", [0.25, 0.1, 0.004], ids=["quarter", "tenth", "eight-workgroups"])
+@pytest.mark.parametrize("chunk", [0, 8192, 16384, 32768, 65536, 524288])
+def test_pipelined_kernels_of_strided_transposing_and_converting_plans(usage, chunk):
+    """Below half the device, strided, transposing and converting tables are moved by
+    persistent workgroups that take whole table entries (in parts of 8, 16 or 32 KiB) through
+    buffer descriptors with 32-bit offsets computed per lane. Batches large enough for a full
+    grid of them, every entry size, both directions, against the oracle."""
+    kvt_amd.set_copy_cu_usage(0, usage)
+    try:
+        for layout, p_tp, d_tp, rank in (("flash", 2, 1, 1), ("ragged", 4, 2, 3), ("ragged", 1, 4, 0),
+                                         ("hnd", 2, 1, 1)):
+            w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=4, src_pool=500, dst_pool=600,
+                                   n_req=6, min_tok=200, max_tok=1400)
+            plan, runs = pipeline.build_plan_runs(w, 0, chunk)
+            tr._check(w, plan, tr._oracle_ranges(w), 91, None)
+        for layout, p_tp, d_tp, rank in (("flash", 2, 1, 1), ("ragged", 8, 2, 5)):
+            w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=4, src_pool=500, dst_pool=600,
+                                   n_req=6, min_tok=200, max_tok=1400, fp8_dst=True)
+            tr._check_converting(w, chunk, "raw")
+        if chunk in (0, 32768, 65536):   # a chunk holds whole token rows of the transform
+            w = workloads.llama70b_flashinfer(n_layers=4, pool=400, n_req=4, tokens=1500)
+            plan, lists = pipeline.build_plan(w, 0, chunk)
+            tp._transposing(w, plan=plan, lists=lists)
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)

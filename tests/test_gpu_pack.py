@@ -152,9 +152,10 @@ def test_chunked_prefill_steps_and_ragged_tail():
     _check_pack_unpack(w)
 
 
-def _transposing(w_t, seed=3):
+def _transposing(w_t, seed=3, plan=None, lists=None):
     heads, ntpb, row = w_t.xform
-    plan, lists = pipeline.build_plan(w_t, 0)
+    if plan is None:
+        plan, lists = pipeline.build_plan(w_t, 0)
     runs = lists.tensor(0)
     B = 2 * heads * ntpb * row
     ids = np.concatenate([np.arange(r[0] // B, (r[0] + r[2]) // B) for r in runs]).astype(np.uint32)

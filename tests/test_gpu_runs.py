@@ -214,6 +214,10 @@ def test_converting_run_plan_bf16_sender_fp8_receiver(layout, p_tp, d_tp, rank, 
     (NaNs, infinities, denormals) likely."""
     w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=2, src_pool=300, dst_pool=400,
                            n_req=4, min_tok=60, max_tok=900, fp8_dst=True)
+    _check_converting(w, chunk, content)
+
+
+def _check_converting(w, chunk, content):
     plan, runs = pipeline.build_plan_runs(w, 0, chunk)
     assert plan.num_strided_chunks > 0
     src_i, dst_i = w.worker_infos()

@@ -52,6 +52,12 @@ def emulate(table, chunk_bytes, shapes, caches, tensor_offset, packed, pack, con
             w = np.arange(n // 4, dtype=np.uint64)                             # word-wise path
             assert np.array_equal((w * np.uint64(int(s["inv_wlen"]))) >> np.uint64(32),
                                   w // np.uint64(4 * vlen))
+            inv_inner = int(s["inv_inner"])                                    # pipelined kernels
+            if n_inner == 1:
+                assert inv_inner == 0
+            else:
+                assert np.array_equal((rec * np.uint64(inv_inner)) >> np.uint64(32),
+                                      rec // np.uint64(n_inner))
             col = v - rec * np.uint64(vlen)
             o, i = rec // np.uint64(n_inner), rec % np.uint64(n_inner)
             at = (o * np.uint64(int(s["outer"][side])) + i * np.uint64(int(s["inner"][side]))
