@@ -857,13 +857,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "e296c7bff5072869475b8982ee6877249a5849504a82c1ac888db6217ef376a5"
+KERNELS_SHA256 = "f7a1009550404fca309ca216f033c8b2359cdba678127b6591fbf1a974b639f2"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134263594, "unpack": 134277546},
-    (2, "ranges"): {"pack": 71013059763, "unpack": 73358396750},
-    (3, "ranges"): {"pack": 85983093249, "unpack": 85983584168},
-    (4, "ranges"): {"pack": 22690381169, "unpack": 22690437702},
-    (5, "ranges"): {"pack": 45141190235, "unpack": 45141384964},
+    (1, "ranges"): {"pack": 134277001, "unpack": 134277086},
+    (2, "ranges"): {"pack": 71013155209, "unpack": 73358401899},
+    (3, "ranges"): {"pack": 85983097442, "unpack": 85983590068},
+    (4, "ranges"): {"pack": 22690396284, "unpack": 22690440529},
+    (5, "ranges"): {"pack": 45141195254, "unpack": 45141390453},
 }
 
 
@@ -1043,7 +1043,7 @@ def run_config(args, headline):
     elif first[0][0].num_chunks <= 64:
         kernel = "kvt::copy_chunks_small_kernel<true, false> (pack)"
     else:
-        kernel = "kvt::copy_chunks_kernel<true, false> (pack)"
+        kernel = "kvt::copy_chunks_kernel<true, 0> (pack)"
     out = {
         "metric": "pack+unpack GB/s (bytes read + bytes written per second, whole job)",
         "value": round(value, 1),

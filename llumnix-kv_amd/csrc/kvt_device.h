@@ -58,7 +58,9 @@ struct StrideTable {
 // max_wgs > 0: at most that many workgroups (a multiple of 8), striding over the same items,
 // for a caller that wants the copy to leave part of the device to other kernels.
 // temporal: plain instead of non-temporal loads, for a launch whose data may sit in the
-// memory-side cache (ignored by a capped launch).
+// memory-side cache (ignored by a capped launch). pipelined (launch_copy_chunks): a capped
+// launch keeps the loads of its next trip in flight across the stores of the last one; for
+// grids of at most 4 workgroups per CU (the kernel then needs more registers than 8 per CU fit).
 hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
@@ -88,8 +90,8 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
-                              hipStream_t stream);
+                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
+                              bool temporal, hipStream_t stream);
 // The capped launch of a plain table with 16-byte aligned entries of at most 16 KiB
 // (sub_shift 2) or 32 KiB (sub_shift 3): `wgs` persistent workgroups (a multiple of 8), one
 // table entry per trip, software-pipelined. Every address and length involved must be a

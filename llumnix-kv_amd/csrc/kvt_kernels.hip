@@ -111,9 +111,35 @@ __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst,
 // item paying for three dependent loads in a row (table entry, layer pointer, data). So it
 // takes kBatch items per trip in phases: the kBatch table entries (independent scalar
 // loads), then the kBatch layer pointers, then the lanes' addresses, then the kBatch vector
-// loads back to back and only then the stores: a lane has kBatch x 16 bytes in flight.
+// loads back to back; the stores of a trip are issued only after the loads of the next one
+// (three register sets in rotation), so a lane has up to 2 x kBatch x 16 bytes in flight.
+
+// Three register sets in rotation: the loads of item k+1 are issued before the stores of item k,
+// and a set is loaded again only two trips after its stores were issued.
+#define KVT_ROTATE3(NEXT, LOAD, STORE) \
+  if (!NEXT(0)) return;                \
+  LOAD(0);                             \
+  for (;;) {                           \
+    const bool l1 = NEXT(1);           \
+    LOAD(1);                           \
+    STORE(0);                          \
+    if (!l1) break;                    \
+    const bool l2 = NEXT(2);           \
+    LOAD(2);                           \
+    STORE(1);                          \
+    if (!l2) break;                    \
+    const bool l0 = NEXT(0);           \
+    LOAD(0);                           \
+    STORE(2);                          \
+    if (!l0) break;                    \
+  }
 
 constexpr int kBatch = 4;
+// How a chunk kernel walks its items: one workgroup per (slice, layer); a capped grid striding
+// over them kBatch at a time; the same with the trips software-pipelined. Twice the bytes in
+// flight pay below half the device (config 4 at a quarter: 4.8 / 4.5 -> 5.2 / 5.2 TB/s) and
+// cost from there on (at one half 5.6 / 5.5 -> 5.1 / 5.2), so the launcher picks by grid size.
+enum { kOnePerSlice = 0, kStriding = 1, kPipelined = 2 };
 constexpr uint32_t kTemporalFlag = 0x100u;  // in a kernel's sub_shift argument: Launch::temporal
 
 // The uniform arguments of a chunk launch.
@@ -174,11 +200,11 @@ struct Move {
 };
 #define KVT_NO_MOVE (Move{nullptr, nullptr, 0, 0, false})
 
-// `fetch(entry)` reads a table entry; `place(item)` turns an item into the lane's move. Odd
+// `fetch_table(entry)` reads a table entry; `place(item)` turns an item into the lane's move. Odd
 // cases (misaligned slices, stragglers behind the last whole vector) `place` may move itself.
-template <bool CAPPED, class Fetch, class Place>
-__device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place place) {
-  if (!CAPPED) {
+template <int MODE, class Fetch, class Place>
+__device__ __forceinline__ void for_items(const Launch& L, Fetch fetch_table, Place place) {
+  if (MODE == kOnePerSlice) {
     // A workgroup's life is a chain of dependent round trips and then its one vector, and
     // 2 048 resident workgroups have to hide all of it: the chain is kept to three links.
     // (1) every argument; (2) the table entry as ONE 32-byte scalar load and, beside it, the
@@ -194,7 +220,7 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place pl
     uint64_t stride = L.layer_stride, blob = L.blobs->off[0];
     asm volatile("" : "+s"(stride), "+s"(blob));
     uint8_t* const* row = L.layer_ptrs + static_cast<uint64_t>(L.first_layer + layer) * L.n_tensors;
-    u32x8 raw = fetch(bc >> L.sub_shift);
+    u32x8 raw = fetch_table(bc >> L.sub_shift);
     uint8_t* base = row[0];
     asm volatile("" : "+s"(raw), "+s"(base));
     Item it;
@@ -231,7 +257,14 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place pl
   const uint32_t per_layer = (L.n_slices + 7u) & ~7u;
   const uint32_t d_layer = gridDim.x / per_layer, d_slice = gridDim.x - d_layer * per_layer;
   uint32_t layer = blockIdx.x / per_layer, s = blockIdx.x - layer * per_layer;
-  while (layer < L.n_layers) {
+  // kStriding: a trip loads kBatch vectors and stores them. kPipelined: three sets of kBatch
+  // vectors in rotation (KVT_ROTATE3), the loads of the next kBatch items in flight before the
+  // stores of the last ones are issued. What a set keeps until its stores is each vector's
+  // destination (null: no vector).
+  uint8_t* dst[3][kBatch];
+  u32x4 r[3][kBatch];
+  auto fetch = [&](int k) -> bool {
+    const bool live = layer < L.n_layers;
     Item it[kBatch];
     uint32_t lay[kBatch];
     bool valid[kBatch];
@@ -241,7 +274,7 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place pl
       valid[j] = layer < L.n_layers && b < L.n_slices;
       lay[j] = min(layer, L.n_layers - 1u);
       const uint32_t bc = min(b, L.n_slices - 1u);
-      it[j].c = entry_of(fetch(bc >> L.sub_shift));
+      it[j].c = entry_of(fetch_table(bc >> L.sub_shift));
       it[j].sub = bc & ((1u << L.sub_shift) - 1u);
       s += d_slice;
       layer += d_layer;
@@ -263,13 +296,23 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch, Place pl
       m[j] = KVT_NO_MOVE;
       if (valid[j]) m[j] = place(it[j]);
     }
-    u32x4 r[kBatch];
 #pragma unroll
-    for (int j = 0; j < kBatch; ++j) r[j] = load_vec(m[j].on ? m[j].src + m[j].src_off : idle);
+    for (int j = 0; j < kBatch; ++j) r[k][j] = load_vec(m[j].on ? m[j].src + m[j].src_off : idle);
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) dst[k][j] = m[j].on ? m[j].dst + m[j].dst_off : nullptr;
+    return live;
+  };
+  auto nothing = [](int) {};
+  auto store = [&](int k) {
 #pragma unroll
     for (int j = 0; j < kBatch; ++j)
-      if (m[j].on) store_vec(m[j].dst + m[j].dst_off, r[j]);
+      if (dst[k][j]) store_vec(dst[k][j], r[k][j]);
+  };
+  if (MODE == kStriding) {
+    while (fetch(0)) store(0);
+    return;
   }
+  KVT_ROTATE3(fetch, nothing, store)
 }
 
 // The lane's share of one contiguous slice: `on` when the slice is 16-byte aligned on both
@@ -301,14 +344,14 @@ __device__ __forceinline__ Move plain_move(const Item& it) {
                  (sub_shift & kTemporalFlag) != 0}
 
 // Gather (PACK) / scatter of a resident chunk table.
-template <bool PACK, bool CAPPED>
-__global__ __launch_bounds__(kThreads, 8) void copy_chunks_kernel(
+template <bool PACK, int MODE>
+__global__ __launch_bounds__(kThreads, MODE == kPipelined ? 4 : 8) void copy_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); },
-                    [&](const Item& it) { return plain_move<PACK>(it); });
+  for_items<MODE>(L, [&](uint32_t e) { return fetch_entry(chunks, e); },
+                  [&](const Item& it) { return plain_move<PACK>(it); });
 }
 
 // The same for a table short enough to be a kernel argument (read through the scalar cache
@@ -319,7 +362,7 @@ __global__ __launch_bounds__(kThreads, 8) void copy_chunks_small_kernel(
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(table.c, e); },
+  for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(table.c, e); },
                     [&](const Item& it) { return plain_move<PACK>(it); });
 }
 
@@ -443,26 +486,6 @@ struct EntryWalk {
     return live;
   }
 };
-
-// Three register sets in rotation: the loads of item k+1 are issued before the stores of item k,
-// and a set is loaded again only two trips after its stores were issued.
-#define KVT_ROTATE3(NEXT, LOAD, STORE) \
-  if (!NEXT(0)) return;                \
-  LOAD(0);                             \
-  for (;;) {                           \
-    const bool l1 = NEXT(1);           \
-    LOAD(1);                           \
-    STORE(0);                          \
-    if (!l1) break;                    \
-    const bool l2 = NEXT(2);           \
-    LOAD(2);                           \
-    STORE(1);                          \
-    if (!l2) break;                    \
-    const bool l0 = NEXT(0);           \
-    LOAD(0);                           \
-    STORE(2);                          \
-    if (!l0) break;                    \
-  }
 
 template <bool PACK, int V, class CacheOffsets>
 __device__ __forceinline__ void entries_pipeline(
@@ -588,7 +611,7 @@ __global__ __launch_bounds__(kThreads, 8) void strided_chunks_kernel(
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     StrideTable shapes) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
+  for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     if (it.c.shape == 0) return plain_move<PACK>(it);
     const uint32_t off = it.sub << kSliceShift;
     if (off >= it.c.len) return KVT_NO_MOVE;
@@ -637,7 +660,7 @@ __global__ __launch_bounds__(kThreads, 8) void xform_chunks_kernel(
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     XformDev x) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
+  for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     const uint32_t v = (it.sub << 8) + threadIdx.x;  // 256 vectors per slice
     // exact quotients by multiply-high (operands < 2^16); a divisor of 1 has no such constant
     const uint32_t r = x.vrow == 1 ? v : __umulhi(v, x.inv_vrow);  // packed-side row: t_local*heads + h
@@ -767,7 +790,7 @@ __global__ __launch_bounds__(kThreads, 8) void convert_chunks_kernel(
   // that both of its loads and both of its stores are contiguous across the wavefront (a lane
   // that loads 32 contiguous bytes makes every load touch twice the lines it uses: measured
   // 2.7 % slower on the TP2 -> TP1 batch).
-  for_items<CAPPED>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
+  for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
     const uint32_t off = it.sub << kSliceShift;
     if (off >= it.c.len) return KVT_NO_MOVE;
@@ -931,17 +954,23 @@ static ChunkGrid chunk_grid(uint32_t n_slices, uint32_t n_layers, uint32_t max_w
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
-                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
-                              hipStream_t stream) {
+                              uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
+                              bool temporal, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
   const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
 #define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
-  if (pack && !g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, false>), KVT_ARGS);
-  else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, true>), KVT_ARGS);
-  else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, false>), KVT_ARGS);
-  else KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, true>), KVT_ARGS);
+  if (!g.capped) {
+    if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, kOnePerSlice>), KVT_ARGS);
+    else KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, kOnePerSlice>), KVT_ARGS);
+  } else if (!pipelined) {
+    if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, kStriding>), KVT_ARGS);
+    else KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, kStriding>), KVT_ARGS);
+  } else {
+    if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, kPipelined>), KVT_ARGS);
+    else KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, kPipelined>), KVT_ARGS);
+  }
 #undef KVT_ARGS
   return hipGetLastError();
 }

@@ -679,7 +679,8 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
                                      layer_stride, blobs, p->xdev, max_wgs, temporal, s)
                : launch_copy_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                     first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                    layer_stride, blobs, max_wgs, temporal, s);
+                                    layer_stride, blobs, max_wgs,
+                                    max_wgs < 4u * device_cu_count(cache->device), temporal, s);
   if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
   if (p->buf) {
     // remember when the table is last read, so that its storage is not recycled too early
