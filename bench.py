@@ -857,13 +857,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "f7a1009550404fca309ca216f033c8b2359cdba678127b6591fbf1a974b639f2"
+KERNELS_SHA256 = "d18bcfc9f6ecfa57dd4e938f52f8c7e255c03a3bacd6af9f527558aa05a0a750"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134277001, "unpack": 134277086},
-    (2, "ranges"): {"pack": 71013155209, "unpack": 73358401899},
-    (3, "ranges"): {"pack": 85983097442, "unpack": 85983590068},
-    (4, "ranges"): {"pack": 22690396284, "unpack": 22690440529},
-    (5, "ranges"): {"pack": 45141195254, "unpack": 45141390453},
+    (1, "ranges"): {"pack": 134272222, "unpack": 134275422},
+    (2, "ranges"): {"pack": 71013037920, "unpack": 73358402624},
+    (3, "ranges"): {"pack": 85983098765, "unpack": 85983588532},
+    (4, "ranges"): {"pack": 22690334162, "unpack": 22690387367},
+    (5, "ranges"): {"pack": 45141187873, "unpack": 45141390581},
 }
 
 

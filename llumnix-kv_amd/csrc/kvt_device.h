@@ -99,7 +99,11 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
 hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
-                               const BlobOffsets& blobs, uint32_t wgs, hipStream_t stream);
+                               const BlobOffsets& blobs, uint32_t wgs, uint32_t* tickets,
+                               hipStream_t stream);
+// tickets (all the pipelined launchers): nine zeroed 32-bit counters 128 bytes apart that no other
+// running launch uses, from which the workgroups take their work in order (they leave them
+// zeroed again); nullptr: every workgroup strides through a fixed share of the work.
 // The same pipeline for strided and for transposing tables (sub_shift 2 ... 7; larger entries
 // are taken in parts of 16 or 32 KiB). Every entry must be 16-byte aligned on both sides, a multiple
 // of 16 bytes long, and span less than 2 GiB on the cache side.
@@ -107,19 +111,19 @@ hipError_t launch_strided_entries(bool pack, const Chunk* chunks, uint32_t n_chu
                                   uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                   uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                   const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
-                                  hipStream_t stream);
+                                  uint32_t* tickets, hipStream_t stream);
 // ... and for the converting gather (entries a multiple of 16 elements long; sub_shift 1 ... 7;
 // strided entries also from sub_shift 1).
 hipError_t launch_convert_entries(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                   uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                   uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                   const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
-                                  hipStream_t stream);
+                                  uint32_t* tickets, hipStream_t stream);
 hipError_t launch_xform_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                 uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                 uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                 const BlobOffsets& blobs, const XformDev& x, uint32_t wgs,
-                                hipStream_t stream);
+                                uint32_t* tickets, hipStream_t stream);
 hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

@@ -117,22 +117,24 @@ __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst,
 // Three register sets in rotation: the loads of item k+1 are issued before the stores of item k,
 // and a set is loaded again only two trips after its stores were issued.
 #define KVT_ROTATE3(NEXT, LOAD, STORE) \
-  if (!NEXT(0)) return;                \
-  LOAD(0);                             \
-  for (;;) {                           \
-    const bool l1 = NEXT(1);           \
-    LOAD(1);                           \
-    STORE(0);                          \
-    if (!l1) break;                    \
-    const bool l2 = NEXT(2);           \
-    LOAD(2);                           \
-    STORE(1);                          \
-    if (!l2) break;                    \
-    const bool l0 = NEXT(0);           \
+  do {                                 \
+    if (!NEXT(0)) break;               \
     LOAD(0);                           \
-    STORE(2);                          \
-    if (!l0) break;                    \
-  }
+    for (;;) {                         \
+      const bool l1 = NEXT(1);         \
+      LOAD(1);                         \
+      STORE(0);                        \
+      if (!l1) break;                  \
+      const bool l2 = NEXT(2);         \
+      LOAD(2);                         \
+      STORE(1);                        \
+      if (!l2) break;                  \
+      const bool l0 = NEXT(0);         \
+      LOAD(0);                         \
+      STORE(2);                        \
+      if (!l0) break;                  \
+    }                                  \
+  } while (0)
 
 constexpr int kBatch = 4;
 // How a chunk kernel walks its items: one workgroup per (slice, layer); a capped grid striding
@@ -312,7 +314,7 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch_table, Pl
     while (fetch(0)) store(0);
     return;
   }
-  KVT_ROTATE3(fetch, nothing, store)
+  KVT_ROTATE3(fetch, nothing, store);
 }
 
 // The lane's share of one contiguous slice: `on` when the slice is 16-byte aligned on both
@@ -385,65 +387,119 @@ __device__ __forceinline__ rsrc_t make_rsrc(const uint8_t* base, uint32_t bytes)
 // cache-policy operand of the buffer builtins: bit 0 = sc0, bit 1 = nt, bit 4 = sc1
 constexpr int kLoadPolicy = 2, kStorePolicy = 1 | 2 | 16;
 
+// This workgroup's way through the (item, layer) pairs of a launch: the items of a layer are
+// dealt to the XCDs in eighths. Without tickets a workgroup strides through its XCD's pairs by
+// the number of workgroups there. With tickets (eight counters, one per XCD, 128 bytes apart,
+// zero at the start of the launch) it takes whatever pair is next on its XCD: workgroups that
+// fall behind no longer spread the addresses in flight over a widening window, which is worth
+// 16 % on a plain 4 GiB copy by 256 persistent workgroups (5.5 -> 6.4 TB/s). The last
+// workgroup to leave zeroes the counters again (kTicketDone counts the leavers).
+constexpr uint32_t kTicketStride = 32, kTicketDone = 8 * kTicketStride;  // in 32-bit words
+// log2 of the 4 KiB slices one ticket stands for: 32 KiB. Finer tickets run into the rate at
+// which one counter can be bumped (16 KiB entries, one per ticket: 11 % slower than without
+// tickets), coarser ones give the order away again (64 / 128 KiB: -6 / -9 % on config 2).
+constexpr uint32_t kTicketSlicesLog2 = 3;
+struct EntryWalk {
+  uint32_t n_items, n_layers, per8, xcd, step_layer, step_within, layer, within;
+  uint32_t* tickets;
+  uint32_t run_shift;  // a ticket stands for 1 << run_shift consecutive pairs
+  uint32_t pair, left; // tickets: the next pair of the current run, and how many of it are left
+  uint32_t ahead;      // lane 0: the ticket of the next run, asked for one run early
+  // slices_log2: log2 of the 4 KiB slices one item holds
+  __device__ __forceinline__ EntryWalk(uint32_t items, uint32_t layers, uint32_t* ticket_block, uint32_t slices_log2)
+      : n_items(items), n_layers(layers), tickets(ticket_block), pair(0), left(0), ahead(0) {
+    per8 = (n_items + 7u) >> 3;
+    xcd = blockIdx.x & 7u;
+    run_shift = slices_log2 < kTicketSlicesLog2 ? kTicketSlicesLog2 - slices_log2 : 0u;
+    if (tickets && threadIdx.x == 0) ahead = atomicAdd(tickets + xcd * kTicketStride, 1u);
+    const uint32_t nloc = gridDim.x >> 3;  // workgroups per XCD
+    step_layer = nloc / per8;
+    step_within = nloc - step_layer * per8;
+    layer = (blockIdx.x >> 3) / per8;
+    within = (blockIdx.x >> 3) - layer * per8;
+  }
+  // The next pair, clamped to the last one past the end (`valid` false: nothing to move there);
+  // returns false once the workgroup is past the last layer. `k`: which of three slots carries
+  // the ticket from lane 0 to the workgroup (a wavefront is at most one barrier behind).
+  __device__ __forceinline__ bool next(int k, uint32_t& item, uint32_t& lay, bool& valid) {
+    if (tickets) {
+      if (left == 0) {
+        __shared__ uint32_t slot[3];
+        if (threadIdx.x == 0) {
+          slot[k] = ahead;
+          ahead = atomicAdd(tickets + xcd * kTicketStride, 1u);
+        }
+        __syncthreads();
+        pair = __builtin_amdgcn_readfirstlane(slot[k]) << run_shift;
+        left = 1u << run_shift;
+      }
+      layer = pair / per8;
+      within = pair - layer * per8;
+      ++pair;
+      --left;
+    }
+    const bool live = layer < n_layers;
+    const uint32_t b = xcd * per8 + within;
+    valid = live && b < n_items;
+    lay = min(layer, n_layers - 1u);
+    item = min(b, n_items - 1u);
+    if (!tickets) {
+      within += step_within;
+      layer += step_layer;
+      const bool wrap = within >= per8;
+      within -= wrap ? per8 : 0u;
+      layer += wrap ? 1u : 0u;
+    }
+    return live;
+  }
+  // Call once, when next() has returned false.
+  __device__ __forceinline__ void leave() {
+    if (!tickets || threadIdx.x != 0) return;
+    asm volatile("" ::"v"(ahead));  // the last ticket asked for has been handed out: it came back
+    if (atomicAdd(tickets + kTicketDone, 1u) == gridDim.x - 1u) {
+#pragma unroll
+      for (uint32_t x = 0; x < 8; ++x) atomicExch(tickets + x * kTicketStride, 0u);
+      atomicExch(tickets + kTicketDone, 0u);
+    }
+  }
+};
+
 template <bool PACK, int V>
 __global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
-  const uint32_t per8 = (n_chunks + 7u) >> 3;
-  const uint32_t xcd = blockIdx.x & 7u;
-  const uint32_t nloc = gridDim.x >> 3;  // workgroups per XCD
-  const uint32_t step_layer = nloc / per8, step_within = nloc - step_layer * per8;
-  uint32_t layer = (blockIdx.x >> 3) / per8, within = (blockIdx.x >> 3) - layer * per8;
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    uint32_t* tickets) {
+  EntryWalk walk(n_chunks, n_layers, tickets, V == 8 ? 3u : 2u);
   const uint32_t off = threadIdx.x << 4;
   const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  rsrc_t src[3], dst[3];
+  u32x4 r[3][V];
   // this workgroup's next entry as two descriptors (empty ones past the end); false past the end
-  auto next = [&](rsrc_t& src, rsrc_t& dst) -> bool {
-    const bool live = layer < n_layers;
-    const uint32_t b = xcd * per8 + within;
-    const bool valid = live && b < n_chunks;
-    const uint32_t lay = min(layer, n_layers - 1u);
-    const Entry c = table[min(b, n_chunks - 1u)];
+  auto next = [&](int k) -> bool {
+    uint32_t item, lay;
+    bool valid;
+    const bool live = walk.next(k, item, lay, valid);
+    const Entry c = table[item];
     uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
     uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed;
     const uint32_t bytes = valid ? c.len : 0u;
-    src = make_rsrc(PACK ? cache : pk, bytes);
-    dst = make_rsrc(PACK ? pk : cache, bytes);
-    within += step_within;
-    layer += step_layer;
-    const bool wrap = within >= per8;
-    within -= wrap ? per8 : 0u;
-    layer += wrap ? 1u : 0u;
+    src[k] = make_rsrc(PACK ? cache : pk, bytes);
+    dst[k] = make_rsrc(PACK ? pk : cache, bytes);
     return live;
   };
-  auto load = [&](rsrc_t src, u32x4* r) {
+  auto load = [&](int k) {
 #pragma unroll
     for (int v = 0; v < V; ++v)
-      r[v] = __builtin_amdgcn_raw_buffer_load_b128(src, off + (v << kSliceShift), 0, kLoadPolicy);
+      r[k][v] = __builtin_amdgcn_raw_buffer_load_b128(src[k], off + (v << kSliceShift), 0, kLoadPolicy);
   };
-  auto store = [&](rsrc_t dst, const u32x4* r) {
+  auto store = [&](int k) {
 #pragma unroll
     for (int v = 0; v < V; ++v)
-      __builtin_amdgcn_raw_buffer_store_b128(r[v], dst, off + (v << kSliceShift), 0, kStorePolicy);
+      __builtin_amdgcn_raw_buffer_store_b128(r[k][v], dst[k], off + (v << kSliceShift), 0, kStorePolicy);
   };
-  rsrc_t s0, d0, s1, d1, s2, d2;
-  u32x4 r0[V], r1[V], r2[V];
-  if (!next(s0, d0)) return;
-  load(s0, r0);
-  for (;;) {
-    const bool l1 = next(s1, d1);
-    load(s1, r1);
-    store(d0, r0);
-    if (!l1) break;
-    const bool l2 = next(s2, d2);
-    load(s2, r2);
-    store(d1, r1);
-    if (!l2) break;
-    const bool l0 = next(s0, d0);
-    load(s0, r0);
-    store(d2, r2);
-    if (!l0) break;
-  }
+  KVT_ROTATE3(next, load, store);
+  walk.leave();
 }
 
 // The same pipeline for tables whose cache side is not contiguous (strided records, the
@@ -457,43 +513,13 @@ __global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
 constexpr uint32_t kCacheWindow = 0x80000000u;  // bytes a cache-side descriptor covers
 constexpr uint32_t kNoVector = kCacheWindow;    // first offset outside it: loads give zero, stores are dropped
 
-// This workgroup's way through the (item, layer) pairs of a launch: the items of a layer are
-// dealt to the XCDs in eighths, neighbouring workgroups of an XCD take neighbouring items.
-struct EntryWalk {
-  uint32_t n_items, n_layers, per8, xcd, step_layer, step_within, layer, within;
-  __device__ __forceinline__ EntryWalk(uint32_t items, uint32_t layers) : n_items(items), n_layers(layers) {
-    per8 = (n_items + 7u) >> 3;
-    xcd = blockIdx.x & 7u;
-    const uint32_t nloc = gridDim.x >> 3;  // workgroups per XCD
-    step_layer = nloc / per8;
-    step_within = nloc - step_layer * per8;
-    layer = (blockIdx.x >> 3) / per8;
-    within = (blockIdx.x >> 3) - layer * per8;
-  }
-  // The next pair, clamped to the last one past the end (`valid` false: nothing to move there);
-  // returns false once the workgroup is past the last layer.
-  __device__ __forceinline__ bool next(uint32_t& item, uint32_t& lay, bool& valid) {
-    const bool live = layer < n_layers;
-    const uint32_t b = xcd * per8 + within;
-    valid = live && b < n_items;
-    lay = min(layer, n_layers - 1u);
-    item = min(b, n_items - 1u);
-    within += step_within;
-    layer += step_layer;
-    const bool wrap = within >= per8;
-    within -= wrap ? per8 : 0u;
-    layer += wrap ? 1u : 0u;
-    return live;
-  }
-};
-
 template <bool PACK, int V, class CacheOffsets>
 __device__ __forceinline__ void entries_pipeline(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride,
-    const BlobOffsets& blobs, CacheOffsets cache_offsets) {
-  EntryWalk walk(n_chunks << part_shift, n_layers);
+    const BlobOffsets& blobs, uint32_t* tickets, CacheOffsets cache_offsets) {
+  EntryWalk walk(n_chunks << part_shift, n_layers, tickets, V == 8 ? 3u : (V == 4 ? 2u : 1u));
   const uint32_t lane = threadIdx.x << 4;
   const Entry* table = reinterpret_cast<const Entry*>(chunks);
   rsrc_t cdesc[3], pdesc[3];
@@ -502,7 +528,7 @@ __device__ __forceinline__ void entries_pipeline(
   auto next = [&](int k) -> bool {
     uint32_t item, lay;
     bool valid;
-    const bool live = walk.next(item, lay, valid);
+    const bool live = walk.next(k, item, lay, valid);
     const Entry c = table[item >> part_shift];
     const uint32_t begin = (item & ((1u << part_shift) - 1u)) * (static_cast<uint32_t>(V) << kSliceShift);
     uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
@@ -529,7 +555,8 @@ __device__ __forceinline__ void entries_pipeline(
         __builtin_amdgcn_raw_buffer_store_b128(r[k][v], cdesc[k], coff[k][v], 0, kStorePolicy);
     }
   };
-  KVT_ROTATE3(next, load, store)
+  KVT_ROTATE3(next, load, store);
+  walk.leave();
 }
 
 // Strided tables (16-byte vectors only; every entry 16-byte aligned on both sides). The
@@ -543,11 +570,11 @@ __global__ __launch_bounds__(kThreads, 4) void strided_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    StrideTable shapes) {
+    StrideTable shapes, uint32_t* tickets) {
   const uint32_t lane = threadIdx.x << 4;
   entries_pipeline<PACK, V>(
       chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride,
-      blobs, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
+      blobs, tickets, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
         const bool plain = c.shape == 0;
         const u32x16 raw = *reinterpret_cast<const u32x16*>(&shapes.shape[plain ? 0u : c.shape - 1u]);
         // words of a StrideShape: 0 vlen, 1 inv_vlen, 2 n_inner, 4 + 2 side: outer, 8 + 2 side: inner,
@@ -576,11 +603,11 @@ __global__ __launch_bounds__(kThreads, 4) void xform_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    XformDev x) {
+    XformDev x, uint32_t* tickets) {
   const uint32_t lane = threadIdx.x << 4;
   entries_pipeline<PACK, V>(
       chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride,
-      blobs, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
+      blobs, tickets, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
 #pragma unroll
         for (int v = 0; v < V; ++v) {
           const uint32_t at = lane + (v << kSliceShift);
@@ -858,16 +885,16 @@ __global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    StrideTable shapes) {
+    StrideTable shapes, uint32_t* tickets) {
   constexpr int G = 2 * V;  // groups per lane and trip
-  EntryWalk walk(n_chunks << part_shift, n_layers);
+  EntryWalk walk(n_chunks << part_shift, n_layers, tickets, V == 8 ? 3u : (V == 4 ? 2u : 1u));
   const Entry* table = reinterpret_cast<const Entry*>(chunks);
   rsrc_t cdesc[3], pdesc[3];
   u32x4 r[3][G];
   auto next = [&](int k, uint32_t* coff) -> bool {
     uint32_t item, lay;
     bool valid;
-    const bool live = walk.next(item, lay, valid);
+    const bool live = walk.next(k, item, lay, valid);
     const Entry c = table[item >> part_shift];
     const uint32_t begin = (item & ((1u << part_shift) - 1u)) * (static_cast<uint32_t>(V) << kSliceShift);
     uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
@@ -915,7 +942,8 @@ __global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
       __builtin_amdgcn_raw_buffer_store_b64(out, pdesc[k], (threadIdx.x + (j << 8)) << 3, 0, kStorePolicy);
     }
   };
-  KVT_ROTATE3(fetch, nothing, store)
+  KVT_ROTATE3(fetch, nothing, store);
+  walk.leave();
 }
 
 // Plain linear copy with the gather kernel's slice shape (calibration / ceiling).
@@ -978,11 +1006,11 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
 hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
-                               const BlobOffsets& blobs, uint32_t wgs, hipStream_t stream) {
+                               const BlobOffsets& blobs, uint32_t wgs, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   if ((sub_shift != 2 && sub_shift != 3) || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
   const dim3 grid(wgs), block(kThreads);
-#define KVT_ARGS chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+#define KVT_ARGS chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
   if (sub_shift == 3) {
     if (pack) hipLaunchKernelGGL((copy_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);
     else hipLaunchKernelGGL((copy_entries_kernel<false, 8>), grid, block, 0, stream, KVT_ARGS);
@@ -1006,13 +1034,13 @@ hipError_t launch_strided_entries(bool pack, const Chunk* chunks, uint32_t n_chu
                                   uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                   uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                   const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
-                                  hipStream_t stream) {
+                                  uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   int v = 0;
   uint32_t part_shift = 0;
   if (!entries_shape(sub_shift, wgs, 8, &v, &part_shift)) return hipErrorInvalidValue;
   const dim3 grid(wgs), block(kThreads);
-#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets
   if (v == 8) {
     if (pack) hipLaunchKernelGGL((strided_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);
     else hipLaunchKernelGGL((strided_entries_kernel<false, 8>), grid, block, 0, stream, KVT_ARGS);
@@ -1031,13 +1059,13 @@ hipError_t launch_convert_entries(const Chunk* chunks, uint32_t n_chunks, uint32
                                   uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                   uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                   const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
-                                  hipStream_t stream) {
+                                  uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   int v = 0;
   uint32_t part_shift = 0;
   if (!entries_shape(sub_shift, wgs, 4, &v, &part_shift)) return hipErrorInvalidValue;
   const dim3 grid(wgs), block(kThreads);
-#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets
   if (v == 4) hipLaunchKernelGGL((convert_entries_kernel<4>), grid, block, 0, stream, KVT_ARGS);
   else hipLaunchKernelGGL((convert_entries_kernel<2>), grid, block, 0, stream, KVT_ARGS);
 #undef KVT_ARGS
@@ -1048,14 +1076,14 @@ hipError_t launch_xform_entries(bool pack, const Chunk* chunks, uint32_t n_chunk
                                 uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                 uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                 const BlobOffsets& blobs, const XformDev& x, uint32_t wgs,
-                                hipStream_t stream) {
+                                uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   int v = 0;
   uint32_t part_shift = 0;
   // the scatter keeps its offsets until the stores: 8 slices per trip would not fit the registers
   if (sub_shift < 2 || !entries_shape(sub_shift, wgs, pack ? 8 : 4, &v, &part_shift)) return hipErrorInvalidValue;
   const dim3 grid(wgs), block(kThreads);
-#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x
+#define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x, tickets
   if (v == 8) {
     hipLaunchKernelGGL((xform_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);
   } else {

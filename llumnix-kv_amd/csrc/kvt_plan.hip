@@ -520,6 +520,33 @@ uint64_t kvt_plan_layer_bytes(const kvt_plan* p) { return p ? p->layer_bytes : 0
 
 }  // extern "C"
 
+namespace {
+// The ticket block of one pipelined launch (nullptr: none to be had, the launch strides).
+struct LaunchTickets {
+  int device;
+  bool capturing;
+  uint32_t* block;
+  LaunchTickets(int dev, bool cap, bool wanted = true)
+      : device(dev), capturing(cap), block(wanted ? ticket_pool().acquire(dev, cap) : nullptr) {}
+  // the launch is on the stream (or in the graph): eager blocks come back when it has run, a
+  // graph's block stays with the plan's table
+  void launched(const kvt_plan* p, hipStream_t s) {
+    if (!block) return;
+    if (!capturing) {
+      ticket_pool().launched(device, block, s);
+    } else if (p->buf) {
+      std::lock_guard<std::mutex> lock(p->buf->mu);
+      p->buf->graph_tickets.push_back(block);
+    }
+    block = nullptr;
+  }
+  // the launch failed: nothing will ever touch the block
+  ~LaunchTickets() {
+    if (block) ticket_pool().give_back(device, block);
+  }
+};
+}  // namespace
+
 int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t first_layer,
                   uint32_t n_layers, void* packed, uint64_t layer_stride, void* stream,
                   const uint64_t* blob_offsets) {
@@ -616,11 +643,15 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
     const uint32_t cus = device_cu_count(cache->device) & ~7u;
     if ((mis & 15u) == 0 && cus >= 8) {
       const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, cus));
+      // fewer workgroups than CUs: each has to move more than the ticket's barrier lets it
+      // (half the CUs: 4.4 against 5.3 TB/s)
+      LaunchTickets tickets(cache->device, capturing, wgs >= cus);
       const hipError_t e = launch_copy_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                                p->n_tensors, first_layer, n_layers,
                                                static_cast<uint8_t*>(packed), layer_stride, blobs,
-                                               wgs, s);
+                                               wgs, tickets.block, s);
       if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
+      tickets.launched(p, s);
       if (p->buf) {
         if (capturing) p->buf->captured = true;
         else if (int rc = p->buf->mark_use(s)) return rc;
@@ -628,15 +659,14 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       return KVT_OK;
     }
   }
-  // The same for strided, transposing and converting tables (16-byte vectors only), whose
-  // pipeline carries 5.4-5.9 TB/s whatever the share: from half the device on the strided loop
-  // of the chunk kernels is as fast or faster (5.6 / 5.7 TB/s on the TP2 -> TP1 batch), below
-  // that its rate falls with the share (a quarter: 4.4 / 4.2, an eighth: 2.5 / 2.4). The
-  // converting gather, with two loads and a conversion per store, gains at every share (half
-  // the device: 5.1 against 4.3 TB/s of bytes read and written).
+  // The same for strided, transposing and converting tables (16-byte vectors only). Measured
+  // against the strided loop of the chunk kernels (`for_items`), TB/s pack / unpack on the
+  // TP2 -> TP1 batch: half the device 5.9 / 5.9 against 5.8 / 5.9, a quarter 5.9 / 5.9 against
+  // 4.4 / 4.2, an eighth 5.9 / 5.8 against 2.5 / 2.4; the converting gather (bytes read and
+  // written) 5.9 against 4.3 at one half.
   const bool converting = p->convert && pack;
   const uint32_t min_shift = p->xform ? 2u : 1u;  // entries of at least 8 KiB (transposing: 16 KiB)
-  if (max_wgs != 0 && (converting || max_wgs < 4u * device_cu_count(cache->device)) && p->all16 && p->near &&
+  if (max_wgs != 0 && p->all16 && p->near &&
       (p->strided || p->xform || converting) && !words && p->sub_shift >= min_shift &&
       p->sub_shift <= 7 && cache->aligned16 && static_cast<uint64_t>(n) * n_layers > max_wgs) {
     uint64_t mis = reinterpret_cast<uintptr_t>(packed) | (n_layers > 1 ? layer_stride : 0);
@@ -647,17 +677,22 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       const uint32_t per_cu = p->sub_shift == 1 ? 2u : 1u;
       const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, per_cu * cus));
       uint8_t* const pk = static_cast<uint8_t*>(packed);
+      // trips of 8 KiB by a single workgroup per CU are better off without the ticket's barrier
+      // (converting gather at an eighth of the device: 4.4 against 5.1 TB/s), and so is a grid
+      // of fewer workgroups than CUs
+      LaunchTickets tickets(cache->device, capturing, wgs >= cus && (p->sub_shift >= 2 || wgs >= 2 * cus));
       const hipError_t e =
           converting ? launch_convert_entries(table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                               first_layer, n_layers, pk, layer_stride, blobs,
-                                              p->shapes, wgs, s)
+                                              p->shapes, wgs, tickets.block, s)
           : p->xform ? launch_xform_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                             p->n_tensors, first_layer, n_layers, pk, layer_stride,
-                                            blobs, p->xdev, wgs, s)
+                                            blobs, p->xdev, wgs, tickets.block, s)
                      : launch_strided_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                               p->n_tensors, first_layer, n_layers, pk, layer_stride,
-                                              blobs, p->shapes, wgs, s);
+                                              blobs, p->shapes, wgs, tickets.block, s);
       if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
+      tickets.launched(p, s);
       if (p->buf) {
         if (capturing) p->buf->captured = true;
         else if (int rc = p->buf->mark_use(s)) return rc;

@@ -63,6 +63,41 @@ struct DeviceGuard {
 
 inline uint64_t round_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
+// Ticket blocks of the persistent (CU-share limited) kernels: nine 32-bit counters, 128 bytes
+// apart, from which the workgroups of ONE launch take their work (kvt_kernels.hip, EntryWalk).
+// A block is all zero when a launch starts and the launch leaves it all zero, so the only rule
+// is that two launches that may run at the same time never share one. An eager launch borrows
+// a block until the event recorded behind it has completed; a launch recorded into a hipGraph
+// keeps its block for as long as the plan's table lives (every replay uses it again). The
+// blocks of a device are allocated in one piece when a CU share is first set for it -- never
+// during a launch, which may sit inside a stream capture -- and a launch that finds none free
+// runs without tickets (static striding), slower but as correct.
+class TicketPool {
+ public:
+  static constexpr uint32_t kBlockBytes = 2048, kBlocks = 1024;
+  // Allocates the device's blocks (no-op when they exist). Not inside a stream capture.
+  int prepare(int device);
+  // A block no running launch uses, or nullptr. permanent: taken out of circulation until
+  // give_back(); otherwise the caller calls launched() once the kernel is on `stream`.
+  uint32_t* acquire(int device, bool permanent);
+  void launched(int device, uint32_t* block, hipStream_t stream);
+  // A permanent block whose graph is gone, or a borrowed one whose launch never happened.
+  void give_back(int device, uint32_t* block);
+
+ private:
+  enum State : uint8_t { kFree = 0, kLent = 1, kInFlight = 2, kPermanent = 3 };  // kLent: event not recorded yet
+  struct PerDevice {
+    uint8_t* arena = nullptr;
+    std::vector<hipEvent_t> done;
+    std::vector<uint8_t> state;
+    uint32_t cursor = 0;
+  };
+  PerDevice* of(int device);  // under mu_
+  std::mutex mu_;
+  std::vector<PerDevice> devices_;
+};
+TicketPool& ticket_pool();
+
 // Chunk tables are uploaded once per batch and die with the batch. hipMalloc /
 // hipFree per batch would stall (hipFree waits for the whole device), so table
 // storage is recycled: a buffer = device memory + a pinned host twin of the same
@@ -82,6 +117,7 @@ struct TableBuf {
   std::mutex mu;          // a plan may be launched from several threads
   std::vector<Use> uses;  // events are kept across recycling (streams repeat)
   bool captured = false;  // read by a kernel recorded into a hipGraph
+  std::vector<uint32_t*> graph_tickets;  // ticket blocks of launches recorded into a hipGraph (under mu)
 
   // Call after every launch on `stream` that reads `dev`.
   int mark_use(hipStream_t stream) {
@@ -208,6 +244,8 @@ class TablePool {
   static constexpr size_t kMaxIdle = 4096;
   static constexpr size_t kMaxIdleBytes = size_t(256) << 20;  // device memory, and as much pinned
   static void destroy(TableBuf* b) {
+    for (uint32_t* t : b->graph_tickets) ticket_pool().give_back(b->device, t);
+    b->graph_tickets.clear();
     if (b->dev) (void)hipFree(b->dev);
     if (b->host) (void)hipHostFree(b->host);
     for (TableBuf::Use& u : b->uses) (void)hipEventDestroy(u.done);

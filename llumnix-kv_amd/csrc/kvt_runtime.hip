@@ -129,6 +129,89 @@ int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) 
   return KVT_OK;
 }
 
+TicketPool& ticket_pool() {
+  static TicketPool* pool = new TicketPool();  // intentionally leaked, like the table pool
+  return *pool;
+}
+
+TicketPool::PerDevice* TicketPool::of(int device) {
+  if (device < 0) return nullptr;
+  if (device >= static_cast<int>(devices_.size())) devices_.resize(device + 1);
+  return &devices_[device];
+}
+
+int TicketPool::prepare(int device) {
+  std::lock_guard<std::mutex> lock(mu_);
+  PerDevice* d = of(device);
+  if (!d) return fail(KVT_ERR_INVALID, "ticket pool: bad device");
+  if (d->arena) return KVT_OK;
+  DeviceGuard g;
+  if (int rc = g.enter(device)) return rc;
+  uint8_t* arena = nullptr;
+  KVT_HIP(hipMalloc(reinterpret_cast<void**>(&arena), static_cast<size_t>(kBlockBytes) * kBlocks));
+  const hipError_t e = hipMemset(arena, 0, static_cast<size_t>(kBlockBytes) * kBlocks);
+  if (e != hipSuccess) {
+    (void)hipFree(arena);
+    return hip_fail(e, "ticket pool: hipMemset");
+  }
+  d->done.assign(kBlocks, nullptr);
+  d->state.assign(kBlocks, kFree);
+  d->arena = arena;
+  return KVT_OK;
+}
+
+uint32_t* TicketPool::acquire(int device, bool permanent) {
+  std::lock_guard<std::mutex> lock(mu_);
+  PerDevice* d = of(device);
+  if (!d || !d->arena) return nullptr;
+  // a few probes from where the last search ended: blocks come free in the order they were lent
+  for (uint32_t probe = 0; probe < 32; ++probe) {
+    const uint32_t i = (d->cursor + probe) % kBlocks;
+    if (d->state[i] == kPermanent || d->state[i] == kLent) continue;
+    if (d->state[i] == kInFlight) {
+      if (hipEventQuery(d->done[i]) != hipSuccess) {
+        (void)hipGetLastError();
+        continue;
+      }
+      d->state[i] = kFree;
+    }
+    if (!permanent && !d->done[i] &&
+        hipEventCreateWithFlags(&d->done[i], hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      d->done[i] = nullptr;
+      return nullptr;
+    }
+    d->state[i] = permanent ? kPermanent : kLent;
+    d->cursor = (i + 1) % kBlocks;
+    return reinterpret_cast<uint32_t*>(d->arena + static_cast<size_t>(i) * kBlockBytes);
+  }
+  d->cursor = (d->cursor + 32) % kBlocks;
+  return nullptr;
+}
+
+void TicketPool::launched(int device, uint32_t* block, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(mu_);
+  PerDevice* d = of(device);
+  if (!d || !d->arena || !block) return;
+  const size_t i = (reinterpret_cast<uint8_t*>(block) - d->arena) / kBlockBytes;
+  // no event, no way to tell when the launch has ended: the block stays out of circulation
+  if (i >= kBlocks) return;
+  if (!d->done[i] || hipEventRecord(d->done[i], stream) != hipSuccess) {
+    (void)hipGetLastError();
+    d->state[i] = kPermanent;
+    return;
+  }
+  d->state[i] = kInFlight;
+}
+
+void TicketPool::give_back(int device, uint32_t* block) {
+  std::lock_guard<std::mutex> lock(mu_);
+  PerDevice* d = of(device);
+  if (!d || !d->arena || !block) return;
+  const size_t i = (reinterpret_cast<uint8_t*>(block) - d->arena) / kBlockBytes;
+  if (i < kBlocks && (d->state[i] == kPermanent || d->state[i] == kLent)) d->state[i] = kFree;
+}
+
 TablePool& table_pool() {
   static TablePool* pool = new TablePool();  // intentionally leaked: outlives static destruction
   return *pool;
@@ -161,6 +244,9 @@ int kvt_set_copy_cu_usage(int device, double usage) {
       const double wgs = usage * static_cast<double>(cus) * kWgsPerCu;
       cap = std::max<uint32_t>(8u, static_cast<uint32_t>(wgs) & ~7u);
     }
+    // the ticket blocks of the persistent kernels: allocated here, not inside a launch
+    if (cap != 0)
+      if (int rc = ticket_pool().prepare(device)) return rc;
     uint64_t bits = 0;
     std::memcpy(&bits, &usage, sizeof(bits));
     g_usage_bits[device].store(bits, std::memory_order_relaxed);

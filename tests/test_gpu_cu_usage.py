@@ -9,8 +9,10 @@ Needs a real MI355X."""
 import ctypes as C
 import math
 
+import numpy as np
 import pytest
 
+import checkers
 import kvt_amd
 import test_gpu_pack as tp
 import test_gpu_runs as tr
@@ -122,3 +124,28 @@ def test_pipelined_kernels_of_strided_transposing_and_converting_plans(usage, ch
             tp._transposing(w, plan=plan, lists=lists)
     finally:
         kvt_amd.set_copy_cu_usage(0, 1.0)
+
+
+def test_more_limited_launches_in_flight_than_ticket_blocks():
+    """A limited launch of the pipelined kernels borrows a block of counters until it has run.
+    Thousands of launches queued without a wait outnumber the blocks: those that find none run
+    without (every workgroup a fixed share), and every result is still the oracle's."""
+    w = workloads.llama8b_single(n_layers=4, pool=256, tokens=2048)
+    plan, lists = pipeline.build_plan(w, 0)
+    o_lists = tp._oracle_lists(w)
+    src_layers = tp._make_caches(w, "src", 17)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    stride = plan.layer_bytes
+    outs = [torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda") for _ in range(3)]
+    kvt_amd.set_copy_cu_usage(0, 0.004)
+    try:
+        stream = torch.cuda.Stream()
+        for i in range(3000):
+            plan.pack(sc, 0, w.n_layers, outs[i % 3], stride, stream.cuda_stream)
+        stream.synchronize()
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+    for l in range(w.n_layers):
+        blob = checkers.oracle_pack(tp._host(src_layers[l][0]), o_lists[0])
+        for out in outs:
+            assert np.array_equal(tp._host(out)[l * stride:l * stride + len(blob)], blob), l
