@@ -857,13 +857,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "d18bcfc9f6ecfa57dd4e938f52f8c7e255c03a3bacd6af9f527558aa05a0a750"
+KERNELS_SHA256 = "db41ff18da04b93088f3de4996eed7a082903e7c2f3db384905183921bff428e"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134272222, "unpack": 134275422},
-    (2, "ranges"): {"pack": 71013037920, "unpack": 73358402624},
-    (3, "ranges"): {"pack": 85983098765, "unpack": 85983588532},
-    (4, "ranges"): {"pack": 22690334162, "unpack": 22690387367},
-    (5, "ranges"): {"pack": 45141187873, "unpack": 45141390581},
+    (1, "ranges"): {"pack": 134278584, "unpack": 134277773},
+    (2, "ranges"): {"pack": 71012999691, "unpack": 73358406988},
+    (3, "ranges"): {"pack": 85983087420, "unpack": 85983592419},
+    (4, "ranges"): {"pack": 22690386598, "unpack": 22690441296},
+    (5, "ranges"): {"pack": 45141195491, "unpack": 45141395554},
 }
 
 

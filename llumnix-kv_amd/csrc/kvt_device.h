@@ -58,7 +58,8 @@ struct StrideTable {
 // max_wgs > 0: at most that many workgroups (a multiple of 8), striding over the same items,
 // for a caller that wants the copy to leave part of the device to other kernels.
 // temporal: plain instead of non-temporal loads, for a launch whose data may sit in the
-// memory-side cache (ignored by a capped launch). pipelined (launch_copy_chunks): a capped
+// memory-side cache (ignored by a capped launch). tickets: a capped launch's block of counters
+// (see launch_copy_entries), or nullptr; an uncapped launch ignores it and leaves it untouched. pipelined (launch_copy_chunks): a capped
 // launch keeps the loads of its next trip in flight across the stores of the last one; for
 // grids of at most 4 workgroups per CU (the kernel then needs more registers than 8 per CU fit).
 hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
@@ -66,14 +67,15 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
                                  const StrideTable& shapes, bool words, uint32_t max_wgs, bool temporal,
-                                 hipStream_t stream);
+                                 uint32_t* tickets, hipStream_t stream);
 // Converting gather (bf16 -> fp8 E4M3) of a chunk table, plain and strided chunks alike; lengths
 // and packed positions count fp8 bytes, cache offsets and strides bytes of the bf16 cache.
 hipError_t launch_convert_chunks(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                  uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                  uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                  uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, uint32_t max_wgs, hipStream_t stream);
+                                 const StrideTable& shapes, uint32_t max_wgs, uint32_t* tickets,
+                                 hipStream_t stream);
 // A table of at most kSmallTable entries travels in the kernel arguments (2 KiB): a short
 // request then needs no table upload, no upload event and no cross-stream wait before its
 // first launch.
@@ -86,12 +88,12 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
                                     const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
-                                    hipStream_t stream);
+                                    uint32_t* tickets, hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                               uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
-                              bool temporal, hipStream_t stream);
+                              bool temporal, uint32_t* tickets, hipStream_t stream);
 // The capped launch of a plain table with 16-byte aligned entries of at most 16 KiB
 // (sub_shift 2) or 32 KiB (sub_shift 3): `wgs` persistent workgroups (a multiple of 8), one
 // table entry per trip, software-pipelined. Every address and length involved must be a
@@ -128,7 +130,7 @@ hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               uint32_t max_wgs, bool temporal, hipStream_t stream);
+                               uint32_t max_wgs, bool temporal, uint32_t* tickets, hipStream_t stream);
 // rows = workgroups striding over the 4 KiB slices of each range
 hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                               const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,

@@ -114,6 +114,86 @@ __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst,
 // loads back to back; the stores of a trip are issued only after the loads of the next one
 // (three register sets in rotation), so a lane has up to 2 x kBatch x 16 bytes in flight.
 
+// This workgroup's way through the (item, layer) pairs of a launch: the items of a layer are
+// dealt to the XCDs in eighths. Without tickets a workgroup strides through its XCD's pairs by
+// the number of workgroups there. With tickets (eight counters, one per XCD, 128 bytes apart,
+// zero at the start of the launch) it takes whatever pair is next on its XCD: workgroups that
+// fall behind no longer spread the addresses in flight over a widening window, which is worth
+// 16 % on a plain 4 GiB copy by 256 persistent workgroups (5.5 -> 6.4 TB/s). The last
+// workgroup to leave zeroes the counters again (kTicketDone counts the leavers).
+constexpr uint32_t kTicketStride = 32, kTicketDone = 8 * kTicketStride;  // in 32-bit words
+// log2 of the 4 KiB slices one ticket stands for: 32 KiB. Finer tickets run into the rate at
+// which one counter can be bumped (16 KiB entries, one per ticket: 11 % slower than without
+// tickets), coarser ones give the order away again (64 / 128 KiB: -6 / -9 % on config 2).
+constexpr uint32_t kTicketSlicesLog2 = 3;
+struct EntryWalk {
+  uint32_t n_items, n_layers, per8, xcd, step_layer, step_within, layer, within;
+  uint32_t* tickets;
+  uint32_t run_shift;  // a ticket stands for 1 << run_shift consecutive pairs
+  uint32_t pair, left; // tickets: the next pair of the current run, and how many of it are left
+  uint32_t turn;       // which LDS word carries the next ticket
+  uint32_t ahead;      // lane 0: the ticket of the next run, asked for one run early
+  // slices_log2: log2 of the 4 KiB slices one item holds
+  __device__ __forceinline__ EntryWalk(uint32_t items, uint32_t layers, uint32_t* ticket_block, uint32_t slices_log2)
+      : n_items(items), n_layers(layers), tickets(ticket_block), pair(0), left(0), turn(0), ahead(0) {
+    per8 = (n_items + 7u) >> 3;
+    xcd = blockIdx.x & 7u;
+    run_shift = slices_log2 < kTicketSlicesLog2 ? kTicketSlicesLog2 - slices_log2 : 0u;
+    if (tickets && threadIdx.x == 0) ahead = atomicAdd(tickets + xcd * kTicketStride, 1u);
+    const uint32_t nloc = gridDim.x >> 3;  // workgroups per XCD
+    step_layer = nloc / per8;
+    step_within = nloc - step_layer * per8;
+    layer = (blockIdx.x >> 3) / per8;
+    within = (blockIdx.x >> 3) - layer * per8;
+  }
+  // The next pair, clamped to the last one past the end (`valid` false: nothing to move there);
+  // returns false once the workgroup is past the last layer. A ticket travels from lane 0 to
+  // the workgroup through one of two LDS words in turn: lane 0 cannot write a word again
+  // before every wavefront has passed the barrier behind the other one, i.e. has read it.
+  __device__ __forceinline__ bool next(uint32_t& item, uint32_t& lay, bool& valid) {
+    if (tickets) {
+      if (left == 0) {
+        __shared__ uint32_t slot[2];
+        if (threadIdx.x == 0) {
+          slot[turn] = ahead;
+          ahead = atomicAdd(tickets + xcd * kTicketStride, 1u);
+        }
+        __syncthreads();
+        pair = __builtin_amdgcn_readfirstlane(slot[turn]) << run_shift;
+        left = 1u << run_shift;
+        turn ^= 1u;
+      }
+      layer = pair / per8;
+      within = pair - layer * per8;
+      ++pair;
+      --left;
+    }
+    const bool live = layer < n_layers;
+    const uint32_t b = xcd * per8 + within;
+    valid = live && b < n_items;
+    lay = min(layer, n_layers - 1u);
+    item = min(b, n_items - 1u);
+    if (!tickets) {
+      within += step_within;
+      layer += step_layer;
+      const bool wrap = within >= per8;
+      within -= wrap ? per8 : 0u;
+      layer += wrap ? 1u : 0u;
+    }
+    return live;
+  }
+  // Call once, when next() has returned false.
+  __device__ __forceinline__ void leave() {
+    if (!tickets || threadIdx.x != 0) return;
+    asm volatile("" ::"v"(ahead));  // the last ticket asked for has been handed out: it came back
+    if (atomicAdd(tickets + kTicketDone, 1u) == gridDim.x - 1u) {
+#pragma unroll
+      for (uint32_t x = 0; x < 8; ++x) atomicExch(tickets + x * kTicketStride, 0u);
+      atomicExch(tickets + kTicketDone, 0u);
+    }
+  }
+};
+
 // Three register sets in rotation: the loads of item k+1 are issued before the stores of item k,
 // and a set is loaded again only two trips after its stores were issued.
 #define KVT_ROTATE3(NEXT, LOAD, STORE) \
@@ -153,6 +233,7 @@ struct Launch {
   uint64_t layer_stride;
   const BlobOffsets* blobs;
   bool temporal;  // plain instead of non-temporal loads (bit 8 of the sub_shift argument)
+  uint32_t* tickets;  // a capped launch: its block of counters, or nullptr (EntryWalk)
 };
 
 // A table entry as the kernels read it: the Chunk's two 16-bit fields as one word (a 16-bit
@@ -256,9 +337,9 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch_table, Pl
   }
   // lanes without a vector load from here: the layer pointer table, at least 16 bytes long
   const uint8_t* const idle = reinterpret_cast<const uint8_t*>(L.layer_ptrs);
-  const uint32_t per_layer = (L.n_slices + 7u) & ~7u;
-  const uint32_t d_layer = gridDim.x / per_layer, d_slice = gridDim.x - d_layer * per_layer;
-  uint32_t layer = blockIdx.x / per_layer, s = blockIdx.x - layer * per_layer;
+  // the (slice, layer) pairs of this workgroup, one 4 KiB slice each: strided by the grid, or
+  // in runs of eight neighbouring slices by ticket
+  EntryWalk walk(L.n_slices, L.n_layers, L.tickets, 0);
   // kStriding: a trip loads kBatch vectors and stores them. kPipelined: three sets of kBatch
   // vectors in rotation (KVT_ROTATE3), the loads of the next kBatch items in flight before the
   // stores of the last ones are issued. What a set keeps until its stores is each vector's
@@ -266,24 +347,17 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch_table, Pl
   uint8_t* dst[3][kBatch];
   u32x4 r[3][kBatch];
   auto fetch = [&](int k) -> bool {
-    const bool live = layer < L.n_layers;
+    bool live = false;
     Item it[kBatch];
     uint32_t lay[kBatch];
     bool valid[kBatch];
 #pragma unroll
     for (int j = 0; j < kBatch; ++j) {  // which items, and their table entries
-      const uint32_t b = xcd_remap(s, L.n_slices);
-      valid[j] = layer < L.n_layers && b < L.n_slices;
-      lay[j] = min(layer, L.n_layers - 1u);
-      const uint32_t bc = min(b, L.n_slices - 1u);
+      uint32_t bc;
+      const bool more = walk.next(bc, lay[j], valid[j]);
+      if (j == 0) live = more;
       it[j].c = entry_of(fetch_table(bc >> L.sub_shift));
       it[j].sub = bc & ((1u << L.sub_shift) - 1u);
-      s += d_slice;
-      layer += d_layer;
-      if (s >= per_layer) {
-        s -= per_layer;
-        ++layer;
-      }
     }
 #pragma unroll
     for (int j = 0; j < kBatch; ++j) {  // their layer tensors
@@ -312,9 +386,10 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch_table, Pl
   };
   if (MODE == kStriding) {
     while (fetch(0)) store(0);
-    return;
+  } else {
+    KVT_ROTATE3(fetch, nothing, store);
   }
-  KVT_ROTATE3(fetch, nothing, store);
+  walk.leave();
 }
 
 // The lane's share of one contiguous slice: `on` when the slice is 16-byte aligned on both
@@ -343,14 +418,15 @@ __device__ __forceinline__ Move plain_move(const Item& it) {
 
 #define KVT_LAUNCH_STRUCT \
   const Launch L{n_slices, sub_shift & 0xFFu, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, &blobs, \
-                 (sub_shift & kTemporalFlag) != 0}
+                 (sub_shift & kTemporalFlag) != 0, tickets}
 
 // Gather (PACK) / scatter of a resident chunk table.
 template <bool PACK, int MODE>
 __global__ __launch_bounds__(kThreads, MODE == kPipelined ? 4 : 8) void copy_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    uint32_t* tickets) {
   KVT_LAUNCH_STRUCT;
   for_items<MODE>(L, [&](uint32_t e) { return fetch_entry(chunks, e); },
                   [&](const Item& it) { return plain_move<PACK>(it); });
@@ -362,7 +438,8 @@ template <bool PACK, bool CAPPED>
 __global__ __launch_bounds__(kThreads, 8) void copy_chunks_small_kernel(
     const SmallTable table, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs) {
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    uint32_t* tickets) {
   KVT_LAUNCH_STRUCT;
   for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(table.c, e); },
                     [&](const Item& it) { return plain_move<PACK>(it); });
@@ -387,83 +464,6 @@ __device__ __forceinline__ rsrc_t make_rsrc(const uint8_t* base, uint32_t bytes)
 // cache-policy operand of the buffer builtins: bit 0 = sc0, bit 1 = nt, bit 4 = sc1
 constexpr int kLoadPolicy = 2, kStorePolicy = 1 | 2 | 16;
 
-// This workgroup's way through the (item, layer) pairs of a launch: the items of a layer are
-// dealt to the XCDs in eighths. Without tickets a workgroup strides through its XCD's pairs by
-// the number of workgroups there. With tickets (eight counters, one per XCD, 128 bytes apart,
-// zero at the start of the launch) it takes whatever pair is next on its XCD: workgroups that
-// fall behind no longer spread the addresses in flight over a widening window, which is worth
-// 16 % on a plain 4 GiB copy by 256 persistent workgroups (5.5 -> 6.4 TB/s). The last
-// workgroup to leave zeroes the counters again (kTicketDone counts the leavers).
-constexpr uint32_t kTicketStride = 32, kTicketDone = 8 * kTicketStride;  // in 32-bit words
-// log2 of the 4 KiB slices one ticket stands for: 32 KiB. Finer tickets run into the rate at
-// which one counter can be bumped (16 KiB entries, one per ticket: 11 % slower than without
-// tickets), coarser ones give the order away again (64 / 128 KiB: -6 / -9 % on config 2).
-constexpr uint32_t kTicketSlicesLog2 = 3;
-struct EntryWalk {
-  uint32_t n_items, n_layers, per8, xcd, step_layer, step_within, layer, within;
-  uint32_t* tickets;
-  uint32_t run_shift;  // a ticket stands for 1 << run_shift consecutive pairs
-  uint32_t pair, left; // tickets: the next pair of the current run, and how many of it are left
-  uint32_t ahead;      // lane 0: the ticket of the next run, asked for one run early
-  // slices_log2: log2 of the 4 KiB slices one item holds
-  __device__ __forceinline__ EntryWalk(uint32_t items, uint32_t layers, uint32_t* ticket_block, uint32_t slices_log2)
-      : n_items(items), n_layers(layers), tickets(ticket_block), pair(0), left(0), ahead(0) {
-    per8 = (n_items + 7u) >> 3;
-    xcd = blockIdx.x & 7u;
-    run_shift = slices_log2 < kTicketSlicesLog2 ? kTicketSlicesLog2 - slices_log2 : 0u;
-    if (tickets && threadIdx.x == 0) ahead = atomicAdd(tickets + xcd * kTicketStride, 1u);
-    const uint32_t nloc = gridDim.x >> 3;  // workgroups per XCD
-    step_layer = nloc / per8;
-    step_within = nloc - step_layer * per8;
-    layer = (blockIdx.x >> 3) / per8;
-    within = (blockIdx.x >> 3) - layer * per8;
-  }
-  // The next pair, clamped to the last one past the end (`valid` false: nothing to move there);
-  // returns false once the workgroup is past the last layer. `k`: which of three slots carries
-  // the ticket from lane 0 to the workgroup (a wavefront is at most one barrier behind).
-  __device__ __forceinline__ bool next(int k, uint32_t& item, uint32_t& lay, bool& valid) {
-    if (tickets) {
-      if (left == 0) {
-        __shared__ uint32_t slot[3];
-        if (threadIdx.x == 0) {
-          slot[k] = ahead;
-          ahead = atomicAdd(tickets + xcd * kTicketStride, 1u);
-        }
-        __syncthreads();
-        pair = __builtin_amdgcn_readfirstlane(slot[k]) << run_shift;
-        left = 1u << run_shift;
-      }
-      layer = pair / per8;
-      within = pair - layer * per8;
-      ++pair;
-      --left;
-    }
-    const bool live = layer < n_layers;
-    const uint32_t b = xcd * per8 + within;
-    valid = live && b < n_items;
-    lay = min(layer, n_layers - 1u);
-    item = min(b, n_items - 1u);
-    if (!tickets) {
-      within += step_within;
-      layer += step_layer;
-      const bool wrap = within >= per8;
-      within -= wrap ? per8 : 0u;
-      layer += wrap ? 1u : 0u;
-    }
-    return live;
-  }
-  // Call once, when next() has returned false.
-  __device__ __forceinline__ void leave() {
-    if (!tickets || threadIdx.x != 0) return;
-    asm volatile("" ::"v"(ahead));  // the last ticket asked for has been handed out: it came back
-    if (atomicAdd(tickets + kTicketDone, 1u) == gridDim.x - 1u) {
-#pragma unroll
-      for (uint32_t x = 0; x < 8; ++x) atomicExch(tickets + x * kTicketStride, 0u);
-      atomicExch(tickets + kTicketDone, 0u);
-    }
-  }
-};
-
 template <bool PACK, int V>
 __global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks,
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
   auto next = [&](int k) -> bool {
     uint32_t item, lay;
     bool valid;
-    const bool live = walk.next(k, item, lay, valid);
+    const bool live = walk.next(item, lay, valid);
     const Entry c = table[item];
     uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
     uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed;
@@ -528,7 +528,7 @@ __device__ __forceinline__ void entries_pipeline(
   auto next = [&](int k) -> bool {
     uint32_t item, lay;
     bool valid;
-    const bool live = walk.next(k, item, lay, valid);
+    const bool live = walk.next(item, lay, valid);
     const Entry c = table[item >> part_shift];
     const uint32_t begin = (item & ((1u << part_shift) - 1u)) * (static_cast<uint32_t>(V) << kSliceShift);
     uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
@@ -636,7 +636,7 @@ __global__ __launch_bounds__(kThreads, 8) void strided_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    StrideTable shapes) {
+    StrideTable shapes, uint32_t* tickets) {
   KVT_LAUNCH_STRUCT;
   for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     if (it.c.shape == 0) return plain_move<PACK>(it);
@@ -685,7 +685,7 @@ __global__ __launch_bounds__(kThreads, 8) void xform_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    XformDev x) {
+    XformDev x, uint32_t* tickets) {
   KVT_LAUNCH_STRUCT;
   for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(chunks, e); }, [&](const Item& it) -> Move {
     const uint32_t v = (it.sub << 8) + threadIdx.x;  // 256 vectors per slice
@@ -810,7 +810,7 @@ __global__ __launch_bounds__(kThreads, 8) void convert_chunks_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    StrideTable shapes) {
+    StrideTable shapes, uint32_t* tickets) {
   KVT_LAUNCH_STRUCT;
   // a conversion between load and store: `place` moves everything itself. A slice is 4096
   // elements = 512 groups of 8 (16 bytes in, 8 bytes out); lane t takes groups t and t + 256, so
@@ -894,7 +894,7 @@ __global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
   auto next = [&](int k, uint32_t* coff) -> bool {
     uint32_t item, lay;
     bool valid;
-    const bool live = walk.next(k, item, lay, valid);
+    const bool live = walk.next(item, lay, valid);
     const Entry c = table[item >> part_shift];
     const uint32_t begin = (item & ((1u << part_shift) - 1u)) * (static_cast<uint32_t>(V) << kSliceShift);
     uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
@@ -983,12 +983,13 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                               uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
-                              bool temporal, hipStream_t stream) {
+                              bool temporal, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+  if (!g.capped) tickets = nullptr;
   const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
-#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
   if (!g.capped) {
     if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, kOnePerSlice>), KVT_ARGS);
     else KVT_LAUNCH_CHUNKS((copy_chunks_kernel<false, kOnePerSlice>), KVT_ARGS);
@@ -1099,12 +1100,13 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
                                     const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
-                                    hipStream_t stream) {
+                                    uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+  if (!g.capped) tickets = nullptr;
   const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
-#define KVT_ARGS table, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+#define KVT_ARGS table, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
   if (pack && !g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, false>), KVT_ARGS);
   else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, true>), KVT_ARGS);
   else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, false>), KVT_ARGS);
@@ -1118,12 +1120,13 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
                                  const StrideTable& shapes, bool words, uint32_t max_wgs, bool temporal,
-                                 hipStream_t stream) {
+                                 uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+  if (!g.capped) tickets = nullptr;
   const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
-#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets
 #define KVT_STRIDED(P, W)                                                                       \
   do {                                                                                          \
     if (g.capped) KVT_LAUNCH_CHUNKS((strided_chunks_kernel<P, W, true>), KVT_ARGS);             \
@@ -1142,12 +1145,13 @@ hipError_t launch_convert_chunks(const Chunk* chunks, uint32_t n_chunks, uint32_
                                  uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                  uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                  uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, uint32_t max_wgs,
+                                 const StrideTable& shapes, uint32_t max_wgs, uint32_t* tickets,
                                  hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
-#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes
+  if (!g.capped) tickets = nullptr;
+#define KVT_ARGS chunks, n_slices, sub_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets
   if (g.capped) KVT_LAUNCH_CHUNKS((convert_chunks_kernel<true>), KVT_ARGS);
   else KVT_LAUNCH_CHUNKS((convert_chunks_kernel<false>), KVT_ARGS);
 #undef KVT_ARGS
@@ -1158,12 +1162,13 @@ hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               uint32_t max_wgs, bool temporal, hipStream_t stream) {
+                               uint32_t max_wgs, bool temporal, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
+  if (!g.capped) tickets = nullptr;
   const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
-#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x
+#define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x, tickets
   if (pack && !g.capped) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, false>), KVT_ARGS);
   else if (pack) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, true>), KVT_ARGS);
   else if (!g.capped) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<false, false>), KVT_ARGS);

@@ -612,7 +612,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
     const hipError_t e = launch_copy_chunks_small(
         pack, pack ? p->small_pack : p->small_unpack, static_cast<uint32_t>(p->n_chunks),
         p->sub_shift, cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
-        static_cast<uint8_t*>(packed), layer_stride, blobs, max_wgs, temporal, s);
+        static_cast<uint8_t*>(packed), layer_stride, blobs, max_wgs, temporal, nullptr, s);
     if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
     return KVT_OK;
   }
@@ -700,22 +700,31 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       return KVT_OK;
     }
   }
+  // A launch that ends up capped (more (slice, layer) pairs than the limit) and has at least
+  // two workgroups per CU takes its slices by ticket, eight neighbours at a time (config 4,
+  // TB/s pack / unpack: half the device 5.6 / 5.5 -> 5.9 / 5.7, a quarter 5.2 / 5.2 ->
+  // 5.7 / 5.1; with one workgroup per CU the ticket's barrier costs more than the order
+  // brings, 4.4 / 3.4 -> 3.8 / 3.1).
+  const uint32_t grid_cap = max_wgs == 0 ? 0u : std::max(8u, max_wgs & ~7u);
+  const uint64_t pairs = ((static_cast<uint64_t>(n) << p->sub_shift) + 7u) / 8u * 8u * n_layers;
+  const uint32_t n_cus = device_cu_count(cache->device);
+  LaunchTickets tickets(cache->device, capturing, grid_cap != 0 && pairs > grid_cap && n_cus != 0 && grid_cap >= 2 * n_cus);
+  uint8_t* const pk8 = static_cast<uint8_t*>(packed);
   const hipError_t e =
       p->convert && pack ? launch_convert_chunks(table, n, p->sub_shift, cache->dev_ptrs,
-                                                 p->n_tensors, first_layer, n_layers,
-                                                 static_cast<uint8_t*>(packed), layer_stride,
-                                                 blobs, p->shapes, max_wgs, s) :
+                                                 p->n_tensors, first_layer, n_layers, pk8,
+                                                 layer_stride, blobs, p->shapes, max_wgs,
+                                                 tickets.block, s) :
       p->strided ? launch_strided_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs,
-                                         p->n_tensors, first_layer, n_layers,
-                                         static_cast<uint8_t*>(packed), layer_stride, blobs,
-                                         p->shapes, words, max_wgs, temporal, s) :
+                                         p->n_tensors, first_layer, n_layers, pk8, layer_stride,
+                                         blobs, p->shapes, words, max_wgs, temporal, tickets.block, s) :
       p->xform ? launch_xform_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
-                                     first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                     layer_stride, blobs, p->xdev, max_wgs, temporal, s)
+                                     first_layer, n_layers, pk8, layer_stride, blobs, p->xdev,
+                                     max_wgs, temporal, tickets.block, s)
                : launch_copy_chunks(pack, table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
-                                    first_layer, n_layers, static_cast<uint8_t*>(packed),
-                                    layer_stride, blobs, max_wgs,
-                                    max_wgs < 4u * device_cu_count(cache->device), temporal, s);
+                                    first_layer, n_layers, pk8, layer_stride, blobs, max_wgs,
+                                    max_wgs < 4u * n_cus, temporal, tickets.block, s);
+  if (e == hipSuccess) tickets.launched(p, s);
   if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
   if (p->buf) {
     // remember when the table is last read, so that its storage is not recycled too early
