@@ -388,7 +388,12 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
  * workgroups, rounded down to a multiple of 8 and at least 8, that stride over the same
  * work; results are identical. Takes effect for launches issued after the call (a launch
  * captured into a graph keeps the shape it was captured with). Passing num_wg > 0 to a
- * launcher still bounds that launch further. */
+ * launcher still bounds that launch further.
+ * The first call with usage < 1 for a device allocates 2 MiB of device memory there (blocks
+ * of counters from which the persistent workgroups of a launch take their work in order; a
+ * launch borrows one until it has run, a launch recorded into a hipGraph keeps one until its
+ * plan is destroyed): call it at start-up, not inside a stream capture. A graph that holds
+ * limited launches must not run at the same time as a second instantiation of itself. */
 int kvt_set_copy_cu_usage(int device, double usage);
 /* The current setting and the workgroup limit it stands for (0 = none); either may be NULL. */
 int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
