@@ -995,6 +995,8 @@ def run_config(args, headline):
             first[i][0].pack(sides[i].src_cache, 0, wls[i].n_layers, packed[i], strides[i], sh)
     keep = [first]
     plans = first
+    if args.cu_usage < 1.0:
+        kvt.set_copy_cu_usage(0, args.cu_usage)
     for _ in range(args.warmup):
         launch(plans, [new_event() for _ in range(3)])
         plans = [prepare(i) for i in range(len(wls))]
@@ -1023,6 +1025,7 @@ def run_config(args, headline):
         host_ms.append((time.perf_counter() - h0) * 1e3)
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    kvt.set_copy_cu_usage(0, 1.0)
     ms_per_step = wall / args.steps * 1e3
     pack_ms = [ev_ms(lib, e[0], e[1]) for e in events]
     unpack_ms = [ev_ms(lib, e[1], e[2]) for e in events]
@@ -1061,6 +1064,7 @@ def run_config(args, headline):
                    "scale": args.scale, "layers": [w.n_layers for w in wls],
                    "requests": [len(w.tasks) for w in wls], "payload_bytes_per_step": P,
                    "chunk_bytes": args.chunk_bytes or "auto", "plan": args.plan,
+                   "cu_usage": args.cu_usage,
                    "table_entries_per_layer": [p.num_chunks for p, _ in first]},
         "frac_hbm_peak": round(value * 1e9 / HBM_PEAK, 4),
         "pack_ms": round(pack_avg, 4),
@@ -1145,6 +1149,9 @@ def main():
     ap.add_argument("--cpu-layers", type=int, default=16,
                     help="layers in the CPU baseline sample (16 layers x 5 passes of config 2 are "
                          "about 10 s of single-thread CPU work)")
+    ap.add_argument("--cu-usage", type=float, default=1.0,
+                    help="limit the timed pack / unpack launches to this share of the device "
+                         "(kvt_set_copy_cu_usage; the reference's BLLM_KVTRANS_KERNEL_COPY_SM_USAGE)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
     ap.add_argument("--calibrate-copy-gib", type=float, default=0.0,
