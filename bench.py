@@ -414,7 +414,7 @@ def leg_cu_usage(c, out):
     pay0 = sum(plan0.tensor_bytes(t) for t in range(w.n_tensors)) * w.n_layers
     rows = []
     try:
-        for usage in (1.0, 0.5, 0.25, 0.125, 0.0625):
+        for usage in (1.0, 0.5, 0.25, 0.125, 0.0625) if c.headline else (1.0, 0.5, 0.125):
             kvt.set_copy_cu_usage(0, usage)
             e = [new_event() for _ in range(3)]
             for rep in range(2):   # second run is the measurement
@@ -1086,14 +1086,14 @@ def run_config(args, headline):
                               wls=wls, sides=sides, full_wls=full_wls, full_sides=full_sides,
                               mixed=mixed, infos=infos, tasks=tasks, first=first, strides=strides,
                               packed=packed, stream=stream, sh=sh, new_event=new_event, keep=keep,
-                              senders=senders, keep_objs=keep_objs)
+                              senders=senders, keep_objs=keep_objs, headline=headline)
     # The timed region is over: a failure in a side leg must not take the measured line with
     # it. It is reported in "errors" (and on stderr, with the traceback) and fails the run.
     legs = [] if args.skip_cpu else [leg_cpu]
     if not args.skip_extras:
-        legs += [leg_latency, leg_staging]
+        legs += [leg_latency, leg_staging, leg_cu_usage]
         if headline:
-            legs += [leg_session, leg_cu_usage, leg_copy_ceilings, leg_launchers, leg_fp8_plan,
+            legs += [leg_session, leg_copy_ceilings, leg_launchers, leg_fp8_plan,
                      leg_frames, leg_store_objects]
     errors = {}
     for leg in legs:
@@ -1217,7 +1217,7 @@ def main():
             for key in ("value", "ms_per_step", "pack_gbps", "unpack_gbps", "pack_ms", "unpack_ms",
                         "frac_hbm_peak", "host_parse_plan_ms", "mode", "parity_vs_oracle",
                         "latency_p50_us", "latency_wall_p50_us", "latency_single_launch_p50_us",
-                        "latency_after_last_layer_p50_us",
+                        "latency_after_last_layer_p50_us", "cu_usage",
                         "staging", "roofline", "cpu_baseline", "errors"):
                 if key in r:
                     row[key] = r[key]
