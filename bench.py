@@ -273,7 +273,7 @@ def leg_latency(c, out):
     strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
     w, side = wls[0], sides[0]
     sender = c.senders[0]
-    single, gated, wall, tail = [], [], [], []
+    single, gated, wall, tail, grouped = [], [], [], [], []
     fill = [torch.zeros(256 << 20, dtype=torch.uint8, device="cuda") for _ in range(2)]
     reqs = list(range(len(w.tasks)))
     if len(reqs) < 5:                  # a single-request configuration: the same request again
@@ -323,6 +323,15 @@ def leg_latency(c, out):
         sess.wait_layer(w.n_layers - 1, step)
         lib.kvt_event_synchronize(b)
         tail.append(ev_ms(lib, a, b) * 1e3)
+        # the gated sequence again with one hop per group of four layers
+        step = sess.begin_step()
+        lib.kvt_event_record(a, sh)
+        for l in range(0, w.n_layers, 4):
+            sess.save_layers(l, min(4, w.n_layers - l), sh)
+        lib.kvt_event_record(b, sess.side_stream)
+        sess.wait_layer(w.n_layers - 1, step)
+        lib.kvt_event_synchronize(b)
+        grouped.append(ev_ms(lib, a, b) * 1e3)
         for rep in range(2):   # second run is the measurement
             lib.kvt_event_record(a, sh)
             plan.pack(side.src_cache, 0, w.n_layers, packed[0], plan.layer_bytes, sh)
@@ -334,12 +343,15 @@ def leg_latency(c, out):
     c.keep_objs.append(held)
     out["latency_p50_us"] = round(statistics.median(gated), 2)
     out["latency_wall_p50_us"] = round(statistics.median(wall), 2)
+    out["latency_groups_of_4_layers_p50_us"] = round(statistics.median(grouped), 2)
     out["latency_single_launch_p50_us"] = round(statistics.median(single), 2)
     out["latency_after_last_layer_p50_us"] = round(statistics.median(tail), 2)
     del fill
     out["latency_note"] = ("per request (%d timed): latency_p50_us = GPU time from the first "
                            "pack launch of layer 0 to the completion of layer %d on the side "
-                           "stream, one event-gated launch per layer; latency_wall_p50_us = host "
+                           "stream, one event-gated launch per layer "
+                           "(latency_groups_of_4_layers_p50_us: per four layers, "
+                           "kvt_session_save_layers); latency_wall_p50_us = host "
                            "clock from before ParseBlock (plan built cold) until the wait for the "
                            "last layer returns; latency_single_launch_p50_us = one warm launch "
                            "covering all layers; latency_after_last_layer_p50_us = the gated "
@@ -1217,6 +1229,7 @@ def main():
             for key in ("value", "ms_per_step", "pack_gbps", "unpack_gbps", "pack_ms", "unpack_ms",
                         "frac_hbm_peak", "host_parse_plan_ms", "mode", "parity_vs_oracle",
                         "latency_p50_us", "latency_wall_p50_us", "latency_single_launch_p50_us",
+                        "latency_groups_of_4_layers_p50_us",
                         "latency_after_last_layer_p50_us", "cu_usage",
                         "staging", "roofline", "cpu_baseline", "errors"):
                 if key in r:

@@ -66,13 +66,15 @@ struct kvt_stager {
 
 namespace {
 
-// One lane: this layer's completion count, bumped in device memory and mirrored to the host.
-// The pack kernel in front of it on the stream has ended, so its stores have left the caches.
-__global__ void publish_layer_kernel(uint32_t* count_dev, uint32_t* count_host) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  const uint32_t c = *count_dev + 1u;
-  *count_dev = c;
-  __hip_atomic_store(count_host, c, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+// One lane per layer: the layer's completion count, bumped in device memory and mirrored to
+// the host. The pack kernel in front of it on the stream has ended, so its stores have left
+// the caches.
+__global__ void publish_layers_kernel(uint32_t* count_dev, uint32_t* count_host, uint32_t n) {
+  for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+    const uint32_t c = count_dev[i] + 1u;
+    count_dev[i] = c;
+    __hip_atomic_store(count_host + i, c, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+  }
 }
 
 // Starts a new step under s->mu. Layers whose pack lives in a captured graph are counted as
@@ -211,19 +213,19 @@ int kvt_session_begin_step(kvt_session* s, uint64_t* step) {
   });
 }
 
-// The pack of `layer` on the side stream, gated by `ready` (already recorded), and the
-// publication of its completion.
-static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
+// The pack of layers [first, first + n) on the side stream as ONE launch, gated by `ready`
+// (already recorded), and the publication of their completion.
+static int issue_layers(kvt_session* s, uint32_t first, uint32_t n, hipEvent_t ready) {
   auto launch = [&](bool* capturing) -> int {
     KVT_HIP(hipStreamWaitEvent(s->side, ready, 0));
     // a side stream that waits for an event recorded inside a capture has joined that capture
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(s->side, &cap) != hipSuccess) (void)hipGetLastError();
     *capturing = cap != hipStreamCaptureStatusNone;
-    uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(layer) * s->layer_stride;
-    if (int rc = run_plan(true, s->plan, s->cache, layer, 1, dst, s->layer_stride, s->side)) return rc;
-    hipLaunchKernelGGL(publish_layer_kernel, dim3(1), dim3(64), 0, s->side, s->count_dev + layer,
-                       s->count_host + layer);
+    uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(first) * s->layer_stride;
+    if (int rc = run_plan(true, s->plan, s->cache, first, n, dst, s->layer_stride, s->side)) return rc;
+    hipLaunchKernelGGL(publish_layers_kernel, dim3(1), dim3(64), 0, s->side, s->count_dev + first,
+                       s->count_host + first, n);
     KVT_HIP(hipGetLastError());
     return KVT_OK;
   };
@@ -231,13 +233,14 @@ static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
   const int rc = launch(&capturing);
   std::lock_guard<std::mutex> lock(s->mu);
   if (capturing) {
-    // nothing runs now: the pack belongs to every later launch of the graph being recorded
-    if (rc == KVT_OK) s->in_graph[layer] = 1;
+    // nothing runs now: the packs belong to every later launch of the graph being recorded
+    if (rc == KVT_OK)
+      for (uint32_t l = first; l < first + n; ++l) s->in_graph[l] = 1;
   } else {
     if (s->cur_step == 0) begin_step_locked(s);  // a session used for one step needs no begin_step
     kvt_session::Step& st = s->step_slot(s->cur_step);
     if (rc == KVT_OK) {
-      st.target[layer] = ++s->submitted[layer];
+      for (uint32_t l = first; l < first + n; ++l) st.target[l] = ++s->submitted[l];
     } else if (st.error == KVT_OK) {   // latched: threads waiting for this step return it
       st.error = rc;
       st.message = kvt_last_error();
@@ -248,25 +251,37 @@ static int issue_layer(kvt_session* s, uint32_t layer, hipEvent_t ready) {
   return rc;
 }
 
-int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream) {
+static int check_layers(const kvt_session* s, uint32_t first, uint32_t n) {
+  if (n == 0 || first >= s->cache->n_layers || n > s->cache->n_layers - first)
+    return fail(KVT_ERR_OUT_OF_RANGE, "layer range out of range");
+  return KVT_OK;
+}
+
+int kvt_session_save_layers(kvt_session* s, uint32_t first_layer, uint32_t n_layers, void* compute_stream) {
   return guarded([&]() -> int {
-    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_save_layer: null session");
-    if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_save_layers: null session");
+    if (int rc = check_layers(s, first_layer, n_layers)) return rc;
     DeviceGuard g;
     if (int rc = g.enter(s->plan->device)) return rc;
-    KVT_HIP(hipEventRecord(s->ready[layer], static_cast<hipStream_t>(compute_stream)));
-    return issue_layer(s, layer, s->ready[layer]);
+    // the event of the group's last layer: everything before it on the stream has run then
+    hipEvent_t ready = s->ready[first_layer + n_layers - 1];
+    KVT_HIP(hipEventRecord(ready, static_cast<hipStream_t>(compute_stream)));
+    return issue_layers(s, first_layer, n_layers, ready);
   });
+}
+
+int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream) {
+  return kvt_session_save_layers(s, layer, 1, compute_stream);
 }
 
 int kvt_session_save_layer_event(kvt_session* s, uint32_t layer, void* ready_event) {
   return guarded([&]() -> int {
     if (!s || !ready_event)
       return fail(KVT_ERR_INVALID, "kvt_session_save_layer_event: null argument");
-    if (layer >= s->cache->n_layers) return fail(KVT_ERR_OUT_OF_RANGE, "layer out of range");
+    if (int rc = check_layers(s, layer, 1)) return rc;
     DeviceGuard g;
     if (int rc = g.enter(s->plan->device)) return rc;
-    return issue_layer(s, layer, static_cast<hipEvent_t>(ready_event));
+    return issue_layers(s, layer, 1, static_cast<hipEvent_t>(ready_event));
   });
 }
 

@@ -272,3 +272,62 @@ def test_a_bounded_wait_runs_out_and_can_be_repeated():
         assert np.array_equal(got, blob), l
     compute.synchronize()
     sess.close()
+
+
+def test_groups_of_layers_behind_one_event_eager_and_in_a_graph():
+    """kvt_session_save_layers: several layers behind one event, packed by one launch; the
+    transport still waits layer by layer. Eagerly with uneven groups, then the same groups
+    captured once and replayed with other cache contents."""
+    w = workloads.llama8b_single(n_layers=7, pool=96, tokens=700)
+    plan, lists = pipeline.build_plan(w, 0)
+    cap = w.capacities("src")[0]
+    layers = [[_contents(cap, 200 + l)] for l in range(w.n_layers)]
+    cache = kvt_amd.Cache(0, layers, [cap])
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    sess = kvt_amd.Session(plan, cache, packed, stride)
+    ranges = lists.tensor(0)
+    groups = [(0, 3), (3, 1), (4, 3)]
+    with pytest.raises(kvt_amd.KvtError):
+        sess.save_layers(5, 3)                                   # beyond the last layer
+    with pytest.raises(kvt_amd.KvtError):
+        sess.save_layers(2, 0)
+    compute = torch.cuda.Stream()
+
+    def check(step):
+        t = _Transport(sess, packed, stride, plan.tensor_bytes(0), w.n_layers, [step])
+        t.start()
+        return t
+
+    step = sess.begin_step()
+    t = check(step)
+    for first, n in groups:
+        sess.save_layers(first, n, compute.cuda_stream)
+    t.join(60)
+    assert not t.is_alive() and t.error is None, t.error
+    for l in range(w.n_layers):
+        assert np.array_equal(t.got[(step, l)], checkers.oracle_pack(layers[l][0].cpu().numpy(), ranges)), l
+    compute.synchronize()
+    sess.close()
+
+    sess = kvt_amd.Session(plan, cache, packed, stride)
+    graph = torch.cuda.CUDAGraph()
+    cap_stream = torch.cuda.Stream()
+    with torch.cuda.graph(graph, stream=cap_stream):
+        for first, n in groups:
+            sess.save_layers(first, n, cap_stream.cuda_stream)
+        sess.join(cap_stream.cuda_stream)
+    for rep in range(3):
+        for l in range(w.n_layers):
+            layers[l][0].copy_(_contents(cap, 300 + 10 * rep + l))
+        torch.cuda.synchronize()
+        expect = [checkers.oracle_pack(layers[l][0].cpu().numpy(), ranges) for l in range(w.n_layers)]
+        step = sess.begin_step()
+        t = check(step)
+        graph.replay()
+        t.join(60)
+        assert not t.is_alive() and t.error is None, t.error
+        for l in range(w.n_layers):
+            assert np.array_equal(t.got[(step, l)], expect[l]), (rep, l)
+    torch.cuda.synchronize()
+    sess.close()
