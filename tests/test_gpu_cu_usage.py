@@ -149,3 +149,55 @@ def test_more_limited_launches_in_flight_than_ticket_blocks():
         blob = checkers.oracle_pack(tp._host(src_layers[l][0]), o_lists[0])
         for out in outs:
             assert np.array_equal(tp._host(out)[l * stride:l * stride + len(blob)], blob), l
+
+
+@pytest.mark.parametrize("usage", [0.25, 0.004], ids=["quarter", "eight-workgroups"])
+def test_limited_launches_of_every_pipelined_kernel_inside_a_graph(usage):
+    """A limited launch recorded into a hipGraph keeps a block of counters of its own for every
+    replay. Plain, strided, converting and transposing plans, pack and unpack in one graph,
+    replayed with fresh cache contents each time."""
+    kvt_amd.set_copy_cu_usage(0, usage)
+    try:
+        cases = []
+        w = workloads.llama8b_batch(n_layers=3, src_pool=700, dst_pool=900, n_req=6, min_tok=300, max_tok=1500)
+        cases.append((w, pipeline.build_plan(w, 0)[0]))
+        w = workloads.tp_split("flash", 2, 1, 1, n_layers=3, src_pool=500, dst_pool=600, n_req=6,
+                               min_tok=200, max_tok=1400)
+        cases.append((w, pipeline.build_plan_runs(w, 0)[0]))
+        w = workloads.tp_split("flash", 2, 1, 1, n_layers=3, src_pool=500, dst_pool=600, n_req=6,
+                               min_tok=200, max_tok=1400, fp8_dst=True)
+        cases.append((w, pipeline.build_plan_runs(w, 0)[0]))
+        w = workloads.llama70b_flashinfer(n_layers=3, pool=400, n_req=4, tokens=1500)
+        cases.append((w, pipeline.build_plan(w, 0)[0]))
+        for w, plan in cases:
+            plan.ready()
+            src = tp._make_caches(w, "src", 5, dtype="raw" if w.notes.get("fp8") else None)
+            sc = kvt_amd.Cache(0, src, w.capacities("src"))
+            stride = plan.layer_bytes
+            eager = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+            out = torch.zeros_like(eager)
+            dst_e = tp._make_caches(w, "dst", 6, fill=False)
+            dst_g = tp._make_caches(w, "dst", 6, fill=False)
+            de, dg = (kvt_amd.Cache(0, d, w.capacities("dst")) for d in (dst_e, dst_g))
+            graph = torch.cuda.CUDAGraph()
+            cs = torch.cuda.Stream()
+            with torch.cuda.graph(graph, stream=cs):
+                plan.pack(sc, 0, w.n_layers, out, stride, cs.cuda_stream)
+                plan.unpack(dg, 0, w.n_layers, out, stride, cs.cuda_stream)
+            for rep in range(3):
+                for l in range(w.n_layers):
+                    for t in range(w.n_tensors):
+                        src[l][t].copy_(torch.roll(src[l][t], 4096 * (rep + 1)))
+                torch.cuda.synchronize()
+                graph.replay()
+                kvt_amd.set_copy_cu_usage(0, 1.0)       # the unlimited launches as the reference
+                plan.pack(sc, 0, w.n_layers, eager, stride)
+                plan.unpack(de, 0, w.n_layers, eager, stride)
+                kvt_amd.set_copy_cu_usage(0, usage)
+                torch.cuda.synchronize()
+                assert torch.equal(out, eager), (w.name, rep)
+                for l in range(w.n_layers):
+                    for t in range(w.n_tensors):
+                        assert torch.equal(dst_g[l][t], dst_e[l][t]), (w.name, rep, l, t)
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
