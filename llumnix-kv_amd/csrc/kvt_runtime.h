@@ -38,7 +38,9 @@ uint32_t device_cu_count(int device);
 
 // KVT_OK when [ptr, ptr + bytes) is, as far as the runtime can tell, memory the device may
 // touch; KVT_ERR_INVALID / KVT_ERR_OUT_OF_RANGE (message set, starting with `what`) otherwise.
-int check_device_span(const void* ptr, uint64_t bytes, const std::string& what);
+// *host_memory (optional): the pointer is host memory mapped into the device (pinned), i.e.
+// whatever a kernel moves there crosses PCIe.
+int check_device_span(const void* ptr, uint64_t bytes, const std::string& what, bool* host_memory = nullptr);
 // Launches whose payload is at most this many bytes read with plain loads (kvt_set_copy_cached_load_max).
 uint64_t copy_cached_load_max_bytes();
 // Drops every remembered allocation extent (call where device memory is freed).

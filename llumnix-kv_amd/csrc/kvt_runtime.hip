@@ -86,12 +86,14 @@ uint64_t copy_cached_load_max_bytes() { return g_cached_load_max.load(std::memor
 static std::atomic<uint64_t> g_span_epoch{1};
 void forget_device_spans() { g_span_epoch.fetch_add(1, std::memory_order_relaxed); }
 
-int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) {
+int check_device_span(const void* ptr, uint64_t bytes, const std::string& what, bool* host_memory) {
+  if (host_memory) *host_memory = false;
   if (bytes == 0) return KVT_OK;
   struct Span {
     uintptr_t lo = 0, hi = 0;
     unsigned uses = 0;
     uint64_t epoch = 0;
+    bool host = false;
   };
   // Allocations the runtime has answered for lately, per thread: a lookup costs microseconds
   // and the same few buffers come back launch after launch. An answer is trusted for a bounded
@@ -102,6 +104,7 @@ int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) 
   const uint64_t epoch = g_span_epoch.load(std::memory_order_relaxed);
   for (Span& s : seen)
     if (s.epoch == epoch && p >= s.lo && p < s.hi && bytes <= s.hi - p) {
+      if (host_memory) *host_memory = s.host;
       if (++s.uses < 256) return KVT_OK;
       s = Span{};  // ask the runtime again below
       break;
@@ -113,6 +116,7 @@ int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) 
   }
   if (attr.type == hipMemoryTypeUnregistered)
     return fail(KVT_ERR_INVALID, what + " is plain host memory the device cannot address");
+  if (host_memory) *host_memory = attr.type == hipMemoryTypeHost;
   hipDeviceptr_t base = nullptr;
   size_t size = 0;
   if (hipMemGetAddressRange(&base, &size, const_cast<void*>(ptr)) != hipSuccess) {
@@ -125,7 +129,7 @@ int check_device_span(const void* ptr, uint64_t bytes, const std::string& what) 
                 what + ": " + std::to_string(bytes) +
                     " bytes reach beyond the allocation that holds the pointer (" +
                     std::to_string(p < lo || p - lo > size ? 0 : size - (p - lo)) + " bytes left)");
-  seen[next++ % 8] = Span{lo, lo + size, 0, epoch};
+  seen[next++ % 8] = Span{lo, lo + size, 0, epoch, attr.type == hipMemoryTypeHost};
   return KVT_OK;
 }
 
