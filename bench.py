@@ -869,13 +869,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "db41ff18da04b93088f3de4996eed7a082903e7c2f3db384905183921bff428e"
+KERNELS_SHA256 = "af354416d0e114834afca107f99c4e2d3e14cdf1bacb1aae6cc10b054a337422"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134278584, "unpack": 134277773},
-    (2, "ranges"): {"pack": 71012999691, "unpack": 73358406988},
-    (3, "ranges"): {"pack": 85983087420, "unpack": 85983592419},
-    (4, "ranges"): {"pack": 22690386598, "unpack": 22690441296},
-    (5, "ranges"): {"pack": 45141195491, "unpack": 45141395554},
+    (1, "ranges"): {"pack": 134278414, "unpack": 134277048},
+    (2, "ranges"): {"pack": 71013067659, "unpack": 73358407012},
+    (3, "ranges"): {"pack": 85983085843, "unpack": 85983587983},
+    (4, "ranges"): {"pack": 22690395884, "unpack": 22690447212},
+    (5, "ranges"): {"pack": 45141193967, "unpack": 45141393090},
 }
 
 

@@ -11,8 +11,13 @@
 //   * workgroup ids are dealt round-robin to the 8 XCDs, so id b is remapped to
 //     (b % 8) * ceil(n / 8) + b / 8: each XCD then streams through one
 //     contiguous eighth of the work list instead of touching every page.
-// No LDS and no MFMA: the HND<->NHD transform moves whole 16-byte vectors of
-// rows that are contiguous on both sides, so it is a pure index permutation.
+// A launch limited to a share of the device runs instead as a few persistent workgroups (at
+// best one per CU) that pipeline whole table entries over three register sets and take them
+// in order from one counter per XCD: what keeps such a launch fast is that the addresses in
+// flight stay in one narrow window, as the order of dispatch keeps them in the unlimited shape.
+// No MFMA, and LDS only to hand a ticket to the wavefronts of a workgroup: the HND<->NHD
+// transform moves whole 16-byte vectors of rows that are contiguous on both sides, so it is
+// a pure index permutation.
 #include <hip/hip_runtime.h>
 
 #include <cstddef>
