@@ -273,7 +273,7 @@ def leg_latency(c, out):
     strides, packed, stream, sh, new_event = c.strides, c.packed, c.stream, c.sh, c.new_event
     w, side = wls[0], sides[0]
     sender = c.senders[0]
-    single, gated, wall, tail, grouped = [], [], [], [], []
+    single, gated, wall, tail, grouped, tail_inline = [], [], [], [], [], []
     fill = [torch.zeros(256 << 20, dtype=torch.uint8, device="cuda") for _ in range(2)]
     reqs = list(range(len(w.tasks)))
     if len(reqs) < 5:                  # a single-request configuration: the same request again
@@ -323,6 +323,19 @@ def leg_latency(c, out):
         sess.wait_layer(w.n_layers - 1, step)
         lib.kvt_event_synchronize(b)
         tail.append(ev_ms(lib, a, b) * 1e3)
+        # ... and with the last layer packed on the compute stream itself (no hop)
+        step = sess.begin_step()
+        for l in range(w.n_layers):
+            assert lib.kvt_copy_linear(fill[1].data_ptr(), fill[0].data_ptr(), fill[0].numel(), sh) == 0
+            if l == w.n_layers - 1:
+                lib.kvt_event_record(a, sh)
+                sess.save_layers_inline(l, 1, sh)
+                lib.kvt_event_record(b, sh)
+            else:
+                sess.save_layer(l, sh)
+        sess.wait_layer(w.n_layers - 1, step)
+        lib.kvt_event_synchronize(b)
+        tail_inline.append(ev_ms(lib, a, b) * 1e3)
         # the gated sequence again with one hop per group of four layers
         step = sess.begin_step()
         lib.kvt_event_record(a, sh)
@@ -346,6 +359,7 @@ def leg_latency(c, out):
     out["latency_groups_of_4_layers_p50_us"] = round(statistics.median(grouped), 2)
     out["latency_single_launch_p50_us"] = round(statistics.median(single), 2)
     out["latency_after_last_layer_p50_us"] = round(statistics.median(tail), 2)
+    out["latency_after_last_layer_inline_p50_us"] = round(statistics.median(tail_inline), 2)
     del fill
     out["latency_note"] = ("per request (%d timed): latency_p50_us = GPU time from the first "
                            "pack launch of layer 0 to the completion of layer %d on the side "
@@ -357,7 +371,10 @@ def leg_latency(c, out):
                            "covering all layers; latency_after_last_layer_p50_us = the gated "
                            "sequence behind a busy compute stream (a 256 MiB copy per layer as "
                            "the forward pass): GPU time from the end of the last layer's compute "
-                           "to the completion of its pack" % (len(reqs), w.n_layers - 1))
+                           "to the completion of its pack "
+                           "(latency_after_last_layer_inline_p50_us: the last layer packed on "
+                           "the compute stream itself, kvt_session_save_layers_inline)"
+                           % (len(reqs), w.n_layers - 1))
 
 
 def leg_session(c, out):
@@ -1233,7 +1250,8 @@ def main():
                         "frac_hbm_peak", "host_parse_plan_ms", "mode", "parity_vs_oracle",
                         "latency_p50_us", "latency_wall_p50_us", "latency_single_launch_p50_us",
                         "latency_groups_of_4_layers_p50_us",
-                        "latency_after_last_layer_p50_us", "cu_usage",
+                        "latency_after_last_layer_p50_us", "latency_after_last_layer_inline_p50_us",
+                        "cu_usage",
                         "staging", "roofline", "cpu_baseline", "errors"):
                 if key in r:
                     row[key] = r[key]

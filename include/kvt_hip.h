@@ -597,6 +597,16 @@ int kvt_session_save_layer(kvt_session* s, uint32_t layer, void* compute_stream)
  * the layers of a group become ready together. */
 int kvt_session_save_layers(kvt_session* s, uint32_t first_layer, uint32_t n_layers,
                             void* compute_stream);
+/* The same without the hop (no counterpart in the reference): the layers are packed on
+ * compute_stream itself, behind whatever is queued there, and whatever the caller queues next
+ * on that stream runs after the pack. For the last layer(s) of a step, when no further compute
+ * is left for the pack to overlap with: what the transport waits for after the forward pass
+ * then ends one launch behind the last layer's compute instead of one cross-stream hop
+ * (18-27 us on MI355X) behind it. Signals, steps and errors as kvt_session_save_layers;
+ * kvt_session_join does not wait for these launches (they are on the caller's stream
+ * already). Capturable. */
+int kvt_session_save_layers_inline(kvt_session* s, uint32_t first_layer, uint32_t n_layers,
+                                   void* compute_stream);
 /* The same for a caller that owns the per-layer events, as the reference's Python side does:
  * it creates one event per layer, hands their handles to the library at init and records
  * event[layer] itself after the layer's KV is written (blade_kvt/kv_transfer_impl.py:287-291,

@@ -26,6 +26,8 @@ struct kvt_session {
   hipStream_t side = nullptr;
   std::vector<hipEvent_t> ready;
   hipEvent_t joined = nullptr;     // recorded on the side stream by kvt_session_join
+  hipEvent_t inline_done = nullptr;  // behind the last eager inline pack (on the caller's stream)
+  bool inline_any = false;
   bool issued_any = false;
   uint32_t* count_dev = nullptr;   // per layer: packs completed so far (device memory)
   uint32_t* count_host = nullptr;  // the same, mirrored by the device into pinned host memory
@@ -153,6 +155,7 @@ int kvt_session_create(const kvt_plan* plan, const kvt_cache* cache, void* packe
       KVT_HIP(hipEventCreateWithFlags(&s->ready[l], hipEventDisableTiming));
     }
     KVT_HIP(hipEventCreateWithFlags(&s->joined, hipEventDisableTiming));
+    KVT_HIP(hipEventCreateWithFlags(&s->inline_done, hipEventDisableTiming));
     KVT_HIP(hipMalloc(reinterpret_cast<void**>(&s->count_dev), n * sizeof(uint32_t)));
     KVT_HIP(hipMemset(s->count_dev, 0, n * sizeof(uint32_t)));
     KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&s->count_host), n * sizeof(uint32_t),
@@ -175,6 +178,8 @@ void kvt_session_destroy(kvt_session* s) {
     (void)hipStreamSynchronize(s->side);
     (void)hipStreamDestroy(s->side);
   }
+  if (s->inline_any) (void)hipEventSynchronize(s->inline_done);  // packs on the caller's own stream
+  if (s->inline_done) (void)hipEventDestroy(s->inline_done);
   for (hipEvent_t e : s->ready)
     if (e) (void)hipEventDestroy(e);
   if (s->joined) (void)hipEventDestroy(s->joined);
@@ -215,18 +220,25 @@ int kvt_session_begin_step(kvt_session* s, uint64_t* step) {
 
 // The pack of layers [first, first + n) on the side stream as ONE launch, gated by `ready`
 // (already recorded), and the publication of their completion.
-static int issue_layers(kvt_session* s, uint32_t first, uint32_t n, hipEvent_t ready) {
+// ready == nullptr: on `inline_stream` itself, behind whatever is queued there, with no event.
+static int issue_layers(kvt_session* s, uint32_t first, uint32_t n, hipEvent_t ready,
+                        hipStream_t inline_stream = nullptr) {
   auto launch = [&](bool* capturing) -> int {
-    KVT_HIP(hipStreamWaitEvent(s->side, ready, 0));
+    const hipStream_t on = ready ? s->side : inline_stream;
+    if (ready) KVT_HIP(hipStreamWaitEvent(s->side, ready, 0));
     // a side stream that waits for an event recorded inside a capture has joined that capture
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s->side, &cap) != hipSuccess) (void)hipGetLastError();
+    if (hipStreamIsCapturing(on, &cap) != hipSuccess) (void)hipGetLastError();
     *capturing = cap != hipStreamCaptureStatusNone;
     uint8_t* dst = static_cast<uint8_t*>(s->packed) + static_cast<uint64_t>(first) * s->layer_stride;
-    if (int rc = run_plan(true, s->plan, s->cache, first, n, dst, s->layer_stride, s->side)) return rc;
-    hipLaunchKernelGGL(publish_layers_kernel, dim3(1), dim3(64), 0, s->side, s->count_dev + first,
+    if (int rc = run_plan(true, s->plan, s->cache, first, n, dst, s->layer_stride, on)) return rc;
+    hipLaunchKernelGGL(publish_layers_kernel, dim3(1), dim3(64), 0, on, s->count_dev + first,
                        s->count_host + first, n);
     KVT_HIP(hipGetLastError());
+    if (!ready && !*capturing) {   // kvt_session_destroy waits for it: the counters must outlive it
+      KVT_HIP(hipEventRecord(s->inline_done, on));
+      s->inline_any = true;
+    }
     return KVT_OK;
   };
   bool capturing = false;
@@ -246,7 +258,7 @@ static int issue_layers(kvt_session* s, uint32_t first, uint32_t n, hipEvent_t r
       st.message = kvt_last_error();
     }
   }
-  if (rc == KVT_OK) s->issued_any = true;
+  if (rc == KVT_OK && ready) s->issued_any = true;   // what kvt_session_join has to wait for
   s->cv.notify_all();
   return rc;
 }
@@ -267,6 +279,16 @@ int kvt_session_save_layers(kvt_session* s, uint32_t first_layer, uint32_t n_lay
     hipEvent_t ready = s->ready[first_layer + n_layers - 1];
     KVT_HIP(hipEventRecord(ready, static_cast<hipStream_t>(compute_stream)));
     return issue_layers(s, first_layer, n_layers, ready);
+  });
+}
+
+int kvt_session_save_layers_inline(kvt_session* s, uint32_t first_layer, uint32_t n_layers, void* compute_stream) {
+  return guarded([&]() -> int {
+    if (!s) return fail(KVT_ERR_INVALID, "kvt_session_save_layers_inline: null session");
+    if (int rc = check_layers(s, first_layer, n_layers)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(s->plan->device)) return rc;
+    return issue_layers(s, first_layer, n_layers, nullptr, static_cast<hipStream_t>(compute_stream));
   });
 }
 

@@ -123,6 +123,7 @@ SIGNATURES = {
     "kvt_session_save_layer": (_int, [_vp, _u32, _vp]),
     "kvt_session_save_layer_event": (_int, [_vp, _u32, _vp]),
     "kvt_session_save_layers": (_int, [_vp, _u32, _u32, _vp]),
+    "kvt_session_save_layers_inline": (_int, [_vp, _u32, _u32, _vp]),
     "kvt_session_wait_layer": (_int, [_vp, _u32]),
     "kvt_session_wait_layer_step": (_int, [_vp, _u64, _u32]),
     "kvt_session_wait_layer_for": (_int, [_vp, _u64, _u32, _u64]),
@@ -563,6 +564,10 @@ class Session:
     def save_layers(self, first_layer, n_layers, compute_stream=None):
         """Layers [first_layer, first_layer + n_layers) behind one event, packed by one launch."""
         check(lib().kvt_session_save_layers(self.h, first_layer, n_layers, _ptr(compute_stream)))
+
+    def save_layers_inline(self, first_layer, n_layers, compute_stream=None):
+        """The same on compute_stream itself: no hop to the side stream (a step's last layers)."""
+        check(lib().kvt_session_save_layers_inline(self.h, first_layer, n_layers, _ptr(compute_stream)))
 
     def save_layer_event(self, layer, ready_event):
         """ready_event: a hipEvent_t handle the caller has recorded (an int, e.g.

@@ -331,3 +331,33 @@ def test_groups_of_layers_behind_one_event_eager_and_in_a_graph():
             assert np.array_equal(t.got[(step, l)], expect[l]), (rep, l)
     torch.cuda.synchronize()
     sess.close()
+
+
+def test_last_layers_packed_on_the_compute_stream_itself():
+    """kvt_session_save_layers_inline: no hop to the side stream; same signal, same bytes, and
+    the session may be destroyed while such a pack is still queued."""
+    w = workloads.llama8b_single(n_layers=5, pool=96, tokens=600)
+    plan, lists = pipeline.build_plan(w, 0)
+    cap = w.capacities("src")[0]
+    layers = [[_contents(cap, 400 + l)] for l in range(w.n_layers)]
+    cache = kvt_amd.Cache(0, layers, [cap])
+    stride = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
+    sess = kvt_amd.Session(plan, cache, packed, stride)
+    compute = torch.cuda.Stream()
+    for rep in range(2):
+        step = sess.begin_step()
+        t = _Transport(sess, packed, stride, plan.tensor_bytes(0), w.n_layers, [step])
+        t.start()
+        for l in range(3):
+            sess.save_layer(l, compute.cuda_stream)
+        sess.save_layers_inline(3, 2, compute.cuda_stream)
+        t.join(60)
+        assert not t.is_alive() and t.error is None, t.error
+        for l in range(w.n_layers):
+            blob = checkers.oracle_pack(layers[l][0].cpu().numpy(), lists.tensor(0))
+            assert np.array_equal(t.got[(step, l)], blob), (rep, l)
+    sess.begin_step()
+    sess.save_layers_inline(0, w.n_layers, compute.cuda_stream)
+    sess.close()                       # waits for the pack queued on the compute stream
+    compute.synchronize()
