@@ -639,6 +639,8 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
     return fail(KVT_ERR_INVALID,
                 "a converting strided plan needs 16-byte aligned layer tensors, packed buffer, "
                 "stride and blob offsets");
+  // Tickets count (4 KiB slice, layer) pairs at the finest, in 32 bits.
+  const bool few_pairs = (static_cast<uint64_t>(n) << p->sub_shift) * n_layers < (1ull << 31);
   // A capped launch of a plain, fully 16-byte aligned table with entries of 16 or 32 KiB: one
   // persistent workgroup per CU at most (more of them were slower on MI355X: 5.5 TB/s with 256,
   // 5.3 with 512, 5.2 with 1 024), each pipelining whole entries.
@@ -652,7 +654,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, cus));
       // fewer workgroups than CUs: each has to move more than the ticket's barrier lets it
       // (half the CUs: 4.4 against 5.3 TB/s)
-      LaunchTickets tickets(cache->device, capturing, wgs >= cus);
+      LaunchTickets tickets(cache->device, capturing, wgs >= cus && few_pairs);
       const hipError_t e = launch_copy_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                                p->n_tensors, first_layer, n_layers,
                                                static_cast<uint8_t*>(packed), layer_stride, blobs,
@@ -687,7 +689,8 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       // trips of 8 KiB by a single workgroup per CU are better off without the ticket's barrier
       // (converting gather at an eighth of the device: 4.4 against 5.1 TB/s), and so is a grid
       // of fewer workgroups than CUs
-      LaunchTickets tickets(cache->device, capturing, wgs >= cus && (p->sub_shift >= 2 || wgs >= 2 * cus));
+      LaunchTickets tickets(cache->device, capturing,
+                            wgs >= cus && few_pairs && (p->sub_shift >= 2 || wgs >= 2 * cus));
       const hipError_t e =
           converting ? launch_convert_entries(table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                               first_layer, n_layers, pk, layer_stride, blobs,
@@ -715,7 +718,8 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   const uint32_t grid_cap = max_wgs == 0 ? 0u : std::max(8u, max_wgs & ~7u);
   const uint64_t pairs = ((static_cast<uint64_t>(n) << p->sub_shift) + 7u) / 8u * 8u * n_layers;
   const uint32_t n_cus = device_cu_count(cache->device);
-  LaunchTickets tickets(cache->device, capturing, grid_cap != 0 && pairs > grid_cap && n_cus != 0 && grid_cap >= 2 * n_cus);
+  LaunchTickets tickets(cache->device, capturing,
+                        grid_cap != 0 && pairs > grid_cap && few_pairs && n_cus != 0 && grid_cap >= 2 * n_cus);
   uint8_t* const pk8 = static_cast<uint8_t*>(packed);
   const hipError_t e =
       p->convert && pack ? launch_convert_chunks(table, n, p->sub_shift, cache->dev_ptrs,
