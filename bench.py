@@ -886,13 +886,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "af354416d0e114834afca107f99c4e2d3e14cdf1bacb1aae6cc10b054a337422"
+KERNELS_SHA256 = "0a177a312b5c878fa2c55fedc85795a65458519f91b1a1307181031a2f49820a"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134278414, "unpack": 134277048},
-    (2, "ranges"): {"pack": 71013067659, "unpack": 73358407012},
-    (3, "ranges"): {"pack": 85983085843, "unpack": 85983587983},
-    (4, "ranges"): {"pack": 22690395884, "unpack": 22690447212},
-    (5, "ranges"): {"pack": 45141193967, "unpack": 45141393090},
+    (1, "ranges"): {"pack": 134278132, "unpack": 134277748},
+    (2, "ranges"): {"pack": 71013083789, "unpack": 73358418543},
+    (3, "ranges"): {"pack": 85983104936, "unpack": 85983602767},
+    (4, "ranges"): {"pack": 22690383563, "unpack": 22690445045},
+    (5, "ranges"): {"pack": 45141201082, "unpack": 45141402424},
 }
 
 
@@ -1073,7 +1073,7 @@ def run_config(args, headline):
     elif wls[0].xform:
         kernel = "kvt::xform_chunks_kernel<true, false> (pack)"
     elif first[0][0].num_chunks <= 64:
-        kernel = "kvt::copy_chunks_small_kernel<true, false> (pack)"
+        kernel = "kvt::copy_chunks_small_kernel<true, 0> (pack)"
     else:
         kernel = "kvt::copy_chunks_kernel<true, 0> (pack)"
     limited = args.cu_usage < 1.0

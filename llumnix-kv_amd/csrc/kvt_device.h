@@ -87,8 +87,8 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
-                                    const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
-                                    uint32_t* tickets, hipStream_t stream);
+                                    const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
+                                    bool temporal, uint32_t* tickets, hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,

@@ -439,14 +439,14 @@ __global__ __launch_bounds__(kThreads, MODE == kPipelined ? 4 : 8) void copy_chu
 
 // The same for a table short enough to be a kernel argument (read through the scalar cache
 // like any other argument; the index is uniform across the workgroup).
-template <bool PACK, bool CAPPED>
-__global__ __launch_bounds__(kThreads, 8) void copy_chunks_small_kernel(
+template <bool PACK, int MODE>
+__global__ __launch_bounds__(kThreads, MODE == kPipelined ? 4 : 8) void copy_chunks_small_kernel(
     const SmallTable table, uint32_t n_slices, uint32_t sub_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
     uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
     uint32_t* tickets) {
   KVT_LAUNCH_STRUCT;
-  for_items<CAPPED ? kStriding : kOnePerSlice>(L, [&](uint32_t e) { return fetch_entry(table.c, e); },
+  for_items<MODE>(L, [&](uint32_t e) { return fetch_entry(table.c, e); },
                     [&](const Item& it) { return plain_move<PACK>(it); });
 }
 
@@ -1104,18 +1104,24 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
-                                    const BlobOffsets& blobs, uint32_t max_wgs, bool temporal,
-                                    uint32_t* tickets, hipStream_t stream) {
+                                    const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
+                                    bool temporal, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
   if (!g.capped) tickets = nullptr;
   const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
 #define KVT_ARGS table, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
-  if (pack && !g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, false>), KVT_ARGS);
-  else if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, true>), KVT_ARGS);
-  else if (!g.capped) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, false>), KVT_ARGS);
-  else KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, true>), KVT_ARGS);
+  if (!g.capped) {
+    if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, kOnePerSlice>), KVT_ARGS);
+    else KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, kOnePerSlice>), KVT_ARGS);
+  } else if (!pipelined) {
+    if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, kStriding>), KVT_ARGS);
+    else KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, kStriding>), KVT_ARGS);
+  } else {
+    if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, kPipelined>), KVT_ARGS);
+    else KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<false, kPipelined>), KVT_ARGS);
+  }
 #undef KVT_ARGS
   return hipGetLastError();
 }

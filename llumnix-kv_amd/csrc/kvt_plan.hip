@@ -616,10 +616,14 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   for (uint32_t t = 0; t < p->n_tensors; ++t) payload += p->tensor_bytes[t];
   const bool temporal = payload * n_layers <= copy_cached_load_max_bytes();
   if (p->small) {
+    // No tickets for a short table: the launch is over before their order pays (a 64 MiB
+    // request at half the device: 31 -> 44 us with them); the pipelined loop does pay below
+    // half the device (a quarter: 35 -> 30 us, an eighth: 47 -> 34 us).
     const hipError_t e = launch_copy_chunks_small(
         pack, pack ? p->small_pack : p->small_unpack, static_cast<uint32_t>(p->n_chunks),
         p->sub_shift, cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
-        static_cast<uint8_t*>(packed), layer_stride, blobs, max_wgs, temporal, nullptr, s);
+        static_cast<uint8_t*>(packed), layer_stride, blobs, max_wgs,
+        max_wgs < 4u * device_cu_count(cache->device), temporal, nullptr, s);
     if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
     return KVT_OK;
   }
