@@ -164,8 +164,8 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
   // choice (memcpy loop or kernel) from a profile it takes at start-up
   // (copy_kernels.cpp:495-619); so does kvt_initialize_copy_method_profile here, and before it
   // has run the thresholds decide, fixed from measurements on one MI355X: against pinned host
-  // memory a copy of 128 MiB runs at 57 GB/s where the kernel's stores across PCIe reach 54,
-  // the kernel wins below about 8 MiB per copy (2 MiB: 53 against 33 GB/s).
+  // memory a copy of 128 MiB runs at 57 GB/s and occupies no CU, where the kernel's stores
+  // across PCIe reach 56; the kernel wins below about 8 MiB per copy (2 MiB: 53 against 33 GB/s).
   if (route == kRouteDma ||
       (route == kRouteAuto && !halve && list_to_dma(direction, n, total, shortest))) {
     uint64_t cursor = 0;
