@@ -201,3 +201,42 @@ def test_limited_launches_of_every_pipelined_kernel_inside_a_graph(usage):
                         assert torch.equal(dst_g[l][t], dst_e[l][t]), (w.name, rep, l, t)
     finally:
         kvt_amd.set_copy_cu_usage(0, 1.0)
+
+
+def test_limited_launches_of_one_plan_from_several_threads_at_once():
+    """Launches that may run at the same time never share a block of counters: four threads,
+    each on a stream of its own, pack the same plan under a limit into their own buffers."""
+    import threading
+    w = workloads.llama8b_batch(n_layers=2, src_pool=700, dst_pool=900, n_req=6, min_tok=300, max_tok=1500)
+    plan, lists = pipeline.build_plan(w, 0)
+    plan.ready()
+    src_layers = tp._make_caches(w, "src", 23)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    stride = plan.layer_bytes
+    outs = [torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda") for _ in range(4)]
+    errors = []
+
+    def worker(i):
+        try:
+            st = torch.cuda.Stream()
+            for _ in range(60):
+                plan.pack(sc, 0, w.n_layers, outs[i], stride, st.cuda_stream)
+            st.synchronize()
+        except Exception as e:          # noqa: BLE001 - handed to the main thread
+            errors.append(e)
+
+    kvt_amd.set_copy_cu_usage(0, 0.25)
+    try:
+        threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(120)
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+    assert not errors, errors
+    o_lists = tp._oracle_lists(w)
+    for l in range(w.n_layers):
+        blob = checkers.oracle_pack(tp._host(src_layers[l][0]), o_lists[0])
+        for out in outs:
+            assert np.array_equal(tp._host(out)[l * stride:l * stride + len(blob)], blob), l
