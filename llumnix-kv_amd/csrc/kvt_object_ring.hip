@@ -48,6 +48,12 @@ struct kvt_object_ring {
   uint8_t* arena = nullptr;
   hipStream_t copy = nullptr;
   hipEvent_t fence = nullptr;
+  // the kernel route of a transfer that is many short pieces: range metadata (3 int64 per
+  // piece) on the device and in pinned memory, in use until `meta_free` has completed
+  int64_t* meta_dev = nullptr;
+  int64_t* meta_host = nullptr;
+  hipEvent_t meta_free = nullptr;
+  bool meta_used = false;
   std::mutex mu;
   uint64_t handed_out = 0;   // entries assigned so far; the next one is handed_out % n_entries
   uint64_t calls = 0;
@@ -117,6 +123,10 @@ int kvt_object_ring_create(int device, uint64_t entry_bytes, uint32_t n_entries,
       KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&r->arena), total, hipHostMallocDefault));
       KVT_HIP(hipStreamCreateWithFlags(&r->copy, hipStreamNonBlocking));
       KVT_HIP(hipEventCreateWithFlags(&r->fence, hipEventDisableTiming));
+      KVT_HIP(hipEventCreateWithFlags(&r->meta_free, hipEventDisableTiming));
+      const size_t meta_bytes = 3 * sizeof(int64_t) * static_cast<size_t>(n_entries);
+      KVT_HIP(hipMalloc(reinterpret_cast<void**>(&r->meta_dev), meta_bytes));
+      KVT_HIP(hipHostMalloc(reinterpret_cast<void**>(&r->meta_host), meta_bytes, hipHostMallocDefault));
     }
     *out = r.release();
     return KVT_OK;
@@ -131,6 +141,12 @@ void kvt_object_ring_destroy(kvt_object_ring* r) {
   }
   r->entries.clear();   // drops the transfer events
   if (r->fence) (void)hipEventDestroy(r->fence);
+  if (r->meta_free) (void)hipEventDestroy(r->meta_free);
+  if (r->meta_dev) {
+    forget_device_spans();
+    (void)hipFree(r->meta_dev);
+  }
+  if (r->meta_host) (void)hipHostFree(r->meta_host);
   if (r->arena) {
     if (r->device == KVT_DEVICE_NONE)
       std::free(r->arena);
@@ -326,7 +342,29 @@ static int transfer(kvt_object_ring* r, const uint32_t* entries, uint32_t n, voi
   KVT_HIP(hipEventRecord(r->fence, user));
   KVT_HIP(hipStreamWaitEvent(r->copy, r->fence, 0));
   uint8_t* d = static_cast<uint8_t*>(dev);
-  if (int rc = for_runs(r, entries, n, dev_stride, [&](uint32_t first, uint32_t count) -> int {
+  // Pieces: runs of entries that are neighbours on both sides. A few long ones go to the DMA
+  // engines, one copy each; many short ones are moved by ONE launch of the range kernel,
+  // which crosses PCIe at 56 GB/s whatever their length (a DMA copy of 2 MiB reaches 33).
+  static thread_local std::vector<kvt_ipc_block> pieces;
+  pieces.clear();
+  (void)for_runs(r, entries, n, dev_stride, [&](uint32_t first, uint32_t count) -> int {
+    pieces.push_back(kvt_ipc_block{static_cast<uint64_t>(entries[first]) * r->entry_bytes,
+                                   static_cast<uint64_t>(first) * dev_stride,
+                                   static_cast<uint64_t>(count) * r->entry_bytes});
+    return KVT_OK;
+  });
+  const uint64_t moved = static_cast<uint64_t>(n) * r->entry_bytes;
+  if (pieces.size() > 1 && moved / pieces.size() < (8ull << 20) && pieces.size() <= r->n_entries) {
+    if (r->meta_used) KVT_HIP(hipEventSynchronize(r->meta_free));  // the staging area is free again
+    const uint64_t m = pieces.size();
+    if (int rc = kvt_copy_handle_data_kernel_direct(
+            r->arena, d, pieces.data(), m, static_cast<uint64_t>(r->n_entries) * r->entry_bytes,
+            save ? KVT_COPY_D2H : KVT_COPY_H2D, r->device, r->copy, r->meta_dev, r->meta_dev + m,
+            r->meta_dev + 2 * m, r->meta_host, 1))
+      return rc;
+    KVT_HIP(hipEventRecord(r->meta_free, r->copy));
+    r->meta_used = true;
+  } else if (int rc = for_runs(r, entries, n, dev_stride, [&](uint32_t first, uint32_t count) -> int {
         uint8_t* host = r->arena + static_cast<uint64_t>(entries[first]) * r->entry_bytes;
         uint8_t* devp = d + static_cast<uint64_t>(first) * dev_stride;
         const uint64_t bytes = static_cast<uint64_t>(count) * r->entry_bytes;
