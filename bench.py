@@ -815,8 +815,9 @@ def leg_store_objects(c, out):
                         "save_gbps": round(saved * entry / (t_b - t_a) / 1e9, 2),
                         "load_gbps": round(len(hits) * entry / (t_d - t_c) / 1e9, 2),
                         "note": "batches of 256 blocks: reserve by hash, pack the missing blocks "
-                                "(all layers per object), DMA into the ring; load: DMA out of the "
-                                "entries found by hash"}
+                                "(all layers per object), DMA into the ring; load: the entries "
+                                "found by hash, scattered ones by one kernel launch over PCIe, "
+                                "long runs by DMA"}
     ring.close()
     out["kvstore_objects"] = res
 
