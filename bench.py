@@ -670,6 +670,7 @@ def leg_frames(c, out):
     stg = kvt.Stager(0, lay.total_bytes, 2)
     dev = [torch.empty(plan.layer_bytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
     ps = torch.cuda.Stream()
+    cs = [torch.cuda.Stream(), torch.cuda.Stream()]     # a consumer stream per slot
     payload = sum(lay.blob_bytes[t] for t in range(w.n_tensors))
     host_write, host_parse, send_t, recv_t = [], [], [], []
     for phase in range(4):
@@ -704,9 +705,10 @@ def leg_frames(c, out):
             rlists.close()
             for t in range(w.n_tensors):
                 stg.load_at(slot, rlay.blob_offset[t], dev[slot].data_ptr() + plan.tensor_offset(t),
-                            rlay.blob_bytes[t], ps.cuda_stream)
-            plan.unpack(side.dst_cache, int(layer), 1, dev[slot], plan.layer_bytes, ps.cuda_stream)
-        ps.synchronize()
+                            rlay.blob_bytes[t], cs[slot].cuda_stream)
+            plan.unpack(side.dst_cache, int(layer), 1, dev[slot], plan.layer_bytes, cs[slot].cuda_stream)
+        cs[0].synchronize()
+        cs[1].synchronize()
         recv_t.append(time.perf_counter() - t_a)
     out["layer_frames"] = {
         "frame_bytes": int(lay.total_bytes), "metadata_bytes": int(lay.total_bytes - payload),
@@ -844,6 +846,7 @@ def leg_staging(c, out):
         stg = kvt.Stager(0, nbytes, 2)
         bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
         ps = torch.cuda.Stream()
+        cs = [torch.cuda.Stream(), torch.cuda.Stream()]
         d2h_t, h2d_t = [], []
         for phase in range(4):          # first phase warms up
             torch.cuda.synchronize()
@@ -862,10 +865,13 @@ def leg_staging(c, out):
             torch.cuda.synchronize()
             a = time.perf_counter()
             for g in range(n_groups):
+                # a consumer stream per slot: a load waits for what was queued on its consumer
+                # stream, which then is the slot's last unpack and not the other slot's
                 slot = g % 2
-                stg.load(slot, bufs[slot], nbytes, ps.cuda_stream)
-                plan.unpack(side.dst_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
-            ps.synchronize()
+                stg.load(slot, bufs[slot], nbytes, cs[slot].cuda_stream)
+                plan.unpack(side.dst_cache, g * group, group, bufs[slot], lbytes, cs[slot].cuda_stream)
+            cs[0].synchronize()
+            cs[1].synchronize()
             h2d_t.append(time.perf_counter() - a)
         d2h_s, h2d_s = statistics.median(d2h_t[1:]), statistics.median(h2d_t[1:])
         pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * group * n_groups

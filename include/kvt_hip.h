@@ -660,7 +660,12 @@ int kvt_stager_save(kvt_stager* s, uint32_t slot, const void* dev, uint64_t byte
 /* Same, to byte `slot_offset` of the slot (e.g. the blob area of a frame). */
 int kvt_stager_save_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, const void* dev,
                        uint64_t bytes, void* producer_stream);
-/* Slot -> device on the copy stream, then makes consumer_stream wait for it. */
+/* Slot -> device on the copy stream, then makes consumer_stream wait for it. The copy
+ * itself first waits for everything queued on consumer_stream so far (the device buffer may
+ * still be read there). A caller that alternates between two device buffers therefore gives
+ * each its own consumer stream: on a shared one the copy for one buffer would also wait for
+ * the kernels reading the other, and transfer and kernels would take turns (about 2 % of the
+ * PCIe rate for 1 GiB transfers). */
 int kvt_stager_load(kvt_stager* s, uint32_t slot, void* dev, uint64_t bytes,
                     void* consumer_stream);
 int kvt_stager_load_at(kvt_stager* s, uint32_t slot, uint64_t slot_offset, void* dev,

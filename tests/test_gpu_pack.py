@@ -968,6 +968,43 @@ def test_stager_save_load_round_trip_overlapped_with_packing():
     stager.close()
 
 
+def test_stager_loads_with_a_consumer_stream_per_slot():
+    """Two device buffers, each with its own consumer stream and no host synchronisation with the
+    kernels: a load into a buffer waits for the unpack that last read it, and only for that."""
+    w = workloads.llama70b_flashinfer(n_layers=8, pool=96, n_req=3, tokens=400)
+    plan, lists = pipeline.build_plan(w, 0)
+    src_layers = _make_caches(w, "src", 31)
+    dst_layers = _make_caches(w, "dst", 32, fill=False)
+    sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
+    dc = kvt_amd.Cache(0, dst_layers, w.capacities("dst"))
+    nbytes = plan.layer_bytes
+    packed = torch.zeros(w.n_layers * nbytes, dtype=torch.uint8, device="cuda")
+    plan.pack(sc, 0, w.n_layers, packed, nbytes, 0)
+    torch.cuda.synchronize()
+    store = packed.cpu().numpy().reshape(w.n_layers, nbytes)
+    stager = kvt_amd.Stager(0, nbytes, 2)
+    dev_buf = [torch.zeros(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for l in range(w.n_layers):
+        slot = l % 2
+        if l >= 2:
+            stager.wait(slot)                     # the slot's last transfer has left the host memory
+        stager.slot_array(slot, nbytes)[:] = store[l]
+        stager.load(slot, dev_buf[slot], nbytes, streams[slot].cuda_stream)
+        plan.unpack(dc, l, 1, dev_buf[slot], nbytes, streams[slot].cuda_stream)
+    streams[0].synchronize()
+    streams[1].synchronize()
+    o_runs = _oracle_lists(w)[0]
+    heads, ntpb, row = w.xform
+    B = 2 * heads * ntpb * row
+    ids = np.concatenate([np.arange(r[0] // B, (r[0] + r[2]) // B) for r in o_runs]).astype(np.int64)
+    dst_ids = np.concatenate([np.arange(r[1] // B, (r[1] + r[2]) // B) for r in o_runs]).astype(np.int64)
+    for l in range(w.n_layers):
+        got = _host(dst_layers[l][0]).reshape(-1, B)
+        assert np.array_equal(got[dst_ids], _host(src_layers[l][0]).reshape(-1, B)[ids]), l
+    stager.close()
+
+
 def test_measure_pcie_reports_a_plausible_rate():
     lib = kvt_amd.lib()
     for direction in (0, 1):
