@@ -58,7 +58,7 @@ def test_plan_builder_under_sanitizers(tmp_path):
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
            "-I", os.path.join(ROOT, "include"), "-I", CSRC,
            os.path.join(ROOT, "tests", "plan_fuzz.cpp")]
-    cmd += [os.path.join(CSRC, s) for s in ["kvt_plan.hip", "kvt_runtime.hip", "kvt_kernels.hip", "kvt_object_ring.hip"] + HOST_SOURCES]
+    cmd += [os.path.join(CSRC, s) for s in ["kvt_plan.hip", "kvt_runtime.hip", "kvt_kernels.hip", "kvt_object_ring.hip", "kvt_dropin.hip"] + HOST_SOURCES]
     cmd += ["-o", exe]
     subprocess.run(cmd, check=True, capture_output=True)
     # (no leak check: the HIP runtime keeps its own allocations for the life of the process)
