@@ -94,15 +94,21 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                               uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
                               bool temporal, uint32_t* tickets, hipStream_t stream);
-// The capped launch of a plain table with 16-byte aligned entries of at most 16 KiB
-// (sub_shift 2) or 32 KiB (sub_shift 3): `wgs` persistent workgroups (a multiple of 8), one
-// table entry per trip, software-pipelined. Every address and length involved must be a
-// multiple of 16.
+// The capped launch of a plain table with 16-byte aligned entries (sub_shift 0 ... 3: at most
+// 4 ... 32 KiB): `wgs` persistent workgroups (a multiple of 8), software-pipelined, one table
+// entry per trip and workgroup (16 or 32 KiB) or per wavefront (4 or 8 KiB). Every address and
+// length involved must be a multiple of 16.
 hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                const BlobOffsets& blobs, uint32_t wgs, uint32_t* tickets,
                                hipStream_t stream);
+// ... of a table that travels in the kernel arguments (no tickets)
+hipError_t launch_copy_entries_small(bool pack, const SmallTable& table, uint32_t n_chunks,
+                                     uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
+                                     uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
+                                     uint64_t layer_stride, const BlobOffsets& blobs, uint32_t wgs,
+                                     hipStream_t stream);
 // tickets (all the pipelined launchers): nine zeroed 32-bit counters 128 bytes apart that no other
 // running launch uses, from which the workgroups take their work in order (they leave them
 // zeroed again); nullptr: every workgroup strides through a fixed share of the work.

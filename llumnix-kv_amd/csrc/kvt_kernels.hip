@@ -201,25 +201,48 @@ struct EntryWalk {
 
 // Three register sets in rotation: the loads of item k+1 are issued before the stores of item k,
 // and a set is loaded again only two trips after its stores were issued.
-#define KVT_ROTATE3(NEXT, LOAD, STORE) \
+// The compiler may reorder loads and stores that cannot alias, and it does: in some stages it
+// issues a trip's stores in front of the loads that were to overlap them (it also sinks loads
+// from a __restrict__ pointer behind the loop's exit test). FENCE pins the order as written;
+// it needs the loads' base not to be a __restrict__ pointer. Measured, the pinned order gains
+// 1-2 % on the plain tables (a changed kernel body had lost 5 % to a worse reordering) and
+// loses 2 % on the strided ones at one workgroup per CU, which therefore stay as the compiler
+// arranges them.
+#define KVT_ISSUE_FENCE()              \
   do {                                 \
-    if (!NEXT(0)) break;               \
-    LOAD(0);                           \
-    for (;;) {                         \
-      const bool l1 = NEXT(1);         \
-      LOAD(1);                         \
-      STORE(0);                        \
-      if (!l1) break;                  \
-      const bool l2 = NEXT(2);         \
-      LOAD(2);                         \
-      STORE(1);                        \
-      if (!l2) break;                  \
-      const bool l0 = NEXT(0);         \
-      LOAD(0);                         \
-      STORE(2);                        \
-      if (!l0) break;                  \
-    }                                  \
+    asm volatile("" ::: "memory");     \
+    __builtin_amdgcn_sched_barrier(0); \
   } while (0)
+#define KVT_NO_FENCE() \
+  do {                 \
+  } while (0)
+#define KVT_ROTATE3_WITH(NEXT, LOAD, STORE, FENCE) \
+  do {                                             \
+    if (!NEXT(0)) break;                           \
+    LOAD(0);                                       \
+    for (;;) {                                     \
+      const bool l1 = NEXT(1);                     \
+      LOAD(1);                                     \
+      FENCE();                                     \
+      STORE(0);                                    \
+      FENCE();                                     \
+      if (!l1) break;                              \
+      const bool l2 = NEXT(2);                     \
+      LOAD(2);                                     \
+      FENCE();                                     \
+      STORE(1);                                    \
+      FENCE();                                     \
+      if (!l2) break;                              \
+      const bool l0 = NEXT(0);                     \
+      LOAD(0);                                     \
+      FENCE();                                     \
+      STORE(2);                                    \
+      FENCE();                                     \
+      if (!l0) break;                              \
+    }                                              \
+  } while (0)
+#define KVT_ROTATE3(NEXT, LOAD, STORE) KVT_ROTATE3_WITH(NEXT, LOAD, STORE, KVT_NO_FENCE)
+#define KVT_ROTATE3_PINNED(NEXT, LOAD, STORE) KVT_ROTATE3_WITH(NEXT, LOAD, STORE, KVT_ISSUE_FENCE)
 
 constexpr int kBatch = 4;
 // How a chunk kernel walks its items: one workgroup per (slice, layer); a capped grid striding
@@ -469,15 +492,13 @@ __device__ __forceinline__ rsrc_t make_rsrc(const uint8_t* base, uint32_t bytes)
 // cache-policy operand of the buffer builtins: bit 0 = sc0, bit 1 = nt, bit 4 = sc1
 constexpr int kLoadPolicy = 2, kStorePolicy = 1 | 2 | 16;
 
-template <bool PACK, int V>
-__global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
-    const Chunk* __restrict__ chunks, uint32_t n_chunks,
-    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    uint32_t* tickets) {
+template <bool PACK, int V, class Fetch>
+__device__ __forceinline__ void copy_entries(
+    Fetch fetch_table, uint32_t n_chunks, uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors,
+    uint32_t first_layer, uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+    const BlobOffsets& blobs, uint32_t* tickets) {
   EntryWalk walk(n_chunks, n_layers, tickets, V == 8 ? 3u : 2u);
   const uint32_t off = threadIdx.x << 4;
-  const Entry* table = reinterpret_cast<const Entry*>(chunks);
   rsrc_t src[3], dst[3];
   u32x4 r[3][V];
   // this workgroup's next entry as two descriptors (empty ones past the end); false past the end
@@ -485,7 +506,7 @@ __global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
     uint32_t item, lay;
     bool valid;
     const bool live = walk.next(item, lay, valid);
-    const Entry c = table[item];
+    const Entry c = fetch_table(item);
     uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
     uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed;
     const uint32_t bytes = valid ? c.len : 0u;
@@ -503,8 +524,102 @@ __global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(
     for (int v = 0; v < V; ++v)
       __builtin_amdgcn_raw_buffer_store_b128(r[k][v], dst[k], off + (v << kSliceShift), 0, kStorePolicy);
   };
-  KVT_ROTATE3(next, load, store);
+  KVT_ROTATE3_PINNED(next, load, store);
   walk.leave();
+}
+
+#define KVT_ENTRIES_PARAMS                                                                         \
+  uint32_t n_chunks, uint8_t *const *__restrict__ layer_ptrs, uint32_t n_tensors,                  \
+      uint32_t first_layer, uint32_t n_layers, uint8_t *packed, uint64_t layer_stride, \
+      BlobOffsets blobs, uint32_t *tickets
+#define KVT_ENTRIES_ARGS n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
+
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void copy_entries_kernel(const Chunk* __restrict__ chunks,
+                                                                  KVT_ENTRIES_PARAMS) {
+  // read field by field: as one 32-byte load, a gather by fewer workgroups than CUs lost 4-7 %
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  copy_entries<PACK, V>([&](uint32_t e) { return table[e]; }, KVT_ENTRIES_ARGS);
+}
+// ... of a table that travels in the kernel arguments
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void copy_entries_small_kernel(const SmallTable table,
+                                                                        KVT_ENTRIES_PARAMS) {
+  copy_entries<PACK, V>([&](uint32_t e) { return entry_of(fetch_entry(table.c, e)); }, KVT_ENTRIES_ARGS);
+}
+
+// The same for tables with entries of 4 or 8 KiB (V = 4 or 8 vectors per lane of ONE wavefront):
+// with a whole workgroup per entry a lane would hold a single vector or two per trip, and the
+// trip's scalar work (walk, table entry, layer pointer, descriptors), which every wavefront
+// repeats, would outweigh them. Here a trip takes 4 U entries and wavefront w of the workgroup
+// moves the U of them at positions w, w + 4, ... by itself, so it prepares only those.
+template <bool PACK, int V, int U, class Fetch>
+__device__ __forceinline__ void copy_entries_by_wave(
+    Fetch fetch_table, uint32_t n_chunks, uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors,
+    uint32_t first_layer, uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+    const BlobOffsets& blobs, uint32_t* tickets) {
+  EntryWalk walk(n_chunks, n_layers, tickets, V == 8 ? 1u : 0u);
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t off = (threadIdx.x & 63u) << 4;
+  rsrc_t src[3][U], dst[3][U];
+  u32x4 r[3][U][V];
+  auto next = [&](int k) -> bool {
+    bool live = false;
+    uint32_t b[4 * U], l[4 * U];
+    bool ok[4 * U];
+#pragma unroll
+    for (int j = 0; j < 4 * U; ++j) {
+      const bool more = walk.next(b[j], l[j], ok[j]);
+      if (j == 0) live = more;
+    }
+    uint32_t item[U], lay[U];
+    bool valid[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {  // this wavefront's of the trip's entries (uniform selects)
+      item[u] = b[4 * u], lay[u] = l[4 * u], valid[u] = ok[4 * u];
+#pragma unroll
+      for (int w = 1; w < 4; ++w)
+        if (wave == static_cast<uint32_t>(w)) item[u] = b[4 * u + w], lay[u] = l[4 * u + w], valid[u] = ok[4 * u + w];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const Entry c = fetch_table(item[u]);
+      uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay[u]) * n_tensors + c.tensor()] + c.cache;
+      uint8_t* pk = packed + lay[u] * layer_stride + blobs.off[c.tensor()] + c.packed;
+      const uint32_t bytes = valid[u] ? c.len : 0u;
+      src[k][u] = make_rsrc(PACK ? cache : pk, bytes);
+      dst[k][u] = make_rsrc(PACK ? pk : cache, bytes);
+    }
+    return live;
+  };
+  auto load = [&](int k) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int v = 0; v < V; ++v)
+        r[k][u][v] = __builtin_amdgcn_raw_buffer_load_b128(src[k][u], off + (v << 10), 0, kLoadPolicy);
+  };
+  auto store = [&](int k) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int v = 0; v < V; ++v)
+        __builtin_amdgcn_raw_buffer_store_b128(r[k][u][v], dst[k][u], off + (v << 10), 0, kStorePolicy);
+  };
+  KVT_ROTATE3_PINNED(next, load, store);
+  walk.leave();
+}
+
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void copy_entries_by_wave_kernel(const Chunk* __restrict__ chunks,
+                                                                          KVT_ENTRIES_PARAMS) {
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  copy_entries_by_wave<PACK, V, U>([&](uint32_t e) { return table[e]; }, KVT_ENTRIES_ARGS);
+}
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void copy_entries_by_wave_small_kernel(const SmallTable table,
+                                                                                KVT_ENTRIES_PARAMS) {
+  copy_entries_by_wave<PACK, V, U>([&](uint32_t e) { return entry_of(fetch_entry(table.c, e)); }, KVT_ENTRIES_ARGS);
 }
 
 // The same pipeline for tables whose cache side is not contiguous (strided records, the
@@ -1009,24 +1124,46 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
   return hipGetLastError();
 }
 
+// One entry per workgroup and trip (entries of 16 or 32 KiB), or per wavefront (4 or 8 KiB: two
+// entries of 4 KiB or one of 8 KiB per wavefront and trip; more per trip, or five register
+// sets, were slower from one workgroup per CU on).
+#define KVT_LAUNCH_ENTRIES(LARGE, BY_WAVE, TABLE)                                                   \
+  do {                                                                                              \
+    const dim3 grid(wgs), block(kThreads);                                                          \
+    switch ((sub_shift << 1) | (pack ? 1u : 0u)) {                                                  \
+      case 0: hipLaunchKernelGGL((BY_WAVE<false, 4, 2>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break; \
+      case 1: hipLaunchKernelGGL((BY_WAVE<true, 4, 2>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break;  \
+      case 2: hipLaunchKernelGGL((BY_WAVE<false, 8, 1>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break; \
+      case 3: hipLaunchKernelGGL((BY_WAVE<true, 8, 1>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break;  \
+      case 4: hipLaunchKernelGGL((LARGE<false, 4>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break;      \
+      case 5: hipLaunchKernelGGL((LARGE<true, 4>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break;       \
+      case 6: hipLaunchKernelGGL((LARGE<false, 8>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break;      \
+      default: hipLaunchKernelGGL((LARGE<true, 8>), grid, block, 0, stream, TABLE, KVT_ENTRIES_ARGS); break;      \
+    }                                                                                               \
+  } while (0)
+
 hipError_t launch_copy_entries(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                const BlobOffsets& blobs, uint32_t wgs, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
-  if ((sub_shift != 2 && sub_shift != 3) || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
-  const dim3 grid(wgs), block(kThreads);
-#define KVT_ARGS chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
-  if (sub_shift == 3) {
-    if (pack) hipLaunchKernelGGL((copy_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);
-    else hipLaunchKernelGGL((copy_entries_kernel<false, 8>), grid, block, 0, stream, KVT_ARGS);
-  } else {
-    if (pack) hipLaunchKernelGGL((copy_entries_kernel<true, 4>), grid, block, 0, stream, KVT_ARGS);
-    else hipLaunchKernelGGL((copy_entries_kernel<false, 4>), grid, block, 0, stream, KVT_ARGS);
-  }
-#undef KVT_ARGS
+  if (sub_shift > 3 || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+  KVT_LAUNCH_ENTRIES(copy_entries_kernel, copy_entries_by_wave_kernel, chunks);
   return hipGetLastError();
 }
+
+hipError_t launch_copy_entries_small(bool pack, const SmallTable& table, uint32_t n_chunks,
+                                     uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
+                                     uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
+                                     uint64_t layer_stride, const BlobOffsets& blobs, uint32_t wgs,
+                                     hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  if (sub_shift > 3 || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+  uint32_t* const tickets = nullptr;  // a short table's launch is over before their order pays
+  KVT_LAUNCH_ENTRIES(copy_entries_small_kernel, copy_entries_by_wave_small_kernel, table);
+  return hipGetLastError();
+}
+#undef KVT_LAUNCH_ENTRIES
 
 // V slices per trip and the parts an entry is taken in, for entries of 4096 << sub_shift bytes.
 static bool entries_shape(uint32_t sub_shift, uint32_t wgs, int max_v, int* v, uint32_t* part_shift) {

@@ -616,6 +616,25 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   for (uint32_t t = 0; t < p->n_tensors; ++t) payload += p->tensor_bytes[t];
   const bool temporal = payload * n_layers <= copy_cached_load_max_bytes();
   if (p->small) {
+    // Under a limit, a 16-byte aligned table goes entry by entry through persistent workgroups
+    // like a resident one (below), as soon as there is more than one entry per workgroup
+    // (a 64 MiB request, 64 entries x 32 layers, TB/s pack / unpack against the strided loop of
+    // the chunk kernel: half the device 4.6 / 4.4 against 4.4 / 4.2, a quarter 4.8 / 4.8 against
+    // 4.7 / 4.0, an eighth 4.7 / 4.8 against 4.2 / 3.1, a sixteenth 4.2 / 4.0 against 2.5 / 1.9).
+    const uint32_t cus = device_cu_count(cache->device) & ~7u;
+    if (max_wgs != 0 && p->all16 && cache->aligned16 && p->sub_shift <= 3 && cus >= 8) {
+      uint64_t mis = reinterpret_cast<uintptr_t>(packed) | (n_layers > 1 ? layer_stride : 0);
+      for (uint32_t t = 0; t < p->n_tensors; ++t) mis |= blobs.off[t];
+      const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, p->sub_shift <= 1 ? 2 * cus : cus));
+      if ((mis & 15u) == 0 && p->n_chunks * n_layers > wgs) {
+        const hipError_t e = launch_copy_entries_small(
+            pack, pack ? p->small_pack : p->small_unpack, static_cast<uint32_t>(p->n_chunks),
+            p->sub_shift, cache->dev_ptrs, p->n_tensors, first_layer, n_layers,
+            static_cast<uint8_t*>(packed), layer_stride, blobs, wgs, s);
+        if (e != hipSuccess) return hip_fail(e, pack ? "pack launch" : "unpack launch");
+        return KVT_OK;
+      }
+    }
     // No tickets for a short table: the launch is over before their order pays (a 64 MiB
     // request at half the device: 31 -> 44 us with them); the pipelined loop does pay below
     // half the device (a quarter: 35 -> 30 us, an eighth: 47 -> 34 us).
@@ -648,17 +667,23 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   // A capped launch of a plain, fully 16-byte aligned table with entries of 16 or 32 KiB: one
   // persistent workgroup per CU at most (more of them were slower on MI355X: 5.5 TB/s with 256,
   // 5.3 with 512, 5.2 with 1 024), each pipelining whole entries.
+  // Entries of 4 or 8 KiB: the same with a wavefront per entry and up to two workgroups per CU
+  // (config 4, whose 36 KiB and 8 KiB blocks are cut into 4 KiB entries, TB/s pack / unpack
+  // against the strided loop of the chunk kernel: a quarter of the device 6.0 / 5.7 against
+  // 5.8 / 5.1, an eighth 5.4 / 5.4 against 4.3 / 3.6, a sixteenth 4.1 / 4.2 against 2.3 / 1.9).
+  const bool by_wave = p->sub_shift <= 1;
   if (max_wgs != 0 && p->all16 && !p->convert && !p->strided && !p->xform &&
-      (p->sub_shift == 2 || p->sub_shift == 3) && cache->aligned16 &&
-      static_cast<uint64_t>(n) * n_layers > max_wgs) {
+      p->sub_shift <= 3 && cache->aligned16 && static_cast<uint64_t>(n) * n_layers > max_wgs) {
     uint64_t mis = reinterpret_cast<uintptr_t>(packed) | (n_layers > 1 ? layer_stride : 0);
     for (uint32_t t = 0; t < p->n_tensors; ++t) mis |= blobs.off[t];
     const uint32_t cus = device_cu_count(cache->device) & ~7u;
     if ((mis & 15u) == 0 && cus >= 8) {
-      const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, cus));
+      const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, by_wave ? 2 * cus : cus));
       // fewer workgroups than CUs: each has to move more than the ticket's barrier lets it
-      // (half the CUs: 4.4 against 5.3 TB/s)
-      LaunchTickets tickets(cache->device, capturing, wgs >= cus && few_pairs);
+      // (half the CUs: 4.4 against 5.3 TB/s); a wavefront per entry: the same below two
+      // workgroups per CU (one per CU 5.1 / 5.2 with tickets, 5.4 / 5.3 without; two per CU
+      // 6.0 / 5.7 with, 5.2 / 5.2 without)
+      LaunchTickets tickets(cache->device, capturing, few_pairs && wgs >= (by_wave ? 2 * cus : cus));
       const hipError_t e = launch_copy_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                                p->n_tensors, first_layer, n_layers,
                                                static_cast<uint8_t*>(packed), layer_stride, blobs,

@@ -126,6 +126,108 @@ def test_pipelined_kernels_of_strided_transposing_and_converting_plans(usage, ch
         kvt_amd.set_copy_cu_usage(0, 1.0)
 
 
+@pytest.mark.parametrize("usage", [0.5, 0.1, 0.004], ids=["half", "tenth", "eight-workgroups"])
+@pytest.mark.parametrize("chunk", [4096, 8192])
+def test_wavefront_per_entry_kernel_of_plain_tables_with_small_entries(usage, chunk):
+    """A limited launch of a plain, 16-byte aligned table cut into entries of 4 or 8 KiB gives
+    every wavefront entries of its own. Seeded batches of arbitrary 16-byte aligned ranges: 1-3
+    tensors, 1-5 layers, lengths from 16 bytes to 70 000 (entries shorter than a wavefront's
+    reach, tables that do not fill the last trip), shuffled, enough of them for a full grid at
+    half the device (with counters) and at a tenth (without), against the oracle."""
+    kvt_amd.set_copy_cu_usage(0, usage)
+    try:
+        for seed in range(6):
+            rng = np.random.default_rng(77_000 + seed)
+            n_t, n_layers = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+            caps_s = [int(rng.integers(1 << 22, 1 << 23)) // 16 * 16 for _ in range(n_t)]
+            caps_d = [int(rng.integers(1 << 22, 1 << 23)) // 16 * 16 for _ in range(n_t)]
+            lists, all_runs = kvt_amd.BlockLists(), []
+            for t in range(n_t):
+                runs, d = [], 0
+                while len(runs) < 400:
+                    ln = int(rng.choice([16, 48, 1024, 4096, 4112, 5008, 8192, 12288, 36864, 69984]))
+                    gap = int(rng.integers(0, 4)) * 16
+                    if d + gap + ln > caps_d[t]:
+                        break
+                    s_off = int(rng.integers(0, (caps_s[t] - ln) // 16 + 1)) * 16
+                    runs.append((s_off, d + gap, ln))
+                    d += gap + ln
+                runs = [runs[i] for i in rng.permutation(len(runs))]
+                lists.append(t, runs)
+                all_runs.append(np.asarray(runs, np.uint64))
+            plan = kvt_amd.Plan(0, lists, caps_s, caps_d, chunk_bytes=chunk)
+            src = [[tp._dev_bytes(c, seed * 64 + l * 8 + t, "u8") for t, c in enumerate(caps_s)]
+                   for l in range(n_layers)]
+            dst = [[torch.full((c,), 0xA5, device="cuda", dtype=torch.uint8) for c in caps_d]
+                   for _ in range(n_layers)]
+            sc, dc = kvt_amd.Cache(0, src, caps_s), kvt_amd.Cache(0, dst, caps_d)
+            stride = plan.layer_bytes + 256
+            packed = torch.zeros(n_layers * stride, dtype=torch.uint8, device="cuda")
+            plan.pack(sc, 0, n_layers, packed, stride)
+            plan.unpack(dc, 0, n_layers, packed, stride)
+            torch.cuda.synchronize()
+            ph = tp._host(packed)
+            for l in range(n_layers):
+                for t in range(n_t):
+                    blob = checkers.oracle_pack(tp._host(src[l][t]), all_runs[t])
+                    off = l * stride + plan.tensor_offset(t)
+                    assert np.array_equal(ph[off:off + len(blob)], blob), (seed, l, t)
+                    exp = np.full(caps_d[t], 0xA5, dtype=np.uint8)
+                    checkers.oracle_unpack(exp, all_runs[t], blob)
+                    assert np.array_equal(tp._host(dst[l][t]), exp), (seed, l, t)
+            plan.close()
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+
+
+@pytest.mark.parametrize("usage", [0.1, 0.004], ids=["tenth", "eight-workgroups"])
+@pytest.mark.parametrize("chunk", [4096, 8192, 16384, 32768])
+def test_short_tables_in_kernel_arguments_entry_by_entry_under_a_limit(usage, chunk):
+    """A table of at most 64 entries travels in the kernel arguments; under a limit, with more
+    (entry, layer) pairs than workgroups, the persistent kernels read it from there. Every entry
+    size, entries shorter than the size, two tensors, 40 layers, against the oracle."""
+    kvt_amd.set_copy_cu_usage(0, usage)
+    try:
+        for seed, n_ranges in enumerate((3, 32)):
+            rng = np.random.default_rng(88_000 + seed)
+            caps = [1 << 21, 1 << 21]
+            n_layers = 40
+            lists, all_runs = kvt_amd.BlockLists(), []
+            for t in range(2):
+                runs, d = [], 0
+                for _ in range(n_ranges):
+                    ln = int(rng.choice([16, 2048, chunk - 16, chunk]))
+                    s_off = int(rng.integers(0, (caps[t] - ln) // 16)) * 16
+                    runs.append((s_off, d, ln))
+                    d += ln + int(rng.integers(0, 3)) * 16
+                runs = [runs[i] for i in rng.permutation(len(runs))]
+                lists.append(t, runs)
+                all_runs.append(np.asarray(runs, np.uint64))
+            plan = kvt_amd.Plan(0, lists, caps, caps, chunk_bytes=chunk)
+            src = [[tp._dev_bytes(c, seed * 640 + l * 8 + t, "u8") for t, c in enumerate(caps)]
+                   for l in range(n_layers)]
+            dst = [[torch.full((c,), 0x5A, device="cuda", dtype=torch.uint8) for c in caps]
+                   for _ in range(n_layers)]
+            sc, dc = kvt_amd.Cache(0, src, caps), kvt_amd.Cache(0, dst, caps)
+            stride = plan.layer_bytes
+            packed = torch.zeros(n_layers * stride, dtype=torch.uint8, device="cuda")
+            plan.pack(sc, 0, n_layers, packed, stride)
+            plan.unpack(dc, 0, n_layers, packed, stride)
+            torch.cuda.synchronize()
+            ph = tp._host(packed)
+            for l in range(n_layers):
+                for t in range(2):
+                    blob = checkers.oracle_pack(tp._host(src[l][t]), all_runs[t])
+                    off = l * stride + plan.tensor_offset(t)
+                    assert np.array_equal(ph[off:off + len(blob)], blob), (seed, l, t)
+                    exp = np.full(caps[t], 0x5A, dtype=np.uint8)
+                    checkers.oracle_unpack(exp, all_runs[t], blob)
+                    assert np.array_equal(tp._host(dst[l][t]), exp), (seed, l, t)
+            plan.close()
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+
+
 def test_more_limited_launches_in_flight_than_ticket_blocks():
     """A limited launch of the pipelined kernels borrows a block of counters until it has run.
     Thousands of launches queued without a wait outnumber the blocks: those that find none run
@@ -154,12 +256,15 @@ def test_more_limited_launches_in_flight_than_ticket_blocks():
 @pytest.mark.parametrize("usage", [0.25, 0.004], ids=["quarter", "eight-workgroups"])
 def test_limited_launches_of_every_pipelined_kernel_inside_a_graph(usage):
     """A limited launch recorded into a hipGraph keeps a block of counters of its own for every
-    replay. Plain, strided, converting and transposing plans, pack and unpack in one graph,
+    replay. Plain (entries of 32 KiB and of 4 KiB), strided, converting and transposing plans,
+    pack and unpack in one graph,
     replayed with fresh cache contents each time."""
     kvt_amd.set_copy_cu_usage(0, usage)
     try:
         cases = []
         w = workloads.llama8b_batch(n_layers=3, src_pool=700, dst_pool=900, n_req=6, min_tok=300, max_tok=1500)
+        cases.append((w, pipeline.build_plan(w, 0)[0]))
+        w = workloads.deepseek_mla(n_layers=3, pool=700, n_req=4, tokens=8192)   # 4 KiB entries
         cases.append((w, pipeline.build_plan(w, 0)[0]))
         w = workloads.tp_split("flash", 2, 1, 1, n_layers=3, src_pool=500, dst_pool=600, n_req=6,
                                min_tok=200, max_tok=1400)
