@@ -893,13 +893,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "0a177a312b5c878fa2c55fedc85795a65458519f91b1a1307181031a2f49820a"
+KERNELS_SHA256 = "a10df6406be38edac587c842a5af4777d31116983d1735f9d600e7c61a173fab"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134278132, "unpack": 134277748},
-    (2, "ranges"): {"pack": 71013083789, "unpack": 73358418543},
-    (3, "ranges"): {"pack": 85983104936, "unpack": 85983602767},
-    (4, "ranges"): {"pack": 22690383563, "unpack": 22690445045},
-    (5, "ranges"): {"pack": 45141201082, "unpack": 45141402424},
+    (1, "ranges"): {"pack": 134278348, "unpack": 134277153},
+    (2, "ranges"): {"pack": 71013098083, "unpack": 73358415712},
+    (3, "ranges"): {"pack": 85983114112, "unpack": 85983602300},
+    (4, "ranges"): {"pack": 22690381642, "unpack": 22690446879},
+    (5, "ranges"): {"pack": 45141201201, "unpack": 45141402287},
 }
 
 

@@ -12,7 +12,8 @@
 //     (b % 8) * ceil(n / 8) + b / 8: each XCD then streams through one
 //     contiguous eighth of the work list instead of touching every page.
 // A launch limited to a share of the device runs instead as a few persistent workgroups (at
-// best one per CU) that pipeline whole table entries over three register sets and take them
+// best one per CU) that pipeline whole table entries over three register sets (an entry per
+// workgroup, or per wavefront where entries are 4 or 8 KiB) and take them
 // in order from one counter per XCD: what keeps such a launch fast is that the addresses in
 // flight stay in one narrow window, as the order of dispatch keeps them in the unlimited shape.
 // No MFMA, and LDS only to hand a ticket to the wavefronts of a workgroup: the HND<->NHD
