@@ -65,11 +65,13 @@ def build_workload(cfg, scale):
         return [W.qwen3next_tp_split(2, 1, 0, n_layers=max(2, int(12 * scale)),
                                      pool=max(16, int(1024 * scale)),
                                      n_req=max(2, int(128 * scale)))]
-    if cfg in (6, 7, 8):
+    if cfg in (6, 7, 8, 11):
         # TP-remapping batches (not among the baseline configurations): config 2's batch with
         # the sender on TP2 and the receiver on TP1 (6), TP1 -> TP2 on the ragged layout (7),
-        # TP2 -> TP1 on FlashInfer HND pages (8: per-head rows, whole segments of 4 KiB)
-        layout, p_tp, d_tp = {6: ("flash", 2, 1), 7: ("ragged", 1, 2), 8: ("hnd", 2, 1)}[cfg]
+        # TP2 -> TP1 on FlashInfer HND pages (8: per-head rows, whole segments of 4 KiB),
+        # TP8 -> TP1 (11: one KV head per sender, table entries of 4 KiB)
+        layout, p_tp, d_tp = {6: ("flash", 2, 1), 7: ("ragged", 1, 2), 8: ("hnd", 2, 1),
+                              11: ("flash", 8, 1)}[cfg]
         return [W.tp_split(layout, p_tp, d_tp, 0, n_layers=max(2, int(32 * scale)),
                            src_pool=max(1024, int(16384 * scale)),
                            dst_pool=max(1536, int(24576 * scale)), n_req=max(2, int(64 * scale)),
@@ -563,11 +565,11 @@ def leg_launchers(c, out):
 
 
 def leg_fp8_plan(c, out):
-    """Config 6 only (TP2 -> TP1): the same batch with an fp8 receiver. The sender's plan
+    """Configs 6 and 11 only (TP2 / TP8 -> TP1): the same batch with an fp8 receiver. The sender's plan
     converts bf16 to fp8 while it gathers (per-token arithmetic still in the kernel); checked
     against the oracle on the first layer."""
     torch, np, kvt, lib, args, pipeline = c.torch, c.np, c.kvt, c.lib, c.args, c.pipeline
-    if args.config != 6 or args.plan != "runs":
+    if args.config not in (6, 11) or args.plan != "runs":
         return
     import dataclasses
     sys.path.insert(0, os.path.join(ROOT, "tests"))
@@ -1175,7 +1177,7 @@ def main():
                     help="0 (default): the headline configuration 2 as the JSON line, followed by "
                          "the other four baseline configurations as rows of its \"configs\" list; "
                          "1-5: that baseline configuration alone (1 = the CPU-runnable case, 2 = "
-                         "the headline); 6-8: TP-remapping batches; 9: config 5 with the "
+                         "the headline); 6-8, 11: TP-remapping batches; 9: config 5 with the "
                          "reference's uniform 2 MiB pages; 10: the same model TP2 -> TP1")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging)")
     ap.add_argument("--chunk-bytes", type=int, default=0)

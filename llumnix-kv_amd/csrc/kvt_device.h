@@ -120,8 +120,14 @@ hipError_t launch_strided_entries(bool pack, const Chunk* chunks, uint32_t n_chu
                                   uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
                                   const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
                                   uint32_t* tickets, hipStream_t stream);
-// ... and for the converting gather (entries a multiple of 16 elements long; sub_shift 1 ... 7;
-// strided entries also from sub_shift 1).
+// ... strided tables with entries of 4 or 8 KiB (sub_shift 0 or 1): a wavefront per entry
+hipError_t launch_strided_entries_by_wave(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                          uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                          uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                          const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
+                                          uint32_t* tickets, hipStream_t stream);
+// ... and for the converting gather (entries a multiple of 16 elements long; sub_shift 0 ... 7,
+// at sub_shift 0 a wavefront per entry).
 hipError_t launch_convert_entries(const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
                                   uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
                                   uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,

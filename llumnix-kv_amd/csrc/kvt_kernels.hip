@@ -686,6 +686,32 @@ __device__ __forceinline__ void entries_pipeline(
 // zero, so that its vectors are all "column" (both multipliers zero), and a divisor of 1,
 // which has no 32-bit reciprocal, adds the dividend itself instead.
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+// The lane's V cache-side offsets for the vectors at packed offsets begin + lane + (v << VSHIFT)
+// of a strided (or, shape 0, contiguous) entry.
+template <bool PACK, int V, int VSHIFT>
+__device__ __forceinline__ void strided_offsets(const StrideTable& shapes, const Entry& c, uint32_t begin,
+                                                uint32_t bytes, uint32_t lane, uint32_t* coff) {
+  const bool plain = c.shape == 0;
+  const u32x16 raw = *reinterpret_cast<const u32x16*>(&shapes.shape[plain ? 0u : c.shape - 1u]);
+  // words of a StrideShape: 0 vlen, 1 inv_vlen, 2 n_inner, 4 + 2 side: outer, 8 + 2 side: inner,
+  // 12 inv_inner (low halves of the strides: the entry spans less than 2 GiB)
+  const uint32_t vlen = plain ? 0u : raw[0];
+  const uint32_t rec_mul = plain || raw[0] == 1u ? 0u : raw[1], rec_add = !plain && raw[0] == 1u ? 1u : 0u;
+  const uint32_t n_inner = plain ? 1u : raw[2];
+  const uint32_t o_mul = raw[12], o_add = n_inner == 1u ? 1u : 0u;
+  const uint32_t outer = raw[PACK ? 4 : 6], inner = raw[PACK ? 8 : 10];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    const uint32_t at = lane + (v << VSHIFT);
+    const uint32_t vi = (begin + at) >> 4;  // vector index inside the entry, < 2^15
+    const uint32_t rec = __umulhi(vi, rec_mul) + vi * rec_add;
+    const uint32_t col = vi - rec * vlen;
+    const uint32_t o = __umulhi(rec, o_mul) + rec * o_add;
+    const uint32_t i = rec - o * n_inner;
+    coff[v] = at < bytes ? o * outer + i * inner + (col << 4) : kNoVector;
+  }
+}
+
 template <bool PACK, int V>
 __global__ __launch_bounds__(kThreads, 4) void strided_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
@@ -696,26 +722,73 @@ __global__ __launch_bounds__(kThreads, 4) void strided_entries_kernel(
   entries_pipeline<PACK, V>(
       chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride,
       blobs, tickets, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
-        const bool plain = c.shape == 0;
-        const u32x16 raw = *reinterpret_cast<const u32x16*>(&shapes.shape[plain ? 0u : c.shape - 1u]);
-        // words of a StrideShape: 0 vlen, 1 inv_vlen, 2 n_inner, 4 + 2 side: outer, 8 + 2 side: inner,
-        // 12 inv_inner (low halves of the strides: the entry spans less than 2 GiB)
-        const uint32_t vlen = plain ? 0u : raw[0];
-        const uint32_t rec_mul = plain || raw[0] == 1u ? 0u : raw[1], rec_add = !plain && raw[0] == 1u ? 1u : 0u;
-        const uint32_t n_inner = plain ? 1u : raw[2];
-        const uint32_t o_mul = raw[12], o_add = n_inner == 1u ? 1u : 0u;
-        const uint32_t outer = raw[PACK ? 4 : 6], inner = raw[PACK ? 8 : 10];
-#pragma unroll
-        for (int v = 0; v < V; ++v) {
-          const uint32_t at = lane + (v << kSliceShift);
-          const uint32_t vi = (begin + at) >> 4;  // vector index inside the entry, < 2^15
-          const uint32_t rec = __umulhi(vi, rec_mul) + vi * rec_add;
-          const uint32_t col = vi - rec * vlen;
-          const uint32_t o = __umulhi(rec, o_mul) + rec * o_add;
-          const uint32_t i = rec - o * n_inner;
-          coff[v] = at < bytes ? o * outer + i * inner + (col << 4) : kNoVector;
-        }
+        strided_offsets<PACK, V, kSliceShift>(shapes, c, begin, bytes, lane, coff);
       });
+}
+
+// Strided tables with entries of 4 or 8 KiB (senders or receivers on TP8: a block's share of
+// one rank is that small): a wavefront per entry, as in copy_entries_by_wave_kernel, with the
+// cache side through a 2 GiB window and per-lane offsets as above.
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void strided_entries_by_wave_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes, uint32_t* tickets) {
+  EntryWalk walk(n_chunks, n_layers, tickets, V == 8 ? 1u : 0u);
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane = (threadIdx.x & 63u) << 4;
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  rsrc_t cdesc[3][U], pdesc[3][U];
+  uint32_t coff[3][U][V];
+  u32x4 r[3][U][V];
+  auto next = [&](int k) -> bool {
+    bool live = false;
+    uint32_t b[4 * U], l[4 * U];
+    bool ok[4 * U];
+#pragma unroll
+    for (int j = 0; j < 4 * U; ++j) {
+      const bool more = walk.next(b[j], l[j], ok[j]);
+      if (j == 0) live = more;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {  // this wavefront's of the trip's entries (uniform selects)
+      uint32_t item = b[4 * u], lay = l[4 * u];
+      bool valid = ok[4 * u];
+#pragma unroll
+      for (int w = 1; w < 4; ++w)
+        if (wave == static_cast<uint32_t>(w)) item = b[4 * u + w], lay = l[4 * u + w], valid = ok[4 * u + w];
+      const Entry c = table[item];
+      uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
+      uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed;
+      const uint32_t bytes = valid ? c.len : 0u;
+      pdesc[k][u] = make_rsrc(pk, bytes);
+      cdesc[k][u] = make_rsrc(cache, bytes ? kCacheWindow : 0u);
+      strided_offsets<PACK, V, 10>(shapes, c, 0u, bytes, lane, coff[k][u]);
+    }
+    return live;
+  };
+  auto load = [&](int k) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int v = 0; v < V; ++v)
+        r[k][u][v] = PACK ? __builtin_amdgcn_raw_buffer_load_b128(cdesc[k][u], coff[k][u][v], 0, kLoadPolicy)
+                          : __builtin_amdgcn_raw_buffer_load_b128(pdesc[k][u], lane + (v << 10), 0, kLoadPolicy);
+  };
+  auto store = [&](int k) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        if (PACK)
+          __builtin_amdgcn_raw_buffer_store_b128(r[k][u][v], pdesc[k][u], lane + (v << 10), 0, kStorePolicy);
+        else
+          __builtin_amdgcn_raw_buffer_store_b128(r[k][u][v], cdesc[k][u], coff[k][u][v], 0, kStorePolicy);
+      }
+  };
+  KVT_ROTATE3(next, load, store);
+  walk.leave();
 }
 
 // The HND <-> NHD transform (index arithmetic of xform_chunks_kernel).
@@ -1067,6 +1140,81 @@ __global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
   walk.leave();
 }
 
+// Converting tables with entries of 4096 elements: a wavefront per entry (see
+// copy_entries_by_wave_kernel), lane t of the wavefront the groups t, t + 64, ... t + 448.
+template <int U>
+__global__ __launch_bounds__(kThreads, 4) void convert_entries_by_wave_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes, uint32_t* tickets) {
+  constexpr int G = 8;  // groups per lane and entry
+  EntryWalk walk(n_chunks, n_layers, tickets, 0u);
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane = threadIdx.x & 63u;
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  rsrc_t pdesc[3][U];
+  u32x4 r[3][U][G];
+  // the cache-side descriptor and the offsets are used up by the loads that follow at once
+  auto fetch = [&](int k) -> bool {
+    bool live = false;
+    uint32_t b[4 * U], l[4 * U];
+    bool ok[4 * U];
+#pragma unroll
+    for (int j = 0; j < 4 * U; ++j) {
+      const bool more = walk.next(b[j], l[j], ok[j]);
+      if (j == 0) live = more;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      uint32_t item = b[4 * u], lay = l[4 * u];
+      bool valid = ok[4 * u];
+#pragma unroll
+      for (int w = 1; w < 4; ++w)
+        if (wave == static_cast<uint32_t>(w)) item = b[4 * u + w], lay = l[4 * u + w], valid = ok[4 * u + w];
+      const Entry c = table[item];
+      uint8_t* cache = layer_ptrs[static_cast<uint64_t>(first_layer + lay) * n_tensors + c.tensor()] + c.cache;
+      uint8_t* pk = packed + lay * layer_stride + blobs.off[c.tensor()] + c.packed;
+      const uint32_t bytes = valid ? c.len : 0u;
+      pdesc[k][u] = make_rsrc(pk, bytes);
+      const rsrc_t cdesc = make_rsrc(cache, bytes ? kCacheWindow : 0u);
+      const bool plain = c.shape == 0;
+      const u32x16 raw = *reinterpret_cast<const u32x16*>(&shapes.shape[plain ? 0u : c.shape - 1u]);
+      const uint32_t vlen = plain ? 0u : raw[0];
+      const uint32_t rec_mul = plain || raw[0] == 1u ? 0u : raw[1], rec_add = !plain && raw[0] == 1u ? 1u : 0u;
+      const uint32_t n_inner = plain ? 1u : raw[2];
+      const uint32_t o_mul = raw[12], o_add = n_inner == 1u ? 1u : 0u;
+      const uint32_t outer = raw[4], inner = raw[8];
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        const uint32_t q = lane + (j << 6);  // group inside the entry
+        const uint32_t half = q >> 1;        // 16-element vector inside the entry
+        const uint32_t rec = __umulhi(half, rec_mul) + half * rec_add;
+        const uint32_t col = q - rec * (vlen << 1);
+        const uint32_t o = __umulhi(rec, o_mul) + rec * o_add;
+        const uint32_t i = rec - o * n_inner;
+        const uint32_t coff = (q << 3) < bytes ? o * outer + i * inner + (col << 4) : kNoVector;
+        r[k][u][j] = __builtin_amdgcn_raw_buffer_load_b128(cdesc, coff, 0, kLoadPolicy);
+      }
+    }
+    return live;
+  };
+  auto nothing = [&](int) {};
+  auto store = [&](int k) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int j = 0; j < G; ++j) {
+        u32x2 out;
+        out.x = cvt4(r[k][u][j].x, r[k][u][j].y);
+        out.y = cvt4(r[k][u][j].z, r[k][u][j].w);
+        __builtin_amdgcn_raw_buffer_store_b64(out, pdesc[k][u], (lane + (j << 6)) << 3, 0, kStorePolicy);
+      }
+  };
+  KVT_ROTATE3(fetch, nothing, store);
+  walk.leave();
+}
+
 // Plain linear copy with the gather kernel's slice shape (calibration / ceiling).
 __global__ __launch_bounds__(kThreads) void copy_linear_kernel(uint8_t* __restrict__ dst,
                                                                const uint8_t* __restrict__ src,
@@ -1192,8 +1340,27 @@ hipError_t launch_strided_entries(bool pack, const Chunk* chunks, uint32_t n_chu
     if (pack) hipLaunchKernelGGL((strided_entries_kernel<true, 4>), grid, block, 0, stream, KVT_ARGS);
     else hipLaunchKernelGGL((strided_entries_kernel<false, 4>), grid, block, 0, stream, KVT_ARGS);
   } else {
-    if (pack) hipLaunchKernelGGL((strided_entries_kernel<true, 2>), grid, block, 0, stream, KVT_ARGS);
-    else hipLaunchKernelGGL((strided_entries_kernel<false, 2>), grid, block, 0, stream, KVT_ARGS);
+    return hipErrorInvalidValue;  // entries of 4 or 8 KiB: launch_strided_entries_by_wave
+  }
+#undef KVT_ARGS
+  return hipGetLastError();
+}
+
+hipError_t launch_strided_entries_by_wave(bool pack, const Chunk* chunks, uint32_t n_chunks, uint32_t sub_shift,
+                                          uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                                          uint32_t n_layers, uint8_t* packed, uint64_t layer_stride,
+                                          const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
+                                          uint32_t* tickets, hipStream_t stream) {
+  if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  if (sub_shift > 1 || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+  const dim3 grid(wgs), block(kThreads);
+#define KVT_ARGS chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets
+  if (sub_shift == 0) {
+    if (pack) hipLaunchKernelGGL((strided_entries_by_wave_kernel<true, 4, 2>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((strided_entries_by_wave_kernel<false, 4, 2>), grid, block, 0, stream, KVT_ARGS);
+  } else {
+    if (pack) hipLaunchKernelGGL((strided_entries_by_wave_kernel<true, 8, 1>), grid, block, 0, stream, KVT_ARGS);
+    else hipLaunchKernelGGL((strided_entries_by_wave_kernel<false, 8, 1>), grid, block, 0, stream, KVT_ARGS);
   }
 #undef KVT_ARGS
   return hipGetLastError();
@@ -1205,10 +1372,16 @@ hipError_t launch_convert_entries(const Chunk* chunks, uint32_t n_chunks, uint32
                                   const BlobOffsets& blobs, const StrideTable& shapes, uint32_t wgs,
                                   uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
+  const dim3 grid(wgs), block(kThreads);
+  if (sub_shift == 0) {  // entries of 4096 elements: a wavefront each
+    if (wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((convert_entries_by_wave_kernel<1>), grid, block, 0, stream, chunks, n_chunks, layer_ptrs,
+                       n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets);
+    return hipGetLastError();
+  }
   int v = 0;
   uint32_t part_shift = 0;
   if (!entries_shape(sub_shift, wgs, 4, &v, &part_shift)) return hipErrorInvalidValue;
-  const dim3 grid(wgs), block(kThreads);
 #define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets
   if (v == 4) hipLaunchKernelGGL((convert_entries_kernel<4>), grid, block, 0, stream, KVT_ARGS);
   else hipLaunchKernelGGL((convert_entries_kernel<2>), grid, block, 0, stream, KVT_ARGS);

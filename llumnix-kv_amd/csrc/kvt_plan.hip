@@ -701,9 +701,14 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   // against the strided loop of the chunk kernels (`for_items`), TB/s pack / unpack on the
   // TP2 -> TP1 batch: half the device 5.9 / 5.9 against 5.8 / 5.9, a quarter 5.9 / 5.9 against
   // 4.4 / 4.2, an eighth 5.9 / 5.8 against 2.5 / 2.4; the converting gather (bytes read and
-  // written) 5.9 against 4.3 at one half.
+  // written) 5.9 against 4.3 at one half. Strided entries of 4 or 8 KiB and converting ones of
+  // 4096 elements (a sender on TP8: one KV head per rank) go a wavefront per entry, TB/s on a
+  // TP8 -> TP1 batch: a quarter 5.6 / 5.3 against 4.0 / 3.6, an eighth 5.5 / 5.1 against
+  // 2.5 / 2.2, a sixteenth 3.3 / 3.7 against 1.3 / 1.1; converting gather at a quarter 4.2
+  // against 1.9, at an eighth 3.2 against 1.1.
   const bool converting = p->convert && pack;
-  const uint32_t min_shift = p->xform ? 2u : 1u;  // entries of at least 8 KiB (transposing: 16 KiB)
+  const bool strided_by_wave = p->strided && !converting && !p->xform && p->sub_shift <= 1;
+  const uint32_t min_shift = p->xform ? 2u : 0u;  // transposing: entries of at least 16 KiB
   if (max_wgs != 0 && p->all16 && p->near &&
       (p->strided || p->xform || converting) && !words && p->sub_shift >= min_shift &&
       p->sub_shift <= 7 && cache->aligned16 && static_cast<uint64_t>(n) * n_layers > max_wgs) {
@@ -712,7 +717,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
     const uint32_t cus = device_cu_count(cache->device) & ~7u;
     if ((mis & 15u) == 0 && cus >= 8) {
       // one workgroup per CU; two where a trip moves only 8 KiB
-      const uint32_t per_cu = p->sub_shift == 1 ? 2u : 1u;
+      const uint32_t per_cu = p->sub_shift <= 1 ? 2u : 1u;
       const uint32_t wgs = std::max(8u, std::min(max_wgs & ~7u, per_cu * cus));
       uint8_t* const pk = static_cast<uint8_t*>(packed);
       // trips of 8 KiB by a single workgroup per CU are better off without the ticket's barrier
@@ -721,6 +726,9 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       LaunchTickets tickets(cache->device, capturing,
                             wgs >= cus && few_pairs && (p->sub_shift >= 2 || wgs >= 2 * cus));
       const hipError_t e =
+          strided_by_wave ? launch_strided_entries_by_wave(pack, table, n, p->sub_shift, cache->dev_ptrs,
+                                              p->n_tensors, first_layer, n_layers, pk, layer_stride, blobs,
+                                              p->shapes, wgs, tickets.block, s) :
           converting ? launch_convert_entries(table, n, p->sub_shift, cache->dev_ptrs, p->n_tensors,
                                               first_layer, n_layers, pk, layer_stride, blobs,
                                               p->shapes, wgs, tickets.block, s)

@@ -100,16 +100,16 @@ def test_sessions_and_graphs_under_a_limit(limited):
 
 
 @pytest.mark.parametrize("usage", [0.25, 0.1, 0.004], ids=["quarter", "tenth", "eight-workgroups"])
-@pytest.mark.parametrize("chunk", [0, 8192, 16384, 32768, 65536, 524288])
+@pytest.mark.parametrize("chunk", [0, 4096, 8192, 16384, 32768, 65536, 524288])
 def test_pipelined_kernels_of_strided_transposing_and_converting_plans(usage, chunk):
     """Below half the device, strided, transposing and converting tables are moved by
-    persistent workgroups that take whole table entries (in parts of 8, 16 or 32 KiB) through
-    buffer descriptors with 32-bit offsets computed per lane. Batches large enough for a full
+    persistent workgroups that take whole table entries (in parts of 16 or 32 KiB; entries of
+    4 or 8 KiB: a wavefront each) through buffer descriptors with 32-bit offsets computed per lane. Batches large enough for a full
     grid of them, every entry size, both directions, against the oracle."""
     kvt_amd.set_copy_cu_usage(0, usage)
     try:
         for layout, p_tp, d_tp, rank in (("flash", 2, 1, 1), ("ragged", 4, 2, 3), ("ragged", 1, 4, 0),
-                                         ("hnd", 2, 1, 1)):
+                                         ("hnd", 2, 1, 1), ("flash", 8, 1, 3), ("ragged", 2, 8, 1)):
             w = workloads.tp_split(layout, p_tp, d_tp, rank, n_layers=4, src_pool=500, dst_pool=600,
                                    n_req=6, min_tok=200, max_tok=1400)
             plan, runs = pipeline.build_plan_runs(w, 0, chunk)
