@@ -726,15 +726,16 @@ __global__ __launch_bounds__(kThreads, 4) void strided_entries_kernel(
       });
 }
 
-// Strided tables with entries of 4 or 8 KiB (senders or receivers on TP8: a block's share of
-// one rank is that small): a wavefront per entry, as in copy_entries_by_wave_kernel, with the
-// cache side through a 2 GiB window and per-lane offsets as above.
-template <bool PACK, int V, int U>
-__global__ __launch_bounds__(kThreads, 4) void strided_entries_by_wave_kernel(
-    const Chunk* __restrict__ chunks, uint32_t n_chunks,
-    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    StrideTable shapes, uint32_t* tickets) {
+// Strided and transposing tables with entries of 4 or 8 KiB (senders or receivers on TP4 / TP8:
+// a block's share of one rank is that small): a wavefront per entry, as in
+// copy_entries_by_wave_kernel, with the cache side through a 2 GiB window and per-lane offsets.
+// `cache_offsets(entry, bytes, off)` fills the lane's V offsets for the vectors at packed
+// offsets lane * 16 + v * 1024 of the entry (lane = lane of the wavefront).
+template <bool PACK, int V, int U, class CacheOffsets>
+__device__ __forceinline__ void entries_pipeline_by_wave(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks, uint8_t* const* __restrict__ layer_ptrs,
+    uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers, uint8_t* __restrict__ packed,
+    uint64_t layer_stride, const BlobOffsets& blobs, uint32_t* tickets, CacheOffsets cache_offsets) {
   EntryWalk walk(n_chunks, n_layers, tickets, V == 8 ? 1u : 0u);
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t lane = (threadIdx.x & 63u) << 4;
@@ -764,7 +765,7 @@ __global__ __launch_bounds__(kThreads, 4) void strided_entries_by_wave_kernel(
       const uint32_t bytes = valid ? c.len : 0u;
       pdesc[k][u] = make_rsrc(pk, bytes);
       cdesc[k][u] = make_rsrc(cache, bytes ? kCacheWindow : 0u);
-      strided_offsets<PACK, V, 10>(shapes, c, 0u, bytes, lane, coff[k][u]);
+      cache_offsets(c, bytes, coff[k][u]);
     }
     return live;
   };
@@ -791,7 +792,41 @@ __global__ __launch_bounds__(kThreads, 4) void strided_entries_by_wave_kernel(
   walk.leave();
 }
 
-// The HND <-> NHD transform (index arithmetic of xform_chunks_kernel).
+#define KVT_BY_WAVE_PARAMS                                                                            \
+  const Chunk *__restrict__ chunks, uint32_t n_chunks, uint8_t *const *__restrict__ layer_ptrs,        \
+      uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers, uint8_t *__restrict__ packed,       \
+      uint64_t layer_stride, BlobOffsets blobs
+#define KVT_BY_WAVE_ARGS chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs
+
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void strided_entries_by_wave_kernel(KVT_BY_WAVE_PARAMS,
+                                                                             StrideTable shapes,
+                                                                             uint32_t* tickets) {
+  const uint32_t lane = (threadIdx.x & 63u) << 4;
+  entries_pipeline_by_wave<PACK, V, U>(KVT_BY_WAVE_ARGS, tickets,
+                                       [&](const Entry& c, uint32_t bytes, uint32_t* coff) {
+                                         strided_offsets<PACK, V, 10>(shapes, c, 0u, bytes, lane, coff);
+                                       });
+}
+
+// The HND <-> NHD transform (index arithmetic of xform_chunks_kernel): the lane's V cache-side
+// offsets for the vectors at packed offsets begin + lane + (v << VSHIFT) of an entry.
+template <int V, int VSHIFT>
+__device__ __forceinline__ void xform_offsets(const XformDev& x, const Entry& c, uint32_t begin,
+                                              uint32_t bytes, uint32_t lane, uint32_t* coff) {
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    const uint32_t at = lane + (v << VSHIFT);
+    const uint32_t vi = (begin + at) >> 4;
+    const uint32_t r = x.vrow == 1 ? vi : __umulhi(vi, x.inv_vrow);
+    const uint32_t col = vi - r * x.vrow;
+    const uint32_t t_local = x.heads == 1 ? r : __umulhi(r, x.inv_heads);
+    const uint32_t h = r - t_local * x.heads;
+    const uint32_t cidx = (h * x.ntpb + c.t0() + t_local) * x.vrow + col;
+    coff[v] = at < bytes ? cidx << 4 : kNoVector;
+  }
+}
+
 template <bool PACK, int V>
 __global__ __launch_bounds__(kThreads, 4) void xform_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
@@ -802,18 +837,18 @@ __global__ __launch_bounds__(kThreads, 4) void xform_entries_kernel(
   entries_pipeline<PACK, V>(
       chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride,
       blobs, tickets, [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
-#pragma unroll
-        for (int v = 0; v < V; ++v) {
-          const uint32_t at = lane + (v << kSliceShift);
-          const uint32_t vi = (begin + at) >> 4;
-          const uint32_t r = x.vrow == 1 ? vi : __umulhi(vi, x.inv_vrow);
-          const uint32_t col = vi - r * x.vrow;
-          const uint32_t t_local = x.heads == 1 ? r : __umulhi(r, x.inv_heads);
-          const uint32_t h = r - t_local * x.heads;
-          const uint32_t cidx = (h * x.ntpb + c.t0() + t_local) * x.vrow + col;
-          coff[v] = at < bytes ? cidx << 4 : kNoVector;
-        }
+        xform_offsets<V, kSliceShift>(x, c, begin, bytes, lane, coff);
       });
+}
+
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void xform_entries_by_wave_kernel(KVT_BY_WAVE_PARAMS, XformDev x,
+                                                                           uint32_t* tickets) {
+  const uint32_t lane = (threadIdx.x & 63u) << 4;
+  entries_pipeline_by_wave<PACK, V, U>(KVT_BY_WAVE_ARGS, tickets,
+                                       [&](const Entry& c, uint32_t bytes, uint32_t* coff) {
+                                         xform_offsets<V, 10>(x, c, 0u, bytes, lane, coff);
+                                       });
 }
 
 // Gather / scatter of a table whose chunks may be strided on the cache side:
@@ -1397,9 +1432,22 @@ hipError_t launch_xform_entries(bool pack, const Chunk* chunks, uint32_t n_chunk
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   int v = 0;
   uint32_t part_shift = 0;
-  // the scatter keeps its offsets until the stores: 8 slices per trip would not fit the registers
-  if (sub_shift < 2 || !entries_shape(sub_shift, wgs, pack ? 8 : 4, &v, &part_shift)) return hipErrorInvalidValue;
   const dim3 grid(wgs), block(kThreads);
+  if (sub_shift <= 1) {  // half pages of 4 or 8 KiB: a wavefront per entry
+    if (wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+#define KVT_ARGS chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x, tickets
+    if (sub_shift == 0) {
+      if (pack) hipLaunchKernelGGL((xform_entries_by_wave_kernel<true, 4, 2>), grid, block, 0, stream, KVT_ARGS);
+      else hipLaunchKernelGGL((xform_entries_by_wave_kernel<false, 4, 2>), grid, block, 0, stream, KVT_ARGS);
+    } else {
+      if (pack) hipLaunchKernelGGL((xform_entries_by_wave_kernel<true, 8, 1>), grid, block, 0, stream, KVT_ARGS);
+      else hipLaunchKernelGGL((xform_entries_by_wave_kernel<false, 8, 1>), grid, block, 0, stream, KVT_ARGS);
+    }
+#undef KVT_ARGS
+    return hipGetLastError();
+  }
+  // the scatter keeps its offsets until the stores: 8 slices per trip would not fit the registers
+  if (!entries_shape(sub_shift, wgs, pack ? 8 : 4, &v, &part_shift)) return hipErrorInvalidValue;
 #define KVT_ARGS chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x, tickets
   if (v == 8) {
     hipLaunchKernelGGL((xform_entries_kernel<true, 8>), grid, block, 0, stream, KVT_ARGS);

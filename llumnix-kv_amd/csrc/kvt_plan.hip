@@ -705,13 +705,12 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   // 4096 elements (a sender on TP8: one KV head per rank) go a wavefront per entry, TB/s on a
   // TP8 -> TP1 batch: a quarter 5.6 / 5.3 against 4.0 / 3.6, an eighth 5.5 / 5.1 against
   // 2.5 / 2.2, a sixteenth 3.3 / 3.7 against 1.3 / 1.1; converting gather at a quarter 4.2
-  // against 1.9, at an eighth 3.2 against 1.1.
+  // against 1.9, at an eighth 3.2 against 1.1; transposing half pages of 8 KiB (two KV heads
+  // per rank) at a quarter 6.3 / 6.1 against 5.0 / 5.1, at an eighth 5.6 / 5.6 against 3.3 / 3.2.
   const bool converting = p->convert && pack;
   const bool strided_by_wave = p->strided && !converting && !p->xform && p->sub_shift <= 1;
-  const uint32_t min_shift = p->xform ? 2u : 0u;  // transposing: entries of at least 16 KiB
   if (max_wgs != 0 && p->all16 && p->near &&
-      (p->strided || p->xform || converting) && !words && p->sub_shift >= min_shift &&
-      p->sub_shift <= 7 && cache->aligned16 && static_cast<uint64_t>(n) * n_layers > max_wgs) {
+      (p->strided || p->xform || converting) && !words && p->sub_shift <= 7 && cache->aligned16 && static_cast<uint64_t>(n) * n_layers > max_wgs) {
     uint64_t mis = reinterpret_cast<uintptr_t>(packed) | (n_layers > 1 ? layer_stride : 0);
     for (uint32_t t = 0; t < p->n_tensors; ++t) mis |= blobs.off[t];
     const uint32_t cus = device_cu_count(cache->device) & ~7u;

@@ -93,14 +93,16 @@ def llama8b_batch(n_layers=32, src_pool=16384, dst_pool=24576, n_req=64, min_tok
 
 
 def llama70b_flashinfer(n_layers=80, pool=8192, n_req=32, tokens=4096, transpose=True,
-                        seed=20253):
-    """Config 3: FlashInfer pages, HND in the cache ([pool, 2, 8, 16, 128] bf16).
+                        seed=20253, heads=8):
+    """Config 3: FlashInfer pages, HND in the cache ([pool, 2, 8, 16, 128] bf16; `heads` KV
+    heads instead of 8 for one rank of a tensor-parallel instance).
 
     transpose=True: whole-page plan (the page parse of the NHD page layout) with
     the HND->NHD transform applied while packing. transpose=False: the plain
     FlashInfer HND parse (per-head ranges, merged)."""
     rng = np.random.default_rng(seed)
-    T, ntpb, heads, row = 4096, 16, 8, 256
+    ntpb, row = 16, 256
+    T = 2 * heads * row
     src, dst = _tables(rng, n_req, [tokens] * n_req, ntpb, pool, pool)
     info = dict(block_sizes=[T * ntpb], token_sizes=[T], layer_num_blocks=pool, num_kv_heads=heads,
                 num_layers=n_layers, num_gdn_layers=0)

@@ -193,3 +193,12 @@ def assert_dispatch(parser_name, src, dst, valid=None, tp_size=None, tp_rank=Non
         exp, got_o, got_p = exp[3:], (got_o[0],) + got_o[4:], got_p[3:]
     assert got_o == (0,) + exp, ("oracle dispatch", parser_name, got_o, exp)
     assert got_p == exp, ("product dispatch", parser_name, got_p, exp)
+
+
+def side_stream():
+    """A stream of its own for a GPU test. The device is synchronized first: what the test has
+    queued on torch's default stream so far (fills, seeded contents) is not ordered against
+    work on any other stream, and a launch there could otherwise overtake it."""
+    import torch
+    torch.cuda.synchronize()
+    return torch.cuda.Stream()

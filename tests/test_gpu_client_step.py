@@ -11,6 +11,7 @@ on the layer's event on a side stream). Needs a real MI355X."""
 import numpy as np
 import pytest
 
+import checkers
 import kvt_amd
 from kvt_amd import pipeline
 from kvt_amd.channel import LoopbackChannel
@@ -26,7 +27,7 @@ KB = 1024
 def test_kernel_sync_and_data_transfer():
     num_layers, block_size, nblk = 2, 16 * KB, 128
     data_size = nblk * block_size
-    stream = torch.cuda.Stream()
+    stream = checkers.side_stream()
     layers = [torch.zeros(data_size, dtype=torch.uint8, device="cuda") for _ in range(num_layers)]
     host_layers = [torch.zeros(data_size, dtype=torch.uint8, pin_memory=True)
                    for _ in range(num_layers)]
@@ -91,7 +92,7 @@ def test_cuda_kernel_sync_over_four_steps():
     import threading
 
     num_layers, data_size = 2, 128 * (1 << 14)
-    stream = torch.cuda.Stream()
+    stream = checkers.side_stream()
     layers = [torch.zeros(data_size, dtype=torch.uint8, device="cuda") for _ in range(num_layers)]
     lists = kvt_amd.BlockLists()
     lists.append(0, [(0, 0, data_size)])

@@ -122,6 +122,11 @@ def test_pipelined_kernels_of_strided_transposing_and_converting_plans(usage, ch
             w = workloads.llama70b_flashinfer(n_layers=4, pool=400, n_req=4, tokens=1500)
             plan, lists = pipeline.build_plan(w, 0, chunk)
             tp._transposing(w, plan=plan, lists=lists)
+        if chunk in (0, 4096, 8192):     # one rank of TP4 / TP8: half pages of 8 / 4 KiB
+            for heads in (2, 1):
+                w = workloads.llama70b_flashinfer(n_layers=4, pool=1200, n_req=6, tokens=3000, heads=heads)
+                plan, lists = pipeline.build_plan(w, 0, chunk)
+                tp._transposing(w, plan=plan, lists=lists)
     finally:
         kvt_amd.set_copy_cu_usage(0, 1.0)
 
@@ -241,7 +246,7 @@ def test_more_limited_launches_in_flight_than_ticket_blocks():
     outs = [torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda") for _ in range(3)]
     kvt_amd.set_copy_cu_usage(0, 0.004)
     try:
-        stream = torch.cuda.Stream()
+        stream = checkers.side_stream()
         for i in range(3000):
             plan.pack(sc, 0, w.n_layers, outs[i % 3], stride, stream.cuda_stream)
         stream.synchronize()
@@ -285,7 +290,7 @@ def test_limited_launches_of_every_pipelined_kernel_inside_a_graph(usage):
             dst_g = tp._make_caches(w, "dst", 6, fill=False)
             de, dg = (kvt_amd.Cache(0, d, w.capacities("dst")) for d in (dst_e, dst_g))
             graph = torch.cuda.CUDAGraph()
-            cs = torch.cuda.Stream()
+            cs = checkers.side_stream()
             with torch.cuda.graph(graph, stream=cs):
                 plan.pack(sc, 0, w.n_layers, out, stride, cs.cuda_stream)
                 plan.unpack(dg, 0, w.n_layers, out, stride, cs.cuda_stream)
@@ -323,7 +328,7 @@ def test_limited_launches_of_one_plan_from_several_threads_at_once():
 
     def worker(i):
         try:
-            st = torch.cuda.Stream()
+            st = checkers.side_stream()
             for _ in range(60):
                 plan.pack(sc, 0, w.n_layers, outs[i], stride, st.cuda_stream)
             st.synchronize()

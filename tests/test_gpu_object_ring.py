@@ -6,6 +6,7 @@ and one unpack launch. Checked against torch's own kvcache[:, b] slices. Needs a
 import numpy as np
 import pytest
 
+import checkers
 import kvt_amd
 
 pytestmark = pytest.mark.gpu
@@ -72,7 +73,7 @@ def test_save_by_hash_skips_stored_blocks_and_load_restores_them_elsewhere():
     kv = _caches(5)
     cache = _cache_handle(kv)
     ring = kvt_amd.ObjectRing(0, ENTRY, 8, 16)
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     blocks1, keys1 = [7, 3, 20, 11, 0], [key(i) for i in range(5)]
     e1, new1 = _save(ring, kv, cache, blocks1, keys1, s)
     assert e1.tolist() == [0, 1, 2, 3, 4] and new1.all()
@@ -125,7 +126,7 @@ def test_objects_spaced_wider_than_an_entry_and_the_error_cases():
     kv = _caches(6)
     cache = _cache_handle(kv)
     ring = kvt_amd.ObjectRing(0, ENTRY, 4, 16)
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     blocks, keys = [4, 17, 9], [key(i) for i in (40, 41, 42)]
     e, new = _save(ring, kv, cache, blocks, keys, s, pad=4096)
     assert new.all()
@@ -173,7 +174,7 @@ def test_a_ring_that_wraps_many_times_under_overlapping_saves_and_loads():
     kv = _caches(7)
     cache = _cache_handle(kv)
     ring = kvt_amd.ObjectRing(0, ENTRY, 6, 16)
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     rng = np.random.default_rng(3)
     for step in range(40):
         blocks = rng.permutation(NBLK)[:4].tolist()

@@ -313,7 +313,7 @@ def test_short_plans_travel_in_the_kernel_arguments(n_ranges):
     sc, dc = kvt_amd.Cache(0, src, [cap]), kvt_amd.Cache(0, dst, [cap])
     stride = plan.layer_bytes
     packed = torch.zeros(2 * stride, dtype=torch.uint8, device="cuda")
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     torch.cuda.synchronize()
     if n_ranges <= 64:
         graph = torch.cuda.CUDAGraph()
@@ -410,7 +410,7 @@ def test_reference_launcher_names_link_level_stand_in():
     meta_d = torch.zeros(3 * n, dtype=torch.int64, device="cuda")
     out = torch.zeros(total, dtype=torch.uint8, device="cuda")
     torch.cuda.synchronize()
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     st = s.cuda_stream
     shim.launch_copy_int64_array_h2d_kernel(meta_h.data_ptr(), meta_d.data_ptr(), 3 * n, 2048, 512, st)
     so, do, ln = (meta_d.data_ptr() + 8 * n * k for k in range(3))
@@ -500,7 +500,7 @@ def _few_very_large_ranges(lib, expect_dma=True):
     pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
     dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
     host_meta = torch.zeros(3 * 8192, dtype=torch.int64).pin_memory()
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(), runs.ctypes.data,
                                               len(runs), total, 1, 0, s.cuda_stream,
                                               dev_meta.data_ptr(), host_meta.data_ptr(), 0)
@@ -532,7 +532,7 @@ def test_launch_copy_int64_array_h2d(n):
     host = torch.from_numpy(rng.integers(-2**62, 2**62, size=n + 1, dtype=np.int64)).pin_memory()
     dev = torch.full((n + 3,), -7, dtype=torch.int64, device="cuda")
     torch.cuda.synchronize()
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     for shift in (0, 1):
         rc = lib.kvt_launch_copy_int64_array_h2d(host.data_ptr() + 8 * shift, dev.data_ptr() + 8,
                                                  n, 0, 0, s.cuda_stream)
@@ -561,7 +561,7 @@ def test_memcpy_route_thresholds_decide_between_dma_and_kernel():
     gather = np.stack([runs[:, 1], runs[:, 1], runs[:, 2]], axis=1)
     blob = checkers.oracle_pack(_host(layer), gather)
     dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
 
     def gather_once():
         pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
@@ -609,7 +609,7 @@ def test_mixed_lists_send_their_long_ranges_to_the_dma_engines(max_block_num):
     dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
     host_meta = torch.zeros(3 * 8192, dtype=torch.int64).pin_memory()
     pinned = torch.zeros(total, dtype=torch.uint8).pin_memory()
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     try:
         assert lib.kvt_set_copy_memcpy_thresholds(1 << 20, 16) == 0
         rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(),
@@ -751,7 +751,7 @@ def test_copy_handle_data_with_kernel_pinned_host_buffer(max_block_num):
     # sender convention: kernel blocks carry the GPU offset in dst_offset (tcp_channel.cpp:538-542)
     kb = np.stack([np.zeros(n, dtype=np.uint64), runs[:, 0], runs[:, 2]], axis=1).copy()
     lib = kvt_amd.lib()
-    st = torch.cuda.Stream()
+    st = checkers.side_stream()
     rc = lib.kvt_copy_handle_data_with_kernel(pinned.data_ptr(), layer.data_ptr(), kb.ctypes.data,
                                               n, total, 1, 0, st.cuda_stream, dev_meta.data_ptr(),
                                               host_meta.data_ptr(), max_block_num)
@@ -832,7 +832,7 @@ def test_per_layer_session_on_side_stream():
     stride = plan.layer_bytes
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     sess = kvt_amd.Session(plan, cache, packed, stride)
-    compute = torch.cuda.Stream()
+    compute = checkers.side_stream()
     fresh = [_dev_bytes(w.capacities("src")[0], 50 + l) for l in range(w.n_layers)]
     with torch.cuda.stream(compute):
         for l in range(w.n_layers):
@@ -861,7 +861,7 @@ def test_per_layer_session_gated_by_the_callers_own_events():
     stride = plan.layer_bytes
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     events = [torch.cuda.Event() for _ in range(w.n_layers)]
-    compute = torch.cuda.Stream()
+    compute = checkers.side_stream()
     for step in range(2):                          # the same events serve every step
         sess = kvt_amd.Session(plan, cache, packed, stride)
         fresh = [_dev_bytes(cap, 70 + 10 * step + l) for l in range(w.n_layers)]
@@ -893,7 +893,7 @@ def test_session_inside_hip_graph_replays():
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     sess = kvt_amd.Session(plan, cache, packed, stride)
     graph = torch.cuda.CUDAGraph()
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     with torch.cuda.stream(s):
         with torch.cuda.graph(graph, stream=s):
             for l in range(w.n_layers):
@@ -925,7 +925,7 @@ def test_stager_save_load_round_trip_overlapped_with_packing():
     nbytes = plan.layer_bytes
     stager = kvt_amd.Stager(0, nbytes, 2)
     dev_buf = [torch.zeros(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
-    pack_stream = torch.cuda.Stream()
+    pack_stream = checkers.side_stream()
     store = []                                    # the "KV store": host copies per layer
     for l in range(w.n_layers):
         slot = l % 2
@@ -951,7 +951,7 @@ def test_stager_save_load_round_trip_overlapped_with_packing():
                                  blob.ctypes.data)
         assert np.array_equal(store[l][:len(blob)], blob), l
     # load path: host -> slot -> device -> unpack
-    un_stream = torch.cuda.Stream()
+    un_stream = checkers.side_stream()
     for l in range(w.n_layers):
         slot = l % 2
         stager.wait(slot)
@@ -984,7 +984,7 @@ def test_stager_loads_with_a_consumer_stream_per_slot():
     store = packed.cpu().numpy().reshape(w.n_layers, nbytes)
     stager = kvt_amd.Stager(0, nbytes, 2)
     dev_buf = [torch.zeros(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
-    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    streams = [checkers.side_stream(), checkers.side_stream()]
     for l in range(w.n_layers):
         slot = l % 2
         if l >= 2:
@@ -1037,7 +1037,7 @@ def test_plan_used_on_two_streams_then_destroyed_while_launches_are_queued():
     stride = plan.layer_bytes
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     junk = torch.zeros(w.n_layers * stride * 2, dtype=torch.uint8, device="cuda")
-    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    a, b = checkers.side_stream(), checkers.side_stream()
     plan.pack(sc, 0, w.n_layers, packed, stride, a.cuda_stream)
     done = torch.cuda.Event()
     done.record(a)
@@ -1094,7 +1094,7 @@ def test_copy_handle_data_kernel_direct(explicit):
     dev = [torch.zeros(n, dtype=torch.int64, device="cuda") for _ in range(3)]
     host_meta = torch.zeros(3 * n, dtype=torch.int64).pin_memory()
     lib = kvt_amd.lib()
-    st = torch.cuda.Stream()
+    st = checkers.side_stream()
 
     def call(buf, gpu, direction, data_size=size):
         return lib.kvt_copy_handle_data_kernel_direct(
@@ -1208,7 +1208,7 @@ def test_many_threads_build_launch_and_drop_plans_at_once():
 
     def work(i):
         try:
-            stream = torch.cuda.Stream()
+            stream = checkers.side_stream()
             for r in range(rounds):
                 w = workloads.llama8b_batch(n_layers=4, src_pool=1024, dst_pool=4096, n_req=4,
                                             min_tok=200, max_tok=1500, seed=1000 + 17 * i + r)

@@ -39,7 +39,7 @@ class _Transport(threading.Thread):
 
     def run(self):
         try:
-            stream = torch.cuda.Stream()
+            stream = checkers.side_stream()
             for step in self.steps:
                 for l in range(self.n_layers):
                     self.sess.wait_layer(l, step)
@@ -71,7 +71,7 @@ def test_graph_replays_signal_every_layer_to_a_waiting_thread():
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     sess = kvt_amd.Session(plan, cache, packed, stride)
     graph = torch.cuda.CUDAGraph()
-    s = torch.cuda.Stream()
+    s = checkers.side_stream()
     with torch.cuda.stream(s):
         with torch.cuda.graph(graph, stream=s):
             for l in range(w.n_layers):
@@ -133,7 +133,7 @@ def test_eager_steps_share_one_session_and_waits_may_come_first():
     blob_len = plan.tensor_bytes(0)
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     sess = kvt_amd.Session(plan, cache, packed, stride)
-    compute = torch.cuda.Stream()
+    compute = checkers.side_stream()
     transport = _Transport(sess, packed, stride, blob_len, w.n_layers, (1, 2, 3))
     transport.start()                                   # parks in wait_layer(0, step 1)
     time.sleep(0.05)
@@ -191,7 +191,7 @@ def test_a_failed_layer_wakes_the_waiting_thread_with_the_error():
 
     t = threading.Thread(target=waiter)
     t.start()
-    compute = torch.cuda.Stream()
+    compute = checkers.side_stream()
     sess.begin_step()
     sess.save_layer(0, compute.cuda_stream)
     sess.save_layer(1, compute.cuda_stream)
@@ -250,7 +250,7 @@ def test_a_bounded_wait_runs_out_and_can_be_repeated():
     cache = kvt_amd.Cache(0, layers, [cap])
     packed = torch.zeros(w.n_layers * plan.layer_bytes, dtype=torch.uint8, device="cuda")
     sess = kvt_amd.Session(plan, cache, packed, plan.layer_bytes)
-    compute = torch.cuda.Stream()
+    compute = checkers.side_stream()
     for step, layer in ((1, 0), (3, 1)):             # step 1 has not begun; step 3 is far off
         t0 = time.perf_counter()
         with pytest.raises(kvt_amd.KvtError) as err:
@@ -292,7 +292,7 @@ def test_groups_of_layers_behind_one_event_eager_and_in_a_graph():
         sess.save_layers(5, 3)                                   # beyond the last layer
     with pytest.raises(kvt_amd.KvtError):
         sess.save_layers(2, 0)
-    compute = torch.cuda.Stream()
+    compute = checkers.side_stream()
 
     def check(step):
         t = _Transport(sess, packed, stride, plan.tensor_bytes(0), w.n_layers, [step])
@@ -312,7 +312,7 @@ def test_groups_of_layers_behind_one_event_eager_and_in_a_graph():
 
     sess = kvt_amd.Session(plan, cache, packed, stride)
     graph = torch.cuda.CUDAGraph()
-    cap_stream = torch.cuda.Stream()
+    cap_stream = checkers.side_stream()
     with torch.cuda.graph(graph, stream=cap_stream):
         for first, n in groups:
             sess.save_layers(first, n, cap_stream.cuda_stream)
@@ -344,7 +344,7 @@ def test_last_layers_packed_on_the_compute_stream_itself():
     stride = plan.layer_bytes
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     sess = kvt_amd.Session(plan, cache, packed, stride)
-    compute = torch.cuda.Stream()
+    compute = checkers.side_stream()
     for rep in range(2):
         step = sess.begin_step()
         t = _Transport(sess, packed, stride, plan.tensor_bytes(0), w.n_layers, [step])

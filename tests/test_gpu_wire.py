@@ -55,7 +55,7 @@ def test_framed_layers_sender_to_receiver(fmt, direct):
     frame_bytes = lay.total_bytes
     offs = list(lay.blob_offset)
     stager = kvt_amd.Stager(0, frame_bytes + 64, 2)
-    stream = torch.cuda.Stream()
+    stream = checkers.side_stream()
     dev_buf = torch.zeros(plan.layer_bytes, dtype=torch.uint8, device="cuda")
     sent = []
     # ---- sender
@@ -217,7 +217,7 @@ def test_framed_layers_of_a_tp_remapping_batch_with_run_plans():
     lay = binding.wire_layout_of(WIRE_RDMA_STAGED, lists)
     assert lay.blob_offset[0] % 16 in (4, 12)
     stager = kvt_amd.Stager(0, lay.total_bytes, 2)
-    stream = torch.cuda.Stream()
+    stream = checkers.side_stream()
     for l in range(w.n_layers):
         slot = l % 2
         binding.wire_write_frame(WIRE_RDMA_STAGED, stager.slot_ptr(slot), stager.slot_bytes, 7, l,

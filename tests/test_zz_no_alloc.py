@@ -7,6 +7,7 @@ row of which the second is smaller, in both directions. Needs a real MI355X."""
 import numpy as np
 import pytest
 
+import checkers
 import kvt_amd
 
 pytestmark = pytest.mark.gpu
@@ -63,7 +64,7 @@ def _both_entry_points(lib, st, blocks, size, layer, explicit):
 def test_static_metadata_entry_point_equals_the_existing_one(explicit):
     lib = kvt_amd.lib()
     assert lib.kvt_initialize_copy_method_profile(0) == 0, lib.kvt_last_error()
-    st = torch.cuda.Stream()
+    st = checkers.side_stream()
     g = torch.Generator(device="cuda")
     g.manual_seed(91)
     layer = torch.randint(0, 256, (CAP,), generator=g, device="cuda", dtype=torch.uint8)
@@ -91,7 +92,7 @@ def test_static_metadata_entry_point_equals_the_existing_one(explicit):
 
 def test_static_metadata_entry_point_refuses_what_it_cannot_hold():
     lib = kvt_amd.lib()
-    st = torch.cuda.Stream()
+    st = checkers.side_stream()
     n = 8193
     blocks = np.ascontiguousarray(np.stack([np.zeros(n, np.uint64), np.arange(n, dtype=np.uint64) * 16,
                                             np.full(n, 16, np.uint64)], axis=1))
