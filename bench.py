@@ -895,13 +895,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "a10df6406be38edac587c842a5af4777d31116983d1735f9d600e7c61a173fab"
+KERNELS_SHA256 = "b0bcf67531ad8861a543fdb2f9920bd205e8a0ce11bdb71fe7341ec5bcb2a17e"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134278348, "unpack": 134277153},
-    (2, "ranges"): {"pack": 71013098083, "unpack": 73358415712},
-    (3, "ranges"): {"pack": 85983114112, "unpack": 85983602300},
-    (4, "ranges"): {"pack": 22690381642, "unpack": 22690446879},
-    (5, "ranges"): {"pack": 45141201201, "unpack": 45141402287},
+    (1, "ranges"): {"pack": 134275715, "unpack": 134277891},
+    (2, "ranges"): {"pack": 71013141385, "unpack": 73358402584},
+    (3, "ranges"): {"pack": 85983097435, "unpack": 85983584556},
+    (4, "ranges"): {"pack": 22690383614, "unpack": 22690451539},
+    (5, "ranges"): {"pack": 45141192424, "unpack": 45141392870},
 }
 
 
