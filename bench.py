@@ -529,6 +529,30 @@ def leg_launchers(c, out):
         res["note"] = ("%d launches of %d ranges each; GB/s = bytes read + bytes written; the "
                        "fp8 gather reads 2 bytes and writes 1 per element" %
                        (w.n_layers, len(runs0)))
+        # the same launches limited to a share of the CUs (the reference's SM-usage knob)
+        shares = []
+        try:
+            for usage in (0.5, 0.25, 0.125):
+                kvt.set_copy_cu_usage(0, usage)
+                row = {"usage": usage, "workgroups": kvt.get_copy_cu_usage(0)[1]}
+                for name, fn, offs, lens, moved in (
+                        ("launch_copy_d2h_direct", lib.kvt_launch_copy_d2h_direct, do, ln, 2 * nb),
+                        ("launch_copy_d2h_bf16_to_fp8", lib.kvt_launch_copy_d2h_bf16_to_fp8, do_e,
+                         ln_e, nb + nb // 2)):
+                    for rep in range(2):
+                        lib.kvt_event_record(a, sh)
+                        for l in range(w.n_layers):
+                            rc = fn(side.src[l][0].data_ptr(), packed[0].data_ptr() + l * strides[0],
+                                    so.data_ptr(), offs.data_ptr(), lens.data_ptr(), len(runs0), 0, 0,
+                                    sh)
+                            assert rc == 0, lib.kvt_last_error()
+                        lib.kvt_event_record(b, sh)
+                    lib.kvt_event_synchronize(b)
+                    row[name + "_gbps"] = round(moved * w.n_layers / (ev_ms(lib, a, b) * 1e-3) / 1e9, 1)
+                shares.append(row)
+        finally:
+            kvt.set_copy_cu_usage(0, 1.0)
+        res["cu_usage"] = shares
         # the reference's host entry point, called the way TCPChannel::send_data /
         # handle_kv_cache_data call it: pinned host buffer on the contiguous side, metadata
         # uploaded per call through the caller's two 8192-range buffers
@@ -895,13 +919,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "b0bcf67531ad8861a543fdb2f9920bd205e8a0ce11bdb71fe7341ec5bcb2a17e"
+KERNELS_SHA256 = "40bbb4a7be1feb56629b543e25972d64bd72e4c062f47718ce016ed2422db99b"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134275715, "unpack": 134277891},
-    (2, "ranges"): {"pack": 71013141385, "unpack": 73358402584},
-    (3, "ranges"): {"pack": 85983097435, "unpack": 85983584556},
-    (4, "ranges"): {"pack": 22690383614, "unpack": 22690451539},
-    (5, "ranges"): {"pack": 45141192424, "unpack": 45141392870},
+    (1, "ranges"): {"pack": 134276860, "unpack": 134277714},
+    (2, "ranges"): {"pack": 71013009630, "unpack": 73358386948},
+    (3, "ranges"): {"pack": 85983085394, "unpack": 85983578361},
+    (4, "ranges"): {"pack": 22690381710, "unpack": 22690433849},
+    (5, "ranges"): {"pack": 45141191545, "unpack": 45141373772},
 }
 
 

@@ -29,6 +29,7 @@
 namespace kvt {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kThreads = 256;
 constexpr uint32_t kSlice = kThreads * 16;  // bytes moved by one workgroup
@@ -951,6 +952,72 @@ __global__ __launch_bounds__(kThreads) void copy_ranges_kernel(
   }
 }
 
+// The same list under a CU-share limit: persistent workgroups whose wavefronts each walk ranges
+// of their own (the ranges are dealt to the XCDs in eighths, the wavefronts of an XCD stride
+// through its eighth), 8 KiB of a range per trip through range-checked buffer descriptors,
+// software-pipelined over three register sets like copy_entries_by_wave_kernel. With one
+// vector per lane in flight (copy_ranges_kernel on a limited grid) the rate follows the wave
+// slots: 4.7 TB/s at a quarter of the device, 2.7 at an eighth. Lengths and addresses live on
+// the device, so alignment is found out here: a range that is not 16-byte aligned on both
+// sides and a multiple of 16 bytes long is copied by its wavefront on the spot, byte-wise.
+__device__ __forceinline__ void copy_range_odd_by_wave(uint8_t* d, const uint8_t* s, uint64_t len, uint32_t lane) {
+#pragma clang loop vectorize(disable) unroll(disable)
+  for (uint64_t j = lane; j < len; j += 64) d[j] = s[j];
+}
+__global__ __launch_bounds__(kThreads, 4) void copy_ranges_persistent_kernel(
+    const uint8_t* src_base, uint8_t* dst_base, const int64_t* __restrict__ src_off,
+    const int64_t* __restrict__ dst_off, const int64_t* __restrict__ lens, uint32_t n) {
+  constexpr int V = 8;
+  constexpr uint32_t kTrip = static_cast<uint32_t>(V) << 10;  // bytes of a range per trip
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane64 = threadIdx.x & 63u, off = lane64 << 4;
+  const uint32_t per8 = (n + 7u) >> 3, xcd = blockIdx.x & 7u;
+  const uint32_t step = (gridDim.x >> 3) * 4u;        // wavefronts per XCD
+  uint32_t within = (blockIdx.x >> 3) * 4u + wave;    // this wavefront's next range inside the eighth
+  const uint8_t* s = nullptr;
+  uint8_t* d = nullptr;
+  uint64_t len = 0, begin = 0;
+  rsrc_t src[3], dst[3];
+  u32x4 r[3][V];
+  auto next = [&](int k) -> bool {
+    bool live = true;
+    if (begin >= len) {  // on to the next range
+      const uint32_t i = xcd * per8 + within;
+      live = within < per8 && i < n;
+      within += step;
+      len = 0;
+      begin = 0;
+      if (live) {
+        const uint64_t l = static_cast<uint64_t>(lens[i]);
+        s = src_base + src_off[i];
+        d = dst_base + dst_off[i];
+        if (((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d) | l) & 15u) == 0) {
+          len = l;
+        } else {
+          copy_range_odd_by_wave(d, s, l, lane64);
+        }
+      }
+    }
+    const uint64_t left = len - begin;  // 0 when there is nothing (more) to move: empty descriptors
+    const uint32_t bytes = left < kTrip ? static_cast<uint32_t>(left) : kTrip;
+    src[k] = make_rsrc(s + begin, bytes);
+    dst[k] = make_rsrc(d + begin, bytes);
+    begin += bytes;
+    return live;
+  };
+  auto load = [&](int k) {
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      r[k][v] = __builtin_amdgcn_raw_buffer_load_b128(src[k], off + (v << 10), 0, kLoadPolicy);
+  };
+  auto store = [&](int k) {
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      __builtin_amdgcn_raw_buffer_store_b128(r[k][v], dst[k], off + (v << 10), 0, kStorePolicy);
+  };
+  KVT_ROTATE3_PINNED(next, load, store);
+}
+
 // bf16 -> fp8 E4M3 (OCP "fn" variant: no infinities, 0x7F = NaN), round to
 // nearest even, finite values and infinities saturate to +-448 (0x7E), NaN
 // stays NaN (sign kept). `pair` holds two bf16; the two fp8 bytes go to the low
@@ -1026,6 +1093,70 @@ __global__ __launch_bounds__(kThreads) void convert_ranges_kernel(
         d8[j] = static_cast<uint8_t>(bf16_to_e4m3(s16[j]));
     }
   }
+}
+
+// The converting gather by persistent workgroups, a wavefront per range (see
+// copy_ranges_persistent_kernel): 4096 elements of a range per trip, lane t of the wavefront
+// the groups of 8 elements t, t + 64, ... t + 448. A range that is not 16-byte aligned on both
+// sides and a multiple of 8 elements long is converted by its wavefront on the spot, element-wise.
+__global__ __launch_bounds__(kThreads, 4) void convert_ranges_persistent_kernel(
+    const uint8_t* src_base, uint8_t* dst_base, const int64_t* __restrict__ src_off,
+    const int64_t* __restrict__ dst_off, const int64_t* __restrict__ lens, uint32_t n) {
+  constexpr int G = 8;
+  constexpr uint32_t kTrip = static_cast<uint32_t>(G) << 9;  // elements of a range per trip
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane64 = threadIdx.x & 63u;
+  const uint32_t per8 = (n + 7u) >> 3, xcd = blockIdx.x & 7u;
+  const uint32_t step = (gridDim.x >> 3) * 4u;
+  uint32_t within = (blockIdx.x >> 3) * 4u + wave;
+  const uint8_t* s = nullptr;
+  uint8_t* d = nullptr;
+  uint64_t count = 0, begin = 0;
+  rsrc_t src[3], dst[3];
+  u32x4 r[3][G];
+  auto next = [&](int k) -> bool {
+    bool live = true;
+    if (begin >= count) {  // on to the next range
+      const uint32_t i = xcd * per8 + within;
+      live = within < per8 && i < n;
+      within += step;
+      count = 0;
+      begin = 0;
+      if (live) {
+        const uint64_t c = static_cast<uint64_t>(lens[i]);
+        s = src_base + src_off[i];
+        d = dst_base + dst_off[i];
+        if (((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) & 15u) == 0 && (c & 7u) == 0) {
+          count = c;
+        } else {
+          const uint16_t* s16 = reinterpret_cast<const uint16_t*>(s);
+#pragma clang loop vectorize(disable) unroll(disable)
+          for (uint64_t j = lane64; j < c; j += 64) d[j] = static_cast<uint8_t>(bf16_to_e4m3(s16[j]));
+        }
+      }
+    }
+    const uint64_t left = count - begin;
+    const uint32_t elems = left < kTrip ? static_cast<uint32_t>(left) : kTrip;
+    src[k] = make_rsrc(s + 2 * begin, 2 * elems);
+    dst[k] = make_rsrc(d + begin, elems);
+    begin += elems;
+    return live;
+  };
+  auto load = [&](int k) {
+#pragma unroll
+    for (int j = 0; j < G; ++j)
+      r[k][j] = __builtin_amdgcn_raw_buffer_load_b128(src[k], (lane64 + (j << 6)) << 4, 0, kLoadPolicy);
+  };
+  auto store = [&](int k) {
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+      u32x2 out;
+      out.x = cvt4(r[k][j].x, r[k][j].y);
+      out.y = cvt4(r[k][j].z, r[k][j].w);
+      __builtin_amdgcn_raw_buffer_store_b64(out, dst[k], (lane64 + (j << 6)) << 3, 0, kStorePolicy);
+    }
+  };
+  KVT_ROTATE3_PINNED(next, load, store);
 }
 
 // Converting gather of a resident chunk table (the pack direction of a plan whose source
@@ -1108,7 +1239,6 @@ __global__ __launch_bounds__(kThreads, 8) void convert_chunks_kernel(
 // through the cache-side descriptor at an offset computed when the part is fetched, and an
 // 8-byte store through the packed-side descriptor. Record arithmetic as in
 // strided_entries_kernel, in groups: a record of vlen * 16 elements is 2 * vlen groups.
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 template <int V>
 __global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
@@ -1558,6 +1688,22 @@ static dim3 range_grid(int num_wg, int rows, uint32_t max_wgs) {
     if (gy > max_wgs / gx) gy = max_wgs / gx;
   }
   return dim3(gx, gy);
+}
+
+hipError_t launch_copy_ranges_persistent(bool convert, const void* src_base, void* dst_base,
+                                         const int64_t* src_off, const int64_t* dst_off,
+                                         const int64_t* lens, int64_t n, uint32_t wgs, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  if (n > 0x7FFFFFF0ll || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+  if (convert)
+    hipLaunchKernelGGL(convert_ranges_persistent_kernel, dim3(wgs), dim3(kThreads), 0, stream,
+                       static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off,
+                       dst_off, lens, static_cast<uint32_t>(n));
+  else
+    hipLaunchKernelGGL(copy_ranges_persistent_kernel, dim3(wgs), dim3(kThreads), 0, stream,
+                       static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off,
+                       dst_off, lens, static_cast<uint32_t>(n));
+  return hipGetLastError();
 }
 
 hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,

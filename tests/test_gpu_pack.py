@@ -383,6 +383,71 @@ def test_launch_copy_direct_gather_and_scatter(n, maxlen):
     assert np.array_equal(_host(dst), exp)
 
 
+@pytest.mark.parametrize("usage", [1.0, 0.25, 0.004], ids=["unlimited", "quarter", "eight-workgroups"])
+def test_long_range_lists_go_through_the_persistent_range_kernels(usage):
+    """A list of thousands of ranges is moved by persistent workgroups, a wavefront per range,
+    8 KiB (converting: 4096 elements) per trip: ranges shorter, longer and much longer than a
+    trip, empty ones, ranges that are not 16-byte aligned or not whole vectors long (copied on
+    the spot), gather, scatter and the converting gather, against the oracle."""
+    lib = kvt_amd.lib()
+    o = checkers.oracle()
+    rng = np.random.default_rng(4242)
+    n, cap = 3000, 384 << 20
+    lens = rng.choice([0, 16, 48, 1000, 4096, 8192, 8208, 16384, 39936, 100000, 13, 4099], size=n,
+                      p=[.03, .05, .05, .05, .2, .2, .1, .1, .1, .02, .05, .05]).astype(np.int64)
+    slot = cap // n // 1024 * 1024                        # one slot per range: nothing overlaps
+    gpu_off = np.arange(n, dtype=np.int64) * slot
+    lens = np.minimum(lens, slot - 64)
+    mis = rng.random(n) < 0.1
+    gpu_off[mis] += rng.choice([1, 2, 4, 8], size=int(mis.sum()))
+    order = rng.permutation(n)                            # the list is not sorted by address
+    gpu_off, lens = gpu_off[order], lens[order]
+    contig = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    contig16 = np.concatenate([[0], np.cumsum((lens + 15) // 16 * 16)[:-1]])   # aligned packed positions
+    src = _dev_bytes(cap, 78, "raw")
+    kvt_amd.set_copy_cu_usage(0, usage)
+    try:
+        for packed_off in (contig, contig16):
+            total = int(packed_off[-1] + lens[-1])
+            out = torch.zeros(total, dtype=torch.uint8, device="cuda")
+            so, do, ln = _soa(np.stack([gpu_off, packed_off, lens], axis=1))
+            assert lib.kvt_launch_copy_d2h_direct(src.data_ptr(), out.data_ptr(), so.data_ptr(),
+                                                  do.data_ptr(), ln.data_ptr(), n, 0, 0, None) == 0
+            torch.cuda.synchronize()
+            src_h, out_h = _host(src), _host(out)
+            exp = np.zeros(total, dtype=np.uint8)
+            for g, p, l in zip(gpu_off, packed_off, lens):
+                exp[p:p + l] = src_h[g:g + l]
+            assert np.array_equal(out_h, exp)
+            dst = torch.full((cap,), 0x3C, dtype=torch.uint8, device="cuda")
+            assert lib.kvt_launch_copy_h2d_direct(out.data_ptr(), dst.data_ptr(), do.data_ptr(),
+                                                  so.data_ptr(), ln.data_ptr(), n, 0, 0, None) == 0
+            torch.cuda.synchronize()
+            exp_d = np.full(cap, 0x3C, dtype=np.uint8)
+            for g, p, l in zip(gpu_off, packed_off, lens):
+                exp_d[g:g + l] = exp[p:p + l]
+            assert np.array_equal(_host(dst), exp_d)
+        # converting gather: lengths count elements, source offsets bytes of bf16
+        elems = lens // 2
+        e_off = np.concatenate([[0], np.cumsum((elems + 15) // 16 * 16 + 16)[:-1]])
+        e_off[rng.random(n) < 0.05] += 4                  # some destinations not 16-byte aligned
+        total_e = int(e_off[-1] + elems[-1])
+        out8 = torch.zeros(total_e, dtype=torch.uint8, device="cuda")
+        g_even = gpu_off // 2 * 2                          # bf16 elements start at even bytes
+        so, do, ln = _soa(np.stack([g_even, e_off, elems], axis=1))
+        assert lib.kvt_launch_copy_d2h_bf16_to_fp8(src.data_ptr(), out8.data_ptr(), so.data_ptr(),
+                                                   do.data_ptr(), ln.data_ptr(), n, 0, 0, None) == 0
+        torch.cuda.synchronize()
+        table = np.array([o.kvto_bf16_to_fp8(int(b)) for b in range(65536)], dtype=np.uint8)
+        src16 = _host(src).view(np.uint16)
+        exp8 = np.zeros(total_e, dtype=np.uint8)
+        for g, p, l in zip(g_even, e_off, elems):
+            exp8[p:p + l] = table[src16[g // 2:g // 2 + l]]
+        assert np.array_equal(_host(out8), exp8)
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+
+
 def test_reference_launcher_names_link_level_stand_in():
     """libkvt_blade_launchers.so exports the four extern "C" names that the reference's
     copy_kernels.cpp calls (copy_kernels.cpp:52-85, 101-108), with its argument order and a
