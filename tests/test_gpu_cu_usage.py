@@ -261,8 +261,8 @@ def test_more_limited_launches_in_flight_than_ticket_blocks():
 @pytest.mark.parametrize("usage", [0.25, 0.004], ids=["quarter", "eight-workgroups"])
 def test_limited_launches_of_every_pipelined_kernel_inside_a_graph(usage):
     """A limited launch recorded into a hipGraph keeps a block of counters of its own for every
-    replay. Plain (entries of 32 KiB and of 4 KiB), strided, converting and transposing plans,
-    pack and unpack in one graph,
+    replay. Plain, strided, converting and transposing plans (entries a workgroup takes and
+    entries a wavefront takes), pack and unpack in one graph,
     replayed with fresh cache contents each time."""
     kvt_amd.set_copy_cu_usage(0, usage)
     try:
@@ -278,6 +278,15 @@ def test_limited_launches_of_every_pipelined_kernel_inside_a_graph(usage):
                                min_tok=200, max_tok=1400, fp8_dst=True)
         cases.append((w, pipeline.build_plan_runs(w, 0)[0]))
         w = workloads.llama70b_flashinfer(n_layers=3, pool=400, n_req=4, tokens=1500)
+        cases.append((w, pipeline.build_plan(w, 0)[0]))
+        # entries of 4 and 8 KiB (one or two KV heads per rank): a wavefront per entry
+        w = workloads.tp_split("flash", 8, 1, 3, n_layers=3, src_pool=900, dst_pool=1000, n_req=6,
+                               min_tok=400, max_tok=2400)
+        cases.append((w, pipeline.build_plan_runs(w, 0)[0]))
+        w = workloads.tp_split("flash", 8, 1, 3, n_layers=3, src_pool=900, dst_pool=1000, n_req=6,
+                               min_tok=400, max_tok=2400, fp8_dst=True)
+        cases.append((w, pipeline.build_plan_runs(w, 0)[0]))
+        w = workloads.llama70b_flashinfer(n_layers=3, pool=1200, n_req=6, tokens=3000, heads=2)
         cases.append((w, pipeline.build_plan(w, 0)[0]))
         for w, plan in cases:
             plan.ready()
