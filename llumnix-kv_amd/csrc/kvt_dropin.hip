@@ -46,13 +46,17 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
   // with its trips software-pipelined: faster than the grid above even without a limit (config
   // 2's 35 014 ranges per layer: 6.39 against 6.24 TB/s), and under a limit it keeps that rate
   // where the grid's follows the wave slots (6.4 against 4.7 TB/s at a quarter of the device,
-  // against 2.7 at an eighth). Every wavefront should find a few ranges of its own.
+  // against 2.7 at an eighth). Every wavefront should find ranges of its own: two under a limit
+  // (where this shape wins at any length: 3 000 ranges of 64 KiB at a quarter 5.5 against 4.1,
+  // 100 000 of 4 KiB 5.4 against 1.7), sixteen without one, because a wavefront's unit of work is
+  // a whole range and few long ones leave an uneven rest (2 100 ranges of 1 MiB: 4.7 against
+  // 5.3 TB/s on the grid; 100 000 of 4 KiB: 5.4 against 3.8).
   const uint32_t cus = device_cu_count(device) & ~7u;
   if (cus >= 8) {
     const uint32_t pw = cap == 0 ? cus : std::max(8u, std::min(cap & ~7u, cus));
     // (the converting gather without a limit stays on the grid: 6.49 against 6.25 TB/s; under a
     // limit 6.25 against 4.96 at one half, 3.40 at a quarter, 2.19 at an eighth)
-    if (static_cast<uint64_t>(n) >= 8ull * pw && (!convert || cap != 0)) {
+    if (static_cast<uint64_t>(n) >= (cap != 0 ? 8ull : 64ull) * pw && (!convert || cap != 0)) {
       const hipError_t pe = launch_copy_ranges_persistent(convert, src, dst, so, dof, len, n, pw, s);
       if (pe != hipSuccess) return hip_fail(pe, "range copy launch");
       return KVT_OK;

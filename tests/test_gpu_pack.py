@@ -392,7 +392,7 @@ def test_long_range_lists_go_through_the_persistent_range_kernels(usage):
     lib = kvt_amd.lib()
     o = checkers.oracle()
     rng = np.random.default_rng(4242)
-    n, cap = 3000, 384 << 20
+    n, cap = 17000, 1088 << 20                            # unlimited: sixteen ranges per wavefront
     lens = rng.choice([0, 16, 48, 1000, 4096, 8192, 8208, 16384, 39936, 100000, 13, 4099], size=n,
                       p=[.03, .05, .05, .05, .2, .2, .1, .1, .1, .02, .05, .05]).astype(np.int64)
     slot = cap // n // 1024 * 1024                        # one slot per range: nothing overlaps
