@@ -46,6 +46,7 @@ def test_kernel_sync_and_data_transfer():
     assert ch.is_active()
     ch.register_data(lists, tp_kind, num_layers,
                      lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda"))
+    torch.cuda.synchronize()          # what the default stream still holds comes first
     with torch.cuda.stream(stream):
         layers[0].fill_(10)                       # mock layer 0
         ch.send_data(0, stream.cuda_stream)       # event record + notify_event_record
@@ -115,6 +116,7 @@ def test_cuda_kernel_sync_over_four_steps():
 
         t = threading.Thread(target=consumer)     # waits before the layers are even launched
         t.start()
+        torch.cuda.synchronize()          # what the default stream still holds comes first
         with torch.cuda.stream(stream):
             layers[0].fill_(step + 1)
             session.save_layer(0, stream.cuda_stream)

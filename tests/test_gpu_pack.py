@@ -317,6 +317,7 @@ def test_short_plans_travel_in_the_kernel_arguments(n_ranges):
     torch.cuda.synchronize()
     if n_ranges <= 64:
         graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()          # what the default stream still holds comes first
         with torch.cuda.stream(s):
             with torch.cuda.graph(graph, stream=s):
                 plan.pack(sc, 0, 2, packed, stride, s.cuda_stream)
@@ -899,6 +900,7 @@ def test_per_layer_session_on_side_stream():
     sess = kvt_amd.Session(plan, cache, packed, stride)
     compute = checkers.side_stream()
     fresh = [_dev_bytes(w.capacities("src")[0], 50 + l) for l in range(w.n_layers)]
+    torch.cuda.synchronize()          # what the default stream still holds comes first
     with torch.cuda.stream(compute):
         for l in range(w.n_layers):
             layers[l][0].copy_(fresh[l])           # the "forward pass" writes layer l
@@ -930,6 +932,7 @@ def test_per_layer_session_gated_by_the_callers_own_events():
     for step in range(2):                          # the same events serve every step
         sess = kvt_amd.Session(plan, cache, packed, stride)
         fresh = [_dev_bytes(cap, 70 + 10 * step + l) for l in range(w.n_layers)]
+        torch.cuda.synchronize()          # what the default stream still holds comes first
         with torch.cuda.stream(compute):
             for l in range(w.n_layers):
                 layers[l][0].copy_(fresh[l])
@@ -959,6 +962,7 @@ def test_session_inside_hip_graph_replays():
     sess = kvt_amd.Session(plan, cache, packed, stride)
     graph = torch.cuda.CUDAGraph()
     s = checkers.side_stream()
+    torch.cuda.synchronize()          # what the default stream still holds comes first
     with torch.cuda.stream(s):
         with torch.cuda.graph(graph, stream=s):
             for l in range(w.n_layers):

@@ -45,6 +45,7 @@ class _Transport(threading.Thread):
                     self.sess.wait_layer(l, step)
                     self.returned_at[(step, l)] = time.perf_counter()
                     host = torch.empty(self.blob_len, dtype=torch.uint8).pin_memory()
+                    torch.cuda.synchronize()          # what the default stream still holds comes first
                     with torch.cuda.stream(stream):
                         host.copy_(self.packed[l * self.stride:l * self.stride + self.blob_len],
                                    non_blocking=True)
@@ -72,6 +73,7 @@ def test_graph_replays_signal_every_layer_to_a_waiting_thread():
     sess = kvt_amd.Session(plan, cache, packed, stride)
     graph = torch.cuda.CUDAGraph()
     s = checkers.side_stream()
+    torch.cuda.synchronize()          # what the default stream still holds comes first
     with torch.cuda.stream(s):
         with torch.cuda.graph(graph, stream=s):
             for l in range(w.n_layers):
@@ -85,12 +87,14 @@ def test_graph_replays_signal_every_layer_to_a_waiting_thread():
     expected, still_running = {}, []
     for rep in range(n_replays):
         contents = [_contents(cap, 900 + 10 * rep + l) for l in range(w.n_layers)]
+        torch.cuda.synchronize()          # what the default stream still holds comes first
         with torch.cuda.stream(s):                      # eager work between the replays
             for l in range(w.n_layers):
                 staging[l].copy_(contents[l])
         step = sess.begin_step()
         assert step == rep + 1
         finished = torch.cuda.Event()
+        torch.cuda.synchronize()          # what the default stream still holds comes first
         with torch.cuda.stream(s):
             graph.replay()
             finished.record(s)
@@ -140,6 +144,7 @@ def test_eager_steps_share_one_session_and_waits_may_come_first():
     for step in (1, 2, 3):
         fresh = [_contents(cap, 70 + 10 * step + l) for l in range(w.n_layers)]
         assert sess.begin_step() == step
+        torch.cuda.synchronize()          # what the default stream still holds comes first
         with torch.cuda.stream(compute):
             for l in range(w.n_layers):
                 layers[l][0].copy_(fresh[l])
