@@ -22,6 +22,33 @@ int range_launch_shape(int64_t n, int num_wg, int* wgs) {
   return KVT_OK;
 }
 
+// One list of device-resident ranges between two device buffers: the grid of (rows x ranges)
+// workgroups, or persistent workgroups for a long list.
+// A long list goes through persistent workgroups, one per CU at most, a wavefront per range
+// with its trips software-pipelined: faster than the grid even without a limit (config
+// 2's 35 014 ranges per layer: 6.39 against 6.24 TB/s), and under a limit it keeps that rate
+// where the grid's follows the wave slots (6.4 against 4.7 TB/s at a quarter of the device,
+// against 2.7 at an eighth). Every wavefront should find ranges of its own: two under a limit
+// (where this shape wins at any length: 3 000 ranges of 64 KiB at a quarter 5.5 against 4.1,
+// 100 000 of 4 KiB 5.4 against 1.7), sixteen without one, because a wavefront's unit of work is
+// a whole range and few long ones leave an uneven rest (2 100 ranges of 1 MiB: 4.7 against
+// 5.3 TB/s on the grid; 100 000 of 4 KiB: 5.4 against 3.8).
+// (The converting gather without a limit stays on the grid: 6.49 against 6.25 TB/s; under a
+// limit 6.25 against 4.96 at one half, 3.40 at a quarter, 2.19 at an eighth.)
+hipError_t launch_device_ranges(bool convert, int device, const void* src, void* dst, const int64_t* so,
+                                const int64_t* dof, const int64_t* len, int64_t n, int wgs, int rows,
+                                hipStream_t s) {
+  const uint32_t cap = copy_wg_cap(device);
+  const uint32_t cus = device_cu_count(device) & ~7u;
+  if (cus >= 8) {
+    const uint32_t pw = cap == 0 ? cus : std::max(8u, std::min(cap & ~7u, cus));
+    if (static_cast<uint64_t>(n) >= (cap != 0 ? 8ull : 64ull) * pw && (!convert || cap != 0))
+      return launch_copy_ranges_persistent(convert, src, dst, so, dof, len, n, pw, s);
+  }
+  return convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s)
+                 : launch_copy_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s);
+}
+
 int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, const int64_t* dof,
                   const int64_t* len, int64_t n, int num_wg, int threads_per_wg, void* stream) {
   (void)threads_per_wg;  // workgroups are always 256 lanes (4 wavefronts)
@@ -41,29 +68,7 @@ int launch_ranges(bool convert, const void* src, void* dst, const int64_t* so, c
   const hipStream_t s = static_cast<hipStream_t>(stream);
   int device = 0;   // these entry points name no device: the caller's current one
   KVT_HIP(hipGetDevice(&device));
-  const uint32_t cap = copy_wg_cap(device);
-  // A long list goes through persistent workgroups, one per CU at most, a wavefront per range
-  // with its trips software-pipelined: faster than the grid above even without a limit (config
-  // 2's 35 014 ranges per layer: 6.39 against 6.24 TB/s), and under a limit it keeps that rate
-  // where the grid's follows the wave slots (6.4 against 4.7 TB/s at a quarter of the device,
-  // against 2.7 at an eighth). Every wavefront should find ranges of its own: two under a limit
-  // (where this shape wins at any length: 3 000 ranges of 64 KiB at a quarter 5.5 against 4.1,
-  // 100 000 of 4 KiB 5.4 against 1.7), sixteen without one, because a wavefront's unit of work is
-  // a whole range and few long ones leave an uneven rest (2 100 ranges of 1 MiB: 4.7 against
-  // 5.3 TB/s on the grid; 100 000 of 4 KiB: 5.4 against 3.8).
-  const uint32_t cus = device_cu_count(device) & ~7u;
-  if (cus >= 8) {
-    const uint32_t pw = cap == 0 ? cus : std::max(8u, std::min(cap & ~7u, cus));
-    // (the converting gather without a limit stays on the grid: 6.49 against 6.25 TB/s; under a
-    // limit 6.25 against 4.96 at one half, 3.40 at a quarter, 2.19 at an eighth)
-    if (static_cast<uint64_t>(n) >= (cap != 0 ? 8ull : 64ull) * pw && (!convert || cap != 0)) {
-      const hipError_t pe = launch_copy_ranges_persistent(convert, src, dst, so, dof, len, n, pw, s);
-      if (pe != hipSuccess) return hip_fail(pe, "range copy launch");
-      return KVT_OK;
-    }
-  }
-  const hipError_t e = convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s)
-                               : launch_copy_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s);
+  const hipError_t e = launch_device_ranges(convert, device, src, dst, so, dof, len, n, wgs, rows, s);
   if (e != hipSuccess) return hip_fail(e, "range copy launch");
   return KVT_OK;
 }
@@ -248,7 +253,13 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     const int rows = rows_for(slices, m);
     const uint32_t cap = pcie_wg_cap(device, over_pcie);
     hipError_t e;
-    if (halve)
+    if (!over_pcie)  // both sides in device memory: the choice of the device-array launchers
+      e = halve || direction == KVT_COPY_D2H
+              ? launch_device_ranges(halve, device, layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
+                                     static_cast<int64_t>(m), wgs, rows, s)
+              : launch_device_ranges(false, device, tensor_buf, layer_gpu_ptr, d_contig, d_gpu, d_lens,
+                                     static_cast<int64_t>(m), wgs, rows, s);
+    else if (halve)
       e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
                                 static_cast<int64_t>(m), wgs, rows, cap, s);
     else if (direction == KVT_COPY_D2H)
@@ -324,7 +335,13 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
   }
   const int rows = rows_for(slices, n);
   const hipError_t e =
-      direction == KVT_COPY_D2H
+      !over_pcie
+          ? (direction == KVT_COPY_D2H
+                 ? launch_device_ranges(false, device, layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
+                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s)
+                 : launch_device_ranges(false, device, tensor_buf, layer_gpu_ptr, src_dev, dst_dev, len_dev,
+                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s))
+      : direction == KVT_COPY_D2H
           ? launch_copy_ranges(layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
                                static_cast<int64_t>(n), static_cast<int>(n), rows, pcie_wg_cap(device, over_pcie), s)
           : launch_copy_ranges(tensor_buf, layer_gpu_ptr, src_dev, dst_dev, len_dev,

@@ -1189,6 +1189,61 @@ def test_copy_handle_data_kernel_direct(explicit):
     assert call(pinned, dst, 0, data_size=int((host_off + lens).max()) - 1) != 0
 
 
+@pytest.mark.parametrize("usage", [1.0, 0.25], ids=["unlimited", "quarter"])
+def test_handle_data_between_two_device_buffers_with_a_long_list(usage):
+    """The contiguous side of copy_handle_data_kernel_direct and copy_handle_data_with_kernel
+    may be device memory (a staging buffer registered for RDMA): a long list then takes the
+    persistent range kernels like the device-array launchers. 20 000 ranges, some unaligned,
+    gather and scatter, unlimited and under a limit."""
+    rng = np.random.default_rng(13)
+    n, slot = 20000, 12288
+    cap = n * slot
+    lens = rng.choice([16, 256, 4096, 8192, 8208, 4099, 12000], size=n).astype(np.uint64)
+    gpu_off = (np.arange(n, dtype=np.uint64) * slot)[rng.permutation(n)]
+    gpu_off[rng.random(n) < 0.05] += 4
+    host_off = (np.cumsum(lens) - lens).astype(np.uint64)
+    total = int(lens.sum())
+    blocks = np.ascontiguousarray(np.stack([np.zeros(n, np.uint64), gpu_off, lens], axis=1))
+    layer = _dev_bytes(cap, 45, "u8")
+    staged = torch.zeros(total, dtype=torch.uint8, device="cuda")
+    dev = [torch.zeros(n, dtype=torch.int64, device="cuda") for _ in range(3)]
+    host_meta = torch.zeros(3 * n, dtype=torch.int64).pin_memory()
+    dev_meta = torch.zeros(3 * 8192, dtype=torch.int64, device="cuda")
+    lib = kvt_amd.lib()
+    st = checkers.side_stream()
+    layer_h = _host(layer)
+    exp = np.zeros(total, dtype=np.uint8)
+    for a, b, m in zip(host_off, gpu_off, lens):
+        exp[int(a):int(a + m)] = layer_h[int(b):int(b + m)]
+    exp_d = np.full(cap, 0x33, dtype=np.uint8)
+    for b, m in zip(gpu_off, lens):
+        exp_d[int(b):int(b + m)] = layer_h[int(b):int(b + m)]
+    kvt_amd.set_copy_cu_usage(0, usage)
+    try:
+        for direct in (True, False):
+            def call(gpu, direction):
+                if direct:
+                    return lib.kvt_copy_handle_data_kernel_direct(
+                        staged.data_ptr(), gpu.data_ptr(), blocks.ctypes.data, n, total, direction, 0,
+                        st.cuda_stream, dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(),
+                        host_meta.data_ptr(), 0)
+                return lib.kvt_copy_handle_data_with_kernel(
+                    staged.data_ptr(), gpu.data_ptr(), blocks.ctypes.data, n, total, direction, 0,
+                    st.cuda_stream, dev_meta.data_ptr(), host_meta.data_ptr(), 8192)
+            staged.zero_()
+            torch.cuda.synchronize()
+            assert call(layer, 1) == 0, lib.kvt_last_error()
+            st.synchronize()
+            assert np.array_equal(_host(staged), exp), direct
+            dst = torch.full((cap,), 0x33, dtype=torch.uint8, device="cuda")
+            torch.cuda.synchronize()
+            assert call(dst, 0) == 0, lib.kvt_last_error()
+            st.synchronize()
+            assert np.array_equal(_host(dst), exp_d), direct
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+
+
 def test_random_range_lists_sweep():
     """80 seeded batches of arbitrary ranges: 1-3 tensors, 1-3 layers, lengths from 1 byte to
     70 000, alignments 1 / 4 / 16 / 256, shuffled list order, every chunk size, packed buffer
