@@ -919,13 +919,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "40bbb4a7be1feb56629b543e25972d64bd72e4c062f47718ce016ed2422db99b"
+KERNELS_SHA256 = "6bec095577269b429bbd1e4544b07e04b85b1ff9e03636a739813f473ca6c631"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134276860, "unpack": 134277714},
-    (2, "ranges"): {"pack": 71013009630, "unpack": 73358386948},
-    (3, "ranges"): {"pack": 85983085394, "unpack": 85983578361},
-    (4, "ranges"): {"pack": 22690381710, "unpack": 22690433849},
-    (5, "ranges"): {"pack": 45141191545, "unpack": 45141373772},
+    (1, "ranges"): {"pack": 134275671, "unpack": 134276951},
+    (2, "ranges"): {"pack": 71013181533, "unpack": 73358399679},
+    (3, "ranges"): {"pack": 85983094148, "unpack": 85983583018},
+    (4, "ranges"): {"pack": 22690385904, "unpack": 22690444784},
+    (5, "ranges"): {"pack": 45141191548, "unpack": 45141394298},
 }
 
 

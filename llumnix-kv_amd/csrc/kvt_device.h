@@ -148,10 +148,12 @@ hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_
                               const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,
                               int rows, uint32_t max_wgs, hipStream_t stream);
 // The same list through `wgs` persistent workgroups (a multiple of 8), a wavefront per range:
-// the shape of a launch of many ranges, limited to a share of the device or not.
+// the shape of a launch of many ranges, limited to a share of the device or not. walkers:
+// ranges a wavefront moves side by side, 1, 2 or 4 (the copy; more for shorter ranges).
 hipError_t launch_copy_ranges_persistent(bool convert, const void* src_base, void* dst_base,
                                          const int64_t* src_off, const int64_t* dst_off,
-                                         const int64_t* lens, int64_t n, uint32_t wgs, hipStream_t stream);
+                                         const int64_t* lens, int64_t n, uint32_t wgs, int walkers,
+                                         hipStream_t stream);
 hipError_t launch_convert_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                                  const int64_t* dst_off, const int64_t* lens, int64_t n,
                                  int num_wg, int rows, uint32_t max_wgs, hipStream_t stream);

@@ -35,15 +35,22 @@ int range_launch_shape(int64_t n, int num_wg, int* wgs) {
 // 5.3 TB/s on the grid; 100 000 of 4 KiB: 5.4 against 3.8).
 // (The converting gather without a limit stays on the grid: 6.49 against 6.25 TB/s; under a
 // limit 6.25 against 4.96 at one half, 3.40 at a quarter, 2.19 at an eighth.)
+// avg_len: the mean range length where the caller knows it (host lists), else 0: a wavefront
+// then moves 2 ranges side by side from 65 536 ranges on and 4 from 262 144 (a list that long
+// holds short ranges; 4 KiB and less is where it pays, 16 KiB and more where it costs 1-9 %).
 hipError_t launch_device_ranges(bool convert, int device, const void* src, void* dst, const int64_t* so,
                                 const int64_t* dof, const int64_t* len, int64_t n, int wgs, int rows,
-                                hipStream_t s) {
+                                hipStream_t s, uint64_t avg_len = 0) {
   const uint32_t cap = copy_wg_cap(device);
   const uint32_t cus = device_cu_count(device) & ~7u;
   if (cus >= 8) {
     const uint32_t pw = cap == 0 ? cus : std::max(8u, std::min(cap & ~7u, cus));
     if (static_cast<uint64_t>(n) >= (cap != 0 ? 8ull : 64ull) * pw && (!convert || cap != 0))
-      return launch_copy_ranges_persistent(convert, src, dst, so, dof, len, n, pw, s);
+    {
+      const int walkers = avg_len != 0 ? (avg_len <= 1536 ? 4 : avg_len <= 8192 ? 2 : 1)
+                                       : (n >= 262144 ? 4 : n >= 65536 ? 2 : 1);
+      return launch_copy_ranges_persistent(convert, src, dst, so, dof, len, n, pw, walkers, s);
+    }
   }
   return convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s)
                  : launch_copy_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s);
@@ -237,9 +244,10 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     int64_t* gpu = host_meta + m;
     int64_t* lens = host_meta + 2 * m;
     const uint64_t unit = halve ? 8192 : 4096;  // source bytes of one workgroup's slice
-    uint64_t slices = 0;
+    uint64_t slices = 0, batch_bytes = 0;
     for (uint64_t i = 0; i < m; ++i) {
       const kvt_ipc_block& b = work[first + i];
+      batch_bytes += b.length;
       contig[i] = static_cast<int64_t>(b.src_offset);
       gpu[i] = static_cast<int64_t>(b.dst_offset);
       lens[i] = static_cast<int64_t>(halve ? b.length / 2 : b.length);
@@ -256,9 +264,9 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     if (!over_pcie)  // both sides in device memory: the choice of the device-array launchers
       e = halve || direction == KVT_COPY_D2H
               ? launch_device_ranges(halve, device, layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
-                                     static_cast<int64_t>(m), wgs, rows, s)
+                                     static_cast<int64_t>(m), wgs, rows, s, batch_bytes / m + 1)
               : launch_device_ranges(false, device, tensor_buf, layer_gpu_ptr, d_contig, d_gpu, d_lens,
-                                     static_cast<int64_t>(m), wgs, rows, s);
+                                     static_cast<int64_t>(m), wgs, rows, s, batch_bytes / m + 1);
     else if (halve)
       e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
                                 static_cast<int64_t>(m), wgs, rows, cap, s);
@@ -338,9 +346,9 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
       !over_pcie
           ? (direction == KVT_COPY_D2H
                  ? launch_device_ranges(false, device, layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
-                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s)
+                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s, cursor / n + 1)
                  : launch_device_ranges(false, device, tensor_buf, layer_gpu_ptr, src_dev, dst_dev, len_dev,
-                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s))
+                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s, cursor / n + 1))
       : direction == KVT_COPY_D2H
           ? launch_copy_ranges(layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
                                static_cast<int64_t>(n), static_cast<int>(n), rows, pcie_wg_cap(device, over_pcie), s)

@@ -964,56 +964,75 @@ __device__ __forceinline__ void copy_range_odd_by_wave(uint8_t* d, const uint8_t
 #pragma clang loop vectorize(disable) unroll(disable)
   for (uint64_t j = lane; j < len; j += 64) d[j] = s[j];
 }
+template <int U>
 __global__ __launch_bounds__(kThreads, 4) void copy_ranges_persistent_kernel(
     const uint8_t* src_base, uint8_t* dst_base, const int64_t* __restrict__ src_off,
     const int64_t* __restrict__ dst_off, const int64_t* __restrict__ lens, uint32_t n) {
-  constexpr int V = 8;
+  // U ranges at a time per wavefront, each in trips of 8 / U KiB: the same bytes in flight, and
+  // more ranges a second where they are short, since a range costs a trip however short it is
+  // (TB/s with 1 / 2 / 4: ranges of 256 B 0.55 / 0.92 / 1.42, of 1 KiB 2.1 / 3.3 / 4.8, of 4 KiB
+  // 5.4 / 6.1 / 5.4, of 16 KiB 6.4 / 6.3 / 5.6)
+  constexpr int V = 8 / U;
   constexpr uint32_t kTrip = static_cast<uint32_t>(V) << 10;  // bytes of a range per trip
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t lane64 = threadIdx.x & 63u, off = lane64 << 4;
   const uint32_t per8 = (n + 7u) >> 3, xcd = blockIdx.x & 7u;
-  const uint32_t step = (gridDim.x >> 3) * 4u;        // wavefronts per XCD
-  uint32_t within = (blockIdx.x >> 3) * 4u + wave;    // this wavefront's next range inside the eighth
-  const uint8_t* s = nullptr;
-  uint8_t* d = nullptr;
-  uint64_t len = 0, begin = 0;
-  rsrc_t src[3], dst[3];
-  u32x4 r[3][V];
+  const uint32_t step = (gridDim.x >> 3) * 4u * U;   // range walkers per XCD
+  uint32_t within[U];                                 // each walker's next range inside the eighth
+  const uint8_t* s[U];
+  uint8_t* d[U];
+  uint64_t len[U], begin[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    within[u] = ((blockIdx.x >> 3) * 4u + wave) * U + u;
+    s[u] = nullptr, d[u] = nullptr, len[u] = 0, begin[u] = 0;
+  }
+  rsrc_t src[3][U], dst[3][U];
+  u32x4 r[3][U][V];
   auto next = [&](int k) -> bool {
-    bool live = true;
-    if (begin >= len) {  // on to the next range
-      const uint32_t i = xcd * per8 + within;
-      live = within < per8 && i < n;
-      within += step;
-      len = 0;
-      begin = 0;
-      if (live) {
-        const uint64_t l = static_cast<uint64_t>(lens[i]);
-        s = src_base + src_off[i];
-        d = dst_base + dst_off[i];
-        if (((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d) | l) & 15u) == 0) {
-          len = l;
-        } else {
-          copy_range_odd_by_wave(d, s, l, lane64);
+    bool any = false;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      bool live = true;
+      if (begin[u] >= len[u]) {  // on to the next range
+        const uint32_t i = xcd * per8 + within[u];
+        live = within[u] < per8 && i < n;
+        within[u] += step;
+        len[u] = 0;
+        begin[u] = 0;
+        if (live) {
+          const uint64_t l = static_cast<uint64_t>(lens[i]);
+          s[u] = src_base + src_off[i];
+          d[u] = dst_base + dst_off[i];
+          if (((reinterpret_cast<uintptr_t>(s[u]) | reinterpret_cast<uintptr_t>(d[u]) | l) & 15u) == 0) {
+            len[u] = l;
+          } else {
+            copy_range_odd_by_wave(d[u], s[u], l, lane64);
+          }
         }
       }
+      const uint64_t left = len[u] - begin[u];  // 0 when there is nothing (more) to move: empty descriptors
+      const uint32_t bytes = left < kTrip ? static_cast<uint32_t>(left) : kTrip;
+      src[k][u] = make_rsrc(s[u] + begin[u], bytes);
+      dst[k][u] = make_rsrc(d[u] + begin[u], bytes);
+      begin[u] += bytes;
+      any = any || live;
     }
-    const uint64_t left = len - begin;  // 0 when there is nothing (more) to move: empty descriptors
-    const uint32_t bytes = left < kTrip ? static_cast<uint32_t>(left) : kTrip;
-    src[k] = make_rsrc(s + begin, bytes);
-    dst[k] = make_rsrc(d + begin, bytes);
-    begin += bytes;
-    return live;
+    return any;
   };
   auto load = [&](int k) {
 #pragma unroll
-    for (int v = 0; v < V; ++v)
-      r[k][v] = __builtin_amdgcn_raw_buffer_load_b128(src[k], off + (v << 10), 0, kLoadPolicy);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int v = 0; v < V; ++v)
+        r[k][u][v] = __builtin_amdgcn_raw_buffer_load_b128(src[k][u], off + (v << 10), 0, kLoadPolicy);
   };
   auto store = [&](int k) {
 #pragma unroll
-    for (int v = 0; v < V; ++v)
-      __builtin_amdgcn_raw_buffer_store_b128(r[k][v], dst[k], off + (v << 10), 0, kStorePolicy);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int v = 0; v < V; ++v)
+        __builtin_amdgcn_raw_buffer_store_b128(r[k][u][v], dst[k][u], off + (v << 10), 0, kStorePolicy);
   };
   KVT_ROTATE3_PINNED(next, load, store);
 }
@@ -1692,17 +1711,25 @@ static dim3 range_grid(int num_wg, int rows, uint32_t max_wgs) {
 
 hipError_t launch_copy_ranges_persistent(bool convert, const void* src_base, void* dst_base,
                                          const int64_t* src_off, const int64_t* dst_off,
-                                         const int64_t* lens, int64_t n, uint32_t wgs, hipStream_t stream) {
+                                         const int64_t* lens, int64_t n, uint32_t wgs, int walkers,
+                                         hipStream_t stream) {
   if (n <= 0) return hipSuccess;
   if (n > 0x7FFFFFF0ll || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+#define KVT_RANGES(U)                                                                              \
+  hipLaunchKernelGGL(copy_ranges_persistent_kernel<U>, dim3(wgs), dim3(kThreads), 0, stream,       \
+                     static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off, \
+                     dst_off, lens, static_cast<uint32_t>(n))
   if (convert)
     hipLaunchKernelGGL(convert_ranges_persistent_kernel, dim3(wgs), dim3(kThreads), 0, stream,
                        static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off,
                        dst_off, lens, static_cast<uint32_t>(n));
+  else if (walkers >= 4)
+    KVT_RANGES(4);
+  else if (walkers >= 2)
+    KVT_RANGES(2);
   else
-    hipLaunchKernelGGL(copy_ranges_persistent_kernel, dim3(wgs), dim3(kThreads), 0, stream,
-                       static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off,
-                       dst_off, lens, static_cast<uint32_t>(n));
+    KVT_RANGES(1);
+#undef KVT_RANGES
   return hipGetLastError();
 }
 

@@ -449,6 +449,41 @@ def test_long_range_lists_go_through_the_persistent_range_kernels(usage):
         kvt_amd.set_copy_cu_usage(0, 1.0)
 
 
+@pytest.mark.parametrize("n", [70000, 270000])
+def test_very_long_lists_of_short_ranges_through_the_launchers(n):
+    """From 65 536 ranges on a wavefront of the persistent range kernel moves two ranges side by
+    side, from 262 144 on four: short ranges of every alignment, gather and scatter."""
+    lib = kvt_amd.lib()
+    rng = np.random.default_rng(n)
+    slot = 1024
+    cap = n * slot
+    lens = rng.choice([16, 48, 256, 512, 1008, 13, 1000], size=n).astype(np.int64)
+    gpu_off = (np.arange(n, dtype=np.int64) * slot)[rng.permutation(n)]
+    gpu_off[rng.random(n) < 0.05] += 8
+    contig = np.concatenate([[0], np.cumsum((lens + 15) // 16 * 16)[:-1]])
+    total = int(contig[-1] + lens[-1])
+    src = _dev_bytes(cap, 79, "raw")
+    out = torch.zeros(total, dtype=torch.uint8, device="cuda")
+    so, do, ln = _soa(np.stack([gpu_off, contig, lens], axis=1))
+    assert lib.kvt_launch_copy_d2h_direct(src.data_ptr(), out.data_ptr(), so.data_ptr(),
+                                          do.data_ptr(), ln.data_ptr(), n, 0, 0, None) == 0
+    torch.cuda.synchronize()
+    # expected: every range's bytes, by one fancy-indexed copy
+    idx_src = np.concatenate([np.arange(g, g + l) for g, l in zip(gpu_off, lens)])
+    idx_dst = np.concatenate([np.arange(p, p + l) for p, l in zip(contig, lens)])
+    src_h = _host(src)
+    exp = np.zeros(total, dtype=np.uint8)
+    exp[idx_dst] = src_h[idx_src]
+    assert np.array_equal(_host(out), exp)
+    dst = torch.full((cap,), 0x3C, dtype=torch.uint8, device="cuda")
+    assert lib.kvt_launch_copy_h2d_direct(out.data_ptr(), dst.data_ptr(), do.data_ptr(),
+                                          so.data_ptr(), ln.data_ptr(), n, 0, 0, None) == 0
+    torch.cuda.synchronize()
+    exp_d = np.full(cap, 0x3C, dtype=np.uint8)
+    exp_d[idx_src] = src_h[idx_src]
+    assert np.array_equal(_host(dst), exp_d)
+
+
 def test_reference_launcher_names_link_level_stand_in():
     """libkvt_blade_launchers.so exports the four extern "C" names that the reference's
     copy_kernels.cpp calls (copy_kernels.cpp:52-85, 101-108), with its argument order and a
@@ -1189,8 +1224,10 @@ def test_copy_handle_data_kernel_direct(explicit):
     assert call(pinned, dst, 0, data_size=int((host_off + lens).max()) - 1) != 0
 
 
+@pytest.mark.parametrize("choice", [[16, 256, 1024, 4099, 48], [16, 256, 4096, 8192, 8208, 4099],
+                                    [4096, 8192, 8208, 4099, 12000, 12272]], ids=["short", "medium", "long"])
 @pytest.mark.parametrize("usage", [1.0, 0.25], ids=["unlimited", "quarter"])
-def test_handle_data_between_two_device_buffers_with_a_long_list(usage):
+def test_handle_data_between_two_device_buffers_with_a_long_list(usage, choice):
     """The contiguous side of copy_handle_data_kernel_direct and copy_handle_data_with_kernel
     may be device memory (a staging buffer registered for RDMA): a long list then takes the
     persistent range kernels like the device-array launchers. 20 000 ranges, some unaligned,
@@ -1198,7 +1235,8 @@ def test_handle_data_between_two_device_buffers_with_a_long_list(usage):
     rng = np.random.default_rng(13)
     n, slot = 20000, 12288
     cap = n * slot
-    lens = rng.choice([16, 256, 4096, 8192, 8208, 4099, 12000], size=n).astype(np.uint64)
+    # (short: four ranges side by side per wavefront; medium: two; long: one)
+    lens = rng.choice(choice, size=n).astype(np.uint64)
     gpu_off = (np.arange(n, dtype=np.uint64) * slot)[rng.permutation(n)]
     gpu_off[rng.random(n) < 0.05] += 4
     host_off = (np.cumsum(lens) - lens).astype(np.uint64)
