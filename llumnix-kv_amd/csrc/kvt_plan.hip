@@ -672,7 +672,8 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   // against the strided loop of the chunk kernel: a quarter of the device 6.0 / 5.7 against
   // 5.8 / 5.1, an eighth 5.4 / 5.4 against 4.3 / 3.6, a sixteenth 4.1 / 4.2 against 2.3 / 1.9).
   const bool by_wave = p->sub_shift <= 1;
-  if (max_wgs != 0 && p->all16 && !p->convert && !p->strided && !p->xform &&
+  // (the unpack of a converting plan moves plain fp8 bytes)
+  if (max_wgs != 0 && p->all16 && !(p->convert && pack) && !p->strided && !p->xform &&
       p->sub_shift <= 3 && cache->aligned16 && static_cast<uint64_t>(n) * n_layers > max_wgs) {
     uint64_t mis = reinterpret_cast<uintptr_t>(packed) | (n_layers > 1 ? layer_stride : 0);
     for (uint32_t t = 0; t < p->n_tensors; ++t) mis |= blobs.off[t];

@@ -233,6 +233,41 @@ def test_short_tables_in_kernel_arguments_entry_by_entry_under_a_limit(usage, ch
         kvt_amd.set_copy_cu_usage(0, 1.0)
 
 
+@pytest.mark.parametrize("usage", [0.25, 0.004], ids=["quarter", "eight-workgroups"])
+@pytest.mark.parametrize("block", [4096, 32768])
+def test_converting_plan_of_plain_aligned_ranges_under_a_limit(usage, block):
+    """Same TP on both sides, bf16 sender and fp8 receiver: plain ranges of whole blocks. The
+    pack converts through the persistent converting kernels (entries of 4096 elements: a
+    wavefront each), the unpack moves plain fp8 bytes through the persistent copy kernels."""
+    rng = np.random.default_rng(block)
+    n_blocks, n_layers, pool = 700, 3, 1000
+    src_ids = rng.permutation(pool)[:n_blocks]
+    dst_ids = rng.permutation(pool)[:n_blocks]
+    elems = block // 2                                         # a block holds bf16
+    ranges = np.stack([src_ids * block, dst_ids * elems, np.full(n_blocks, elems)], axis=1).astype(np.uint64)
+    lists = kvt_amd.BlockLists()
+    lists.append(0, ranges)
+    cap_s, cap_d = pool * block, pool * elems
+    plan = kvt_amd.Plan(0, kvt_amd.RunLists.compress(lists), [cap_s], [cap_d], bf16_to_fp8=True)
+    src = [[tp._dev_bytes(cap_s, 30 + l, "raw")] for l in range(n_layers)]
+    dst = [[torch.full((cap_d,), 0xA5, dtype=torch.uint8, device="cuda")] for _ in range(n_layers)]
+    stride = plan.layer_bytes
+    packed = torch.zeros(n_layers * stride, dtype=torch.uint8, device="cuda")
+    kvt_amd.set_copy_cu_usage(0, usage)
+    try:
+        plan.pack(kvt_amd.Cache(0, src, [cap_s]), 0, n_layers, packed, stride)
+        plan.unpack(kvt_amd.Cache(0, dst, [cap_d]), 0, n_layers, packed, stride)
+        torch.cuda.synchronize()
+    finally:
+        kvt_amd.set_copy_cu_usage(0, 1.0)
+    for l in range(n_layers):
+        blob = tr._oracle_pack_fp8(tp._host(src[l][0]), ranges)
+        assert np.array_equal(tp._host(packed)[l * stride:l * stride + len(blob)], blob), l
+        exp = np.full(cap_d, 0xA5, dtype=np.uint8)
+        checkers.oracle_unpack(exp, ranges, blob)
+        assert np.array_equal(tp._host(dst[l][0]), exp), l
+
+
 def test_more_limited_launches_in_flight_than_ticket_blocks():
     """A limited launch of the pipelined kernels borrows a block of counters until it has run.
     Thousands of launches queued without a wait outnumber the blocks: those that find none run
