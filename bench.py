@@ -919,13 +919,13 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "6bec095577269b429bbd1e4544b07e04b85b1ff9e03636a739813f473ca6c631"
+KERNELS_SHA256 = "96cc727430f2a47695f2dc58f5311b51ecf65fb0c5dc15ab7a47e61444203041"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134275671, "unpack": 134276951},
-    (2, "ranges"): {"pack": 71013181533, "unpack": 73358399679},
-    (3, "ranges"): {"pack": 85983094148, "unpack": 85983583018},
-    (4, "ranges"): {"pack": 22690385904, "unpack": 22690444784},
-    (5, "ranges"): {"pack": 45141191548, "unpack": 45141394298},
+    (1, "ranges"): {"pack": 134267182, "unpack": 134277593},
+    (2, "ranges"): {"pack": 71013168478, "unpack": 73358403376},
+    (3, "ranges"): {"pack": 85983095771, "unpack": 85983579778},
+    (4, "ranges"): {"pack": 22690375536, "unpack": 22690444271},
+    (5, "ranges"): {"pack": 45141193160, "unpack": 45141392582},
 }
 
 
