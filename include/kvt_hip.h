@@ -288,6 +288,73 @@ int kvt_unpack_at(const kvt_plan* p, const kvt_cache* cache, uint32_t first_laye
                   uint32_t n_layers, const void* base, uint64_t layer_stride,
                   const uint64_t* blob_offsets, void* stream);
 
+/* ------------------------------- plan slots: a new batch per replay of a graph */
+
+/* A plan whose table lives at a FIXED device address and is refilled for every batch, so that
+ * launches recorded once into a hipGraph (kvt_pack / kvt_unpack / kvt_session_save_layer inside
+ * a stream capture) move a new batch on every replay. The reference builds a new range list for
+ * every batch                                     kvtransfer/src/tx_stub.cpp:158-263 (do_task)
+ * and sends it layer by layer                     kvtransfer/src/tx_stub.cpp:395-415,
+ * with the per-layer event recorded every step    blade_kvt/kv_transfer_impl.py:319-327;
+ * a plan made by kvt_plan_create names one batch for good, and a graph that holds its launches
+ * can only ever replay that batch. A slot is the plan for an engine whose forward pass is a
+ * replayed graph.
+ *
+ * What a recorded launch fixes: the slot (table address and capacity), the cache, the packed
+ * buffer and its layer stride, the launch grid -- a slot is always served by persistent
+ * workgroups, at most one or two per CU (fewer under kvt_set_copy_cu_usage as set when the
+ * launch was recorded). What follows the batch: the number of table entries, where each
+ * tensor's blob starts inside a packed layer and the blobs' sizes; the kernels read them from
+ * a header in front of the table.
+ *
+ *   chunk_bytes      size of a table entry: a power of two, 4096 ... 32768 for plain slots
+ *                    (0 = 32768), up to 524288 for transposing ones and for slots made for
+ *                    runs (0 = 32768; a transposing slot holds at least one token row per entry)
+ *   max_entries      table capacity per direction; a batch that needs more is refused
+ *   max_layer_bytes  room of one layer in the packed buffer (what the launches check the
+ *                    buffer against, and the smallest layer_stride accepted); a batch whose
+ *                    packed layer is larger is refused. 0 = max_entries * chunk_bytes + 256 *
+ *                    n_tensors, which no batch that fits the table exceeds
+ * Everything a slot moves must be 16-byte aligned (range offsets and lengths, layer tensors,
+ * packed buffer, layer stride): a batch that is not is refused by the fill, a cache or buffer
+ * that is not by the launch. kvt_pack_at / kvt_unpack_at (caller-chosen blob positions) do
+ * not take a slot. xform as for kvt_plan_create (may be NULL). */
+typedef struct kvt_slot_layout {
+  uint64_t n_entries;                       /* table entries the batch took                     */
+  uint64_t layer_bytes;                     /* bytes of one packed layer of this batch          */
+  uint32_t n_tensors, reserved0;
+  uint64_t tensor_bytes[KVT_MAX_TENSORS];   /* what kvt_plan_tensor_bytes / _offset say of a    */
+  uint64_t tensor_offset[KVT_MAX_TENSORS];  /* plan made from the same lists                    */
+} kvt_slot_layout;
+int kvt_plan_slot_create(int device, uint32_t n_tensors, const uint64_t* src_capacity,
+                         const uint64_t* dst_capacity, const kvt_xform* xform, uint32_t chunk_bytes,
+                         uint64_t max_entries, uint64_t max_layer_bytes, kvt_plan** out);
+/* The same for batches in run form (kvt_parse_block_runs): strided table entries, the per-token
+ * arithmetic done by the kernel; bf16_to_fp8 != 0 as kvt_plan_create_runs_bf16_to_fp8. A run
+ * whose group of records (one token's K and V, or one record) is larger than chunk_bytes makes
+ * the fill fail. */
+int kvt_plan_slot_create_runs(int device, uint32_t n_tensors, const uint64_t* src_capacity,
+                              const uint64_t* dst_capacity, uint32_t chunk_bytes, int bf16_to_fp8,
+                              uint64_t max_entries, uint64_t max_layer_bytes, kvt_plan** out);
+/* Puts a batch into the slot: `lists` as for kvt_plan_create (merged by the caller for PEQD; a
+ * list container without tensors, or with empty lists, is an empty batch: launches then move
+ * nothing and a session still signals every layer). The tables are built in pinned memory and
+ * copied to the device asynchronously on `stream`: work queued on `stream` afterwards -- the
+ * launch of the graph, normally -- sees the new batch, work queued before it the old one.
+ * Launches on other streams: eager ones order themselves behind the fill (and the fill behind
+ * them); a graph launched on another stream must be ordered by the caller. Never inside a
+ * stream capture. Refused, with the slot's contents untouched: a batch that needs more than
+ * max_entries entries or max_layer_bytes per layer (KVT_ERR_OUT_OF_RANGE), ranges outside the
+ * capacities given at creation (KVT_ERR_OUT_OF_RANGE), ranges that are not 16-byte aligned
+ * (KVT_ERR_INVALID). The host may run ahead of the device by one fill without blocking; a third
+ * fill waits until the first one's copy has run. *layout (may be NULL) receives where the
+ * blobs of this batch lie; kvt_plan_tensor_bytes / _offset / _layer_bytes / _num_chunks of the
+ * slot answer for the newest fill. One thread at a time fills a slot. */
+int kvt_plan_slot_fill(kvt_plan* slot, const kvt_block_lists* lists, void* stream,
+                       kvt_slot_layout* layout);
+int kvt_plan_slot_fill_runs(kvt_plan* slot, const kvt_run_lists* lists, void* stream,
+                            kvt_slot_layout* layout);
+
 /* ------------------------------------------ layer-message framing (host) */
 
 /* The per-layer messages of the staged transports:
@@ -397,6 +464,11 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
 int kvt_set_copy_cu_usage(int device, double usage);
 /* The current setting and the workgroup limit it stands for (0 = none); either may be NULL. */
 int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
+/* Counters of the launches limited to a CU share that wanted a block of work counters, since
+ * the first kvt_set_copy_cu_usage(device, < 1): out[0] eager launches that got one, out[1] eager
+ * launches that found none free (they ran with a fixed stride per workgroup instead: slower,
+ * same result), out[2] / out[3] the same for launches recorded into a stream capture. */
+int kvt_get_copy_ticket_stats(int device, uint64_t out[4]);
 
 /* No counterpart in the reference (its copy kernel uses one load flavour). A pack / unpack
  * launch whose payload (bytes moved one way, all layers of the launch) is at most
@@ -574,8 +646,10 @@ void kvt_session_destroy(kvt_session* s);
  * `packed` (stream, events and counters of a session are not cheap to create; a sender keeps
  * one session per destination and gives it each batch's plan). Layers already issued keep
  * what they were issued with. Refused once save_layer calls of this session have been captured
- * into a graph (the graph would go on launching the old plan). Call it from the thread that
- * drives the forward pass, between steps. */
+ * into a graph (the graph would go on launching the old plan) -- unless the session was made
+ * with a plan slot and is given the same slot, buffer and stride again: such a session takes
+ * its next batch through kvt_plan_slot_fill, captured or not, and needs no call here. Call it
+ * from the thread that drives the forward pass, between steps. */
 int kvt_session_set_plan(kvt_session* s, const kvt_plan* plan, void* packed, uint64_t layer_stride);
 /* Host only, never captured: starts step *step (1, 2, ...). Eager use: call before the step's
  * first save_layer. Graph use: call before EACH launch of a graph that holds captured

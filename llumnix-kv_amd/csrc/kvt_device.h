@@ -54,6 +54,31 @@ struct StrideTable {
   StrideShape shape[kMaxShapes];
 };
 
+// What stands in front of a slot's table in device memory (a plan slot: a table at a fixed
+// address that is refilled for every batch, so that launches recorded into a hipGraph find the
+// new batch on every replay): everything a launch would otherwise get as an argument and that
+// changes with the batch.
+struct __attribute__((aligned(256))) SlotHeader {
+  uint32_t n_entries;       // table entries of the batch in the slot (0: nothing to move)
+  uint32_t reserved[3];
+  BlobOffsets blobs;
+  uint8_t pad[256 - 16 - sizeof(BlobOffsets)];
+  StrideTable shapes;       // record shapes of strided entries (slots made for runs)
+};
+static_assert(sizeof(SlotHeader) == 256 + sizeof(StrideTable), "SlotHeader layout");
+constexpr uint64_t kSlotTableOffset = 2048;   // the pack table; the unpack table follows it at capacity entries
+static_assert(sizeof(SlotHeader) <= kSlotTableOffset, "the header must fit in front of the table");
+enum { kSlotPlain = 0, kSlotXform = 1, kSlotStrided = 2, kSlotConvert = 3 };
+// One launch over a slot's table by `wgs` persistent workgroups (a multiple of 8): the
+// pipelined kernels of launch_copy_entries / launch_strided_entries / launch_xform_entries /
+// launch_convert_entries with the entry count, blob positions and record shapes read from `hdr`.
+// Same requirements: everything 16-byte aligned, entries of at most 4096 << sub_shift bytes
+// (plain tables: sub_shift <= 3), less than 2 GiB per entry on the cache side.
+hipError_t launch_slot(int kind, bool pack, const Chunk* chunks, const SlotHeader* hdr, uint32_t sub_shift,
+                       uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                       uint32_t n_layers, uint8_t* packed, uint64_t layer_stride, const XformDev& x,
+                       uint32_t wgs, uint32_t* tickets, hipStream_t stream);
+
 // Chunk launchers. max_wgs = 0: one workgroup per (4 KiB slice, layer), the fastest shape.
 // max_wgs > 0: at most that many workgroups (a multiple of 8), striding over the same items,
 // for a caller that wants the copy to leave part of the device to other kernels.

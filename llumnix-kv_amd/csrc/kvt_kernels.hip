@@ -1289,11 +1289,11 @@ __global__ __launch_bounds__(kThreads, 8) void convert_chunks_kernel(
 // 8-byte store through the packed-side descriptor. Record arithmetic as in
 // strided_entries_kernel, in groups: a record of vlen * 16 elements is 2 * vlen groups.
 template <int V>
-__global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
+__device__ __forceinline__ void convert_entries(
     const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    StrideTable shapes, uint32_t* tickets) {
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, const BlobOffsets& blobs,
+    const StrideTable& shapes, uint32_t* tickets) {
   constexpr int G = 2 * V;  // groups per lane and trip
   EntryWalk walk(n_chunks << part_shift, n_layers, tickets, V == 8 ? 3u : (V == 4 ? 2u : 1u));
   const Entry* table = reinterpret_cast<const Entry*>(chunks);
@@ -1353,15 +1353,24 @@ __global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
   KVT_ROTATE3(fetch, nothing, store);
   walk.leave();
 }
+template <int V>
+__global__ __launch_bounds__(kThreads, 4) void convert_entries_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks, uint32_t part_shift,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes, uint32_t* tickets) {
+  convert_entries<V>(chunks, n_chunks, part_shift, layer_ptrs, n_tensors, first_layer, n_layers, packed,
+                     layer_stride, blobs, shapes, tickets);
+}
 
 // Converting tables with entries of 4096 elements: a wavefront per entry (see
 // copy_entries_by_wave_kernel), lane t of the wavefront the groups t, t + 64, ... t + 448.
 template <int U>
-__global__ __launch_bounds__(kThreads, 4) void convert_entries_by_wave_kernel(
+__device__ __forceinline__ void convert_entries_by_wave(
     const Chunk* __restrict__ chunks, uint32_t n_chunks,
     uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
-    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
-    StrideTable shapes, uint32_t* tickets) {
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, const BlobOffsets& blobs,
+    const StrideTable& shapes, uint32_t* tickets) {
   constexpr int G = 8;  // groups per lane and entry
   EntryWalk walk(n_chunks, n_layers, tickets, 0u);
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1427,6 +1436,97 @@ __global__ __launch_bounds__(kThreads, 4) void convert_entries_by_wave_kernel(
   };
   KVT_ROTATE3(fetch, nothing, store);
   walk.leave();
+}
+template <int U>
+__global__ __launch_bounds__(kThreads, 4) void convert_entries_by_wave_kernel(
+    const Chunk* __restrict__ chunks, uint32_t n_chunks,
+    uint8_t* const* __restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+    uint32_t n_layers, uint8_t* __restrict__ packed, uint64_t layer_stride, BlobOffsets blobs,
+    StrideTable shapes, uint32_t* tickets) {
+  convert_entries_by_wave<U>(chunks, n_chunks, layer_ptrs, n_tensors, first_layer, n_layers, packed,
+                             layer_stride, blobs, shapes, tickets);
+}
+
+// ------------------------------------------------------------------ plan slots
+//
+// A slot is a chunk table at a fixed device address whose contents change from batch to batch:
+// the launches that read it can be recorded into a hipGraph once and replayed for every batch.
+// What varies with the batch -- the number of entries, where each tensor's blob starts in a
+// packed layer, the record shapes of strided entries -- lives in a header in front of the table
+// and is read here, not passed as kernel arguments; what a recorded launch fixes is the grid,
+// so these are the persistent kernels above (whose grid does not depend on the table's length)
+// with the header's values in place of the arguments. An empty batch ends every workgroup at once.
+#define KVT_SLOT_PARAMS                                                                              \
+  const Chunk *__restrict__ chunks, const SlotHeader *__restrict__ hdr,                              \
+      uint8_t *const *__restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,             \
+      uint32_t n_layers, uint8_t *packed, uint64_t layer_stride, uint32_t *tickets
+#define KVT_SLOT_TAIL layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, hdr->blobs
+
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void copy_entries_slot_kernel(KVT_SLOT_PARAMS) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  copy_entries<PACK, V>([&](uint32_t e) { return table[e]; }, n_chunks, KVT_SLOT_TAIL, tickets);
+}
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void copy_entries_by_wave_slot_kernel(KVT_SLOT_PARAMS) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  const Entry* table = reinterpret_cast<const Entry*>(chunks);
+  copy_entries_by_wave<PACK, V, U>([&](uint32_t e) { return table[e]; }, n_chunks, KVT_SLOT_TAIL, tickets);
+}
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void strided_entries_slot_kernel(KVT_SLOT_PARAMS, uint32_t part_shift) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  const uint32_t lane = threadIdx.x << 4;
+  entries_pipeline<PACK, V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL, tickets,
+                            [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
+                              strided_offsets<PACK, V, kSliceShift>(hdr->shapes, c, begin, bytes, lane, coff);
+                            });
+}
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void strided_entries_by_wave_slot_kernel(KVT_SLOT_PARAMS) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  const uint32_t lane = (threadIdx.x & 63u) << 4;
+  entries_pipeline_by_wave<PACK, V, U>(chunks, n_chunks, KVT_SLOT_TAIL, tickets,
+                                       [&](const Entry& c, uint32_t bytes, uint32_t* coff) {
+                                         strided_offsets<PACK, V, 10>(hdr->shapes, c, 0u, bytes, lane, coff);
+                                       });
+}
+template <bool PACK, int V>
+__global__ __launch_bounds__(kThreads, 4) void xform_entries_slot_kernel(KVT_SLOT_PARAMS, uint32_t part_shift,
+                                                                        XformDev x) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  const uint32_t lane = threadIdx.x << 4;
+  entries_pipeline<PACK, V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL, tickets,
+                            [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
+                              xform_offsets<V, kSliceShift>(x, c, begin, bytes, lane, coff);
+                            });
+}
+template <bool PACK, int V, int U>
+__global__ __launch_bounds__(kThreads, 4) void xform_entries_by_wave_slot_kernel(KVT_SLOT_PARAMS, XformDev x) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  const uint32_t lane = (threadIdx.x & 63u) << 4;
+  entries_pipeline_by_wave<PACK, V, U>(chunks, n_chunks, KVT_SLOT_TAIL, tickets,
+                                       [&](const Entry& c, uint32_t bytes, uint32_t* coff) {
+                                         xform_offsets<V, 10>(x, c, 0u, bytes, lane, coff);
+                                       });
+}
+template <int V>
+__global__ __launch_bounds__(kThreads, 4) void convert_entries_slot_kernel(KVT_SLOT_PARAMS, uint32_t part_shift) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  convert_entries<V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL, hdr->shapes, tickets);
+}
+__global__ __launch_bounds__(kThreads, 4) void convert_entries_by_wave_slot_kernel(KVT_SLOT_PARAMS) {
+  const uint32_t n_chunks = hdr->n_entries;
+  if (n_chunks == 0) return;
+  convert_entries_by_wave<1>(chunks, n_chunks, KVT_SLOT_TAIL, hdr->shapes, tickets);
 }
 
 // Plain linear copy with the gather kernel's slice shape (calibration / ceiling).
@@ -1781,6 +1881,73 @@ hipError_t launch_convert_ranges(const void* src_base, void* dst_base, const int
                      stream, static_cast<const uint8_t*>(src_base),
                      static_cast<uint8_t*>(dst_base), src_off, dst_off, lens, n);
   return hipGetLastError();
+}
+
+hipError_t launch_slot(int kind, bool pack, const Chunk* chunks, const SlotHeader* hdr, uint32_t sub_shift,
+                       uint8_t* const* layer_ptrs, uint32_t n_tensors, uint32_t first_layer,
+                       uint32_t n_layers, uint8_t* packed, uint64_t layer_stride, const XformDev& x,
+                       uint32_t wgs, uint32_t* tickets, hipStream_t stream) {
+  if (n_layers == 0) return hipSuccess;
+  if (wgs < 8 || (wgs & 7u) || sub_shift > 7) return hipErrorInvalidValue;
+  const dim3 grid(wgs), block(kThreads);
+#define KVT_ARGS chunks, hdr, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, tickets
+#define KVT_GO(KERNEL, ...) hipLaunchKernelGGL(KERNEL, grid, block, 0, stream, KVT_ARGS, ##__VA_ARGS__)
+#define KVT_EITHER(KERNEL_PACK, KERNEL_UNPACK, ...) \
+  do {                                              \
+    if (pack) KVT_GO(KERNEL_PACK, ##__VA_ARGS__);   \
+    else KVT_GO(KERNEL_UNPACK, ##__VA_ARGS__);      \
+  } while (0)
+  int v = 0;
+  uint32_t part_shift = 0;
+  if (kind == kSlotPlain || (kind == kSlotConvert && !pack)) {
+    // (the unpack of a converting table moves plain fp8 bytes, but its entries may be strided)
+    if (kind == kSlotConvert) goto strided;
+    if (sub_shift > 3) return hipErrorInvalidValue;
+    switch (sub_shift) {
+      case 0: KVT_EITHER((copy_entries_by_wave_slot_kernel<true, 4, 2>), (copy_entries_by_wave_slot_kernel<false, 4, 2>)); break;
+      case 1: KVT_EITHER((copy_entries_by_wave_slot_kernel<true, 8, 1>), (copy_entries_by_wave_slot_kernel<false, 8, 1>)); break;
+      case 2: KVT_EITHER((copy_entries_slot_kernel<true, 4>), (copy_entries_slot_kernel<false, 4>)); break;
+      default: KVT_EITHER((copy_entries_slot_kernel<true, 8>), (copy_entries_slot_kernel<false, 8>)); break;
+    }
+    return hipGetLastError();
+  }
+  if (kind == kSlotXform) {
+    if (sub_shift == 0) {
+      KVT_EITHER((xform_entries_by_wave_slot_kernel<true, 4, 2>), (xform_entries_by_wave_slot_kernel<false, 4, 2>), x);
+    } else if (sub_shift == 1) {
+      KVT_EITHER((xform_entries_by_wave_slot_kernel<true, 8, 1>), (xform_entries_by_wave_slot_kernel<false, 8, 1>), x);
+    } else {
+      // the scatter keeps its offsets until the stores: 8 slices per trip would not fit the registers
+      if (!entries_shape(sub_shift, wgs, pack ? 8 : 4, &v, &part_shift)) return hipErrorInvalidValue;
+      if (v == 8) KVT_GO((xform_entries_slot_kernel<true, 8>), part_shift, x);
+      else KVT_EITHER((xform_entries_slot_kernel<true, 4>), (xform_entries_slot_kernel<false, 4>), part_shift, x);
+    }
+    return hipGetLastError();
+  }
+  if (kind == kSlotConvert) {
+    if (sub_shift == 0) {
+      KVT_GO(convert_entries_by_wave_slot_kernel);
+    } else {
+      if (!entries_shape(sub_shift, wgs, 4, &v, &part_shift)) return hipErrorInvalidValue;
+      if (v == 4) KVT_GO((convert_entries_slot_kernel<4>), part_shift);
+      else KVT_GO((convert_entries_slot_kernel<2>), part_shift);
+    }
+    return hipGetLastError();
+  }
+strided:
+  if (sub_shift == 0) {
+    KVT_EITHER((strided_entries_by_wave_slot_kernel<true, 4, 2>), (strided_entries_by_wave_slot_kernel<false, 4, 2>));
+  } else if (sub_shift == 1) {
+    KVT_EITHER((strided_entries_by_wave_slot_kernel<true, 8, 1>), (strided_entries_by_wave_slot_kernel<false, 8, 1>));
+  } else {
+    if (!entries_shape(sub_shift, wgs, 8, &v, &part_shift)) return hipErrorInvalidValue;
+    if (v == 8) KVT_EITHER((strided_entries_slot_kernel<true, 8>), (strided_entries_slot_kernel<false, 8>), part_shift);
+    else KVT_EITHER((strided_entries_slot_kernel<true, 4>), (strided_entries_slot_kernel<false, 4>), part_shift);
+  }
+  return hipGetLastError();
+#undef KVT_EITHER
+#undef KVT_GO
+#undef KVT_ARGS
 }
 
 hipError_t launch_copy_linear(void* dst, const void* src, uint64_t bytes, hipStream_t stream) {

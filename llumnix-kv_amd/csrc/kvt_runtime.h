@@ -77,11 +77,17 @@ inline uint64_t round_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 class TicketPool {
  public:
   static constexpr uint32_t kBlockBytes = 2048, kBlocks = 1024;
+  // blocks [0, kEagerBlocks) are lent to eager launches, the rest belong to captured ones
+  static constexpr uint32_t kEagerBlocks = 768;
   // Allocates the device's blocks (no-op when they exist). Not inside a stream capture.
   int prepare(int device);
-  // A block no running launch uses, or nullptr. permanent: taken out of circulation until
-  // give_back(); otherwise the caller calls launched() once the kernel is on `stream`.
+  // A block no running launch uses, or nullptr. permanent (a launch that is being recorded
+  // into a stream capture): taken out of circulation until give_back(), found without any
+  // call into the runtime; otherwise the caller calls launched() once the kernel is on `stream`.
   uint32_t* acquire(int device, bool permanent);
+  // {eager launches that got a block, eager launches that found none, captured launches that
+  // got one, captured launches that found none} since the device's blocks were allocated.
+  void stats(int device, uint64_t out[4]);
   void launched(int device, uint32_t* block, hipStream_t stream);
   // A permanent block whose graph is gone, or a borrowed one whose launch never happened.
   void give_back(int device, uint32_t* block);
@@ -92,7 +98,8 @@ class TicketPool {
     uint8_t* arena = nullptr;
     std::vector<hipEvent_t> done;
     std::vector<uint8_t> state;
-    uint32_t cursor = 0;
+    uint32_t cursor = 0, capture_cursor = 0;
+    uint64_t counters[4] = {0, 0, 0, 0};
   };
   PerDevice* of(int device);  // under mu_
   std::mutex mu_;
@@ -245,6 +252,9 @@ class TablePool {
  private:
   static constexpr size_t kMaxIdle = 4096;
   static constexpr size_t kMaxIdleBytes = size_t(256) << 20;  // device memory, and as much pinned
+ public:
+  // Frees what a buffer holds (device memory, pinned twin, events; its graphs' ticket blocks go
+  // back to their pool).
   static void destroy(TableBuf* b) {
     for (uint32_t* t : b->graph_tickets) ticket_pool().give_back(b->device, t);
     b->graph_tickets.clear();
@@ -254,6 +264,8 @@ class TablePool {
     b->uses.clear();
     b->dev = b->host = nullptr;
   }
+
+ private:
   std::mutex mu_;
   std::vector<TableBuf*> idle_;
   size_t idle_bytes_ = 0;
@@ -277,8 +289,31 @@ struct kvt_cache {
   bool aligned4 = true;   // ... on a 4-byte boundary
 };
 
+namespace kvt {
+// A plan slot (kvt_plan_slot_create): the plan's table lives at a fixed device address with a
+// header in front (SlotHeader) and is rewritten for every batch by kvt_plan_slot_fill, through
+// one of two pinned staging copies in turn. The plan's TableBuf holds the device memory (never
+// recycled through the pool) and the record of eager launches that still read it.
+struct Slot {
+  int kind = kSlotPlain;
+  uint64_t max_entries = 0, max_layer_bytes = 0;
+  uint32_t chunk_bytes = 0;
+  uint32_t ntpb = 0;                 // layout transform: tokens per page
+  uint64_t half = 0, tok_bytes = 0;  // ... bytes of a half page and of one token row
+  uint8_t* host[2] = {nullptr, nullptr};
+  hipEvent_t staged[2] = {nullptr, nullptr};  // the copy out of host[i] has run
+  bool staged_rec[2] = {false, false};
+  uint32_t turn = 0;
+  hipEvent_t filled = nullptr;       // the newest contents have reached the device
+  hipStream_t filled_on = nullptr;
+  bool filled_rec = false;
+  std::mutex mu;                     // a fill against launches from other threads
+};
+}  // namespace kvt
+
 struct kvt_plan {
   int device = 0;
+  kvt::Slot* slot = nullptr;       // non-null: a plan slot, refilled per batch
   uint32_t n_tensors = 0;
   uint64_t n_chunks = 0;
   std::vector<uint64_t> tensor_bytes, tensor_offset, src_cap, dst_cap;

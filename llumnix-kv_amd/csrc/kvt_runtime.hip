@@ -168,9 +168,25 @@ uint32_t* TicketPool::acquire(int device, bool permanent) {
   std::lock_guard<std::mutex> lock(mu_);
   PerDevice* d = of(device);
   if (!d || !d->arena) return nullptr;
+  if (permanent) {
+    // For a launch that is being recorded into a stream capture: no runtime call may be made
+    // here (an event query inside a capture can be refused, or end the capture), so these
+    // launches have blocks of their own that are never lent to eager launches and are simply
+    // free or taken.
+    for (uint32_t probe = 0; probe < kBlocks - kEagerBlocks; ++probe) {
+      const uint32_t i = kEagerBlocks + (d->capture_cursor + probe) % (kBlocks - kEagerBlocks);
+      if (d->state[i] != kFree) continue;
+      d->state[i] = kPermanent;
+      d->capture_cursor = (i + 1 - kEagerBlocks) % (kBlocks - kEagerBlocks);
+      ++d->counters[2];
+      return reinterpret_cast<uint32_t*>(d->arena + static_cast<size_t>(i) * kBlockBytes);
+    }
+    ++d->counters[3];
+    return nullptr;
+  }
   // a few probes from where the last search ended: blocks come free in the order they were lent
   for (uint32_t probe = 0; probe < 32; ++probe) {
-    const uint32_t i = (d->cursor + probe) % kBlocks;
+    const uint32_t i = (d->cursor + probe) % kEagerBlocks;
     if (d->state[i] == kPermanent || d->state[i] == kLent) continue;
     if (d->state[i] == kInFlight) {
       if (hipEventQuery(d->done[i]) != hipSuccess) {
@@ -179,18 +195,27 @@ uint32_t* TicketPool::acquire(int device, bool permanent) {
       }
       d->state[i] = kFree;
     }
-    if (!permanent && !d->done[i] &&
+    if (!d->done[i] &&
         hipEventCreateWithFlags(&d->done[i], hipEventDisableTiming) != hipSuccess) {
       (void)hipGetLastError();
       d->done[i] = nullptr;
+      ++d->counters[1];
       return nullptr;
     }
-    d->state[i] = permanent ? kPermanent : kLent;
-    d->cursor = (i + 1) % kBlocks;
+    d->state[i] = kLent;
+    d->cursor = (i + 1) % kEagerBlocks;
+    ++d->counters[0];
     return reinterpret_cast<uint32_t*>(d->arena + static_cast<size_t>(i) * kBlockBytes);
   }
-  d->cursor = (d->cursor + 32) % kBlocks;
+  d->cursor = (d->cursor + 32) % kEagerBlocks;
+  ++d->counters[1];
   return nullptr;
+}
+
+void TicketPool::stats(int device, uint64_t out[4]) {
+  std::lock_guard<std::mutex> lock(mu_);
+  PerDevice* d = of(device);
+  for (int i = 0; i < 4; ++i) out[i] = d ? d->counters[i] : 0;
 }
 
 void TicketPool::launched(int device, uint32_t* block, hipStream_t stream) {
@@ -268,6 +293,13 @@ int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups) {
     if (bits != 0) std::memcpy(usage, &bits, sizeof(bits));
   }
   if (max_workgroups) *max_workgroups = g_wg_cap[device].load(std::memory_order_relaxed);
+  return KVT_OK;
+}
+
+int kvt_get_copy_ticket_stats(int device, uint64_t out[4]) {
+  if (!out) return fail(KVT_ERR_INVALID, "kvt_get_copy_ticket_stats: null argument");
+  if (int rc = check_device(device)) return rc;
+  ticket_pool().stats(device, out);
   return KVT_OK;
 }
 

@@ -71,9 +71,14 @@ namespace {
 // One lane per layer: the layer's completion count, bumped in device memory and mirrored to
 // the host. The pack kernel in front of it on the stream has ended, so its stores have left
 // the caches.
+// The count after `c`: 1, 2, ... 2^32 - 1, 1, ... Zero is left out on both sides (the host's
+// `submitted` and the device's counter step alike), because a step's target of 0 means "not
+// submitted yet".
+__host__ __device__ inline uint32_t next_count(uint32_t c) { return c + 1u != 0u ? c + 1u : 1u; }
+
 __global__ void publish_layers_kernel(uint32_t* count_dev, uint32_t* count_host, uint32_t n) {
   for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
-    const uint32_t c = count_dev[i] + 1u;
+    const uint32_t c = next_count(count_dev[i]);
     count_dev[i] = c;
     __hip_atomic_store(count_host + i, c, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
   }
@@ -89,7 +94,7 @@ uint64_t begin_step_locked(kvt_session* s) {
   st.message.clear();
   st.target.assign(s->cache->n_layers, 0);
   for (uint32_t l = 0; l < s->cache->n_layers; ++l)
-    if (s->in_graph[l]) st.target[l] = ++s->submitted[l];
+    if (s->in_graph[l]) st.target[l] = s->submitted[l] = next_count(s->submitted[l]);
   return id;
 }
 
@@ -105,7 +110,7 @@ int timed_out(uint32_t layer) {
 int poll_layer(kvt_session* s, uint32_t layer, uint32_t target, const Clock::time_point* deadline) {
   const uint32_t* word = s->count_host + layer;
   for (uint32_t spins = 0;; ++spins) {
-    // counts only grow; the comparison survives wrap-around of the 32-bit counter
+    // counts only grow (next_count); the comparison survives wrap-around of the 32-bit counter
     if (static_cast<int32_t>(__atomic_load_n(word, __ATOMIC_ACQUIRE) - target) >= 0) return KVT_OK;
     if (spins < 2000) {
 #if defined(__x86_64__)
@@ -196,8 +201,11 @@ int kvt_session_set_plan(kvt_session* s, const kvt_plan* plan, void* packed, uin
     if (layer_stride < plan->min_layer_stride)
       return fail(KVT_ERR_INVALID, "kvt_session_set_plan: layer_stride smaller than one packed layer");
     std::lock_guard<std::mutex> lock(s->mu);
+    // a plan slot takes its batches through kvt_plan_slot_fill: the same slot, buffer and stride
+    // again change nothing a captured launch has fixed
+    const bool same_slot = plan->slot && plan == s->plan && packed == s->packed && layer_stride == s->layer_stride;
     for (uint8_t g : s->in_graph)
-      if (g)
+      if (g && !same_slot)
         return fail(KVT_ERR_INVALID,
                     "kvt_session_set_plan: a captured graph still launches the session's old plan");
     s->plan = plan;
@@ -252,7 +260,8 @@ static int issue_layers(kvt_session* s, uint32_t first, uint32_t n, hipEvent_t r
     if (s->cur_step == 0) begin_step_locked(s);  // a session used for one step needs no begin_step
     kvt_session::Step& st = s->step_slot(s->cur_step);
     if (rc == KVT_OK) {
-      for (uint32_t l = first; l < first + n; ++l) st.target[l] = ++s->submitted[l];
+      for (uint32_t l = first; l < first + n; ++l)
+        st.target[l] = s->submitted[l] = next_count(s->submitted[l]);
     } else if (st.error == KVT_OK) {   // latched: threads waiting for this step return it
       st.error = rc;
       st.message = kvt_last_error();

@@ -9,11 +9,12 @@ from .binding import (KvtError, LIB_PATH, BlockLists, RunLists, Cache, Parser, P
                       WireLayout, WIRE_TCP, WIRE_RDMA_STAGED, block_object_lists, device_count,
                       lib, select_parser, compute_valid_ranks_pd, merge_interval, validate_bounds,
                       wire_layout_of, wire_parse_frame, wire_write_frame, set_copy_cu_usage,
-                      get_copy_cu_usage, ObjectRing)
+                      get_copy_cu_usage, ObjectRing, PlanSlot, SlotLayout, copy_ticket_stats)
 from . import ctypes_defs
 
 __all__ = ["KvtError", "LIB_PATH", "BlockLists", "Cache", "Parser", "Plan", "Session", "Stager",
            "device_count", "lib", "select_parser", "compute_valid_ranks_pd", "merge_interval",
            "validate_bounds", "ctypes_defs", "WireLayout", "WIRE_TCP", "WIRE_RDMA_STAGED",
            "block_object_lists", "RunLists", "wire_layout_of", "wire_parse_frame", "wire_write_frame",
-           "set_copy_cu_usage", "get_copy_cu_usage", "ObjectRing"]
+           "set_copy_cu_usage", "get_copy_cu_usage", "ObjectRing", "PlanSlot", "SlotLayout",
+           "copy_ticket_stats"]

@@ -23,6 +23,11 @@ class WireLayout(C.Structure):
 WIRE_TCP, WIRE_RDMA_STAGED = 0, 1
 
 
+class SlotLayout(C.Structure):
+    _fields_ = [("n_entries", _u64), ("layer_bytes", _u64), ("n_tensors", _u32), ("reserved0", _u32),
+                ("tensor_bytes", _u64 * 8), ("tensor_offset", _u64 * 8)]
+
+
 class Xform(C.Structure):
     _fields_ = [("kind", _u32), ("heads", _u32), ("ntpb", _u32), ("row_bytes", _u32)]
 
@@ -76,6 +81,13 @@ SIGNATURES = {
     "kvt_plan_num_strided_chunks": (_u64, [_vp]),
     "kvt_plan_create_objects": (_int, [_int, _vp, _P(_u64), _P(_u64), _u64, _u64, _u32, _P(_vp)]),
     "kvt_plan_host_tables": (_int, [_vp, _P(_vp), _P(_u64), _P(_u32), _P(_vp)]),
+    "kvt_plan_slot_create": (_int, [_int, _u32, _P(_u64), _P(_u64), _P(Xform), _u32, _u64, _u64,
+                                    _P(_vp)]),
+    "kvt_plan_slot_create_runs": (_int, [_int, _u32, _P(_u64), _P(_u64), _u32, _int, _u64, _u64,
+                                         _P(_vp)]),
+    "kvt_plan_slot_fill": (_int, [_vp, _vp, _vp, _P(SlotLayout)]),
+    "kvt_plan_slot_fill_runs": (_int, [_vp, _vp, _vp, _P(SlotLayout)]),
+    "kvt_get_copy_ticket_stats": (_int, [_int, _P(_u64)]),
     "kvt_pack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
     "kvt_unpack_at": (_int, [_vp, _vp, _u32, _u32, _vp, _u64, _P(_u64), _vp]),
     "kvt_wire_layout_of": (_int, [_int, _vp, _P(WireLayout)]),
@@ -542,6 +554,46 @@ class Plan:
         offs = (_u64 * 8)(*blob_offsets)
         check(lib().kvt_unpack_at(self.h, cache.h, first_layer, n_layers, _ptr(base), layer_stride,
                                   offs, _ptr(stream)))
+
+
+class PlanSlot(Plan):
+    """A plan at a fixed device address that takes a new batch per fill (kvt_plan_slot_*): what
+    launches recorded into a hipGraph read, so that every replay moves the batch of its step.
+    runs=True: filled with RunLists (strided entries; bf16_to_fp8: converting pack)."""
+
+    def __init__(self, device, n_tensors, src_capacity, dst_capacity, max_entries, xform=None,
+                 chunk_bytes=0, max_layer_bytes=0, runs=False, bf16_to_fp8=False):
+        sc = (_u64 * n_tensors)(*src_capacity)
+        dc = (_u64 * n_tensors)(*dst_capacity)
+        self.h = _vp()
+        self.runs = runs
+        if runs:
+            if xform is not None:
+                raise ValueError("no layout transform for a slot made for runs")
+            check(lib().kvt_plan_slot_create_runs(device, n_tensors, sc, dc, chunk_bytes,
+                                                  1 if bf16_to_fp8 else 0, max_entries,
+                                                  max_layer_bytes, C.byref(self.h)))
+        else:
+            xf = C.byref(Xform(1, *xform)) if xform is not None else None
+            check(lib().kvt_plan_slot_create(device, n_tensors, sc, dc, xf, chunk_bytes,
+                                             max_entries, max_layer_bytes, C.byref(self.h)))
+
+    def fill(self, lists, stream=None):
+        """The next batch (BlockLists, or RunLists for a slot made for runs), copied to the
+        device on `stream` -> SlotLayout. Raises KvtError and leaves the slot as it was when
+        the batch does not fit."""
+        lay = SlotLayout()
+        fn = lib().kvt_plan_slot_fill_runs if self.runs else lib().kvt_plan_slot_fill
+        check(fn(self.h, lists.h, _ptr(stream), C.byref(lay)))
+        return lay
+
+
+def copy_ticket_stats(device):
+    """-> (eager launches with a block of work counters, eager launches that found none,
+    captured launches with one, captured launches that found none)"""
+    out = (_u64 * 4)()
+    check(lib().kvt_get_copy_ticket_stats(device, out))
+    return tuple(out)
 
 
 class Session:

@@ -270,27 +270,53 @@ def test_converting_plan_of_plain_aligned_ranges_under_a_limit(usage, block):
 
 def test_more_limited_launches_in_flight_than_ticket_blocks():
     """A limited launch of the pipelined kernels borrows a block of counters until it has run.
-    Thousands of launches queued without a wait outnumber the blocks: those that find none run
-    without (every workgroup a fixed share), and every result is still the oracle's."""
+    At an eighth of the device such a launch asks for one (a workgroup per CU). Thousands of
+    launches queued behind a kernel that holds the stream back outnumber the blocks: those that
+    find none run without (every workgroup a fixed share), and once the queue has drained the
+    blocks are lent again, each left zeroed by the launch that had it. Every result is the
+    oracle's, and the library's counters show that both paths were taken."""
     w = workloads.llama8b_single(n_layers=4, pool=256, tokens=2048)
     plan, lists = pipeline.build_plan(w, 0)
+    assert plan.num_chunks > 64                      # a resident table, not kernel arguments
     o_lists = tp._oracle_lists(w)
     src_layers = tp._make_caches(w, "src", 17)
     sc = kvt_amd.Cache(0, src_layers, w.capacities("src"))
     stride = plan.layer_bytes
     outs = [torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda") for _ in range(3)]
-    kvt_amd.set_copy_cu_usage(0, 0.004)
+    blobs = [checkers.oracle_pack(tp._host(src_layers[l][0]), o_lists[0]) for l in range(w.n_layers)]
+
+    def check():
+        for l in range(w.n_layers):
+            for out in outs:
+                assert np.array_equal(tp._host(out)[l * stride:l * stride + len(blobs[l])], blobs[l]), l
+
+    kvt_amd.set_copy_cu_usage(0, 0.125)
     try:
         stream = checkers.side_stream()
+        got0, none0 = kvt_amd.copy_ticket_stats(0)[:2]
+        with torch.cuda.stream(stream):
+            torch.cuda._sleep(400_000_000)           # some tenths of a second: the launches pile up
         for i in range(3000):
             plan.pack(sc, 0, w.n_layers, outs[i % 3], stride, stream.cuda_stream)
+        got1, none1 = kvt_amd.copy_ticket_stats(0)[:2]
         stream.synchronize()
+        check()
+        assert got1 - got0 > 0 and none1 - none0 > 0, (got0, none0, got1, none1)
+        assert (got1 - got0) + (none1 - none0) == 3000
+        # every block has been through a launch: the next ones reuse them
+        for out in outs:
+            out.zero_()
+        torch.cuda.synchronize()
+        for i in range(1500):
+            plan.pack(sc, 0, w.n_layers, outs[i % 3], stride, stream.cuda_stream)
+            if i % 100 == 99:
+                stream.synchronize()
+        stream.synchronize()
+        got2, none2 = kvt_amd.copy_ticket_stats(0)[:2]
+        assert got2 - got1 >= 1400, (got1, none1, got2, none2)
+        check()
     finally:
         kvt_amd.set_copy_cu_usage(0, 1.0)
-    for l in range(w.n_layers):
-        blob = checkers.oracle_pack(tp._host(src_layers[l][0]), o_lists[0])
-        for out in outs:
-            assert np.array_equal(tp._host(out)[l * stride:l * stride + len(blob)], blob), l
 
 
 @pytest.mark.parametrize("usage", [0.25, 0.004], ids=["quarter", "eight-workgroups"])

@@ -45,7 +45,9 @@ class _Transport(threading.Thread):
                     self.sess.wait_layer(l, step)
                     self.returned_at[(step, l)] = time.perf_counter()
                     host = torch.empty(self.blob_len, dtype=torch.uint8).pin_memory()
-                    torch.cuda.synchronize()          # what the default stream still holds comes first
+                    # straight after the wait, on this thread's stream alone: the rest of the
+                    # step or replay is still running, so equal bytes mean the layer was
+                    # complete when the wait returned
                     with torch.cuda.stream(stream):
                         host.copy_(self.packed[l * self.stride:l * self.stride + self.blob_len],
                                    non_blocking=True)
