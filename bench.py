@@ -28,19 +28,22 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_workload(cfg, scale):
+def build_workload(cfg, scale, variant=0):
+    """variant (config 2 only): another batch on the same pools (other lengths, other block
+    tables), for the legs that give a captured graph a new batch per replay."""
     from kvt_amd import workloads as W
     if cfg == 1:
         return [W.llama8b_single()]
     if cfg == 2:
+        seed = 20252 + 1000 * variant
         if scale < 1.0:
             return [W.llama8b_batch(n_layers=max(2, int(32 * scale)),
                                     src_pool=max(1024, int(16384 * scale)),
                                     dst_pool=max(1536, int(24576 * scale)),
                                     n_req=max(2, int(64 * scale)),
                                     min_tok=max(64, int(1024 * scale)),
-                                    max_tok=max(128, int(8192 * scale)))]
-        return [W.llama8b_batch()]
+                                    max_tok=max(128, int(8192 * scale)), seed=seed)]
+        return [W.llama8b_batch(seed=seed)]
     if cfg == 3:
         return [W.llama70b_flashinfer(n_layers=max(2, int(80 * scale)),
                                       pool=max(512, int(8192 * scale)),
@@ -356,6 +359,59 @@ def leg_latency(c, out):
     torch.cuda.synchronize()
     sess.close()
     c.keep_objs.append(held)
+    # The same per-layer sequence as ONE captured graph over a plan slot: per request ParseBlock,
+    # refill of the slot, launch of the graph, until the transport's wait for the last layer
+    # returns (host clock); and GPU time of the replay alone.
+    if args.plan == "ranges":
+        caps = (w.capacities("src"), w.capacities("dst"))
+        chunk = plan_chunk_bytes(kvt, first[0][1], caps, w.xform, args.chunk_bytes)
+        plan0 = first[0][0]
+        slot = kvt.PlanSlot(0, w.n_tensors, caps[0], caps[1], max_entries=max(1, plan0.num_chunks),
+                            xform=w.xform, chunk_bytes=chunk, max_layer_bytes=strides[0])
+        gsess = kvt.Session(slot, side.src_cache, packed[0], strides[0])
+        gs = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(gs):
+            with torch.cuda.graph(graph, stream=gs):
+                for l in range(w.n_layers):
+                    gsess.save_layer(l, gs.cuda_stream)
+                gsess.join(gs.cuda_stream)
+        g_wall, g_gpu, g_parse = [], [], []
+        with torch.cuda.stream(gs):
+            for r in [reqs[0]] + reqs:           # the first pass warms up
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                lists = sender.parse([tasks[0][r]])
+                t1 = time.perf_counter()
+                slot.fill(lists, gs.cuda_stream)
+                step = gsess.begin_step()
+                lib.kvt_event_record(a, gs.cuda_stream)
+                graph.replay()
+                lib.kvt_event_record(b, gs.cuda_stream)
+                gsess.wait_layer(w.n_layers - 1, step)
+                g_wall.append((time.perf_counter() - t0) * 1e6)
+                g_parse.append((t1 - t0) * 1e6)
+                lib.kvt_event_synchronize(b)
+                g_gpu.append(ev_ms(lib, a, b) * 1e3)
+                lists.close()
+        torch.cuda.synchronize()
+        # the last request once more through a plan of its own: same bytes
+        lists = sender.parse([tasks[0][reqs[-1]]])
+        fresh = kvt.Plan(0, lists, caps[0], caps[1], xform=w.xform, chunk_bytes=chunk)
+        probe = torch.empty(max(1, strides[0]), dtype=torch.uint8, device="cuda")
+        fresh.pack(side.src_cache, w.n_layers - 1, 1, probe, strides[0], gs.cuda_stream)
+        gs.synchronize()
+        nb = fresh.layer_bytes
+        off = (w.n_layers - 1) * strides[0]
+        out["latency_graph_replay_equals_fresh_plan"] = bool(torch.equal(probe[:nb], packed[0][off:off + nb]))
+        out["latency_graph_replay_p50_us"] = round(statistics.median(g_wall[1:]), 2)
+        out["latency_graph_replay_gpu_p50_us"] = round(statistics.median(g_gpu[1:]), 2)
+        out["latency_graph_replay_parse_p50_us"] = round(statistics.median(g_parse[1:]), 2)
+        gsess.close()
+        fresh.close()
+        lists.close()
+        slot.close()
+        del graph, probe
     out["latency_p50_us"] = round(statistics.median(gated), 2)
     out["latency_wall_p50_us"] = round(statistics.median(wall), 2)
     out["latency_groups_of_4_layers_p50_us"] = round(statistics.median(grouped), 2)
@@ -375,7 +431,13 @@ def leg_latency(c, out):
                            "the forward pass): GPU time from the end of the last layer's compute "
                            "to the completion of its pack "
                            "(latency_after_last_layer_inline_p50_us: the last layer packed on "
-                           "the compute stream itself, kvt_session_save_layers_inline)"
+                           "the compute stream itself, kvt_session_save_layers_inline); "
+                           "latency_graph_replay_p50_us = the per-layer sequence captured once "
+                           "into a hipGraph over a plan slot, host clock per request from before "
+                           "ParseBlock (latency_graph_replay_parse_p50_us of it) through "
+                           "kvt_plan_slot_fill and the launch of the graph until the wait for the "
+                           "last layer returns (latency_graph_replay_gpu_p50_us: GPU time of the "
+                           "replay between two events)"
                            % (len(reqs), w.n_layers - 1))
 
 
@@ -434,6 +496,105 @@ def leg_session(c, out):
     torch.cuda.synchronize()
     del graph
     sess.close()
+    if args.config == 2 and args.plan == "ranges":
+        session_new_batches(c, out, g_ms)
+
+
+def plan_chunk_bytes(kvt, lists, caps, xform, chunk_bytes):
+    """The table-entry size kvt_plan_create picks for these lists (read off a host-only plan)."""
+    probe = kvt.Plan(-1, lists, caps[0], caps[1], xform=xform, chunk_bytes=chunk_bytes)
+    chunk = probe.host_tables()[2]
+    probe.close()
+    return chunk
+
+
+def session_new_batches(c, out, frozen_ms):
+    """The per-layer sequence captured ONCE over a plan slot and replayed with a NEW batch every
+    time (kvt_plan_slot_fill before each launch of the graph): three batches on the same pools
+    with different lengths and block tables in turn, ParseBlock + merge + refill inside the
+    loop, the host running ahead of the GPU the way the timed steps do."""
+    torch, kvt, lib, args, pipeline = c.torch, c.kvt, c.lib, c.args, c.pipeline
+    w, side = c.wls[0], c.sides[0]
+    caps = (w.capacities("src"), w.capacities("dst"))
+    variants = [w] + [build_workload(2, args.scale, v)[0] for v in (1, 2)]
+    v_tasks = [v.task_bufs() for v in variants]
+    v_lists = [c.senders[0].parse(t) for t in v_tasks]
+    chunk = plan_chunk_bytes(kvt, v_lists[0], caps, None, args.chunk_bytes)
+    probes = [kvt.Plan(-1, l, caps[0], caps[1], chunk_bytes=chunk) for l in v_lists]
+    entries = max(p.num_chunks for p in probes)
+    room = max(p.layer_bytes for p in probes)
+    payloads = [p.tensor_bytes(0) * w.n_layers for p in probes]
+    for p in probes:
+        p.close()
+    slot = kvt.PlanSlot(0, 1, caps[0], caps[1], max_entries=entries, chunk_bytes=chunk,
+                        max_layer_bytes=room)
+    buf = torch.empty(room * w.n_layers, dtype=torch.uint8, device="cuda")
+    sess = kvt.Session(slot, side.src_cache, buf, room)
+    gs = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    slot.fill(v_lists[0], gs.cuda_stream)
+    with torch.cuda.stream(gs):
+        with torch.cuda.graph(graph, stream=gs):
+            for l in range(w.n_layers):
+                sess.save_layer(l, gs.cuda_stream)
+            sess.join(gs.cuda_stream)
+    res = {}
+    with torch.cuda.stream(gs):
+        for rep in range(2):           # the same batch again and again: the kernels' share
+            torch.cuda.synchronize()
+            t_a = time.perf_counter()
+            for _ in range(5):
+                sess.begin_step()
+                graph.replay()
+            torch.cuda.synchronize()
+            res["graph_replay_slot_same_batch_ms"] = round((time.perf_counter() - t_a) / 5 * 1e3, 4)
+        host = []
+        for rep in range(2):
+            torch.cuda.synchronize()
+            t_a = time.perf_counter()
+            n = 6
+            for i in range(n):
+                h0 = time.perf_counter()
+                k = (i + 1) % len(variants)
+                lists = c.senders[0].parse(v_tasks[k])
+                slot.fill(lists, gs.cuda_stream)
+                lists.close()
+                host.append(time.perf_counter() - h0)
+                sess.begin_step()
+                graph.replay()
+            torch.cuda.synchronize()
+            new_ms = (time.perf_counter() - t_a) / n * 1e3
+        last = (n - 1 + 1) % len(variants)
+    # what the last replay packed against a plan made for that batch alone (first and last layer)
+    fresh = kvt.Plan(0, v_lists[last], caps[0], caps[1], chunk_bytes=chunk)
+    ref = torch.empty(room, dtype=torch.uint8, device="cuda")
+    same = True
+    for l in (0, w.n_layers - 1):
+        fresh.pack(side.src_cache, l, 1, ref, room, gs.cuda_stream)
+        gs.synchronize()
+        nb = fresh.tensor_bytes(0)
+        same &= bool(torch.equal(ref[:nb], buf[l * room:l * room + nb]))
+    mean_pay = sum(payloads[(i + 1) % len(variants)] for i in range(n)) / n
+    res.update({
+        "graph_replay_new_batch_ms": round(new_ms, 4),
+        "graph_replay_new_batch_gbps": round(2.0 * mean_pay / (new_ms * 1e-3) / 1e9, 1),
+        "graph_replay_new_batch_host_ms": round(statistics.median(host) * 1e3, 4),
+        "graph_replay_new_batch_vs_frozen_plan": round(
+            (new_ms / mean_pay) / (frozen_ms / payloads[0]), 4),
+        "graph_replay_new_batch_equals_fresh_plan": same,
+        "graph_replay_new_batch_note":
+            "one graph captured over a plan slot (%d entries of %d KiB), %d replays, each after "
+            "ParseBlock + merge + kvt_plan_slot_fill of another batch (payloads %s MiB per "
+            "launch of all layers), host not waiting for the GPU; vs_frozen_plan = time per "
+            "payload byte against graph_replay_ms_all_layers" %
+            (entries, chunk >> 10, n, [round(p / 2**20) for p in payloads])})
+    out["per_layer_session"].update(res)
+    sess.close()
+    fresh.close()
+    slot.close()
+    for l in v_lists:
+        l.close()
+    del buf, ref, graph
 
 
 def leg_cu_usage(c, out):
@@ -901,11 +1062,78 @@ def leg_staging(c, out):
             h2d_t.append(time.perf_counter() - a)
         d2h_s, h2d_s = statistics.median(d2h_t[1:]), statistics.median(h2d_t[1:])
         pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * group * n_groups
+        # Both directions at once: a saving and a loading stager side by side, against two plain
+        # pinned <-> device copies of the same size running concurrently on two streams.
+        both = [C.c_double(), C.c_double()]
+        assert lib.kvt_measure_pcie_both_ways(0, min(nbytes, 1 << 30), 5, C.byref(both[0]),
+                                              C.byref(both[1])) == 0, lib.kvt_last_error()
+        stg_in = kvt.Stager(0, nbytes, 2)
+        bufs_in = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
+        for slot in range(2):           # what the loading side brings in: the groups saved last
+            stg_in.slot_array(slot, nbytes)[:] = stg.slot_array(slot, nbytes)
+        def both_ways(ps_, cs_, groups):
+            """One pass with the given producer / consumer streams -> (save seconds, load seconds)."""
+            torch.cuda.synchronize()
+            a = time.perf_counter()
+            for g in range(groups):
+                slot = g % 2
+                if g >= 2:
+                    stg.wait(slot)
+                plan.pack(side.src_cache, (g % n_groups) * group, group, bufs[slot], lbytes, ps_.cuda_stream)
+                stg.save(slot, bufs[slot], nbytes, ps_.cuda_stream)
+                stg_in.load(slot, bufs_in[slot], nbytes, cs_[slot].cuda_stream)
+                plan.unpack(side.dst_cache, (g % n_groups) * group, group, bufs_in[slot], lbytes,
+                            cs_[slot].cuda_stream)
+            stg.wait(0)
+            if groups > 1:
+                stg.wait(1)
+            t_save = time.perf_counter() - a
+            cs_[0].synchronize()
+            cs_[1].synchronize()
+            return t_save, time.perf_counter() - a
+
+        # Which streams the caller uses matters: HIP maps streams onto a few hardware queues, and a
+        # consumer stream that waits for a transfer parks that wait in its queue for as long as
+        # the transfer takes; a copy stream mapped to the same queue gets nothing through
+        # meanwhile, and the two directions take turns instead of overlapping. Which streams share
+        # a queue cannot be asked, only measured: four sets of streams are tried with a short
+        # pass each and the best one is used (what a deployment does once at start-up).
+        probe_groups = min(n_groups, 4)
+        sets, quick = [], []
+        for k in range(4):
+            st = (torch.cuda.Stream(), [torch.cuda.Stream(), torch.cuda.Stream()])
+            both_ways(st[0], st[1], min(2, probe_groups))
+            t_s, t_l = both_ways(st[0], st[1], probe_groups)
+            sets.append(st)
+            quick.append(round(2 * pay / n_groups * probe_groups / (t_s + t_l) / 1e9, 2))
+        ps_b, cs_b = sets[max(range(4), key=lambda k: quick[k])]
+        bi_save, bi_load = [], []
+        for phase in range(4):
+            t_s, t_l = both_ways(ps_b, cs_b, n_groups)
+            bi_save.append(t_s)
+            bi_load.append(t_l)
+        bs, bl = statistics.median(bi_save[1:]), statistics.median(bi_load[1:])
+        stg_in.close()
+        del bufs_in
         out["staging"] = {
             "save_gbps": round(pay / d2h_s / 1e9, 2), "load_gbps": round(pay / h2d_s / 1e9, 2),
             "pcie_d2h_gbps": round(ceil["d2h"] / 1e9, 2), "pcie_h2d_gbps": round(ceil["h2d"] / 1e9, 2),
             "save_frac_of_pcie": round(pay / d2h_s / ceil["d2h"], 4),
             "load_frac_of_pcie": round(pay / h2d_s / ceil["h2d"], 4),
+            "bidir_save_gbps": round(pay / bs / 1e9, 2), "bidir_load_gbps": round(pay / bl / 1e9, 2),
+            "bidir_pcie_d2h_gbps": round(both[0].value / 1e9, 2),
+            "bidir_pcie_h2d_gbps": round(both[1].value / 1e9, 2),
+            "bidir_save_frac_of_pcie": round(pay / bs / both[0].value, 4),
+            "bidir_load_frac_of_pcie": round(pay / bl / both[1].value, 4),
+            "bidir_stream_sets_gbps": quick,
+            "bidir_note": "a saving and a loading stager at the same time (pack -> D2H beside H2D "
+                          "-> unpack), each direction's payload over the time until that direction "
+                          "has finished; ceiling: two plain copies of one transfer's size running "
+                          "concurrently on two streams (kvt_measure_pcie_both_ways); "
+                          "bidir_stream_sets_gbps: mean rate per direction of a short pass with "
+                          "each of four sets of producer / consumer streams (streams that share a "
+                          "hardware queue with a copy stream make the directions take turns), the "
+                          "best set is the one measured",
             "sample": "%d transfers of %d layer(s) = %.1f MiB each through 2 pinned slots, "
                       "pack / unpack of the group in one launch; median of 3 passes" %
                       (n_groups, group, nbytes / 2**20),
@@ -1199,7 +1427,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=0,
                     help="0 (default): the headline configuration 2 as the JSON line, followed by "
-                         "the other four baseline configurations as rows of its \"configs\" list; "
+                         "the other four baseline configurations and config 9 (config 5 in the "
+                         "reference's uniform-page arrangement) as rows of its \"configs\" list; "
                          "1-5: that baseline configuration alone (1 = the CPU-runnable case, 2 = "
                          "the headline); 6-8, 11: TP-remapping batches; 9: config 5 with the "
                          "reference's uniform 2 MiB pages; 10: the same model TP2 -> TP1")
@@ -1266,7 +1495,7 @@ def main():
         # the timed steps, parity against the oracle on a sample of layers, the request
         # latencies and the staging path
         rows = []
-        for cfg in (1, 3, 4, 5):
+        for cfg in (1, 3, 4, 5, 9):
             sub = argparse.Namespace(**vars(args))
             sub.config, sub.plan, sub.chunk_bytes = cfg, "ranges", 0
             sub.cpu_layers = min(args.cpu_layers, 4)
@@ -1282,7 +1511,9 @@ def main():
             for key in ("value", "ms_per_step", "pack_gbps", "unpack_gbps", "pack_ms", "unpack_ms",
                         "frac_hbm_peak", "host_parse_plan_ms", "mode", "parity_vs_oracle",
                         "latency_p50_us", "latency_wall_p50_us", "latency_single_launch_p50_us",
-                        "latency_groups_of_4_layers_p50_us",
+                        "latency_groups_of_4_layers_p50_us", "latency_graph_replay_p50_us",
+                        "latency_graph_replay_gpu_p50_us", "latency_graph_replay_parse_p50_us",
+                        "latency_graph_replay_equals_fresh_plan",
                         "latency_after_last_layer_p50_us", "latency_after_last_layer_inline_p50_us",
                         "cu_usage",
                         "staging", "roofline", "cpu_baseline", "errors"):

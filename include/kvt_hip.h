@@ -601,9 +601,14 @@ int kvt_copy_handle_data_kernel_direct(void* tensor_buf, void* layer_gpu_ptr,
  * runtime or the device: the metadata is brought over by a copy kernel reading host_meta.
  * At most 8192 ranges per call: more are refused with KVT_ERR_INVALID. All calls on one GPU
  * share that GPU's array, which keeps the last call's metadata until the next one overwrites
- * it: calls whose execution may overlap on one GPU (different streams, or the same graph
- * launched twice at once) race; calls on one stream do not. host_meta must stay untouched
- * until the stream has run the copy. Errors as kvt_copy_handle_data_kernel_direct. */
+ * it. Eager calls are kept apart by the library: each makes its stream wait for the previous
+ * call on that GPU (whatever stream that was on, through one event per GPU created at
+ * kvt_initialize_copy_method_profile or the first call), so copy threads with a stream each
+ * (kvtransfer/src/copy_utils.cpp:59-95) may call it at will and their copies run one after the
+ * other. Calls recorded into a stream capture are ordered by their graph alone: two graphs
+ * that hold such calls, or one graph launched twice at once, must not run at the same time,
+ * nor beside an eager call. host_meta must stay untouched until the stream has run the copy.
+ * Errors as kvt_copy_handle_data_kernel_direct. */
 int kvt_copy_handle_data_kernel_direct_static(void* tensor_buf, void* layer_gpu_ptr,
                                               const kvt_ipc_block* blocks, uint64_t n,
                                               uint64_t tensor_data_size, int direction, int device,
@@ -750,6 +755,12 @@ int kvt_stager_wait(kvt_stager* s, uint32_t slot);
  * the ceiling the staging path is reported against. */
 int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats,
                      double* bytes_per_s);
+
+/* The same with both directions running at the same time on two streams (a saving and a
+ * loading stager side by side): the rate each direction reaches while the other one is busy,
+ * the ceiling for concurrent save and load. Allocates 2 x bytes of pinned and of device memory. */
+int kvt_measure_pcie_both_ways(int device, uint64_t bytes, uint32_t repeats, double* d2h_bytes_per_s,
+                               double* h2d_bytes_per_s);
 
 /* ---------------------------------------- store objects found by block hash */
 

@@ -571,23 +571,36 @@ static __device__ __align__(256) int64_t scratch[3 * kStaticMaxRanges];
 
 namespace {
 constexpr int kMaxStaticDevices = 64;
+// Per device: the array's address, and what keeps calls that share it apart. Every eager call
+// makes its stream wait for the event the previous call on that GPU recorded behind its
+// kernel, before its own metadata is written, and records the event again behind its own
+// kernel: calls on different streams then run one after the other instead of overwriting each
+// other's metadata. The event is made once, with the address lookup; a call allocates nothing.
+struct StaticScratch {
+  std::mutex mu;            // one call at a time issues (wait, metadata copy, kernel, record)
+  int64_t* ptr = nullptr;
+  hipEvent_t last = nullptr;
+  bool recorded = false;
+};
 std::mutex g_scratch_mu;
-int64_t* g_scratch_ptr[kMaxStaticDevices] = {};
+StaticScratch g_scratch[kMaxStaticDevices];
 
-// The address of `device`'s copy of the array (looked up with that device current).
-int static_scratch(int device, int64_t** out) {
+// `device`'s copy of the array (address looked up with that device current).
+int static_scratch(int device, StaticScratch** out) {
   if (device < 0 || device >= kMaxStaticDevices)
     return fail(KVT_ERR_INVALID, "device index too large for the static metadata array");
   std::lock_guard<std::mutex> lock(g_scratch_mu);
-  if (!g_scratch_ptr[device]) {
+  StaticScratch& sc = g_scratch[device];
+  if (!sc.ptr) {
     DeviceGuard g;
     if (int rc = g.enter(device)) return rc;
     void* p = nullptr;
     KVT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (!p) return fail(KVT_ERR_HIP, "hipGetSymbolAddress gave no address for the static metadata array");
-    g_scratch_ptr[device] = static_cast<int64_t*>(p);
+    if (!sc.last) KVT_HIP(hipEventCreateWithFlags(&sc.last, hipEventDisableTiming));
+    sc.ptr = static_cast<int64_t*>(p);
   }
-  *out = g_scratch_ptr[device];
+  *out = &sc;
   return KVT_OK;
 }
 }  // namespace
@@ -701,7 +714,7 @@ extern "C" {
 int kvt_initialize_copy_method_profile(int device) {
   return guarded([&]() -> int {
     if (int rc = check_device(device)) return rc;
-    int64_t* unused = nullptr;
+    StaticScratch* unused = nullptr;
     if (int rc = static_scratch(device, &unused)) return rc;
     std::lock_guard<std::mutex> lock(g_profile_mu);
     if (g_profile.measured) return KVT_OK;  // once per process, like the reference's call_once
@@ -753,11 +766,28 @@ int kvt_copy_handle_data_kernel_direct_static(void* tensor_buf, void* layer_gpu_
                       std::to_string(n) + " given)");
     if (n == 0) return KVT_OK;
     if (int rc = check_device(device)) return rc;
-    int64_t* meta = nullptr;
-    if (int rc = static_scratch(device, &meta)) return rc;
-    return handle_data_direct(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction,
-                              device, stream, meta, meta + n, meta + 2 * n, host_meta,
-                              use_explicit_host_offsets != 0, true);
+    StaticScratch* sc = nullptr;
+    if (int rc = static_scratch(device, &sc)) return rc;
+    int64_t* meta = sc->ptr;
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    const hipStream_t s = static_cast<hipStream_t>(stream);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess) (void)hipGetLastError();
+    // Inside a stream capture nothing runs now and an outside event can neither be waited for
+    // nor recorded: a recorded call is ordered by its graph alone.
+    const bool capturing = cap != hipStreamCaptureStatusNone;
+    std::lock_guard<std::mutex> lock(sc->mu);
+    if (!capturing && sc->recorded) KVT_HIP(hipStreamWaitEvent(s, sc->last, 0));
+    const int rc = handle_data_direct(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction,
+                                      device, stream, meta, meta + n, meta + 2 * n, host_meta,
+                                      use_explicit_host_offsets != 0, true);
+    // also behind a call that failed half way: its metadata copy may be on the stream
+    if (!capturing) {
+      KVT_HIP(hipEventRecord(sc->last, s));
+      sc->recorded = true;
+    }
+    return rc;
   });
 }
 

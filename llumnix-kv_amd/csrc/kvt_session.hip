@@ -554,4 +554,72 @@ int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats
   });
 }
 
+int kvt_measure_pcie_both_ways(int device, uint64_t bytes, uint32_t repeats, double* d2h_bytes_per_s,
+                               double* h2d_bytes_per_s) {
+  return guarded([&]() -> int {
+    if (!d2h_bytes_per_s || !h2d_bytes_per_s || bytes == 0 || repeats == 0)
+      return fail(KVT_ERR_INVALID, "kvt_measure_pcie_both_ways: bad argument");
+    if (int rc = check_device(device)) return rc;
+    DeviceGuard g;
+    if (int rc = g.enter(device)) return rc;
+    // [0] device -> host, [1] host -> device: a buffer pair, a stream and two events each
+    void *host[2] = {nullptr, nullptr}, *dev[2] = {nullptr, nullptr};
+    hipStream_t st[2] = {nullptr, nullptr};
+    hipEvent_t a[2] = {nullptr, nullptr}, b[2] = {nullptr, nullptr}, go = nullptr;
+    int rc = KVT_OK;
+    auto cleanup = [&]() {
+      for (int d = 0; d < 2; ++d) {
+        if (st[d]) (void)hipStreamSynchronize(st[d]);
+        if (a[d]) (void)hipEventDestroy(a[d]);
+        if (b[d]) (void)hipEventDestroy(b[d]);
+        if (st[d]) (void)hipStreamDestroy(st[d]);
+        if (dev[d]) (void)hipFree(dev[d]);
+        if (host[d]) (void)hipHostFree(host[d]);
+      }
+      if (go) (void)hipEventDestroy(go);
+    };
+#define KVT_TRY(call)                         \
+  do {                                        \
+    const hipError_t _e = (call);             \
+    if (_e != hipSuccess) {                   \
+      rc = hip_fail(_e, #call);               \
+      cleanup();                              \
+      return rc;                              \
+    }                                         \
+  } while (0)
+    for (int d = 0; d < 2; ++d) {
+      KVT_TRY(hipHostMalloc(&host[d], bytes, hipHostMallocDefault));
+      KVT_TRY(hipMalloc(&dev[d], bytes));
+      std::memset(host[d], 0x5a, bytes);
+      KVT_TRY(hipStreamCreateWithFlags(&st[d], hipStreamNonBlocking));
+      KVT_TRY(hipEventCreate(&a[d]));
+      KVT_TRY(hipEventCreate(&b[d]));
+    }
+    KVT_TRY(hipEventCreateWithFlags(&go, hipEventDisableTiming));
+    auto copy = [&](int d) {
+      return d == 0 ? hipMemcpyAsync(host[0], dev[0], bytes, hipMemcpyDeviceToHost, st[0])
+                    : hipMemcpyAsync(dev[1], host[1], bytes, hipMemcpyHostToDevice, st[1]);
+    };
+    for (int d = 0; d < 2; ++d) KVT_TRY(copy(d));   // warm-up, both at once as well
+    // both streams start their timed copies together: the second waits for the first's warm-up
+    KVT_TRY(hipEventRecord(go, st[0]));
+    KVT_TRY(hipStreamWaitEvent(st[1], go, 0));
+    for (int d = 0; d < 2; ++d) KVT_TRY(hipEventRecord(a[d], st[d]));
+    for (uint32_t i = 0; i < repeats; ++i)          // issued alternately, so that neither runs ahead
+      for (int d = 0; d < 2; ++d) KVT_TRY(copy(d));
+    for (int d = 0; d < 2; ++d) KVT_TRY(hipEventRecord(b[d], st[d]));
+    float ms[2] = {0, 0};
+    for (int d = 0; d < 2; ++d) {
+      KVT_TRY(hipEventSynchronize(b[d]));
+      KVT_TRY(hipEventElapsedTime(&ms[d], a[d], b[d]));
+    }
+#undef KVT_TRY
+    *d2h_bytes_per_s = static_cast<double>(bytes) * repeats / (ms[0] * 1e-3);
+    *h2d_bytes_per_s = static_cast<double>(bytes) * repeats / (ms[1] * 1e-3);
+    cleanup();
+    forget_device_spans();
+    return KVT_OK;
+  });
+}
+
 }  // extern "C"

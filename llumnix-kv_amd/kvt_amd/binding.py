@@ -153,6 +153,7 @@ SIGNATURES = {
     "kvt_stager_load": (_int, [_vp, _u32, _vp, _u64, _vp]),
     "kvt_stager_wait": (_int, [_vp, _u32]),
     "kvt_measure_pcie": (_int, [_int, _int, _u64, _u32, _P(C.c_double)]),
+    "kvt_measure_pcie_both_ways": (_int, [_int, _u64, _u32, _P(C.c_double), _P(C.c_double)]),
     "kvt_copy_linear": (_int, [_vp, _vp, _u64, _vp]),
     "kvt_copy_runtime_d2d": (_int, [_vp, _vp, _u64, _vp]),
     "kvt_event_create": (_int, [_P(_vp)]),

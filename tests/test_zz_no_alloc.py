@@ -90,6 +90,50 @@ def test_static_metadata_entry_point_equals_the_existing_one(explicit):
         assert (got_dst[~touched] == 0x33).all()
 
 
+def test_calls_on_two_streams_do_not_overwrite_each_others_metadata():
+    """The reference's callers are several copy threads with a stream each
+    (kvtransfer/src/copy_utils.cpp:59-154). Two streams issue different lists back to back
+    while the first stream is held back by a sleeping kernel, so that without ordering the
+    second call's metadata would replace the first one's before its kernel has run. Every call
+    must still move its own ranges: results equal the existing entry point's."""
+    lib = kvt_amd.lib()
+    s1, s2 = checkers.side_stream(), checkers.side_stream()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(92)
+    layer = torch.randint(0, 256, (CAP,), generator=g, device="cuda", dtype=torch.uint8)
+    cases = [_ranges(5, 700, False), _ranges(6, 400, True), _ranges(7, 90, False)]
+    ref = [_both_entry_points(lib, s1, b, size, layer, ex)[0] for (b, size), ex in
+           zip(cases, (False, True, False))]
+    metas = [torch.zeros(3 * len(b), dtype=torch.int64).pin_memory() for b, _ in cases]
+    bufs = [torch.full((size,), 0x11, dtype=torch.uint8).pin_memory() for _, size in cases]
+    dsts = [torch.full((CAP,), 0x33, dtype=torch.uint8, device="cuda") for _ in cases]
+
+    def call(i, stream, direction, gpu):
+        b, size = cases[i]
+        rc = lib.kvt_copy_handle_data_kernel_direct_static(
+            bufs[i].data_ptr(), gpu.data_ptr(), b.ctypes.data, len(b), size, direction, 0,
+            stream.cuda_stream, metas[i].data_ptr(), 1 if i == 1 else 0)
+        assert rc == 0, lib.kvt_last_error()
+
+    with torch.cuda.stream(s1):
+        torch.cuda._sleep(100_000_000)              # stream 1 falls behind
+    call(0, s1, 1, layer)                           # gathers, alternating streams, no waits
+    call(1, s2, 1, layer)
+    call(2, s1, 1, layer)
+    s1.synchronize()
+    s2.synchronize()
+    with torch.cuda.stream(s2):
+        torch.cuda._sleep(100_000_000)
+    call(0, s2, 0, dsts[0])                         # scatters of what was gathered
+    call(1, s1, 0, dsts[1])
+    call(2, s2, 0, dsts[2])
+    s1.synchronize()
+    s2.synchronize()
+    for i in range(3):
+        assert np.array_equal(bufs[i].numpy(), ref[i][0]), (i, "gather differs")
+        assert np.array_equal(dsts[i].cpu().numpy(), ref[i][1]), (i, "scatter differs")
+
+
 def test_static_metadata_entry_point_refuses_what_it_cannot_hold():
     lib = kvt_amd.lib()
     st = checkers.side_stream()
