@@ -395,7 +395,31 @@ def leg_latency(c, out):
                 g_gpu.append(ev_ms(lib, a, b) * 1e3)
                 lists.close()
         torch.cuda.synchronize()
+        # what the replay costs when there is nothing to move: the same graph over an empty batch
+        # (2 kernel nodes per layer -- the pack, which ends at once, and the signal -- chained
+        # through the side stream): the price of per-layer launches and signals in a graph
+        empty = kvt.BlockLists()
+        g_floor = []
+        with torch.cuda.stream(gs):
+            slot.fill(empty, gs.cuda_stream)
+            for rep in range(6):
+                step = gsess.begin_step()
+                lib.kvt_event_record(a, gs.cuda_stream)
+                graph.replay()
+                lib.kvt_event_record(b, gs.cuda_stream)
+                gsess.wait_layer(w.n_layers - 1, step)
+                lib.kvt_event_synchronize(b)
+                g_floor.append(ev_ms(lib, a, b) * 1e3)
+        empty.close()
+        out["latency_graph_replay_empty_batch_gpu_p50_us"] = round(statistics.median(g_floor[1:]), 2)
         # the last request once more through a plan of its own: same bytes
+        with torch.cuda.stream(gs):
+            lists = sender.parse([tasks[0][reqs[-1]]])
+            slot.fill(lists, gs.cuda_stream)
+            gsess.begin_step()
+            graph.replay()
+        lists.close()
+        torch.cuda.synchronize()
         lists = sender.parse([tasks[0][reqs[-1]]])
         fresh = kvt.Plan(0, lists, caps[0], caps[1], xform=w.xform, chunk_bytes=chunk)
         probe = torch.empty(max(1, strides[0]), dtype=torch.uint8, device="cuda")
@@ -437,7 +461,9 @@ def leg_latency(c, out):
                            "ParseBlock (latency_graph_replay_parse_p50_us of it) through "
                            "kvt_plan_slot_fill and the launch of the graph until the wait for the "
                            "last layer returns (latency_graph_replay_gpu_p50_us: GPU time of the "
-                           "replay between two events)"
+                           "replay between two events; latency_graph_replay_empty_batch_gpu_p50_us: "
+                           "the same replay over an empty batch, i.e. what the launches and "
+                           "signals of the layers cost by themselves)"
                            % (len(reqs), w.n_layers - 1))
 
 
@@ -1514,6 +1540,7 @@ def main():
                         "latency_groups_of_4_layers_p50_us", "latency_graph_replay_p50_us",
                         "latency_graph_replay_gpu_p50_us", "latency_graph_replay_parse_p50_us",
                         "latency_graph_replay_equals_fresh_plan",
+                        "latency_graph_replay_empty_batch_gpu_p50_us",
                         "latency_after_last_layer_p50_us", "latency_after_last_layer_inline_p50_us",
                         "cu_usage",
                         "staging", "roofline", "cpu_baseline", "errors"):

@@ -485,6 +485,15 @@ int kvt_get_copy_ticket_stats(int device, uint64_t out[4]);
  * captured with). Results are identical either way. */
 int kvt_set_copy_cached_load_max(uint64_t payload_bytes);
 uint64_t kvt_get_copy_cached_load_max(void);
+/* The same for the stores (no counterpart in the reference either): a pack / unpack launch
+ * between device buffers whose payload is at most payload_bytes writes with plain stores, which
+ * leave their lines in the memory-side cache, instead of non-temporal write-through ones. For a
+ * caller whose next launch reads what this one wrote while it still fits there (a request packed
+ * and unpacked on the same GPU, a blob packed and at once stored and sent). Default: 0, never.
+ * Process-wide, for launches issued after the call; launches limited to a CU share and launches
+ * whose packed side is pinned host memory keep the streaming stores. Results are identical. */
+int kvt_set_copy_cached_store_max(uint64_t payload_bytes);
+uint64_t kvt_get_copy_cached_store_max(void);
 
 /* replaces launch_copy_int64_array_h2d_kernel()  kvtransfer/src/copy_kernels.cu:93-103
  * (declared for the channels, kvtransfer/src/copy_kernels.cpp:101-108): a kernel reads

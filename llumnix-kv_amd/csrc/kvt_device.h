@@ -47,6 +47,7 @@ struct __attribute__((aligned(16))) StrideShape {
 };
 static_assert(sizeof(StrideShape) == 64, "StrideShape is read as one 64-byte scalar load");
 constexpr uint32_t kMaxShapes = 16;
+enum : uint32_t { kPolicyTemporalLoads = 1u, kPolicyCachedStores = 2u };
 // Default payload (bytes moved one way) up to which a launch reads with plain loads: none.
 // Plain loads pay only when the same data is read again soon (kvt_set_copy_cached_load_max).
 constexpr uint64_t kTemporalMaxBytes = 0;
@@ -82,8 +83,9 @@ hipError_t launch_slot(int kind, bool pack, const Chunk* chunks, const SlotHeade
 // Chunk launchers. max_wgs = 0: one workgroup per (4 KiB slice, layer), the fastest shape.
 // max_wgs > 0: at most that many workgroups (a multiple of 8), striding over the same items,
 // for a caller that wants the copy to leave part of the device to other kernels.
-// temporal: plain instead of non-temporal loads, for a launch whose data may sit in the
-// memory-side cache (ignored by a capped launch). tickets: a capped launch's block of counters
+// policy: kPolicyTemporalLoads = plain instead of non-temporal loads, for a launch whose data may
+// sit in the memory-side cache; kPolicyCachedStores = plain stores, for a launch whose output is
+// read again while it still fits there (both ignored by a capped launch). tickets: a capped launch's block of counters
 // (see launch_copy_entries), or nullptr; an uncapped launch ignores it and leaves it untouched. pipelined (launch_copy_chunks): a capped
 // launch keeps the loads of its next trip in flight across the stores of the last one; for
 // grids of at most 4 workgroups per CU (the kernel then needs more registers than 8 per CU fit).
@@ -91,7 +93,7 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, bool words, uint32_t max_wgs, bool temporal,
+                                 const StrideTable& shapes, bool words, uint32_t max_wgs, uint32_t policy,
                                  uint32_t* tickets, hipStream_t stream);
 // Converting gather (bf16 -> fp8 E4M3) of a chunk table, plain and strided chunks alike; lengths
 // and packed positions count fp8 bytes, cache offsets and strides bytes of the bf16 cache.
@@ -113,12 +115,12 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
                                     const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
-                                    bool temporal, uint32_t* tickets, hipStream_t stream);
+                                    uint32_t policy, uint32_t* tickets, hipStream_t stream);
 hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                               uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
-                              bool temporal, uint32_t* tickets, hipStream_t stream);
+                              uint32_t policy, uint32_t* tickets, hipStream_t stream);
 // The capped launch of a plain table with 16-byte aligned entries (sub_shift 0 ... 3: at most
 // 4 ... 32 KiB): `wgs` persistent workgroups (a multiple of 8), software-pipelined, one table
 // entry per trip and workgroup (16 or 32 KiB) or per wavefront (4 or 8 KiB). Every address and
@@ -167,7 +169,7 @@ hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               uint32_t max_wgs, bool temporal, uint32_t* tickets, hipStream_t stream);
+                               uint32_t max_wgs, uint32_t policy, uint32_t* tickets, hipStream_t stream);
 // rows = workgroups striding over the 4 KiB slices of each range
 hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                               const int64_t* dst_off, const int64_t* lens, int64_t n, int num_wg,

@@ -252,7 +252,9 @@ constexpr int kBatch = 4;
 // flight pay below half the device (config 4 at a quarter: 4.8 / 4.5 -> 5.2 / 5.2 TB/s) and
 // cost from there on (at one half 5.6 / 5.5 -> 5.1 / 5.2), so the launcher picks by grid size.
 enum { kOnePerSlice = 0, kStriding = 1, kPipelined = 2 };
-constexpr uint32_t kTemporalFlag = 0x100u;  // in a kernel's sub_shift argument: Launch::temporal
+// in a kernel's sub_shift argument: Launch::temporal, Launch::cached_store (the launchers'
+// `policy` argument, bits 0 and 1, shifted by 8)
+constexpr uint32_t kTemporalFlag = 0x100u, kCachedStoreFlag = 0x200u;
 
 // The uniform arguments of a chunk launch.
 struct Launch {
@@ -263,6 +265,7 @@ struct Launch {
   uint64_t layer_stride;
   const BlobOffsets* blobs;
   bool temporal;  // plain instead of non-temporal loads (bit 8 of the sub_shift argument)
+  bool cached_store;  // plain stores, which leave their lines in the caches (bit 9)
   uint32_t* tickets;  // a capped launch: its block of counters, or nullptr (EntryWalk)
 };
 
@@ -361,7 +364,10 @@ __device__ __forceinline__ void for_items(const Launch& L, Fetch fetch_table, Pl
                      : "v"(src)
                      : "memory");
       }
-      store_vec(m.dst + m.dst_off, v);
+      if (L.cached_store)
+        *(g_u32x4*)(m.dst + m.dst_off) = v;
+      else
+        store_vec(m.dst + m.dst_off, v);
     }
     return;
   }
@@ -448,7 +454,7 @@ __device__ __forceinline__ Move plain_move(const Item& it) {
 
 #define KVT_LAUNCH_STRUCT \
   const Launch L{n_slices, sub_shift & 0xFFu, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, &blobs, \
-                 (sub_shift & kTemporalFlag) != 0, tickets}
+                 (sub_shift & kTemporalFlag) != 0, (sub_shift & kCachedStoreFlag) != 0, tickets}
 
 // Gather (PACK) / scatter of a resident chunk table.
 template <bool PACK, int MODE>
@@ -472,7 +478,7 @@ __global__ __launch_bounds__(kThreads, MODE == kPipelined ? 4 : 8) void copy_chu
     uint32_t* tickets) {
   KVT_LAUNCH_STRUCT;
   for_items<MODE>(L, [&](uint32_t e) { return fetch_entry(table.c, e); },
-                    [&](const Item& it) { return plain_move<PACK>(it); });
+                  [&](const Item& it) { return plain_move<PACK>(it); });
 }
 
 // The capped launch of a plain table whose entries are whole multiples of 16 bytes, 16-byte
@@ -1461,27 +1467,38 @@ __global__ __launch_bounds__(kThreads, 4) void convert_entries_by_wave_kernel(
       uint8_t *const *__restrict__ layer_ptrs, uint32_t n_tensors, uint32_t first_layer,             \
       uint32_t n_layers, uint8_t *packed, uint64_t layer_stride, uint32_t *tickets
 #define KVT_SLOT_TAIL layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, hdr->blobs
+// A batch so small that no workgroup gets a second trip is dealt out by position: asking for a
+// ticket first would put one more round trip to memory in front of the only load (a request of
+// 64 entries per layer: 7.2 -> 5.8 us per layer in a replayed graph, of which 3.5 are the launch
+// and the signal).
+__device__ __forceinline__ uint32_t* slot_tickets(uint32_t n_chunks, uint32_t n_layers, uint32_t per_trip,
+                                                  uint32_t* tickets) {
+  return static_cast<uint64_t>(n_chunks) * n_layers <= static_cast<uint64_t>(gridDim.x) * per_trip ? nullptr : tickets;
+}
 
 template <bool PACK, int V>
 __global__ __launch_bounds__(kThreads, 4) void copy_entries_slot_kernel(KVT_SLOT_PARAMS) {
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
   const Entry* table = reinterpret_cast<const Entry*>(chunks);
-  copy_entries<PACK, V>([&](uint32_t e) { return table[e]; }, n_chunks, KVT_SLOT_TAIL, tickets);
+  copy_entries<PACK, V>([&](uint32_t e) { return table[e]; }, n_chunks, KVT_SLOT_TAIL,
+                        slot_tickets(n_chunks, n_layers, 1, tickets));
 }
 template <bool PACK, int V, int U>
 __global__ __launch_bounds__(kThreads, 4) void copy_entries_by_wave_slot_kernel(KVT_SLOT_PARAMS) {
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
   const Entry* table = reinterpret_cast<const Entry*>(chunks);
-  copy_entries_by_wave<PACK, V, U>([&](uint32_t e) { return table[e]; }, n_chunks, KVT_SLOT_TAIL, tickets);
+  copy_entries_by_wave<PACK, V, U>([&](uint32_t e) { return table[e]; }, n_chunks, KVT_SLOT_TAIL,
+                                   slot_tickets(n_chunks, n_layers, 4 * U, tickets));
 }
 template <bool PACK, int V>
 __global__ __launch_bounds__(kThreads, 4) void strided_entries_slot_kernel(KVT_SLOT_PARAMS, uint32_t part_shift) {
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
   const uint32_t lane = threadIdx.x << 4;
-  entries_pipeline<PACK, V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL, tickets,
+  entries_pipeline<PACK, V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL,
+                            slot_tickets(n_chunks << part_shift, n_layers, 1, tickets),
                             [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
                               strided_offsets<PACK, V, kSliceShift>(hdr->shapes, c, begin, bytes, lane, coff);
                             });
@@ -1491,7 +1508,7 @@ __global__ __launch_bounds__(kThreads, 4) void strided_entries_by_wave_slot_kern
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
   const uint32_t lane = (threadIdx.x & 63u) << 4;
-  entries_pipeline_by_wave<PACK, V, U>(chunks, n_chunks, KVT_SLOT_TAIL, tickets,
+  entries_pipeline_by_wave<PACK, V, U>(chunks, n_chunks, KVT_SLOT_TAIL, slot_tickets(n_chunks, n_layers, 4 * U, tickets),
                                        [&](const Entry& c, uint32_t bytes, uint32_t* coff) {
                                          strided_offsets<PACK, V, 10>(hdr->shapes, c, 0u, bytes, lane, coff);
                                        });
@@ -1502,7 +1519,8 @@ __global__ __launch_bounds__(kThreads, 4) void xform_entries_slot_kernel(KVT_SLO
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
   const uint32_t lane = threadIdx.x << 4;
-  entries_pipeline<PACK, V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL, tickets,
+  entries_pipeline<PACK, V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL,
+                            slot_tickets(n_chunks << part_shift, n_layers, 1, tickets),
                             [&](const Entry& c, uint32_t begin, uint32_t bytes, uint32_t* coff) {
                               xform_offsets<V, kSliceShift>(x, c, begin, bytes, lane, coff);
                             });
@@ -1512,7 +1530,7 @@ __global__ __launch_bounds__(kThreads, 4) void xform_entries_by_wave_slot_kernel
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
   const uint32_t lane = (threadIdx.x & 63u) << 4;
-  entries_pipeline_by_wave<PACK, V, U>(chunks, n_chunks, KVT_SLOT_TAIL, tickets,
+  entries_pipeline_by_wave<PACK, V, U>(chunks, n_chunks, KVT_SLOT_TAIL, slot_tickets(n_chunks, n_layers, 4 * U, tickets),
                                        [&](const Entry& c, uint32_t bytes, uint32_t* coff) {
                                          xform_offsets<V, 10>(x, c, 0u, bytes, lane, coff);
                                        });
@@ -1521,12 +1539,13 @@ template <int V>
 __global__ __launch_bounds__(kThreads, 4) void convert_entries_slot_kernel(KVT_SLOT_PARAMS, uint32_t part_shift) {
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
-  convert_entries<V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL, hdr->shapes, tickets);
+  convert_entries<V>(chunks, n_chunks, part_shift, KVT_SLOT_TAIL, hdr->shapes,
+                     slot_tickets(n_chunks << part_shift, n_layers, 1, tickets));
 }
 __global__ __launch_bounds__(kThreads, 4) void convert_entries_by_wave_slot_kernel(KVT_SLOT_PARAMS) {
   const uint32_t n_chunks = hdr->n_entries;
   if (n_chunks == 0) return;
-  convert_entries_by_wave<1>(chunks, n_chunks, KVT_SLOT_TAIL, hdr->shapes, tickets);
+  convert_entries_by_wave<1>(chunks, n_chunks, KVT_SLOT_TAIL, hdr->shapes, slot_tickets(n_chunks, n_layers, 4, tickets));
 }
 
 // Plain linear copy with the gather kernel's slice shape (calibration / ceiling).
@@ -1566,12 +1585,12 @@ hipError_t launch_copy_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks,
                               uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                               uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                               uint64_t layer_stride, const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
-                              bool temporal, uint32_t* tickets, hipStream_t stream) {
+                              uint32_t policy, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
   if (!g.capped) tickets = nullptr;
-  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+  const uint32_t shift_arg = sub_shift | (g.capped ? 0u : (policy & 3u) << 8);
 #define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
   if (!g.capped) {
     if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_kernel<true, kOnePerSlice>), KVT_ARGS);
@@ -1743,12 +1762,12 @@ hipError_t launch_copy_chunks_small(bool pack, const SmallTable& table, uint32_t
                                     uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                     uint8_t* packed, uint64_t layer_stride,
                                     const BlobOffsets& blobs, uint32_t max_wgs, bool pipelined,
-                                    bool temporal, uint32_t* tickets, hipStream_t stream) {
+                                    uint32_t policy, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
   if (!g.capped) tickets = nullptr;
-  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+  const uint32_t shift_arg = sub_shift | (g.capped ? 0u : (policy & 3u) << 8);
 #define KVT_ARGS table, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, tickets
   if (!g.capped) {
     if (pack) KVT_LAUNCH_CHUNKS((copy_chunks_small_kernel<true, kOnePerSlice>), KVT_ARGS);
@@ -1768,13 +1787,13 @@ hipError_t launch_strided_chunks(bool pack, const Chunk* chunks, uint32_t n_chun
                                  uint32_t sub_shift, uint8_t* const* layer_ptrs,
                                  uint32_t n_tensors, uint32_t first_layer, uint32_t n_layers,
                                  uint8_t* packed, uint64_t layer_stride, const BlobOffsets& blobs,
-                                 const StrideTable& shapes, bool words, uint32_t max_wgs, bool temporal,
+                                 const StrideTable& shapes, bool words, uint32_t max_wgs, uint32_t policy,
                                  uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
   if (!g.capped) tickets = nullptr;
-  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+  const uint32_t shift_arg = sub_shift | (g.capped ? 0u : (policy & 3u) << 8);
 #define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, shapes, tickets
 #define KVT_STRIDED(P, W)                                                                       \
   do {                                                                                          \
@@ -1811,12 +1830,12 @@ hipError_t launch_xform_chunks(bool pack, const Chunk* chunks, uint32_t n_chunks
                                uint32_t sub_shift, uint8_t* const* layer_ptrs, uint32_t n_tensors,
                                uint32_t first_layer, uint32_t n_layers, uint8_t* packed,
                                uint64_t layer_stride, const BlobOffsets& blobs, const XformDev& x,
-                               uint32_t max_wgs, bool temporal, uint32_t* tickets, hipStream_t stream) {
+                               uint32_t max_wgs, uint32_t policy, uint32_t* tickets, hipStream_t stream) {
   if (n_chunks == 0 || n_layers == 0) return hipSuccess;
   const uint32_t n_slices = n_chunks << sub_shift;
   const ChunkGrid g = chunk_grid(n_slices, n_layers, max_wgs);
   if (!g.capped) tickets = nullptr;
-  const uint32_t shift_arg = sub_shift | (temporal && !g.capped ? kTemporalFlag : 0u);
+  const uint32_t shift_arg = sub_shift | (g.capped ? 0u : (policy & 3u) << 8);
 #define KVT_ARGS chunks, n_slices, shift_arg, layer_ptrs, n_tensors, first_layer, n_layers, packed, layer_stride, blobs, x, tickets
   if (pack && !g.capped) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, false>), KVT_ARGS);
   else if (pack) KVT_LAUNCH_CHUNKS((xform_chunks_kernel<true, true>), KVT_ARGS);

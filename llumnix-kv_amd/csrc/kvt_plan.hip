@@ -1004,7 +1004,9 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   // A launch whose payload fits the memory-side cache reads with plain loads (kvt_kernels.hip).
   uint64_t payload = 0;
   for (uint32_t t = 0; t < p->n_tensors; ++t) payload += p->tensor_bytes[t];
-  const bool temporal = payload * n_layers <= copy_cached_load_max_bytes();
+  // ... and one whose output is read again soon may leave it there (plain stores); not across PCIe
+  const uint32_t temporal = (payload * n_layers <= copy_cached_load_max_bytes() ? kPolicyTemporalLoads : 0u) |
+                            (!over_pcie && payload * n_layers <= copy_cached_store_max_bytes() ? kPolicyCachedStores : 0u);
   if (p->small) {
     // Under a limit, a 16-byte aligned table goes entry by entry through persistent workgroups
     // like a resident one (below), as soon as there is more than one entry per workgroup

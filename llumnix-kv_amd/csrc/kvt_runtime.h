@@ -43,6 +43,8 @@ uint32_t device_cu_count(int device);
 int check_device_span(const void* ptr, uint64_t bytes, const std::string& what, bool* host_memory = nullptr);
 // Launches whose payload is at most this many bytes read with plain loads (kvt_set_copy_cached_load_max).
 uint64_t copy_cached_load_max_bytes();
+// ... write with plain stores (kvt_set_copy_cached_store_max).
+uint64_t copy_cached_store_max_bytes();
 // Drops every remembered allocation extent (call where device memory is freed).
 void forget_device_spans();
 

@@ -73,6 +73,8 @@ uint32_t device_cu_count(int device) {
 
 static std::atomic<uint64_t> g_cached_load_max{kTemporalMaxBytes};
 uint64_t copy_cached_load_max_bytes() { return g_cached_load_max.load(std::memory_order_relaxed); }
+static std::atomic<uint64_t> g_cached_store_max{0};
+uint64_t copy_cached_store_max_bytes() { return g_cached_store_max.load(std::memory_order_relaxed); }
 
 // A kernel that runs past a buffer takes a GPU memory fault, which can cost the whole
 // process (and more) instead of an error code. What the runtime knows about a pointer is
@@ -259,6 +261,11 @@ int kvt_set_copy_cached_load_max(uint64_t payload_bytes) {
   return KVT_OK;
 }
 uint64_t kvt_get_copy_cached_load_max(void) { return copy_cached_load_max_bytes(); }
+int kvt_set_copy_cached_store_max(uint64_t payload_bytes) {
+  g_cached_store_max.store(payload_bytes, std::memory_order_relaxed);
+  return KVT_OK;
+}
+uint64_t kvt_get_copy_cached_store_max(void) { return copy_cached_store_max_bytes(); }
 
 int kvt_set_copy_cu_usage(int device, double usage) {
   return guarded([&]() -> int {

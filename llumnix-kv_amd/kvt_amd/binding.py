@@ -119,6 +119,8 @@ SIGNATURES = {
     "kvt_get_copy_method_profile": (_int, [_int] + [_P(C.c_double)] * 4 + [_P(_u64), _P(_int), _P(C.c_double)]),
     "kvt_set_copy_cached_load_max": (_int, [_u64]),
     "kvt_get_copy_cached_load_max": (_u64, []),
+    "kvt_set_copy_cached_store_max": (_int, [_u64]),
+    "kvt_get_copy_cached_store_max": (_u64, []),
     "kvt_set_copy_cu_usage": (_int, [_int, C.c_double]),
     "kvt_get_copy_cu_usage": (_int, [_int, _P(C.c_double), _P(_u32)]),
     "kvt_get_kernel_copy_buffer": (_int, [_int, _i64, _P(_vp), _P(_vp)]),

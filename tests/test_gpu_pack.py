@@ -1416,3 +1416,21 @@ def test_either_load_flavour_moves_the_same_bytes(limit):
         test_arbitrary_ranges_including_misaligned()
     finally:
         assert lib.kvt_set_copy_cached_load_max(0) == 0
+
+
+@pytest.mark.parametrize("loads", [0, 1 << 40])
+def test_either_store_flavour_moves_the_same_bytes(loads):
+    """kvt_set_copy_cached_store_max: plain stores for every launch between device buffers (a
+    huge limit), with either load flavour -- the same plans give the oracle's bytes."""
+    lib = kvt_amd.lib()
+    assert lib.kvt_get_copy_cached_store_max() == 0
+    assert lib.kvt_set_copy_cached_store_max(1 << 40) == 0 and lib.kvt_set_copy_cached_load_max(loads) == 0
+    try:
+        assert lib.kvt_get_copy_cached_store_max() == 1 << 40
+        test_short_plans_travel_in_the_kernel_arguments(64)
+        test_config2_shape_reduced_pool(0)
+        test_config3_transposing_pack_hnd_to_nhd()
+        test_config4_mla_and_indexer_two_tensors()
+        test_arbitrary_ranges_including_misaligned()
+    finally:
+        assert lib.kvt_set_copy_cached_store_max(0) == 0 and lib.kvt_set_copy_cached_load_max(0) == 0
