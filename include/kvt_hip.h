@@ -429,7 +429,11 @@ int kvt_enlarge_block_ids(const uint32_t* ids, uint64_t n, uint32_t factor, uint
 /* replaces launch_copy_d2h_direct_kernel()      kvtransfer/src/copy_kernels.cu:268-281
  * gather: dst[dst_offsets[i] : +lengths[i]] = gpu_src_base[src_offsets[i] : ...].
  * The three arrays live in device memory. num_wg / threads_per_wg <= 0 pick
- * this library's launch shape. */
+ * this library's launch shape. A long list is moved by persistent workgroups, a wavefront per
+ * range; ranges above 256 KiB (up to 500 of them per launch) are listed by a small kernel in
+ * front and moved by all wavefronts together at the end, so that a list which mixes many short
+ * ranges with a few very long ones (merged runs of hundreds of MiB) does not wait for single
+ * wavefronts. */
 int kvt_launch_copy_d2h_direct(const void* gpu_src_base, void* dst, const int64_t* src_offsets,
                                const int64_t* dst_offsets, const int64_t* lengths, int64_t n,
                                int num_wg, int threads_per_wg, void* stream);

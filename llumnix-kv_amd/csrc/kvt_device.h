@@ -177,10 +177,15 @@ hipError_t launch_copy_ranges(const void* src_base, void* dst_base, const int64_
 // The same list through `wgs` persistent workgroups (a multiple of 8), a wavefront per range:
 // the shape of a launch of many ranges, limited to a share of the device or not. walkers:
 // ranges a wavefront moves side by side, 1, 2 or 4 (the copy; more for shorter ranges).
+// share: a zeroed block of kShareBlockBytes that the launch may use until it has run (it leaves
+// it zeroed), or nullptr. With it the ranges above kLongRange bytes (at most kShareMax of
+// them, else none) are moved by all wavefronts together, in segments, instead of by the one
+// wavefront each that meets them; not for the converting gather.
+constexpr uint32_t kLongRange = 256u << 10, kShareMax = 500, kShareBlockBytes = 2048;
 hipError_t launch_copy_ranges_persistent(bool convert, const void* src_base, void* dst_base,
                                          const int64_t* src_off, const int64_t* dst_off,
                                          const int64_t* lens, int64_t n, uint32_t wgs, int walkers,
-                                         hipStream_t stream);
+                                         uint32_t* share, hipStream_t stream);
 hipError_t launch_convert_ranges(const void* src_base, void* dst_base, const int64_t* src_off,
                                  const int64_t* dst_off, const int64_t* lens, int64_t n,
                                  int num_wg, int rows, uint32_t max_wgs, hipStream_t stream);

@@ -38,18 +38,48 @@ int range_launch_shape(int64_t n, int num_wg, int* wgs) {
 // avg_len: the mean range length where the caller knows it (host lists), else 0: a wavefront
 // then moves 2 ranges side by side from 65 536 ranges on and 4 from 262 144 (a list that long
 // holds short ranges; 4 KiB and less is where it pays, 16 KiB and more where it costs 1-9 %).
+// max_len, n_long: the longest range and how many exceed kLongRange, where the caller knows the
+// lengths. A persistent wavefront's unit of work is a whole range, so a list that also holds a
+// few very long ranges (merged runs of hundreds of blocks among single blocks) would leave
+// those to one wavefront each after all others have finished, and the grid's few rows per
+// range fare no better: such a list goes to the persistent workgroups with a block through
+// which they share the long ranges out (launch_copy_ranges_persistent), whatever its length.
+// Where the lengths are unknown every persistent launch gets a block (about 2 us for the
+// kernel that lists the long ranges). own_share: the block to use (a caller that may not
+// allocate); otherwise one of the device's ticket blocks, none inside a stream capture.
 hipError_t launch_device_ranges(bool convert, int device, const void* src, void* dst, const int64_t* so,
                                 const int64_t* dof, const int64_t* len, int64_t n, int wgs, int rows,
-                                hipStream_t s, uint64_t avg_len = 0) {
+                                hipStream_t s, uint64_t avg_len = 0, uint64_t max_len = 0,
+                                uint64_t n_long = 0, uint32_t* own_share = nullptr) {
   const uint32_t cap = copy_wg_cap(device);
   const uint32_t cus = device_cu_count(device) & ~7u;
   if (cus >= 8) {
     const uint32_t pw = cap == 0 ? cus : std::max(8u, std::min(cap & ~7u, cus));
-    if (static_cast<uint64_t>(n) >= (cap != 0 ? 8ull : 64ull) * pw && (!convert || cap != 0))
+    const bool known = avg_len != 0;
+    const bool skewed = known && !convert && n_long != 0 && n_long <= kShareMax && max_len > 16 * avg_len;
+    if (skewed || (static_cast<uint64_t>(n) >= (cap != 0 ? 8ull : 64ull) * pw && (!convert || cap != 0)))
     {
-      const int walkers = avg_len != 0 ? (avg_len <= 1536 ? 4 : avg_len <= 8192 ? 2 : 1)
-                                       : (n >= 262144 ? 4 : n >= 65536 ? 2 : 1);
-      return launch_copy_ranges_persistent(convert, src, dst, so, dof, len, n, pw, walkers, s);
+      const int walkers = known ? (avg_len <= 1536 ? 4 : avg_len <= 8192 ? 2 : 1)
+                                : (n >= 262144 ? 4 : n >= 65536 ? 2 : 1);
+      uint32_t* share = nullptr;
+      bool lent = false;
+      if (!convert && (skewed || !known)) {
+        share = own_share;
+        if (!share) {
+          hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+          if (hipStreamIsCapturing(s, &st) != hipSuccess) (void)hipGetLastError();
+          if (st == hipStreamCaptureStatusNone && ticket_pool().prepare(device) == KVT_OK) {
+            share = ticket_pool().acquire(device, false);
+            lent = share != nullptr;
+          }
+        }
+      }
+      const hipError_t e = launch_copy_ranges_persistent(convert, src, dst, so, dof, len, n, pw, walkers, share, s);
+      if (lent) {
+        if (e == hipSuccess) ticket_pool().launched(device, share, s);
+        else ticket_pool().give_back(device, share);
+      }
+      return e;
     }
   }
   return convert ? launch_convert_ranges(src, dst, so, dof, len, n, wgs, rows, cap, s)
@@ -244,10 +274,12 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     int64_t* gpu = host_meta + m;
     int64_t* lens = host_meta + 2 * m;
     const uint64_t unit = halve ? 8192 : 4096;  // source bytes of one workgroup's slice
-    uint64_t slices = 0, batch_bytes = 0;
+    uint64_t slices = 0, batch_bytes = 0, batch_longest = 0, batch_long = 0;
     for (uint64_t i = 0; i < m; ++i) {
       const kvt_ipc_block& b = work[first + i];
       batch_bytes += b.length;
+      batch_longest = std::max(batch_longest, b.length);
+      batch_long += b.length > kLongRange;
       contig[i] = static_cast<int64_t>(b.src_offset);
       gpu[i] = static_cast<int64_t>(b.dst_offset);
       lens[i] = static_cast<int64_t>(halve ? b.length / 2 : b.length);
@@ -264,9 +296,9 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
     if (!over_pcie)  // both sides in device memory: the choice of the device-array launchers
       e = halve || direction == KVT_COPY_D2H
               ? launch_device_ranges(halve, device, layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
-                                     static_cast<int64_t>(m), wgs, rows, s, batch_bytes / m + 1)
+                                     static_cast<int64_t>(m), wgs, rows, s, batch_bytes / m + 1, batch_longest, batch_long)
               : launch_device_ranges(false, device, tensor_buf, layer_gpu_ptr, d_contig, d_gpu, d_lens,
-                                     static_cast<int64_t>(m), wgs, rows, s, batch_bytes / m + 1);
+                                     static_cast<int64_t>(m), wgs, rows, s, batch_bytes / m + 1, batch_longest, batch_long);
     else if (halve)
       e = launch_convert_ranges(layer_gpu_ptr, tensor_buf, d_gpu, d_contig, d_lens,
                                 static_cast<int64_t>(m), wgs, rows, cap, s);
@@ -290,7 +322,8 @@ int handle_data(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* bloc
 int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_block* blocks,
                        uint64_t n, uint64_t tensor_data_size, int direction, int device,
                        void* stream, int64_t* src_dev, int64_t* dst_dev, int64_t* len_dev,
-                       int64_t* host_meta, bool explicit_host_offsets, bool meta_by_kernel = false) {
+                       int64_t* host_meta, bool explicit_host_offsets, bool meta_by_kernel = false,
+                       uint32_t* share = nullptr) {
   if (n == 0) return KVT_OK;
   if (!tensor_buf || !layer_gpu_ptr || !blocks || !src_dev || !dst_dev || !len_dev || !host_meta)
     return fail(KVT_ERR_INVALID, "copy_handle_data_kernel_direct: null argument");
@@ -298,9 +331,11 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
     return fail(KVT_ERR_INVALID, "copy_handle_data_kernel_direct: bad direction");
   if (n > 0x7FFFFFFFull) return fail(KVT_ERR_INVALID, "too many ranges");
   if (int rc = check_device(device)) return rc;
-  uint64_t cursor = 0, slices = 0, layer_extent = 0;
+  uint64_t cursor = 0, slices = 0, layer_extent = 0, longest = 0, n_long = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const kvt_ipc_block& b = blocks[i];
+    longest = std::max(longest, b.length);
+    n_long += b.length > kLongRange;
     uint64_t end = 0;
     if (__builtin_add_overflow(b.dst_offset, b.length, &end))
       return fail(KVT_ERR_OUT_OF_RANGE,
@@ -346,9 +381,9 @@ int handle_data_direct(void* tensor_buf, void* layer_gpu_ptr, const kvt_ipc_bloc
       !over_pcie
           ? (direction == KVT_COPY_D2H
                  ? launch_device_ranges(false, device, layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
-                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s, cursor / n + 1)
+                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s, cursor / n + 1, longest, n_long, share)
                  : launch_device_ranges(false, device, tensor_buf, layer_gpu_ptr, src_dev, dst_dev, len_dev,
-                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s, cursor / n + 1))
+                                        static_cast<int64_t>(n), static_cast<int>(n), rows, s, cursor / n + 1, longest, n_long, share))
       : direction == KVT_COPY_D2H
           ? launch_copy_ranges(layer_gpu_ptr, tensor_buf, dst_dev, src_dev, len_dev,
                                static_cast<int64_t>(n), static_cast<int>(n), rows, pcie_wg_cap(device, over_pcie), s)
@@ -563,11 +598,13 @@ int kvt_copy_handle_data_kernel_direct(void* tensor_buf, void* layer_gpu_ptr,
 // ------------------------------------------------ the entry point that allocates nothing
 
 // Device-side range metadata of kvt_copy_handle_data_kernel_direct_static: three int64 arrays
-// of up to kStaticMaxRanges entries, 192 KiB, held by every GPU the library runs on until the
+// of up to kStaticMaxRanges entries, 192 KiB (+ 2 KiB), held by every GPU the library runs on until the
 // process ends. In host code the name is only a handle for hipGetSymbolAddress; each device
 // has its own copy at its own address, looked up once per device (g_scratch_ptr).
 constexpr uint64_t kStaticMaxRanges = 8192;
-static __device__ __align__(256) int64_t scratch[3 * kStaticMaxRanges];
+// Behind them one block of kShareBlockBytes, all zero between launches, through which the
+// persistent workgroups share out very long ranges (launch_copy_ranges_persistent).
+static __device__ __align__(256) int64_t scratch[3 * kStaticMaxRanges + kShareBlockBytes / 8];
 
 namespace {
 constexpr int kMaxStaticDevices = 64;
@@ -781,7 +818,8 @@ int kvt_copy_handle_data_kernel_direct_static(void* tensor_buf, void* layer_gpu_
     if (!capturing && sc->recorded) KVT_HIP(hipStreamWaitEvent(s, sc->last, 0));
     const int rc = handle_data_direct(tensor_buf, layer_gpu_ptr, blocks, n, tensor_data_size, direction,
                                       device, stream, meta, meta + n, meta + 2 * n, host_meta,
-                                      use_explicit_host_offsets != 0, true);
+                                      use_explicit_host_offsets != 0, true,
+                                      reinterpret_cast<uint32_t*>(meta + 3 * kStaticMaxRanges));
     // also behind a call that failed half way: its metadata copy may be on the stream
     if (!capturing) {
       KVT_HIP(hipEventRecord(sc->last, s));

@@ -997,10 +997,100 @@ __device__ __forceinline__ void copy_range_odd_by_wave(uint8_t* d, const uint8_t
     copy_units_by_wave(d, s, len, lane);
   }
 }
+// A wavefront's unit of work is a whole range, so one very long range among short ones (a merged
+// run of hundreds of blocks) would be moved by a single wavefront long after the others have
+// left. With a block of its own (`share`: word 0 the number of listed ranges, word 1 the
+// wavefronts that have left the second kernel, from word 2 the listed indices; all zero
+// between launches) the wavefront that meets a range above kLongRange lists it instead of
+// moving it (when the list is full it moves it after all), and move_listed_ranges_kernel,
+// launched behind, moves the listed ranges with every wavefront, in segments of kSegment dealt
+// out by position: the segments are numbered through all listed ranges and a wavefront takes
+// those whose number is its own modulo the wavefronts. The last wavefront to leave zeroes the
+// words used.
+constexpr uint32_t kSegment = 64u << 10;
+static_assert((2 + kShareMax) * 4 <= kShareBlockBytes, "the list of long ranges must fit its block");
+__global__ __launch_bounds__(kThreads, 2) void move_listed_ranges_kernel(
+    const uint8_t* src_base, uint8_t* dst_base, const int64_t* __restrict__ src_off,
+    const int64_t* __restrict__ dst_off, const int64_t* __restrict__ lens, uint32_t* share) {
+  const uint32_t listed = __builtin_amdgcn_readfirstlane(share[0]);
+  if (listed == 0) return;  // (every wavefront sees the same: nobody counts itself out below)
+  const uint32_t n_long = listed < kShareMax ? listed : kShareMax;
+  constexpr uint32_t kTrip = 8u << 10, kNoSegment = 0xFFFFFFFFu;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint32_t lane64 = threadIdx.x & 63u, off = lane64 << 4;
+  const uint32_t walkers = gridDim.x * 4u, me = blockIdx.x * 4u + wave;
+  const uint32_t* list = share + 2;
+  // j: the listed range the wavefront is at; before: the segments of the ranges in front of it
+  // (mod walkers); seg: its next segment in range j (kNoSegment: not worked out yet)
+  uint32_t j = 0, before = 0, seg = kNoSegment;
+  const uint8_t* s = nullptr;
+  uint8_t* d = nullptr;
+  uint64_t len = 0, begin = 0;
+  rsrc_t src[3], dst[3];
+  u32x4 r[3][8];
+  auto next = [&](int k) -> bool {
+    bool live = true;
+    if (begin >= len) {
+      len = 0;
+      begin = 0;
+      live = false;
+      uint32_t odd = 0;
+      while (j < n_long) {
+        const uint32_t at = __builtin_amdgcn_readfirstlane(list[j]);
+        const uint64_t whole = static_cast<uint64_t>(lens[at]);
+        const uint64_t n_seg = (whole + kSegment - 1) / kSegment;
+        if (seg == kNoSegment) seg = __builtin_amdgcn_readfirstlane((me + walkers - before) % walkers);
+        if (seg < n_seg) {
+          const uint64_t o = static_cast<uint64_t>(seg) * kSegment;
+          const uint64_t l = whole - o < kSegment ? whole - o : kSegment;
+          s = src_base + src_off[at] + o;
+          d = dst_base + dst_off[at] + o;
+          if (((reinterpret_cast<uintptr_t>(s) | reinterpret_cast<uintptr_t>(d)) & 3u) == 0) {
+            len = l & ~15ull;  // whole vectors through the pipeline, the last bytes at once
+            if (lane64 < (l & 15u)) d[len + lane64] = s[len + lane64];
+          } else {
+            odd = static_cast<uint32_t>(l);
+          }
+          seg += walkers;
+          live = true;
+          break;
+        }
+        before = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>((before + n_seg) % walkers));
+        seg = kNoSegment;
+        ++j;
+      }
+      // a segment that is not 4-byte aligned on both sides: byte by byte, on the spot
+#pragma unroll 8
+      for (uint32_t b = lane64; b < odd; b += 64u) d[b] = s[b];
+    }
+    const uint64_t left = len - begin;
+    const uint32_t bytes = left < kTrip ? static_cast<uint32_t>(left) : kTrip;
+    src[k] = make_rsrc(s + begin, bytes);
+    dst[k] = make_rsrc(d + begin, bytes);
+    begin += bytes;
+    return live;
+  };
+  auto load = [&](int k) {
+#pragma unroll
+    for (int v = 0; v < 8; ++v)
+      r[k][v] = __builtin_amdgcn_raw_buffer_load_b128(src[k], off + (v << 10), 0, kLoadPolicy);
+  };
+  auto store = [&](int k) {
+#pragma unroll
+    for (int v = 0; v < 8; ++v)
+      __builtin_amdgcn_raw_buffer_store_b128(r[k][v], dst[k], off + (v << 10), 0, kStorePolicy);
+  };
+  KVT_ROTATE3_PINNED(next, load, store);
+  uint32_t left = 0;
+  if (lane64 == 0) left = atomicAdd(share + 1, 1u);
+  if (static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(left)) == walkers - 1u)  // the last wavefront out
+    for (uint32_t w = lane64; w < 2u + n_long; w += 64u) share[w] = 0;
+}
 template <int U>
 __global__ __launch_bounds__(kThreads, 4) void copy_ranges_persistent_kernel(
     const uint8_t* src_base, uint8_t* dst_base, const int64_t* __restrict__ src_off,
-    const int64_t* __restrict__ dst_off, const int64_t* __restrict__ lens, uint32_t n) {
+    const int64_t* __restrict__ dst_off, const int64_t* __restrict__ lens, uint32_t n,
+    uint32_t* share) {
   // U ranges at a time per wavefront, each in trips of 8 / U KiB: the same bytes in flight, and
   // more ranges a second where they are short, since a range costs a trip however short it is
   // (TB/s with 1 / 2 / 4: ranges of 256 B 0.55 / 0.92 / 1.42, of 1 KiB 2.1 / 3.3 / 4.8, of 4 KiB
@@ -1022,6 +1112,23 @@ __global__ __launch_bounds__(kThreads, 4) void copy_ranges_persistent_kernel(
   }
   rsrc_t src[3][U], dst[3][U];
   u32x4 r[3][U][V];
+  // the walker's current range is (s, d, l): whole vectors through the pipeline, the last bytes
+  // and a range that is not 4-byte aligned on the spot
+  auto begin_range = [&](int u, uint64_t l) {
+    if (((reinterpret_cast<uintptr_t>(s[u]) | reinterpret_cast<uintptr_t>(d[u])) & 3u) == 0) {
+      len[u] = l & ~15ull;
+      if (lane64 < (l & 15u)) d[u][len[u] + lane64] = s[u][len[u] + lane64];
+    } else {
+      copy_range_odd_by_wave(d[u], s[u], l, lane64);
+    }
+  };
+  auto trip = [&](int k, int u) {
+    const uint64_t left = len[u] - begin[u];  // 0 when there is nothing (more) to move: empty descriptors
+    const uint32_t bytes = left < kTrip ? static_cast<uint32_t>(left) : kTrip;
+    src[k][u] = make_rsrc(s[u] + begin[u], bytes);
+    dst[k][u] = make_rsrc(d[u] + begin[u], bytes);
+    begin[u] += bytes;
+  };
   auto next = [&](int k) -> bool {
     bool any = false;
 #pragma unroll
@@ -1037,19 +1144,18 @@ __global__ __launch_bounds__(kThreads, 4) void copy_ranges_persistent_kernel(
           const uint64_t l = static_cast<uint64_t>(lens[i]);
           s[u] = src_base + src_off[i];
           d[u] = dst_base + dst_off[i];
-          if (((reinterpret_cast<uintptr_t>(s[u]) | reinterpret_cast<uintptr_t>(d[u])) & 3u) == 0) {
-            len[u] = l & ~15ull;  // whole vectors through the pipeline, the last bytes at once
-            if (lane64 < (l & 15u)) d[u][len[u] + lane64] = s[u][len[u] + lane64];
-          } else {
-            copy_range_odd_by_wave(d[u], s[u], l, lane64);
+          bool mine = true;
+          if (share && l > kLongRange) {  // everybody's, later, if the list has room
+            uint32_t at = 0;
+            if (lane64 == 0) at = atomicAdd(share, 1u);
+            at = __builtin_amdgcn_readfirstlane(at);
+            mine = at >= kShareMax;
+            if (!mine && lane64 == 0) share[2 + at] = i;
           }
+          if (mine) begin_range(u, l);
         }
       }
-      const uint64_t left = len[u] - begin[u];  // 0 when there is nothing (more) to move: empty descriptors
-      const uint32_t bytes = left < kTrip ? static_cast<uint32_t>(left) : kTrip;
-      src[k][u] = make_rsrc(s[u] + begin[u], bytes);
-      dst[k][u] = make_rsrc(d[u] + begin[u], bytes);
-      begin[u] += bytes;
+      trip(k, u);
       any = any || live;
     }
     return any;
@@ -1861,13 +1967,14 @@ static dim3 range_grid(int num_wg, int rows, uint32_t max_wgs) {
 hipError_t launch_copy_ranges_persistent(bool convert, const void* src_base, void* dst_base,
                                          const int64_t* src_off, const int64_t* dst_off,
                                          const int64_t* lens, int64_t n, uint32_t wgs, int walkers,
-                                         hipStream_t stream) {
+                                         uint32_t* share, hipStream_t stream) {
   if (n <= 0) return hipSuccess;
   if (n > 0x7FFFFFF0ll || wgs < 8 || (wgs & 7u)) return hipErrorInvalidValue;
+  if (convert) share = nullptr;
 #define KVT_RANGES(U)                                                                              \
   hipLaunchKernelGGL(copy_ranges_persistent_kernel<U>, dim3(wgs), dim3(kThreads), 0, stream,       \
                      static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off, \
-                     dst_off, lens, static_cast<uint32_t>(n))
+                     dst_off, lens, static_cast<uint32_t>(n), share)
   if (convert)
     hipLaunchKernelGGL(convert_ranges_persistent_kernel, dim3(wgs), dim3(kThreads), 0, stream,
                        static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off,
@@ -1879,6 +1986,10 @@ hipError_t launch_copy_ranges_persistent(bool convert, const void* src_base, voi
   else
     KVT_RANGES(1);
 #undef KVT_RANGES
+  if (share)
+    hipLaunchKernelGGL(move_listed_ranges_kernel, dim3(wgs), dim3(kThreads), 0, stream,
+                       static_cast<const uint8_t*>(src_base), static_cast<uint8_t*>(dst_base), src_off,
+                       dst_off, lens, share);
   return hipGetLastError();
 }
 

@@ -1282,6 +1282,119 @@ def test_handle_data_between_two_device_buffers_with_a_long_list(usage, choice):
         kvt_amd.set_copy_cu_usage(0, 1.0)
 
 
+@pytest.mark.parametrize("short,longs,starts", [
+    ([4096, 8192, 16384], [48 << 20, 48 << 20, (48 << 20) + 1000], (0, 4, 16)),   # one range per wavefront
+    ([4096, 4099, 2048], [(20 << 20) + 5, 300 << 10], (0, 1)),                     # two side by side
+    ([256, 512, 1000, 13], [3 << 20, (1 << 20) + 7, 262145, 262144], (4, 0, 16, 1))],   # four
+    ids=["one", "two", "four"])
+def test_a_long_list_with_a_few_very_long_ranges(short, longs, starts):
+    """Merged runs of many blocks among single blocks: 20 000 short ranges and a few of up to
+    48 MiB, some of them not 16-byte aligned or not whole vectors long. A persistent
+    wavefront's unit of work is a whole range; the ranges above 256 KiB are listed by the
+    wavefronts that meet them and moved by a kernel behind, by all wavefronts together, in
+    64 KiB segments. Through the host-list
+    entry point (which sees the lengths), the device-array launchers (which do not) and the
+    entry point that allocates nothing: the oracle's bytes, and the list takes at most three
+    times what the same bytes take as even ranges (it took eight times that)."""
+    rng = np.random.default_rng(14)
+    n, slot = 20000, 16384
+    lens = rng.choice(short, size=n).astype(np.uint64)
+    gpu_off = (np.arange(n, dtype=np.uint64) * slot)[rng.permutation(n)]
+    gpu_off[rng.random(n) < 0.05] += 4
+    where = rng.choice(n, size=len(longs), replace=False)  # the long ranges sit anywhere in the list
+    at = n * slot
+    for k, i in enumerate(where):
+        lens[i] = longs[k]
+        gpu_off[i] = at + starts[k]
+        at += (longs[k] + 4096 + 255) // 256 * 256
+    cap = int(at)
+    host_off = (np.cumsum(lens) - lens).astype(np.uint64)
+    total = int(lens.sum())
+    blocks = np.ascontiguousarray(np.stack([np.zeros(n, np.uint64), gpu_off, lens], axis=1))
+    layer = _dev_bytes(cap, 46, "raw")
+    staged = torch.zeros(total, dtype=torch.uint8, device="cuda")
+    dev = [torch.zeros(n, dtype=torch.int64, device="cuda") for _ in range(3)]
+    host_meta = torch.zeros(3 * n, dtype=torch.int64).pin_memory()
+    lib = kvt_amd.lib()
+    st = checkers.side_stream()
+    layer_h = _host(layer)
+    idx_src = np.concatenate([np.arange(int(g), int(g + l)) for g, l in zip(gpu_off, lens)])
+    exp = layer_h[idx_src]                                  # the packed side has no gaps
+    exp_d = np.full(cap, 0x33, dtype=np.uint8)
+    exp_d[idx_src] = exp
+
+    def call(gpu, direction, blk=blocks, count=n, size=total):
+        return lib.kvt_copy_handle_data_kernel_direct(
+            staged.data_ptr(), gpu.data_ptr(), blk.ctypes.data, count, size, direction, 0,
+            st.cuda_stream, dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(),
+            host_meta.data_ptr(), 0)
+
+    for _ in range(2):                                      # the second launch finds the block zeroed
+        staged.zero_()
+        torch.cuda.synchronize()
+        assert call(layer, 1) == 0, lib.kvt_last_error()
+        st.synchronize()
+        assert np.array_equal(_host(staged), exp)
+    dst = torch.full((cap,), 0x33, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    assert call(dst, 0) == 0, lib.kvt_last_error()
+    st.synchronize()
+    assert np.array_equal(_host(dst), exp_d)
+    # the device-array launchers
+    so, do, ln = _soa(np.stack([gpu_off, host_off, lens], axis=1).astype(np.int64))
+    for _ in range(2):
+        staged.zero_()
+        assert lib.kvt_launch_copy_d2h_direct(layer.data_ptr(), staged.data_ptr(), so.data_ptr(),
+                                              do.data_ptr(), ln.data_ptr(), n, 0, 0, None) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(_host(staged), exp)
+    dst.fill_(0x33)
+    assert lib.kvt_launch_copy_h2d_direct(staged.data_ptr(), dst.data_ptr(), do.data_ptr(),
+                                          so.data_ptr(), ln.data_ptr(), n, 0, 0, None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(_host(dst), exp_d)
+    # the entry point that allocates nothing (8192 ranges at most): the first 8000 and the long ones
+    keep = np.unique(np.concatenate([np.arange(8000), where]))
+    sub = np.ascontiguousarray(blocks[keep])
+    sub_total = int(sub[:, 2].sum())
+    pinned_meta = torch.zeros(3 * len(keep), dtype=torch.int64).pin_memory()
+    for _ in range(2):
+        staged.zero_()
+        torch.cuda.synchronize()
+        assert lib.kvt_copy_handle_data_kernel_direct_static(
+            staged.data_ptr(), layer.data_ptr(), sub.ctypes.data, len(keep), sub_total, 1, 0,
+            st.cuda_stream, pinned_meta.data_ptr(), 0) == 0, lib.kvt_last_error()
+        st.synchronize()
+        idx_sub = np.concatenate([np.arange(int(g), int(g + l)) for g, l in zip(sub[:, 1], sub[:, 2])])
+        assert np.array_equal(_host(staged)[:sub_total], layer_h[idx_sub])
+    del dst
+
+    # the same bytes as even ranges (every range 16 KiB) for the time
+    m = total // 16384
+    even = np.ascontiguousarray(np.stack([np.zeros(m, np.uint64), np.arange(m, dtype=np.uint64) * 16384,
+                                          np.full(m, 16384, np.uint64)], axis=1))
+    if m > n:
+        dev = [torch.zeros(m, dtype=torch.int64, device="cuda") for _ in range(3)]
+        host_meta = torch.zeros(3 * m, dtype=torch.int64).pin_memory()
+
+    def timed(blk, count, size=total):
+        best = 1e9
+        for _ in range(4):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            with torch.cuda.stream(st):
+                e0.record()
+                assert call(layer, 1, blk, count, size) == 0, lib.kvt_last_error()
+                e1.record()
+            st.synchronize()
+            best = min(best, e0.elapsed_time(e1))
+        return best
+
+    t_even, t_skew = timed(even, m, m * 16384), timed(blocks, n)
+    print(f"skewed list {t_skew * 1e3:.0f} us, even list of the same bytes {t_even * 1e3:.0f} us")
+    if short[0] == 4096 and len(short) == 3 and short[1] == 8192:
+        assert t_skew < 3 * t_even
+
+
 def test_random_range_lists_sweep():
     """80 seeded batches of arbitrary ranges: 1-3 tensors, 1-3 layers, lengths from 1 byte to
     70 000, alignments 1 / 4 / 16 / 256, shuffled list order, every chunk size, packed buffer
