@@ -650,6 +650,68 @@ def leg_cu_usage(c, out):
     out["cu_usage"] = rows
 
 
+def leg_small_launch(c, out):
+    """A launch small enough for the 256 MiB memory-side cache (config 1: 64 MiB) under the four
+    load / store policies of kvt_set_copy_cached_load_max / kvt_set_copy_cached_store_max,
+    against plain copies of the same size. Event intervals per launch, launches back to back on
+    one stream. cold: 24 different requests of that size one after the other (1.5 GiB of blobs,
+    so nothing a launch reads or writes is left in a cache from the launch before); pack_then_
+    unpack: a request's unpack right behind its pack, requests cycling."""
+    torch, kvt, lib, sh, new_event, pipeline = c.torch, c.kvt, c.lib, c.sh, c.new_event, c.pipeline
+    from kvt_amd import workloads as W
+    w, side = c.wls[0], c.sides[0]
+    reps = 24
+    ws = [W.llama8b_single(seed=20251 + 7 * r) for r in range(reps)]
+    plans = [pipeline.build_plan(x, 0) for x in ws]
+    stride = plans[0][0].layer_bytes
+    nbytes = stride * w.n_layers
+    blobs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(reps)]
+    evs = [new_event() for _ in range(2 * reps + 1)]
+
+    def timed(fns):
+        for _ in range(3):              # the last pass is the measurement
+            lib.kvt_event_record(evs[0], sh)
+            for i, f in enumerate(fns):
+                f()
+                lib.kvt_event_record(evs[i + 1], sh)
+            lib.kvt_event_synchronize(evs[len(fns)])
+        return [ev_ms(lib, evs[i], evs[i + 1]) * 1e3 for i in range(len(fns))]
+
+    def pk(r):
+        return lambda: plans[r][0].pack(side.src_cache, 0, w.n_layers, blobs[r], stride, sh)
+
+    def un(r):
+        return lambda: plans[r][0].unpack(side.dst_cache, 0, w.n_layers, blobs[r], stride, sh)
+
+    rows = []
+    try:
+        for loads, stores in ((0, 0), (0, 1), (1, 0), (1, 1)):
+            lib.kvt_set_copy_cached_load_max(loads << 30)
+            lib.kvt_set_copy_cached_store_max(stores << 30)
+            cold_pack = statistics.median(timed([pk(r) for r in range(reps)]))
+            cold_unpack = statistics.median(timed([un(r) for r in range(reps)]))
+            seq = timed([f for r in range(reps // 2) for f in (pk(r), un(r))])
+            rows.append({"loads": "plain" if loads else "nt", "stores": "plain" if stores else "sc0 sc1 nt",
+                         "cold_pack_us": round(cold_pack, 2), "cold_unpack_us": round(cold_unpack, 2),
+                         "pack_then_unpack_us": [round(statistics.median(seq[0::2]), 2),
+                                                 round(statistics.median(seq[1::2]), 2)]})
+    finally:
+        lib.kvt_set_copy_cached_load_max(0)
+        lib.kvt_set_copy_cached_store_max(0)
+    res = {"policies": rows, "bytes_per_launch": nbytes}
+    others = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(reps)]
+    for fn_name in ("kvt_copy_linear", "kvt_copy_runtime_d2d"):
+        fn = getattr(lib, fn_name)
+        t = timed([(lambda i=i: fn(others[i].data_ptr(), blobs[i].data_ptr(), nbytes, sh)) for i in range(reps)])
+        res[fn_name + "_cold_us"] = round(statistics.median(t), 2)
+    res["note"] = ("us per launch by event interval (launch gap included); the library's default is "
+                   "the first row; the two copies are the cold ceilings for a launch of this size")
+    for pl, ls in plans:
+        pl.close()
+        ls.close()
+    out["small_launch"] = res
+
+
 def leg_copy_ceilings(c, out):
     """Plain copies of the sizes the launches here have, by this library's linear copy kernel
     and by the runtime's own device-to-device hipMemcpyAsync: what the part gives a copy that
@@ -1173,13 +1235,14 @@ def leg_staging(c, out):
 # chunk size, and only for the kernel source they were measured with: tests/test_bench_contract.py
 # compares KERNELS_SHA256 with llumnix-kv_amd/csrc/kvt_kernels.hip and fails when the file has
 # changed since, so a stale table cannot pass unnoticed.
-KERNELS_SHA256 = "96cc727430f2a47695f2dc58f5311b51ecf65fb0c5dc15ab7a47e61444203041"
+KERNELS_SHA256 = "aa1123ba9e7332ed676cb512bcb5997d9402593a554fe0ea56256a9a1a5cd47c"
 MEASURED_TRAFFIC = {
-    (1, "ranges"): {"pack": 134267182, "unpack": 134277593},
-    (2, "ranges"): {"pack": 71013168478, "unpack": 73358403376},
-    (3, "ranges"): {"pack": 85983095771, "unpack": 85983579778},
-    (4, "ranges"): {"pack": 22690375536, "unpack": 22690444271},
-    (5, "ranges"): {"pack": 45141193160, "unpack": 45141392582},
+    (1, "ranges"): {"pack": 134268079, "unpack": 134278234},
+    (2, "ranges"): {"pack": 71013152265, "unpack": 73358397596},
+    (3, "ranges"): {"pack": 85983237339, "unpack": 85984011093},
+    (4, "ranges"): {"pack": 22690361783, "unpack": 22690413793},
+    (5, "ranges"): {"pack": 45141172606, "unpack": 45141395495},
+    (9, "ranges"): {"pack": 45141104254, "unpack": 45141166035},
 }
 
 
@@ -1411,9 +1474,19 @@ def run_config(args, headline):
     legs = [] if args.skip_cpu else [leg_cpu]
     if not args.skip_extras:
         legs += [leg_latency, leg_staging, leg_cu_usage]
+        if args.config == 1:
+            legs += [leg_small_launch]
         if headline:
             legs += [leg_session, leg_copy_ceilings, leg_launchers, leg_fp8_plan,
                      leg_frames, leg_store_objects]
+    if args.legs:   # a profiling run of chosen legs only
+        want = {"leg_" + name for name in args.legs.split(",")}
+        every = [leg_latency, leg_staging, leg_cu_usage, leg_small_launch, leg_session, leg_copy_ceilings,
+                 leg_launchers, leg_fp8_plan, leg_frames, leg_store_objects]
+        unknown = want - {leg.__name__ for leg in every}
+        if unknown:
+            raise SystemExit("bench.py: --legs knows %s" % ", ".join(l.__name__[4:] for l in every))
+        legs = [leg for leg in every if leg.__name__ in want]
     errors = {}
     for leg in legs:
         try:
@@ -1474,6 +1547,10 @@ def main():
                          "(kvt_set_copy_cu_usage; the reference's BLLM_KVTRANS_KERNEL_COPY_SM_USAGE)")
     ap.add_argument("--skip-cpu", action="store_true")
     ap.add_argument("--skip-extras", action="store_true", help="no latency / staging legs")
+    ap.add_argument("--legs", default="",
+                    help="comma-separated side legs to run instead of the default set (for a "
+                         "profile of one of them): latency, staging, cu_usage, small_launch, session, "
+                         "copy_ceilings, launchers, fp8_plan, frames, store_objects")
     ap.add_argument("--calibrate-copy-gib", type=float, default=0.0,
                     help="only run the plain linear copy kernel on this many GiB (profiler "
                          "counter calibration: its HBM traffic is known, 1 read + 1 write)")
@@ -1542,7 +1619,7 @@ def main():
                         "latency_graph_replay_equals_fresh_plan",
                         "latency_graph_replay_empty_batch_gpu_p50_us",
                         "latency_after_last_layer_p50_us", "latency_after_last_layer_inline_p50_us",
-                        "cu_usage",
+                        "cu_usage", "small_launch",
                         "staging", "roofline", "cpu_baseline", "errors"):
                 if key in r:
                     row[key] = r[key]
