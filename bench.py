@@ -1113,6 +1113,7 @@ def leg_staging(c, out):
         group = max(1, min(w.n_layers, -(-(256 << 20) // lbytes)))
         n_groups = max(1, min(8, w.n_layers // group))
         nbytes = group * lbytes
+        pay_group = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * group
         ceil = {}
         for name, d in (("d2h", 1), ("h2d", 0)):
             r = C.c_double()
@@ -1120,34 +1121,53 @@ def leg_staging(c, out):
             ceil[name] = r.value
         stg = kvt.Stager(0, nbytes, 2)
         bufs = [torch.empty(nbytes, dtype=torch.uint8, device="cuda") for _ in range(2)]
-        ps = torch.cuda.Stream()
-        cs = [torch.cuda.Stream(), torch.cuda.Stream()]
-        d2h_t, h2d_t = [], []
-        for phase in range(4):          # first phase warms up
+
+        def save_pass(ps_, groups):
             torch.cuda.synchronize()
             a = time.perf_counter()
-            for g in range(n_groups):
+            for g in range(groups):
                 slot = g % 2
                 if g >= 2:
                     stg.wait(slot)
-                plan.pack(side.src_cache, g * group, group, bufs[slot], lbytes, ps.cuda_stream)
-                stg.save(slot, bufs[slot], nbytes, ps.cuda_stream)
+                plan.pack(side.src_cache, g * group, group, bufs[slot], lbytes, ps_.cuda_stream)
+                stg.save(slot, bufs[slot], nbytes, ps_.cuda_stream)
             stg.wait(0)
-            if n_groups > 1:
+            if groups > 1:
                 stg.wait(1)
-            d2h_t.append(time.perf_counter() - a)
-        for phase in range(4):
+            return time.perf_counter() - a
+
+        def load_pass(cs_, groups):
             torch.cuda.synchronize()
             a = time.perf_counter()
-            for g in range(n_groups):
+            for g in range(groups):
                 # a consumer stream per slot: a load waits for what was queued on its consumer
                 # stream, which then is the slot's last unpack and not the other slot's
                 slot = g % 2
-                stg.load(slot, bufs[slot], nbytes, cs[slot].cuda_stream)
-                plan.unpack(side.dst_cache, g * group, group, bufs[slot], lbytes, cs[slot].cuda_stream)
-            cs[0].synchronize()
-            cs[1].synchronize()
-            h2d_t.append(time.perf_counter() - a)
+                stg.load(slot, bufs[slot], nbytes, cs_[slot].cuda_stream)
+                plan.unpack(side.dst_cache, g * group, group, bufs[slot], lbytes, cs_[slot].cuda_stream)
+            cs_[0].synchronize()
+            cs_[1].synchronize()
+            return time.perf_counter() - a
+
+        # Which streams the caller uses matters: HIP maps streams onto a few hardware queues, and a
+        # stream that waits (a consumer stream for its transfer, the copy stream for a pack)
+        # parks that wait in its queue for as long as it takes; another stream mapped to the same
+        # queue gets nothing through meanwhile, and what should overlap takes turns. Which
+        # streams share a queue cannot be asked, only measured: four sets of producer / consumer
+        # streams are tried with a short pass each and the best one is used (what a deployment
+        # does once at start-up).
+        probe_groups = min(n_groups, 4)
+        sets = [(torch.cuda.Stream(), [torch.cuda.Stream(), torch.cuda.Stream()]) for _ in range(4)]
+        one_way = []
+        for st in sets:
+            save_pass(st[0], min(2, probe_groups))
+            t_s = save_pass(st[0], probe_groups)
+            load_pass(st[1], min(2, probe_groups))
+            t_l = load_pass(st[1], probe_groups)
+            one_way.append(round(2 * pay_group * probe_groups / (t_s + t_l) / 1e9, 2))
+        ps, cs = sets[max(range(4), key=lambda k: one_way[k])]
+        d2h_t = [save_pass(ps, n_groups) for phase in range(4)]      # the first pass warms up
+        h2d_t = [load_pass(cs, n_groups) for phase in range(4)]
         d2h_s, h2d_s = statistics.median(d2h_t[1:]), statistics.median(h2d_t[1:])
         pay = sum(plan.tensor_bytes(t) for t in range(w.n_tensors)) * group * n_groups
         # Both directions at once: a saving and a loading stager side by side, against two plain
@@ -1180,27 +1200,22 @@ def leg_staging(c, out):
             cs_[1].synchronize()
             return t_save, time.perf_counter() - a
 
-        # Which streams the caller uses matters: HIP maps streams onto a few hardware queues, and a
-        # consumer stream that waits for a transfer parks that wait in its queue for as long as
-        # the transfer takes; a copy stream mapped to the same queue gets nothing through
-        # meanwhile, and the two directions take turns instead of overlapping. Which streams share
-        # a queue cannot be asked, only measured: four sets of streams are tried with a short
-        # pass each and the best one is used (what a deployment does once at start-up).
-        probe_groups = min(n_groups, 4)
-        sets, quick = [], []
-        for k in range(4):
-            st = (torch.cuda.Stream(), [torch.cuda.Stream(), torch.cuda.Stream()])
-            both_ways(st[0], st[1], min(2, probe_groups))
-            t_s, t_l = both_ways(st[0], st[1], probe_groups)
-            sets.append(st)
-            quick.append(round(2 * pay / n_groups * probe_groups / (t_s + t_l) / 1e9, 2))
+        # (the same four sets of streams, tried with both stagers at work; at least four
+        # transfers each way, the groups repeating, so that there is something to overlap)
+        bi_groups = max(n_groups, 4)
+        quick = []
+        for st in sets:
+            both_ways(st[0], st[1], 2)
+            t_s, t_l = both_ways(st[0], st[1], 4)
+            quick.append(round(2 * pay_group * 4 / (t_s + t_l) / 1e9, 2))
         ps_b, cs_b = sets[max(range(4), key=lambda k: quick[k])]
         bi_save, bi_load = [], []
         for phase in range(4):
-            t_s, t_l = both_ways(ps_b, cs_b, n_groups)
+            t_s, t_l = both_ways(ps_b, cs_b, bi_groups)
             bi_save.append(t_s)
             bi_load.append(t_l)
-        bs, bl = statistics.median(bi_save[1:]), statistics.median(bi_load[1:])
+        bs, bl = (statistics.median(bi_save[1:]) * n_groups / bi_groups,
+                  statistics.median(bi_load[1:]) * n_groups / bi_groups)
         stg_in.close()
         del bufs_in
         out["staging"] = {
@@ -1213,15 +1228,16 @@ def leg_staging(c, out):
             "bidir_pcie_h2d_gbps": round(both[1].value / 1e9, 2),
             "bidir_save_frac_of_pcie": round(pay / bs / both[0].value, 4),
             "bidir_load_frac_of_pcie": round(pay / bl / both[1].value, 4),
+            "stream_sets_gbps": one_way,
             "bidir_stream_sets_gbps": quick,
             "bidir_note": "a saving and a loading stager at the same time (pack -> D2H beside H2D "
                           "-> unpack), each direction's payload over the time until that direction "
                           "has finished; ceiling: two plain copies of one transfer's size running "
                           "concurrently on two streams (kvt_measure_pcie_both_ways); "
-                          "bidir_stream_sets_gbps: mean rate per direction of a short pass with "
-                          "each of four sets of producer / consumer streams (streams that share a "
-                          "hardware queue with a copy stream make the directions take turns), the "
-                          "best set is the one measured",
+                          "stream_sets_gbps / bidir_stream_sets_gbps: mean rate per direction of a "
+                          "short pass with each of four sets of producer / consumer streams, one "
+                          "direction at a time / both at once (streams that share a hardware queue "
+                          "take turns where they should overlap), the best set is the one measured",
             "sample": "%d transfers of %d layer(s) = %.1f MiB each through 2 pinned slots, "
                       "pack / unpack of the group in one launch; median of 3 passes" %
                       (n_groups, group, nbytes / 2**20),

@@ -732,9 +732,13 @@ void* kvt_session_side_stream(kvt_session* s);
 
 /* ------------------------------------ pinned-host staging (KVStore path) */
 
-/* A ring of pinned host slots fed by hipMemcpyAsync on its own copy stream, so
+/* A ring of pinned host slots fed by hipMemcpyAsync on a copy stream of the library's, so
  * that D2H of layer L overlaps the pack of layer L+1 (and H2D of L+1 overlaps
- * the unpack of L). Stands where the reference's KVStore backends hand packed
+ * the unpack of L). The copy streams are four per device, made together with the first
+ * stager, kept until the process ends and handed to the stagers in turn: stagers made one
+ * after the other (a saving and a loading one) then copy through different hardware queues,
+ * which is what lets the two directions overlap; from the fifth on stagers share streams.
+ * Stands where the reference's KVStore backends hand packed
  * layers to a host-side store                   blade_kvt/hybrid_connector/kvsbackend.py:268-357,
  *                                               blade_kvt/hybrid_connector/file_backend.py:222-283.
  * slot_bytes bounds one transfer; n_slots >= 2. One stager serves one caller
@@ -771,7 +775,10 @@ int kvt_measure_pcie(int device, int direction, uint64_t bytes, uint32_t repeats
 
 /* The same with both directions running at the same time on two streams (a saving and a
  * loading stager side by side): the rate each direction reaches while the other one is busy,
- * the ceiling for concurrent save and load. Allocates 2 x bytes of pinned and of device memory. */
+ * the ceiling for concurrent save and load. The rate of two concurrent copies depends on which
+ * streams carry them (streams share a few hardware queues), so four pairs out of four new
+ * streams are measured, `repeats` copies each way per pair, and the pair with the highest sum
+ * is reported. Allocates 2 x bytes of pinned and of device memory. */
 int kvt_measure_pcie_both_ways(int device, uint64_t bytes, uint32_t repeats, double* d2h_bytes_per_s,
                                double* h2d_bytes_per_s);
 
