@@ -70,15 +70,33 @@ def _caches(w, seed):
     return src, dst
 
 
-def _run_plain(w, seed):
-    plan, lists = pipeline.build_plan(w, 0)
+def _run_plain(w, seed, earlier=None, chunk=0):
+    """earlier: another batch on the same pools. The plan then is a plan slot that held that
+    batch first and was refilled with w's (kvt_plan_slot_fill), launched through the persistent
+    kernels that read the batch's entry count and blob positions from the slot's header.
+    chunk: the size the slot's table entries are cut to."""
+    plan, lists = pipeline.build_plan(w, 0, chunk)
     o_lists = _oracle_lists(w)
     for t in range(w.n_tensors):
         assert np.array_equal(lists.tensor(t), o_lists[t])
+    if earlier is not None:
+        fresh = plan
+        old_plan, old_lists = pipeline.build_plan(earlier, 0, chunk)
+        room = max(fresh.layer_bytes, old_plan.layer_bytes)   # a layer's stride holds any batch of the slot
+        plan = kvt_amd.PlanSlot(0, w.n_tensors, w.capacities("src"), w.capacities("dst"),
+                                max_entries=max(fresh.num_chunks, old_plan.num_chunks),
+                                max_layer_bytes=room, chunk_bytes=chunk)
+        assert plan.fill(old_lists).n_entries == old_plan.num_chunks
+        lay = plan.fill(lists)
+        assert (lay.n_entries, lay.layer_bytes) == (fresh.num_chunks, fresh.layer_bytes)
+        for t in range(w.n_tensors):
+            assert (lay.tensor_bytes[t], lay.tensor_offset[t]) == (fresh.tensor_bytes(t), fresh.tensor_offset(t))
+        old_plan.close()
+        fresh.close()
     src, dst = _caches(w, seed)
     sc = kvt_amd.Cache(0, src, w.capacities("src"))
     dc = kvt_amd.Cache(0, dst, w.capacities("dst"))
-    stride = plan.layer_bytes
+    stride = plan.layer_bytes if earlier is None else room
     packed = torch.zeros(w.n_layers * stride, dtype=torch.uint8, device="cuda")
     plan.pack(sc, 0, w.n_layers, packed, stride)
     plan.unpack(dc, 0, w.n_layers, packed, stride)
@@ -109,6 +127,16 @@ def test_config2_full_size():
 
 def test_config4_full_size():
     _run_plain(workloads.deepseek_mla(), 4)        # 61 layers, MLA latent + indexer, 10.5 GiB
+
+
+def test_config2_full_size_through_a_refilled_plan_slot():
+    w = workloads.llama8b_batch()
+    _run_plain(w, 12, earlier=workloads.llama8b_batch(seed=4711), chunk=32768)
+
+
+def test_config4_full_size_through_a_refilled_plan_slot():
+    # two tensors per layer, entries of 4 KiB: a wavefront per entry
+    _run_plain(workloads.deepseek_mla(), 14, earlier=workloads.deepseek_mla(n_req=9, tokens=9000), chunk=4096)
 
 
 def test_config5_full_size():
