@@ -575,22 +575,27 @@ def session_new_batches(c, out, frozen_ms):
             torch.cuda.synchronize()
             res["graph_replay_slot_same_batch_ms"] = round((time.perf_counter() - t_a) / 5 * 1e3, 4)
         host = []
+        e_a, e_b = c.new_event(), c.new_event()
         for rep in range(2):
             torch.cuda.synchronize()
-            t_a = time.perf_counter()
             n = 6
-            for i in range(n):
+            for i in range(n + 1):
+                # steady state: the clock starts behind the first replay, whose batch the host
+                # prepared with the GPU idle; from then on the host works while the GPU replays
                 h0 = time.perf_counter()
-                k = (i + 1) % len(variants)
+                k = i % len(variants)
                 lists = c.senders[0].parse(v_tasks[k])
                 slot.fill(lists, gs.cuda_stream)
                 lists.close()
                 host.append(time.perf_counter() - h0)
                 sess.begin_step()
                 graph.replay()
-            torch.cuda.synchronize()
-            new_ms = (time.perf_counter() - t_a) / n * 1e3
-        last = (n - 1 + 1) % len(variants)
+                if i == 0:
+                    lib.kvt_event_record(e_a, gs.cuda_stream)
+            lib.kvt_event_record(e_b, gs.cuda_stream)
+            lib.kvt_event_synchronize(e_b)
+            new_ms = ev_ms(lib, e_a, e_b) / n
+        last = n % len(variants)
     # what the last replay packed against a plan made for that batch alone (first and last layer)
     fresh = kvt.Plan(0, v_lists[last], caps[0], caps[1], chunk_bytes=chunk)
     ref = torch.empty(room, dtype=torch.uint8, device="cuda")
@@ -600,19 +605,22 @@ def session_new_batches(c, out, frozen_ms):
         gs.synchronize()
         nb = fresh.tensor_bytes(0)
         same &= bool(torch.equal(ref[:nb], buf[l * room:l * room + nb]))
-    mean_pay = sum(payloads[(i + 1) % len(variants)] for i in range(n)) / n
+    mean_pay = sum(payloads[i % len(variants)] for i in range(1, n + 1)) / n
     res.update({
         "graph_replay_new_batch_ms": round(new_ms, 4),
         "graph_replay_new_batch_gbps": round(2.0 * mean_pay / (new_ms * 1e-3) / 1e9, 1),
-        "graph_replay_new_batch_host_ms": round(statistics.median(host) * 1e3, 4),
+        # (the fastest: a fill that finds the staging copy of two fills ago still unread waits
+        # for the GPU, which is the back-pressure that keeps the host at most two steps ahead)
+        "graph_replay_new_batch_host_ms": round(min(host) * 1e3, 4),
         "graph_replay_new_batch_vs_frozen_plan": round(
             (new_ms / mean_pay) / (frozen_ms / payloads[0]), 4),
         "graph_replay_new_batch_equals_fresh_plan": same,
         "graph_replay_new_batch_note":
             "one graph captured over a plan slot (%d entries of %d KiB), %d replays, each after "
             "ParseBlock + merge + kvt_plan_slot_fill of another batch (payloads %s MiB per "
-            "launch of all layers), host not waiting for the GPU; vs_frozen_plan = time per "
-            "payload byte against graph_replay_ms_all_layers" %
+            "launch of all layers), the host preparing the next batch while the GPU replays "
+            "(HIP events from behind the first replay to behind the last); vs_frozen_plan = "
+            "time per payload byte against graph_replay_ms_all_layers" %
             (entries, chunk >> 10, n, [round(p / 2**20) for p in payloads])})
     out["per_layer_session"].update(res)
     sess.close()
