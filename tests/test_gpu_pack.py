@@ -1282,15 +1282,23 @@ def test_handle_data_between_two_device_buffers_with_a_long_list(usage, choice):
         kvt_amd.set_copy_cu_usage(0, 1.0)
 
 
-@pytest.mark.parametrize("short,longs,starts", [
-    ([4096, 8192, 16384], [48 << 20, 48 << 20, (48 << 20) + 1000], (0, 4, 16)),   # one range per wavefront
-    ([4096, 4099, 2048], [(20 << 20) + 5, 300 << 10], (0, 1)),                     # two side by side
-    ([256, 512, 1000, 13], [3 << 20, (1 << 20) + 7, 262145, 262144], (4, 0, 16, 1)),    # four
+_SKEWED = {
+    # one range per wavefront
+    "one": ([4096, 8192, 16384], [48 << 20, 48 << 20, (48 << 20) + 1000], (0, 4, 16)),
+    # two side by side
+    "two": ([4096, 4099, 2048], [(20 << 20) + 5, 300 << 10], (0, 1)),
+    # four
+    "four": ([256, 512, 1000, 13], [3 << 20, (1 << 20) + 7, 262145, 262144], (4, 0, 16, 1)),
     # more long ranges than the list of a launch holds (500): the rest stay with their owners
-    ([4096, 8192], [(300 << 10) + 16 * k for k in range(600)], tuple(16 * (k % 3) for k in range(600)))],
-    ids=["one", "two", "four", "more than the list holds"])
-@pytest.mark.parametrize("usage", [1.0, 0.25], ids=["unlimited", "quarter"])
-def test_a_long_list_with_a_few_very_long_ranges(short, longs, starts, usage, request):
+    "more than the list holds": ([4096, 8192], [(300 << 10) + 16 * k for k in range(600)],
+                                 tuple(16 * (k % 3) for k in range(600))),
+}
+
+
+@pytest.mark.parametrize("shape,usage", [("one", 1.0), ("two", 1.0), ("four", 1.0),
+                                         ("more than the list holds", 1.0), ("one", 0.25),
+                                         ("more than the list holds", 0.25)])
+def test_a_long_list_with_a_few_very_long_ranges(shape, usage, request):
     """Merged runs of many blocks among single blocks: 20 000 short ranges and a few of up to
     48 MiB, some of them not 16-byte aligned or not whole vectors long. A persistent
     wavefront's unit of work is a whole range; the ranges above 256 KiB are listed by the
@@ -1299,8 +1307,7 @@ def test_a_long_list_with_a_few_very_long_ranges(short, longs, starts, usage, re
     entry point (which sees the lengths), the device-array launchers (which do not) and the
     entry point that allocates nothing: the oracle's bytes, and the list takes at most three
     times what the same bytes take as even ranges (it took eight times that)."""
-    if usage != 1.0 and len(longs) not in (3, 600):
-        pytest.skip("under a limit: the first and the last shape")
+    short, longs, starts = _SKEWED[shape]
     request.addfinalizer(lambda: kvt_amd.set_copy_cu_usage(0, 1.0))
     kvt_amd.set_copy_cu_usage(0, usage)
     rng = np.random.default_rng(14)
