@@ -462,16 +462,19 @@ int kvt_launch_copy_d2h_bf16_to_fp8(const void* gpu_src_base, void* dst,
  * launcher still bounds that launch further.
  * The first call with usage < 1 for a device allocates 2 MiB of device memory there (blocks
  * of counters from which the persistent workgroups of a launch take their work in order; a
- * launch borrows one until it has run, a launch recorded into a hipGraph keeps one until its
- * plan is destroyed): call it at start-up, not inside a stream capture. A graph that holds
- * limited launches must not run at the same time as a second instantiation of itself. */
+ * launch borrows one until it has run; the launches of a plan that are recorded into one
+ * stream capture on one stream share one, which stays with the plan until it is destroyed;
+ * 256 of the device's 1024 blocks are kept for captures): call it at start-up, not inside a
+ * stream capture. A graph that holds limited launches must not run at the same time as a
+ * second instantiation of itself. */
 int kvt_set_copy_cu_usage(int device, double usage);
 /* The current setting and the workgroup limit it stands for (0 = none); either may be NULL. */
 int kvt_get_copy_cu_usage(int device, double* usage, uint32_t* max_workgroups);
 /* Counters of the launches limited to a CU share that wanted a block of work counters, since
  * the first kvt_set_copy_cu_usage(device, < 1): out[0] eager launches that got one, out[1] eager
  * launches that found none free (they ran with a fixed stride per workgroup instead: slower,
- * same result), out[2] / out[3] the same for launches recorded into a stream capture. */
+ * same result), out[2] blocks handed to stream captures (one per plan, capture and stream), out[3]
+ * launches recorded into a capture that found none. */
 int kvt_get_copy_ticket_stats(int device, uint64_t out[4]);
 
 /* No counterpart in the reference (its copy kernel uses one load flavour). A pack / unpack

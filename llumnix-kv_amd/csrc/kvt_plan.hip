@@ -840,16 +840,47 @@ int kvt_plan_slot_fill_runs(kvt_plan* p, const kvt_run_lists* lists, void* strea
 
 namespace {
 // The ticket block of one pipelined launch (nullptr: none to be had, the launch strides).
+// An eager launch borrows a block until it has run. A launch that is being recorded into a
+// stream capture keeps its block for the life of the plan's table, and shares it with the
+// plan's other launches recorded into the same capture on the same stream: those become a
+// chain of kernel nodes, which never run at the same time, and each leaves the block zeroed
+// (a graph of 80 per-layer launches holds one block, not 80; an engine that captures one graph
+// per batch-size bucket would otherwise run the device's 256 capture blocks dry).
 struct LaunchTickets {
   int device;
   bool capturing;
-  uint32_t* block;
-  LaunchTickets(int dev, bool cap, bool wanted = true)
-      : device(dev), capturing(cap), block(wanted ? ticket_pool().acquire(dev, cap) : nullptr) {}
+  bool shared = false;   // a block this capture already holds: nothing to hand over or back
+  uint32_t* block = nullptr;
+  LaunchTickets(const kvt_plan* p, int dev, bool cap, hipStream_t s, bool wanted = true)
+      : device(dev), capturing(cap) {
+    if (!wanted) return;
+    if (capturing && p->buf) {
+      hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+      unsigned long long id = 0;
+      if (hipStreamGetCaptureInfo(s, &st, &id) == hipSuccess && st == hipStreamCaptureStatusActive) {
+        std::lock_guard<std::mutex> lock(p->buf->mu);
+        for (const TableBuf::CaptureTickets& c : p->buf->capture_tickets)
+          if (c.capture == id && c.stream == s) {
+            block = c.block;
+            shared = true;
+            return;
+          }
+        block = ticket_pool().acquire(dev, true);
+        if (block) {
+          p->buf->capture_tickets.push_back({id, s, block});
+          p->buf->graph_tickets.push_back(block);
+          shared = true;   // the table owns it from here on
+        }
+        return;
+      }
+      (void)hipGetLastError();
+    }
+    block = ticket_pool().acquire(dev, cap);
+  }
   // the launch is on the stream (or in the graph): eager blocks come back when it has run, a
   // graph's block stays with the plan's table
   void launched(const kvt_plan* p, hipStream_t s) {
-    if (!block) return;
+    if (!block || shared) return;
     if (!capturing) {
       ticket_pool().launched(device, block, s);
     } else if (p->buf) {
@@ -860,7 +891,7 @@ struct LaunchTickets {
   }
   // the launch failed: nothing will ever touch the block
   ~LaunchTickets() {
-    if (block) ticket_pool().give_back(device, block);
+    if (block && !shared) ticket_pool().give_back(device, block);
   }
 };
 }  // namespace
@@ -916,7 +947,7 @@ static int run_slot(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32
   const uint32_t wgs = max_wgs == 0 ? full : std::max(8u, std::min(max_wgs & ~7u, full));
   const bool few_pairs = (sl->max_entries << p->sub_shift) * n_layers < (1ull << 31);
   const bool plain = sl->kind == kSlotPlain;
-  LaunchTickets tickets(cache->device, capturing,
+  LaunchTickets tickets(p, cache->device, capturing, s,
                         few_pairs && (plain ? wgs >= full : wgs >= cus && (p->sub_shift >= 2 || wgs >= 2 * cus)));
   const uint8_t* dev = static_cast<const uint8_t*>(p->buf->dev);
   const Chunk* table = p->dev_chunks + (pack ? 0 : sl->max_entries);
@@ -1076,7 +1107,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       // (half the CUs: 4.4 against 5.3 TB/s); a wavefront per entry: the same below two
       // workgroups per CU (one per CU 5.1 / 5.2 with tickets, 5.4 / 5.3 without; two per CU
       // 6.0 / 5.7 with, 5.2 / 5.2 without)
-      LaunchTickets tickets(cache->device, capturing, few_pairs && wgs >= (by_wave ? 2 * cus : cus));
+      LaunchTickets tickets(p, cache->device, capturing, s, few_pairs && wgs >= (by_wave ? 2 * cus : cus));
       const hipError_t e = launch_copy_entries(pack, table, n, p->sub_shift, cache->dev_ptrs,
                                                p->n_tensors, first_layer, n_layers,
                                                static_cast<uint8_t*>(packed), layer_stride, blobs,
@@ -1115,7 +1146,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
       // trips of 8 KiB by a single workgroup per CU are better off without the ticket's barrier
       // (converting gather at an eighth of the device: 4.4 against 5.1 TB/s), and so is a grid
       // of fewer workgroups than CUs
-      LaunchTickets tickets(cache->device, capturing,
+      LaunchTickets tickets(p, cache->device, capturing, s,
                             wgs >= cus && few_pairs && (p->sub_shift >= 2 || wgs >= 2 * cus));
       const hipError_t e =
           strided_by_wave ? launch_strided_entries_by_wave(pack, table, n, p->sub_shift, cache->dev_ptrs,
@@ -1147,7 +1178,7 @@ int kvt::run_plan(bool pack, const kvt_plan* p, const kvt_cache* cache, uint32_t
   const uint32_t grid_cap = max_wgs == 0 ? 0u : std::max(8u, max_wgs & ~7u);
   const uint64_t pairs = ((static_cast<uint64_t>(n) << p->sub_shift) + 7u) / 8u * 8u * n_layers;
   const uint32_t n_cus = device_cu_count(cache->device);
-  LaunchTickets tickets(cache->device, capturing,
+  LaunchTickets tickets(p, cache->device, capturing, s,
                         grid_cap != 0 && pairs > grid_cap && few_pairs && n_cus != 0 && grid_cap >= 2 * n_cus);
   uint8_t* const pk8 = static_cast<uint8_t*>(packed);
   const hipError_t e =

@@ -129,6 +129,14 @@ struct TableBuf {
   std::vector<Use> uses;  // events are kept across recycling (streams repeat)
   bool captured = false;  // read by a kernel recorded into a hipGraph
   std::vector<uint32_t*> graph_tickets;  // ticket blocks of launches recorded into a hipGraph (under mu)
+  // which of them serves which capture: launches recorded into one capture on one stream share
+  // a block (under mu)
+  struct CaptureTickets {
+    unsigned long long capture;
+    hipStream_t stream;
+    uint32_t* block;
+  };
+  std::vector<CaptureTickets> capture_tickets;
 
   // Call after every launch on `stream` that reads `dev`.
   int mark_use(hipStream_t stream) {
@@ -260,6 +268,7 @@ class TablePool {
   static void destroy(TableBuf* b) {
     for (uint32_t* t : b->graph_tickets) ticket_pool().give_back(b->device, t);
     b->graph_tickets.clear();
+    b->capture_tickets.clear();
     if (b->dev) (void)hipFree(b->dev);
     if (b->host) (void)hipHostFree(b->host);
     for (TableBuf::Use& u : b->uses) (void)hipEventDestroy(u.done);

@@ -593,7 +593,7 @@ class PlanSlot(Plan):
 
 def copy_ticket_stats(device):
     """-> (eager launches with a block of work counters, eager launches that found none,
-    captured launches with one, captured launches that found none)"""
+    blocks handed to stream captures, captured launches that found none)"""
     out = (_u64 * 4)()
     check(lib().kvt_get_copy_ticket_stats(device, out))
     return tuple(out)

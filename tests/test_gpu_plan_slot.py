@@ -324,6 +324,7 @@ def test_one_captured_graph_packs_a_new_batch_on_every_replay(usage):
         sess = kvt_amd.Session(send, sc, packed, stride)
         s = checkers.side_stream()
         graph, ungraph = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+        blocks_before = kvt_amd.copy_ticket_stats(0)
         with torch.cuda.stream(s):
             with torch.cuda.graph(graph, stream=s):
                 for l in range(n_layers):
@@ -334,6 +335,10 @@ def test_one_captured_graph_packs_a_new_batch_on_every_replay(usage):
             with torch.cuda.graph(ungraph, stream=s):
                 for l in range(n_layers):
                     recv.unpack(dc, l, 1, packed.data_ptr() + l * stride, stride, s.cuda_stream)
+        # the per-layer launches of a capture are a chain of kernel nodes: they share ONE block of
+        # work counters per plan, capture and stream instead of holding one each for good
+        blocks_after = kvt_amd.copy_ticket_stats(0)
+        assert blocks_after[2] - blocks_before[2] == 2 and blocks_after[3] == blocks_before[3]
     finally:
         kvt_amd.set_copy_cu_usage(0, 1.0)
     # once launches of the session have been captured, only its own slot may be named again
